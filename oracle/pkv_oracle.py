@@ -1,0 +1,272 @@
+"""ctypes/numpy front end of the CPU oracle (``libpkv_oracle.so``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, by ``__graft_entry__.smoke()``
+and by the ``cpu_baseline`` leg of ``bench.py`` as the checker / timed CPU
+baseline.  The product package never imports this module.
+
+All arrays are numpy, key-major: ``codes [n,16] u8``, ``nib [n,16,4] u8``,
+``weight [n,16] f32`` (bf16-representable values).  Helpers at the bottom
+convert to the reference's subspace-major tensors
+(``cache_hub/polar_cache.py:288-307``).
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+import os
+import subprocess
+
+import numpy as np
+
+F32, BF16 = 0, 1
+D, B, M, KW = 128, 16, 8, 256
+TIER_RATIOS = (0.05, 0.15, 0.30, 0.50, 0.75, 1.0)  # polar_cache.py:1221
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libpkv_oracle.so")
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with gcc (idempotent)."""
+    src = os.path.join(_HERE, "pkv_oracle.c")
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-s", "-B", "-C", _HERE, "libpkv_oracle.so"])
+    return _SO
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            build()
+        _lib = C.CDLL(_SO)
+        _lib.pkv_o_bf16_round.restype = C.c_float
+        _lib.pkv_o_bf16_round.argtypes = [C.c_float]
+        _lib.pkv_o_expf.restype = C.c_float
+        _lib.pkv_o_expf.argtypes = [C.c_float]
+        _lib.pkv_o_select_candidates.restype = C.c_int
+        _lib.pkv_o_adaptive_topk.restype = C.c_int64
+    return _lib
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _i64(a):
+    return np.ascontiguousarray(a, dtype=np.int64)
+
+
+def bf16_round(x):
+    """Round fp32 array to bfloat16 (RNE), returned as fp32 (numpy restatement)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    u = x.view(np.uint32).astype(np.uint64)
+    lsb = (u >> 16) & 1
+    r = ((u + 0x7FFF + lsb) & 0xFFFF0000).astype(np.uint32)
+    return r.view(np.float32).reshape(x.shape)
+
+
+def mag_constants():
+    th = np.zeros(7, np.float32)
+    ce = np.zeros(8, np.float32)
+    lib().pkv_o_mag_constants(_p(th), _p(ce))
+    return th, ce
+
+
+def fwht128(x):
+    x = _f32(x).copy()
+    flat = x.reshape(-1, D)
+    for i in range(flat.shape[0]):
+        row = np.ascontiguousarray(flat[i])
+        lib().pkv_o_fwht128(_p(row))
+        flat[i] = row
+    return flat.reshape(x.shape)
+
+
+def encode(keys, signs, dtype):
+    """keys [n,128] -> (codes [n,16] u8, nib [n,16,4] u8, weight [n,16] f32)."""
+    keys = _f32(keys).reshape(-1, D)
+    n = keys.shape[0]
+    codes = np.zeros((n, B), np.uint8)
+    nib = np.zeros((n, B, 4), np.uint8)
+    w = np.zeros((n, B), np.float32)
+    lib().pkv_o_encode(_p(keys), C.c_int64(n), _p(_f32(signs)), C.c_int(dtype), _p(codes), _p(nib), _p(w))
+    return codes, nib, w
+
+
+def count_cluster_keys(codes, counts=None):
+    codes = np.ascontiguousarray(codes, dtype=np.uint8).reshape(-1, B)
+    if counts is None:
+        counts = np.zeros((B, KW), np.int32)
+    assert counts.dtype == np.int32 and counts.flags.c_contiguous
+    lib().pkv_o_count_cluster_keys(_p(codes), C.c_int64(codes.shape[0]), _p(counts))
+    return counts
+
+
+def query_prep(q, signs, dtype):
+    """q [G,128] -> (qhat [128] f32, qnorm float)."""
+    q = _f32(q).reshape(-1, D)
+    qhat = np.zeros(D, np.float32)
+    qn = np.zeros(1, np.float32)
+    lib().pkv_o_query_prep(_p(q), C.c_int(q.shape[0]), _p(_f32(signs)), C.c_int(dtype), _p(qhat), _p(qn))
+    return qhat, float(qn[0])
+
+
+def rank_centroids(qhat, dtype):
+    ids = np.zeros((B, KW), np.int64)
+    lib().pkv_o_rank_centroids(_p(_f32(qhat)), C.c_int(dtype), _p(ids))
+    return ids
+
+
+def tier_counts(kv_len: int, collision_ratio: float, ratios=TIER_RATIOS):
+    """polar_cache.py:1221-1222, evaluated with Python doubles left to right."""
+    return [int(math.ceil(kv_len * collision_ratio * r)) for r in ratios]
+
+
+def tier_lut(sorted_ids, counts, tiers):
+    sorted_ids = _i64(sorted_ids).reshape(-1, KW)
+    counts = np.ascontiguousarray(counts, dtype=np.int32).reshape(-1, KW)
+    n_sub = sorted_ids.shape[0]
+    t = np.asarray(tiers, dtype=np.uint32)
+    lut = np.zeros((n_sub, KW), np.uint8)
+    lib().pkv_o_tier_lut(_p(sorted_ids), _p(counts), C.c_int(n_sub), _p(t), C.c_int(len(t)), _p(lut))
+    return lut
+
+
+def collision_count(codes, lut):
+    """codes [n,n_sub] u8 (key-major), lut [n_sub,256] -> cnt [n] i32."""
+    codes = np.ascontiguousarray(codes, dtype=np.uint8)
+    n, n_sub = codes.shape
+    lut = np.ascontiguousarray(lut, dtype=np.uint8)
+    cnt = np.zeros(n, np.int32)
+    lib().pkv_o_collision_count(_p(codes), C.c_int64(n), C.c_int64(n_sub), C.c_int64(1), C.c_int(n_sub), _p(lut), _p(cnt))
+    return cnt
+
+
+def select_candidates(cnt, k):
+    cnt = np.ascontiguousarray(cnt, dtype=np.int32)
+    out = np.zeros(k, np.int64)
+    theta = lib().pkv_o_select_candidates(_p(cnt), C.c_int64(cnt.shape[0]), C.c_int64(k), _p(out))
+    return out, theta
+
+
+def rerank(cand, nib, weight, qhat, qnorm, centers=None):
+    """nib [n,16,4] u8, weight [n,16] f32 (key-major) -> scores [len(cand)] f32."""
+    cand = _i64(cand)
+    nib = np.ascontiguousarray(nib, dtype=np.uint8)
+    weight = _f32(weight)
+    if centers is None:
+        centers = mag_constants()[1]
+    scores = np.zeros(cand.shape[0], np.float32)
+    lib().pkv_o_rerank(_p(cand), C.c_int64(cand.shape[0]), _p(nib), C.c_int64(64), C.c_int64(4), _p(weight),
+                       C.c_int64(16), C.c_int64(1), _p(_f32(qhat)), C.c_float(qnorm), _p(_f32(centers)), _p(scores))
+    return scores
+
+
+def topk_f32(scores, ids, k):
+    scores = _f32(scores)
+    n = scores.shape[0]
+    ids_c = _i64(ids) if ids is not None else None
+    out_ids = np.zeros(k, np.int64)
+    out_pos = np.zeros(k, np.int64)
+    lib().pkv_o_topk_f32(_p(scores), _p(ids_c), C.c_int64(n), C.c_int64(k), _p(out_ids), _p(out_pos))
+    return out_ids, out_pos
+
+
+def gather_rows(src, idx):
+    src = np.ascontiguousarray(src)
+    idx = _i64(idx)
+    row_bytes = src.strides[0]
+    dst = np.zeros((idx.shape[0],) + src.shape[1:], src.dtype)
+    lib().pkv_o_gather_rows(_p(src), _p(idx), C.c_int64(idx.shape[0]), C.c_int64(row_bytes), _p(dst))
+    return dst
+
+
+def expf(x):
+    x = _f32(x)
+    out = np.empty_like(x)
+    f = lib().pkv_o_expf
+    flat_in, flat_out = x.reshape(-1), out.reshape(-1)
+    for i in range(flat_in.shape[0]):
+        flat_out[i] = f(C.c_float(float(flat_in[i])))
+    return out
+
+
+def adaptive_topk(sl_logits, sl_vnorm, cand_logits, cand_vnorm, cand_ids, threshold, k_out):
+    sl_logits, sl_vnorm = _f32(sl_logits), _f32(sl_vnorm)
+    cand_logits, cand_vnorm, cand_ids = _f32(cand_logits), _f32(cand_vnorm), _i64(cand_ids)
+    out = np.zeros(k_out, np.int64)
+    k = lib().pkv_o_adaptive_topk(_p(sl_logits), _p(sl_vnorm), C.c_int64(sl_logits.shape[0]), _p(cand_logits),
+                                  _p(cand_vnorm), _p(cand_ids), C.c_int64(cand_logits.shape[0]),
+                                  C.c_float(threshold), C.c_int64(k_out), _p(out))
+    return int(k), out
+
+
+def retrieve_row(q, signs, dtype, codes, nib, weight, cluster_counts, tiers, n_cand, k):
+    """Whole retrieval (query prep .. final top-k) for one (batch, kv-head) row."""
+    q = _f32(q).reshape(-1, D)
+    codes = np.ascontiguousarray(codes, dtype=np.uint8)
+    nib = np.ascontiguousarray(nib, dtype=np.uint8)
+    weight = _f32(weight)
+    cc = np.ascontiguousarray(cluster_counts, dtype=np.int32)
+    t = np.asarray(tiers, dtype=np.uint32)
+    kk = min(k, n_cand)
+    out = np.zeros(kk, np.int64)
+    lib().pkv_o_retrieve_row(_p(q), C.c_int(q.shape[0]), _p(_f32(signs)), C.c_int(dtype), _p(codes), _p(nib),
+                             _p(weight), _p(cc), C.c_int64(codes.shape[0]), _p(t), C.c_int(len(t)),
+                             C.c_int64(n_cand), C.c_int64(k), _p(out))
+    return out
+
+
+# ------------------------------------------------------------------ fixtures
+
+
+def srht_signs(seed: int = 42):
+    """SRHT diagonal D in {+-1}^128.  The reference draws it from the CUDA
+    generator (polar_cache.py:59-63), which a CPU cannot reproduce; the build
+    fixes it as this CPU-generator draw."""
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randint(0, 2, (D,), generator=g).to(torch.float32) * 2 - 1).numpy()
+
+
+def synth_keys(n, seed, outliers=(7, 31, 64, 101), bf16=False, drift_deg_per_1k=0.0):
+    """Synthetic keys ~N(0,1) with 4 fixed outlier channels x10; optional slow
+    rotation of the key mean in the (0,1) plane."""
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    k = torch.randn(n, D, generator=g, dtype=torch.float32)
+    k[:, list(outliers)] *= 10.0
+    if drift_deg_per_1k:
+        ang = torch.arange(n, dtype=torch.float32) * (drift_deg_per_1k / 1000.0) * (math.pi / 180.0)
+        k[:, 0] += 3.0 * torch.cos(ang)
+        k[:, 1] += 3.0 * torch.sin(ang)
+    k = k.numpy()
+    return bf16_round(k) if bf16 else k
+
+
+def synth_queries(keys, G, seed, bf16=False):
+    """queries = key mean + N(0, 0.5), one per q-head of the group."""
+    import torch
+
+    g = torch.Generator().manual_seed(seed + 1000003)
+    q = torch.from_numpy(keys.mean(axis=0, dtype=np.float64).astype(np.float32)).unsqueeze(0) + 0.5 * torch.randn(
+        G, D, generator=g, dtype=torch.float32)
+    q = q.numpy()
+    return bf16_round(q) if bf16 else q
+
+
+def to_reference_layout(codes, nib, weight):
+    """key-major -> reference tensors: codebook [16,n], key_4bit [16,n,4],
+    block_weight [16,n] (per (b,h) row)."""
+    return (np.ascontiguousarray(codes.T), np.ascontiguousarray(nib.transpose(1, 0, 2)),
+            np.ascontiguousarray(weight.T))

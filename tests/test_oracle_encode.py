@@ -1,0 +1,153 @@
+"""Pins the oracle's append path (encode, cluster counts, query prep) against
+closed forms and library routines.  CPU only."""
+import json
+import os
+
+import numpy as np
+import pytest
+import scipy.linalg
+import torch
+
+import refforms
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def test_bf16_round_matches_torch(oracle):
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(100000, generator=g) * torch.exp(torch.randn(100000, generator=g) * 8)
+    x = torch.cat([x, torch.tensor([0.0, -0.0, 1.0, 65504.0, 3.3895e38, 1e-40, float("inf")])])
+    ref = x.to(torch.bfloat16).float().numpy()
+    assert np.array_equal(oracle.bf16_round(x.numpy()).view(np.uint32), ref.view(np.uint32))
+    for v in x[:2000].tolist():
+        assert np.float32(oracle.lib().pkv_o_bf16_round(v)).view(np.uint32) == np.float32(
+            torch.tensor(v).to(torch.bfloat16).float().item()).view(np.uint32)
+
+
+def test_mag_constants_match_torch_and_reference_data(oracle):
+    th, ce = oracle.mag_constants()
+    assert np.array_equal(th, torch.tensor(refforms.MAG_THRESHOLDS, dtype=torch.bfloat16).float().numpy())
+    assert np.array_equal(ce, torch.tensor(refforms.MAG_CENTERS, dtype=torch.bfloat16).float().numpy())
+    # known bf16 values
+    assert th.tolist() == [0.08447265625, 0.169921875, 0.2578125, 0.349609375, 0.44921875, 0.55859375, 0.69140625]
+    assert ce.tolist() == [0.0419921875, 0.126953125, 0.212890625, 0.302734375, 0.396484375, 0.5, 0.6171875, 0.76171875]
+    # the literals agree with the reference's Lloyd-Max data file to Monte-Carlo noise
+    data = json.load(open(os.path.join(GOLD, "magnitude_levels_m8_4bit.json")))
+    np.testing.assert_allclose(data["thresholds"], refforms.MAG_THRESHOLDS, atol=5e-4)
+    np.testing.assert_allclose(data["centers"], refforms.MAG_CENTERS, atol=5e-4)
+
+
+def test_sign_codebook_is_bit_enumeration():
+    cb = json.load(open(os.path.join(GOLD, "codebook_d128_m8_Kr1_Kw256_rabitq_sign.json")))
+    assert cb["config"]["d"] == 128 and cb["config"]["m"] == 8 and cb["config"]["K_omega"] == 256
+    s = np.array(cb["angular_signs"])
+    for c in range(256):
+        for j in range(8):
+            assert (s[c, j] > 0) == bool((c >> j) & 1)
+
+
+def test_fwht_matches_hadamard_matrix(oracle):
+    H = scipy.linalg.hadamard(128).astype(np.float64)
+    g = np.random.default_rng(0)
+    xi = g.integers(-50, 50, size=(64, 128)).astype(np.float32)  # exact in fp32
+    assert np.array_equal(oracle.fwht128(xi), (xi.astype(np.float64) @ H).astype(np.float32))
+    x = g.standard_normal((64, 128)).astype(np.float32)
+    y = oracle.fwht128(x)
+    err = np.abs(y - x.astype(np.float64) @ H)
+    assert (err <= 2e-6 * np.abs(x).sum(axis=1, keepdims=True)).all()
+    np.testing.assert_allclose(oracle.fwht128(y) / 128.0, x, atol=1e-5)  # involution
+    e = np.zeros((1, 128), np.float32)
+    e[0, 5] = 1.0
+    assert np.array_equal(oracle.fwht128(e)[0], H[5].astype(np.float32))  # row of H, natural order
+
+
+@pytest.mark.parametrize("dtype_name", ["f32", "bf16"])
+def test_encode_matches_library_restatement(oracle, signs, dtype_name):
+    bf = dtype_name == "bf16"
+    keys = oracle.synth_keys(6000, seed=3, bf16=bf)
+    codes, nib, w = oracle.encode(keys, signs, oracle.BF16 if bf else oracle.F32)
+    tk = torch.from_numpy(keys)
+    if bf:
+        tk = tk.to(torch.bfloat16)
+    rc, rp, rw = refforms.batch_encode(tk, torch.from_numpy(signs))
+    rc, rp, rw = rc.numpy(), rp.numpy(), rw.float().numpy()
+    # codes and nibbles hinge on fp32 round-off only where a rotated coordinate
+    # or a direction sits on a boundary: near-total agreement is the pin
+    assert (codes == rc).mean() > 0.9995
+    assert (nib == rp).mean() > 0.995
+    agree = (nib == rp).all(axis=2)
+    rel = np.abs(w - rw) / np.maximum(np.abs(rw), 1e-6)
+    assert np.median(rel) == 0.0 or np.median(rel) < 1e-2
+    assert rel[agree].max() <= 2 ** -7  # at most one bf16 ulp where the codes agree
+    # invariants
+    assert w.min() > 0 and np.array_equal(oracle.bf16_round(w), w)
+    assert ((nib & 0x07) <= 7).all()
+
+
+def test_encode_exact_closed_form_cases(oracle):
+    """Inputs for which every fp step is exact, so the codes have a closed form."""
+    ones = np.ones(128, np.float32)
+    # key = c * e_0 with all-ones signs: rotated vector is constant 1/sqrt(128) > 0
+    k = np.zeros((1, 128), np.float32)
+    k[0, 0] = 4.0
+    codes, nib, w = oracle.encode(k, ones, oracle.F32)
+    assert (codes == 255).all()
+    # direction of each block is 1/sqrt(8)=0.3536 in every dim -> bucket 4 (0.3496 < u <= 0.4492), sign bit set
+    assert (nib == ((8 | 4) << 4 | (8 | 4))).all()
+    th, ce = oracle.mag_constants()
+    r = np.sqrt(8.0 / 128.0)
+    alpha = 8 * ce[4] * (1 / np.sqrt(8.0))
+    np.testing.assert_allclose(w, np.full_like(w, oracle.bf16_round(np.float32([r / alpha * 4.0]))[0]), rtol=2 ** -7)
+    # flipping the SRHT sign of dim 0 negates everything: all sign bits clear
+    s = ones.copy()
+    s[0] = -1
+    codes2, nib2, _ = oracle.encode(k, s, oracle.F32)
+    assert (codes2 == 0).all() and (nib2 == (4 << 4 | 4)).all()
+    # zero key: no NaNs, codes 255 (0 >= 0), magnitude bucket 0, weight 0
+    codes3, nib3, w3 = oracle.encode(np.zeros((1, 128), np.float32), ones, oracle.BF16)
+    assert (codes3 == 255).all() and (nib3 == 0x88).all() and (w3 == 0).all()
+
+
+def test_encode_brute_force_nearest_sign_centroid(oracle, signs):
+    """Sign bit-pack == argmax over the 256 sign centroids of <V_c, y_b>."""
+    keys = oracle.synth_keys(300, seed=11)
+    codes, _, _ = oracle.encode(keys, signs, oracle.F32)
+    V = np.array([[1.0 if (c >> j) & 1 else -1.0 for j in range(8)] for c in range(256)])
+    y = (keys / np.linalg.norm(keys, axis=1, keepdims=True) * signs) @ scipy.linalg.hadamard(128) / np.sqrt(128)
+    best = (y.reshape(-1, 16, 8) @ V.T).argmax(axis=-1)
+    assert (best == codes).mean() > 0.9999
+
+
+def test_nibble_pack_roundtrip_exhaustive():
+    allb = torch.arange(256, dtype=torch.uint8).view(-1, 1).repeat(1, 4)
+    s, t = refforms.unpack_4bit(allb)
+    assert torch.equal(refforms.pack_4bit(s > 0, t.to(torch.uint8)), allb)
+
+
+def test_count_cluster_keys_is_bincount(oracle):
+    g = np.random.default_rng(5)
+    codes = g.integers(0, 256, size=(5000, 16), dtype=np.uint8)
+    counts = oracle.count_cluster_keys(codes)
+    for b in range(16):
+        assert np.array_equal(counts[b], np.bincount(codes[:, b], minlength=256))
+    more = oracle.count_cluster_keys(codes[:100], counts.copy())  # accumulates (polar_cache.py:774-775)
+    assert more.sum() == counts.sum() + 1600
+
+
+@pytest.mark.parametrize("dtype_name", ["f32", "bf16"])
+def test_query_prep_matches_library_restatement(oracle, signs, dtype_name):
+    bf = dtype_name == "bf16"
+    keys = oracle.synth_keys(512, seed=7, bf16=bf)
+    bad = 0
+    for s in range(20):
+        q = oracle.synth_queries(keys, 4, seed=s, bf16=bf)
+        qhat, qn = oracle.query_prep(q, signs, oracle.BF16 if bf else oracle.F32)
+        tq = torch.from_numpy(q).to(torch.bfloat16 if bf else torch.float32)
+        rh, rn = refforms.encode_query(tq, torch.from_numpy(signs))
+        tol = 2 ** -7 if bf else 1e-5
+        assert abs(qn - float(rn)) <= tol * abs(float(rn))
+        np.testing.assert_allclose(qhat, rh.float().numpy(), rtol=0, atol=tol)
+        bad += int((qhat != rh.float().numpy()).sum())
+        assert abs(np.linalg.norm(qhat.astype(np.float64)) - 1.0) < (2e-2 if bf else 1e-5)  # rotation keeps the unit norm
+    if bf:  # bf16 rounding hides the summation order except at rounding boundaries
+        assert bad <= 20 * 128 * 0.02
