@@ -1,0 +1,292 @@
+/*
+ * pariskv_hip.h -- C ABI of libpariskv_hip.so: ParisKV's per-decode-step KV
+ * retrieval path as hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * Conventions
+ *   - Every function returns 0 on success or a negative PKV_E* code;
+ *     pkv_last_error() gives the message of the calling thread's last failure
+ *     (the Python shims raise RuntimeError with it, like the reference's
+ *     TORCH_CHECKs).
+ *   - The caller owns every buffer, workspaces and outputs included; nothing
+ *     is allocated or freed behind the caller's back (pkv_host_alloc_mapped /
+ *     pkv_host_free excepted, which exist to allocate).
+ *   - All device work is enqueued on `stream` (a hipStream_t passed as void*);
+ *     no call synchronises, none touches the default stream on its own.
+ *   - Strides are in ELEMENTS of the pointed-to type unless a name says bytes.
+ *   - "row" means one (batch, kv-head) pair; R = bs * n_kv_heads.
+ *   - Geometry is the reference's default codebook: head_dim 128 = 16 subspaces
+ *     x 8 dims, 256 sign centroids per subspace
+ *     (turboquant/codebooks/codebook_d128_m8_Kr1_Kw256_rabitq_sign.json).
+ *
+ * Each entry point cites the reference interface it replaces
+ * (paths relative to the ParisKV checkout).
+ */
+#ifndef PARISKV_HIP_H
+#define PARISKV_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+#pragma GCC visibility push(default)
+
+#define PKV_OK 0
+#define PKV_EINVAL (-22)   /* bad argument (shape, stride, alignment, range) */
+#define PKV_ENOMEM (-12)   /* workspace too small / host allocation failed */
+#define PKV_EHIP (-5)      /* a HIP runtime call failed */
+
+#define PKV_DTYPE_F32 0
+#define PKV_DTYPE_BF16 1
+
+#define PKV_HEAD_DIM 128
+#define PKV_SUBSPACES 16
+#define PKV_SUBDIM 8
+#define PKV_CLUSTERS 256
+#define PKV_MAX_TIERS 8
+
+int pkv_version(void);
+const char *pkv_last_error(void);
+
+/* ------------------------------------------------------------------ append */
+
+/* Replaces polar_cache.batch_encode + _count_cluster_keys
+ * (cache_hub/polar_cache.py:924-978, 980-996; call sites :484-494, :768-775).
+ * keys: [bs][h][n_keys][128] of `dtype` addressed with the given strides
+ * (last dim contiguous).  signs: device float[128] of +-1 (SRHT diagonal).
+ * For key i of row (b,h), subspace s:
+ *   codes[b*cs_b + h*cs_h + i*cs_key + s*cs_sub]            (u8 sign code)
+ *   nib  [b*ns_b + h*ns_h + i*ns_key + s*ns_sub + 0..3]     (u8 packed 4-bit)
+ *   weight[b*ws_b + h*ws_h + i*ws_key + s*ws_sub]           (bf16 bits)
+ * so both the reference's subspace-major tensors and key-major storage are
+ * expressible.  cluster_counts (int32 [bs][h][16][256], strides cc_b, cc_h) is
+ * incremented (+=, polar_cache.py:775) when non-NULL.  nib/weight may be NULL
+ * (return_rabitq=False). */
+int pkv_encode_append(const void *keys, int dtype, int bs, int n_kv_heads, int64_t n_keys,
+                      int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_key,
+                      const float *signs,
+                      uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t cs_key, int64_t cs_sub,
+                      uint8_t *nib, int64_t ns_b, int64_t ns_h, int64_t ns_key, int64_t ns_sub,
+                      uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key, int64_t ws_sub,
+                      int32_t *cluster_counts, int64_t cc_b, int64_t cc_h,
+                      void *stream);
+
+/* polar_cache._count_cluster_keys on its own (cache_hub/polar_cache.py:980-996):
+ * cluster_counts[b][h][s][code] += 1 for every key and subspace. */
+int pkv_count_cluster_keys(const uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t cs_key, int64_t cs_sub,
+                           int bs, int n_kv_heads, int64_t n_keys,
+                           int32_t *cluster_counts, int64_t cc_b, int64_t cc_h, void *stream);
+
+/* ------------------------------------------------------------- query side */
+
+/* Replaces the query half of polar_cache.compute / _encode_query_blocks and the
+ * centroid ranking of get_cache_cnt_fused, plus convert_to_bits
+ * (cache_hub/polar_cache.py:1027-1031, 905-922, 1216-1222;
+ *  cache_hub/collision_fused/collision.cu:71-151).
+ * q: [bs][n_kv_heads*group][128] contiguous of `dtype` (the [bs,1,Hq,D] decode
+ * query).  cluster_counts as above.  tier_counts: HOST array of n_tiers (1..8)
+ * cumulative key thresholds.  Outputs (device): qhat float [R][128],
+ * qnorm float [R], lut u8 [R][16][256] (votes a key gets per subspace for each
+ * centroid), sorted_ids int64 [R][16][256] or NULL. */
+int pkv_query_prep_lut(const void *q, int dtype, int bs, int n_kv_heads, int group,
+                       const float *signs,
+                       const int32_t *cluster_counts, int64_t cc_b, int64_t cc_h,
+                       const uint32_t *tier_counts, int n_tiers,
+                       float *qhat, float *qnorm, uint8_t *lut, int64_t *sorted_ids,
+                       void *stream);
+
+/* Replaces update_cache_cnt (cache_hub/collision_fused/collision.cu:250-411;
+ * python: collison_interface.py:60-86 update_cache_cnt_cuda_interface).
+ * sorted_ids int64 [bs][h][16][256] (strides si_b, si_h, si_sub; last dim
+ * contiguous), cluster_counts likewise, codes u8 addressed as in
+ * pkv_encode_append, tier_counts HOST array (n_tiers 1 or 6 in the reference;
+ * 1..8 here).  lut_ws: device workspace of R*16*256 bytes.
+ * cnt: int32 [bs][h][n_keys] contiguous. */
+int pkv_update_cache_cnt(const int64_t *sorted_ids, int64_t si_b, int64_t si_h, int64_t si_sub,
+                         const int32_t *cluster_counts, int64_t cc_b, int64_t cc_h, int64_t cc_sub,
+                         const uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t cs_key, int64_t cs_sub,
+                         int bs, int n_kv_heads, int64_t n_keys,
+                         const uint32_t *tier_counts, int n_tiers,
+                         uint8_t *lut_ws, int32_t *cnt, void *stream);
+
+/* Legacy single-tier form: cache_hub/collision/collision.cu:146-276,
+ * collision.py:87-98 (update_cache_cnt_cuda).  sorted_ids int32
+ * [bs][h][16][256] contiguous, topk_cluster_cnt int32 [bs][h][16], codebook
+ * int32 [bs][h][16][n_keys] contiguous.  A key scores 1 per subspace whose
+ * code is among the first topk_cluster_cnt ranked clusters. */
+int pkv_update_cache_cnt_legacy(const int32_t *sorted_ids, const int32_t *topk_cluster_cnt,
+                                const int32_t *codebook, int bs, int n_kv_heads, int64_t n_keys,
+                                uint8_t *lut_ws, int32_t *cnt, void *stream);
+
+/* The scan stage of the fused pipeline: votes per key from a ready LUT
+ * (the per-key loop of cache_hub/collision_fused/collision.cu:204-228).
+ * cnt_u8 [R][n_keys] and/or cnt_i32 [R][n_keys] (either may be NULL, not both);
+ * chunk_hist uint16 [R][n_chunks][128] (NULL to skip) receives the histogram of
+ * each `chunk_keys`-key chunk, n_chunks = ceil(n_keys / chunk_keys);
+ * chunk_keys must be a multiple of 2048 and at most 32768. */
+int pkv_collision_scan(const uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t cs_key, int64_t cs_sub,
+                       int bs, int n_kv_heads, int64_t n_keys, const uint8_t *lut,
+                       uint8_t *cnt_u8, int32_t *cnt_i32, uint16_t *chunk_hist, int chunk_keys,
+                       void *stream);
+
+/* pkv_collision_scan (u8 counts, row stride cnt_u8_stride) as ONE launch whose
+ * own begin/end timestamps are returned in *kernel_us: the call blocks until
+ * the kernel has finished.  Measurement aid for the benchmark's roofline line;
+ * no counterpart in the reference. */
+int pkv_collision_scan_timed(const uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t cs_key, int64_t cs_sub,
+                             int bs, int n_kv_heads, int64_t n_keys, const uint8_t *lut,
+                             uint8_t *cnt_u8, int64_t cnt_u8_stride, uint16_t *chunk_hist, int chunk_keys,
+                             float *kernel_us, void *stream);
+
+/* ------------------------------------------------------------- selections */
+
+/* Replaces bucket_topk / bucket_topk_3d and the integer use of radix_topk_3d
+ * (cache_hub/topk/radix_topk.cu:39-120, 258-319; hot call
+ * cache_hub/polar_cache.py:1241).  x: int32 [rows][len] (row stride x_stride),
+ * values clamped to [0,127].  out: int64 [rows][k]: every index whose value is
+ * above the k-th largest value (ascending index), then the smallest indices at
+ * that value (ascending).  len == k gives 0..len-1.  ws: device workspace of
+ * pkv_bucket_topk_ws_bytes(rows, len) bytes. */
+size_t pkv_bucket_topk_ws_bytes(int rows, int64_t len);
+int pkv_bucket_topk(const int32_t *x, int64_t x_stride, int rows, int64_t len, int64_t k,
+                    int64_t *out, void *ws, size_t ws_bytes, void *stream);
+
+/* Replaces radix_topk / radix_topk_3d on floats (radix_topk.cu:161-239,
+ * 323-382) and torch.topk + gather at cache_hub/polar_cache.py:1300-1302.
+ * Exact: the k largest of x[rows][len] in descending order, ties by smaller
+ * ids[row][i] (by smaller position when ids == NULL).  out_ids int64 [rows][k]
+ * = ids[..] (or positions); out_vals float [rows][k] or NULL.
+ * ws: pkv_topk_f32_ws_bytes(rows, len, k) bytes. */
+size_t pkv_topk_f32_ws_bytes(int rows, int64_t len, int64_t k);
+int pkv_topk_f32(const float *x, int64_t x_stride, const int64_t *ids, int64_t ids_stride,
+                 int rows, int64_t len, int64_t k, int64_t *out_ids, float *out_vals,
+                 void *ws, size_t ws_bytes, void *stream);
+
+/* Replaces partial_rerank (cache_hub/rerank/rerank.cu:141-219; python
+ * rerank.py:214-263 partial_rerank_cuda).  cand int64 [bs][h][n_cand]
+ * contiguous; nib / weight addressed as in pkv_encode_append with n_keys keys
+ * per row; qhat float [R][128], qnorm float [R], centers float[8] (device).
+ * scores float [R][n_cand].  v4b (bf16 bits [R][16][n_cand][8], the unpacked
+ * values the reference also returns) is written when non-NULL.
+ * Candidate indices outside [0,n_keys) score -inf instead of being read. */
+int pkv_rerank4(const int64_t *cand, int bs, int n_kv_heads, int64_t n_cand, int64_t n_keys,
+                const uint8_t *nib, int64_t ns_b, int64_t ns_h, int64_t ns_key, int64_t ns_sub,
+                const uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key, int64_t ws_sub,
+                const float *qhat, const float *qnorm, const float *centers,
+                float *scores, uint16_t *v4b, void *stream);
+
+/* ----------------------------------------------------------------- gathers */
+
+/* Replaces h2d_gather_kv (cache_hub/gather_trans/trans_h2d.cu:79-121; python
+ * trans_h2d.py:65-105).  src_k/src_v: pinned, device-mapped HOST memory
+ * [bs][h][src_len][row_bytes/2 bf16]; idx int64 [bs][h][k] on the device;
+ * dst_k/dst_v device [bs][h][dst_len][...].  Rows are row_bytes bytes
+ * (multiple of 16; 256 for head_dim 128 bf16).  Out-of-range indices produce
+ * zero rows.  idx_offset is added to every index before addressing src
+ * (0 for the offload layout; retrieval_start for pkv_gather_hbm callers,
+ * cache_hub/polar_cache.py:1090). */
+int pkv_gather_uva(const void *src_k, const void *src_v, int64_t src_len,
+                   const int64_t *idx, int64_t k, int64_t idx_offset,
+                   void *dst_k, void *dst_v, int64_t dst_len, int64_t dst_row0,
+                   int bs, int n_kv_heads, int row_bytes, void *stream);
+
+/* Same contract with src in device memory: the no-offload branch
+ * cache_hub/polar_cache.py:1089-1095 (torch.gather over the GPU KV). */
+int pkv_gather_hbm(const void *src_k, const void *src_v, int64_t src_len,
+                   const int64_t *idx, int64_t k, int64_t idx_offset,
+                   void *dst_k, void *dst_v, int64_t dst_len, int64_t dst_row0,
+                   int bs, int n_kv_heads, int row_bytes, void *stream);
+
+/* Ragged form used by the adaptive-k cache variant (kernel source absent from
+ * the reference; contract from the call site
+ * cache_hub/polar_cache_adaptivek_varlen.py:1634-1644, layout :1573-1586).
+ * For virtual head v = b*h_count + h and slot s < cu_topk[v+1]-cu_topk[v]:
+ *   dst row  = cu_k[v] + sink_local_end + s
+ *   src row  = idx_packed[cu_topk[v] + s] of (b,h)
+ * dst_k/dst_v: [total_k][row_bytes]; cu_* are int32 device arrays [V+1];
+ * max_k bounds the per-head slot count (grid bound). */
+int pkv_gather_uva_packed(const void *src_k, const void *src_v, int64_t src_len,
+                          const int64_t *idx_packed, const int32_t *cu_topk, const int32_t *cu_k,
+                          int64_t sink_local_end, int64_t max_k,
+                          void *dst_k, void *dst_v, int64_t total_k,
+                          int bs, int n_kv_heads, int row_bytes, void *stream);
+
+/* Replaces gather_kv_out_cpu (cache_hub/gather/gather_cpu.cpp:116-170): host
+ * gather [B][H][N][D] -> [B][H][K][D], element strides given, `elem_bytes` per
+ * element.  Returns PKV_EINVAL if an index is out of range (bounds are checked
+ * up front, like the reference's release build). */
+int pkv_gather_cpu(const void *src, const int64_t *src_strides4, const int64_t *index,
+                   void *out, const int64_t *out_strides4,
+                   int64_t B, int64_t H, int64_t N, int64_t D, int64_t K, int elem_bytes,
+                   int n_threads);
+
+/* Streaming device copy of `bytes` (multiple of 16) bytes: the known-size kernel
+ * against which the HBM traffic counters are calibrated.  No counterpart in the
+ * reference. */
+int pkv_copy_bytes(const void *src, void *dst, size_t bytes, void *stream);
+
+/* Pinned host memory that kernels can read in place (hipHostMalloc, mapped).
+ * The reference relies on torch's pin_memory=True for the same purpose
+ * (cache_hub/polar_cache.py:226-237). */
+int pkv_host_alloc_mapped(size_t bytes, void **host_ptr);
+int pkv_host_free(void *host_ptr);
+/* Device-visible address of a pinned host pointer (PKV_EINVAL if not pinned). */
+int pkv_host_device_pointer(const void *host_ptr, void **dev_ptr);
+
+/* ------------------------------------------------------- fused decode step */
+
+/* One layer's retrieval for one decode step, key-major storage:
+ * query prep + LUT -> collision scan -> candidate select -> 4-bit rerank ->
+ * exact top-k (-> optional gather).  Equivalent to
+ * polar_cache.collision_based_topk_batch (cache_hub/polar_cache.py:1126-1162)
+ * followed by the gather at :1075-1095.
+ *   codes  u8   [R][cap][16]   (row stride = cap*16),   keys [key0, key0+n_keys)
+ *   nib    u8   [R][cap][64]
+ *   weight bf16 [R][cap][16]
+ * out_ids int64 [R][k] (indices relative to key0, descending score).
+ * If src_k != NULL the selected rows are gathered into dst_k/dst_v
+ * (gather_from_host selects pkv_gather_uva vs pkv_gather_hbm semantics).
+ * ws: pkv_retrieve_ws_bytes(R, n_keys, n_cand, k) bytes of device memory. */
+typedef struct pkv_retrieve_args {
+  const void *q;            /* [bs][n_kv_heads*group][128] */
+  int dtype;                /* PKV_DTYPE_* of q */
+  int bs, n_kv_heads, group;
+  const float *signs;       /* device float[128] */
+  const float *centers;     /* device float[8] */
+  const int32_t *cluster_counts; /* [R][16][256] contiguous */
+  const uint8_t *codes;
+  const uint8_t *nib;
+  const uint16_t *weight;
+  int64_t cap;              /* keys per row in the three arrays above */
+  int64_t key0;             /* first key of the retrieval zone */
+  int64_t n_keys;           /* valid retrieval length N */
+  uint32_t tier_counts[PKV_MAX_TIERS];
+  int n_tiers;
+  int64_t n_cand;           /* C */
+  int64_t k;                /* K (<= C) */
+  int64_t *out_ids;         /* [R][k] */
+  float *out_scores;        /* [R][k] or NULL */
+  /* optional gather */
+  const void *src_k, *src_v;
+  int gather_from_host;
+  int64_t src_len, idx_offset;
+  void *dst_k, *dst_v;
+  int64_t dst_len, dst_row0;
+  int row_bytes;
+} pkv_retrieve_args;
+
+size_t pkv_retrieve_ws_bytes(int rows, int64_t n_keys, int64_t n_cand, int64_t k);
+int pkv_retrieve(const pkv_retrieve_args *args, void *ws, size_t ws_bytes, void *stream);
+
+/* Names and device pointers of the intermediates inside a pkv_retrieve
+ * workspace (for tests and profiling): qhat, qnorm, lut, cnt_u8, chunk_hist,
+ * cand, scores.  Returns PKV_EINVAL for an unknown name. */
+int pkv_retrieve_ws_view(void *ws, int rows, int64_t n_keys, int64_t n_cand, int64_t k,
+                         const char *name, void **ptr, size_t *bytes);
+
+#pragma GCC visibility pop
+#ifdef __cplusplus
+}
+#endif
+#endif

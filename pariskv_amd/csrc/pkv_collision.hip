@@ -1,0 +1,235 @@
+// Collision vote: cnt[key] = sum over the 16 subspaces of lut[subspace][code].
+//
+// Reference: cache_hub/collision_fused/collision.cu:163-229
+// (update_cache_cnt_kernel: 16 byte loads at stride kv_len and 6 LDS bit tests
+// per subspace).  Here the six tier bitsets are one 4 KB byte table per row held
+// in LDS, a key's 16 codes are one 128-bit load (key-major storage), and the
+// same pass also builds the per-chunk histogram that the candidate select needs,
+// so the counts are never re-read to find the threshold.
+//
+// HBM-bound: 16 B read + 1 B written per key.
+#include "pkv_common.h"
+
+namespace {
+
+constexpr int kScanThreads = 256;
+constexpr int kHistCopies = 16;  // replicated LDS histogram: copy = lane & 15
+
+__device__ __forceinline__ int lut_sum16(const uint8_t *__restrict__ l8, pkv_u32x4 v) {
+  int c = 0;
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t code = (w[d] >> (8 * k)) & 0xffu;
+      c += l8[(4 * d + k) * 256 + code];
+    }
+  }
+  return c;
+}
+
+__device__ __forceinline__ void load_lut(uint32_t *s_lut, const uint8_t *__restrict__ lut, int row) {
+  const uint32_t *g = (const uint32_t *)(lut + (int64_t)row * 4096);
+#pragma unroll
+  for (int i = 0; i < 1024 / kScanThreads; ++i) s_lut[threadIdx.x + i * kScanThreads] = g[threadIdx.x + i * kScanThreads];
+}
+
+// Key-major codes ([key][16] bytes, 16-byte aligned).  grid (n_chunks, R).
+__global__ __launch_bounds__(kScanThreads) void pkv_scan_keymajor_kernel(
+    const uint8_t *__restrict__ codes, int64_t cs_b, int64_t cs_h, int n_kv_heads, int64_t n_keys,
+    const uint8_t *__restrict__ lut, uint8_t *__restrict__ cnt_u8, int64_t cnt_u8_stride,
+    int32_t *__restrict__ cnt_i32, uint16_t *__restrict__ chunk_hist, int chunk_keys) {
+  const int row = blockIdx.y;
+  const int chunk = blockIdx.x;
+  const int b = row / n_kv_heads, h = row % n_kv_heads;
+  const int tid = threadIdx.x;
+
+  __shared__ uint32_t s_lut[1024];
+  __shared__ uint32_t s_hist[128 * kHistCopies];
+  load_lut(s_lut, lut, row);
+  for (int i = tid; i < 128 * kHistCopies; i += kScanThreads) s_hist[i] = 0;
+  __syncthreads();
+  const uint8_t *l8 = (const uint8_t *)s_lut;
+  const int copy = tid & (kHistCopies - 1);
+
+  const pkv_u32x4 *base = (const pkv_u32x4 *)(codes + (int64_t)b * cs_b + (int64_t)h * cs_h);
+  const int64_t k0 = (int64_t)chunk * chunk_keys;
+  const int64_t k1 = (k0 + chunk_keys < n_keys) ? k0 + chunk_keys : n_keys;
+  uint8_t *out8 = cnt_u8 ? cnt_u8 + (int64_t)row * cnt_u8_stride : nullptr;
+  int32_t *out32 = cnt_i32 ? cnt_i32 + (int64_t)row * n_keys : nullptr;
+
+  for (int64_t i0 = k0 + tid; i0 < k1; i0 += 4 * kScanThreads) {
+    pkv_u32x4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int64_t i = i0 + u * kScanThreads;
+      v[u] = (i < k1) ? __builtin_nontemporal_load(base + i) : pkv_u32x4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int64_t i = i0 + u * kScanThreads;
+      if (i < k1) {
+        const int c = lut_sum16(l8, v[u]);
+        if (out8) out8[i] = (uint8_t)c;
+        if (out32) out32[i] = c;
+        if (chunk_hist) atomicAdd(&s_hist[c * kHistCopies + copy], 1u);
+      }
+    }
+  }
+  if (chunk_hist) {
+    __syncthreads();
+    if (tid < 128) {
+      uint32_t s = 0;
+#pragma unroll
+      for (int c = 0; c < kHistCopies; ++c) s += s_hist[tid * kHistCopies + c];
+      chunk_hist[((int64_t)row * gridDim.x + chunk) * 128 + tid] = (uint16_t)s;
+    }
+  }
+}
+
+// Any byte strides (e.g. the reference's subspace-major [16][kv_len] tensor).
+__global__ __launch_bounds__(kScanThreads) void pkv_scan_strided_kernel(
+    const uint8_t *__restrict__ codes, int64_t cs_b, int64_t cs_h, int64_t cs_key, int64_t cs_sub, int n_kv_heads,
+    int64_t n_keys, const uint8_t *__restrict__ lut, uint8_t *__restrict__ cnt_u8, int64_t cnt_u8_stride,
+    int32_t *__restrict__ cnt_i32, uint16_t *__restrict__ chunk_hist, int chunk_keys) {
+  const int row = blockIdx.y;
+  const int chunk = blockIdx.x;
+  const int b = row / n_kv_heads, h = row % n_kv_heads;
+  const int tid = threadIdx.x;
+
+  __shared__ uint32_t s_lut[1024];
+  __shared__ uint32_t s_hist[128 * kHistCopies];
+  load_lut(s_lut, lut, row);
+  for (int i = tid; i < 128 * kHistCopies; i += kScanThreads) s_hist[i] = 0;
+  __syncthreads();
+  const uint8_t *l8 = (const uint8_t *)s_lut;
+  const int copy = tid & (kHistCopies - 1);
+
+  const uint8_t *base = codes + (int64_t)b * cs_b + (int64_t)h * cs_h;
+  const int64_t k0 = (int64_t)chunk * chunk_keys;
+  const int64_t k1 = (k0 + chunk_keys < n_keys) ? k0 + chunk_keys : n_keys;
+  uint8_t *out8 = cnt_u8 ? cnt_u8 + (int64_t)row * cnt_u8_stride : nullptr;
+  int32_t *out32 = cnt_i32 ? cnt_i32 + (int64_t)row * n_keys : nullptr;
+
+  for (int64_t i = k0 + tid; i < k1; i += kScanThreads) {
+    int c = 0;
+#pragma unroll
+    for (int s = 0; s < 16; ++s) c += l8[s * 256 + base[i * cs_key + s * cs_sub]];
+    if (out8) out8[i] = (uint8_t)c;
+    if (out32) out32[i] = c;
+    if (chunk_hist) atomicAdd(&s_hist[c * kHistCopies + copy], 1u);
+  }
+  if (chunk_hist) {
+    __syncthreads();
+    if (tid < 128) {
+      uint32_t s = 0;
+#pragma unroll
+      for (int c = 0; c < kHistCopies; ++c) s += s_hist[tid * kHistCopies + c];
+      chunk_hist[((int64_t)row * gridDim.x + chunk) * 128 + tid] = (uint16_t)s;
+    }
+  }
+}
+
+// Legacy int32 codebook [rows][16][n_keys]; codes outside [0,255] get no vote.
+__global__ __launch_bounds__(kScanThreads) void pkv_scan_i32_codes_kernel(const int32_t *__restrict__ codebook,
+                                                                          int64_t n_keys,
+                                                                          const uint8_t *__restrict__ lut,
+                                                                          int32_t *__restrict__ cnt) {
+  const int row = blockIdx.y;
+  __shared__ uint32_t s_lut[1024];
+  load_lut(s_lut, lut, row);
+  __syncthreads();
+  const uint8_t *l8 = (const uint8_t *)s_lut;
+  const int64_t i = (int64_t)blockIdx.x * kScanThreads + threadIdx.x;
+  if (i >= n_keys) return;
+  const int32_t *base = codebook + (int64_t)row * 16 * n_keys;
+  int c = 0;
+#pragma unroll
+  for (int s = 0; s < 16; ++s) {
+    const int32_t code = base[(int64_t)s * n_keys + i];
+    if ((uint32_t)code < 256u) c += l8[s * 256 + code];
+  }
+  cnt[(int64_t)row * n_keys + i] = c;
+}
+
+}  // namespace
+
+static int launch_scan_impl(const uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t cs_key, int64_t cs_sub, int bs,
+                            int n_kv_heads, int64_t n_keys, const uint8_t *lut, uint8_t *cnt_u8,
+                            int64_t cnt_u8_stride, int32_t *cnt_i32, uint16_t *chunk_hist, int chunk_keys,
+                            hipStream_t s, hipEvent_t ev_start, hipEvent_t ev_stop) {
+  PKV_REQUIRE(chunk_keys >= 2048 && chunk_keys % 2048 == 0 && chunk_keys <= 32768,
+              "chunk_keys must be a multiple of 2048 in [2048,32768], got %d", chunk_keys);
+  const int64_t n_chunks = (n_keys + chunk_keys - 1) / chunk_keys;
+  PKV_REQUIRE(n_chunks >= 1 && n_chunks <= 65535 * 16, "too many chunks (%lld)", (long long)n_chunks);
+  PKV_REQUIRE(pkv_aligned(lut, 4), "lut must be 4-byte aligned");
+  dim3 grid((unsigned)n_chunks, (unsigned)(bs * n_kv_heads));
+  const bool keymajor = cs_sub == 1 && cs_key == 16 && pkv_aligned(codes, 16) && cs_b % 16 == 0 && cs_h % 16 == 0;
+  if (keymajor) {
+    // the ext launch ties the two events to this dispatch's own begin/end timestamps
+    hipExtLaunchKernelGGL(pkv_scan_keymajor_kernel, grid, dim3(kScanThreads), 0, s, ev_start, ev_stop, 0, codes, cs_b,
+                          cs_h, n_kv_heads, n_keys, lut, cnt_u8, cnt_u8_stride, cnt_i32, chunk_hist, chunk_keys);
+    PKV_LAUNCH_CHECK("pkv_scan_keymajor_kernel");
+  } else {
+    hipExtLaunchKernelGGL(pkv_scan_strided_kernel, grid, dim3(kScanThreads), 0, s, ev_start, ev_stop, 0, codes, cs_b,
+                          cs_h, cs_key, cs_sub, n_kv_heads, n_keys, lut, cnt_u8, cnt_u8_stride, cnt_i32, chunk_hist,
+                          chunk_keys);
+    PKV_LAUNCH_CHECK("pkv_scan_strided_kernel");
+  }
+  return PKV_OK;
+}
+
+int pkv_launch_scan(const uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t cs_key, int64_t cs_sub, int bs,
+                    int n_kv_heads, int64_t n_keys, const uint8_t *lut, uint8_t *cnt_u8, int64_t cnt_u8_stride,
+                    int32_t *cnt_i32, uint16_t *chunk_hist, int chunk_keys, hipStream_t s) {
+  return launch_scan_impl(codes, cs_b, cs_h, cs_key, cs_sub, bs, n_kv_heads, n_keys, lut, cnt_u8, cnt_u8_stride, cnt_i32,
+                          chunk_hist, chunk_keys, s, nullptr, nullptr);
+}
+
+int pkv_launch_scan_i32_codes(const int32_t *codebook, int rows, int64_t n_keys, const uint8_t *lut, int32_t *cnt,
+                              hipStream_t s) {
+  dim3 grid((unsigned)((n_keys + kScanThreads - 1) / kScanThreads), (unsigned)rows);
+  hipLaunchKernelGGL(pkv_scan_i32_codes_kernel, grid, dim3(kScanThreads), 0, s, codebook, n_keys, lut, cnt);
+  PKV_LAUNCH_CHECK("pkv_scan_i32_codes_kernel");
+  return PKV_OK;
+}
+
+extern "C" int pkv_collision_scan(const uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t cs_key, int64_t cs_sub,
+                                  int bs, int n_kv_heads, int64_t n_keys, const uint8_t *lut, uint8_t *cnt_u8,
+                                  int32_t *cnt_i32, uint16_t *chunk_hist, int chunk_keys, void *stream) {
+  PKV_REQUIRE(codes && lut && (cnt_u8 || cnt_i32), "pkv_collision_scan: null pointer");
+  PKV_REQUIRE(bs > 0 && n_kv_heads > 0 && (int64_t)bs * n_kv_heads <= 65535 && n_keys > 0 &&
+                  n_keys <= PKV_MAX_KEYS_PER_ROW,
+              "bad shape bs=%d kv_heads=%d n_keys=%lld", bs, n_kv_heads, (long long)n_keys);
+  return pkv_launch_scan(codes, cs_b, cs_h, cs_key, cs_sub, bs, n_kv_heads, n_keys, lut, cnt_u8, n_keys, cnt_i32,
+                         chunk_hist, chunk_keys, (hipStream_t)stream);
+}
+
+extern "C" int pkv_collision_scan_timed(const uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t cs_key,
+                                        int64_t cs_sub, int bs, int n_kv_heads, int64_t n_keys, const uint8_t *lut,
+                                        uint8_t *cnt_u8, int64_t cnt_u8_stride, uint16_t *chunk_hist, int chunk_keys,
+                                        float *kernel_us, void *stream) {
+  PKV_REQUIRE(codes && lut && cnt_u8 && kernel_us, "pkv_collision_scan_timed: null pointer");
+  PKV_REQUIRE(bs > 0 && n_kv_heads > 0 && (int64_t)bs * n_kv_heads <= 65535 && n_keys > 0 &&
+                  n_keys <= PKV_MAX_KEYS_PER_ROW && cnt_u8_stride >= n_keys,
+              "bad shape bs=%d kv_heads=%d n_keys=%lld", bs, n_kv_heads, (long long)n_keys);
+  hipEvent_t e0, e1;
+  PKV_HIP(hipEventCreate(&e0));
+  PKV_HIP(hipEventCreate(&e1));
+  int rc = launch_scan_impl(codes, cs_b, cs_h, cs_key, cs_sub, bs, n_kv_heads, n_keys, lut, cnt_u8, cnt_u8_stride,
+                            nullptr, chunk_hist, chunk_keys, (hipStream_t)stream, e0, e1);
+  if (rc == PKV_OK) {
+    float ms = 0.f;
+    hipError_t e = hipEventSynchronize(e1);
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    if (e != hipSuccess) {
+      pkv_set_error("event timing failed: %s", hipGetErrorString(e));
+      rc = PKV_EHIP;
+    }
+    *kernel_us = ms * 1000.f;
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  return rc;
+}

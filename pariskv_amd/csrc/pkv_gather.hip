@@ -1,0 +1,184 @@
+// Row gathers of the selected K/V: out of pinned host memory through the GPU's
+// unified addressing (PCIe reads issued by the kernel), or HBM to HBM.
+//
+// Reference: cache_hub/gather_trans/trans_h2d.cu:19-121 (h2d_gather_kv_kernel:
+// one 32-thread block per selected index, 16 lanes per 256-byte row) and the
+// torch.gather branch cache_hub/polar_cache.py:1089-1095.  Here a wave64 moves
+// four 256-byte rows per instruction and every lane keeps several independent
+// 16-byte reads in flight, which is what a latency-bound PCIe read stream needs.
+#include "pkv_common.h"
+
+namespace {
+
+constexpr int kGatherThreads = 256;
+constexpr int kGatherUnroll = 4;  // independent row reads per lane
+
+// task t in [0, rows*k*2): kv = t & 1, (row, slot) = divmod(t >> 1, k).
+// `vpr` = 16-byte vectors per row; consecutive lanes cover one row.
+__global__ __launch_bounds__(kGatherThreads) void pkv_gather_rows_kernel(
+    const pkv_u32x4 *__restrict__ src_k, const pkv_u32x4 *__restrict__ src_v, int64_t src_len,
+    const int64_t *__restrict__ idx, int64_t k, int64_t idx_offset, pkv_u32x4 *__restrict__ dst_k,
+    pkv_u32x4 *__restrict__ dst_v, int64_t dst_len, int64_t dst_row0, int64_t n_tasks, int vpr) {
+  const int64_t lanes_per_block = kGatherThreads;
+  const int64_t g0 = (int64_t)blockIdx.x * lanes_per_block * kGatherUnroll + threadIdx.x;
+  pkv_u32x4 val[kGatherUnroll];
+  pkv_u32x4 *dst[kGatherUnroll];
+#pragma unroll
+  for (int u = 0; u < kGatherUnroll; ++u) {
+    const int64_t g = g0 + (int64_t)u * lanes_per_block;
+    const int64_t task = g / vpr;
+    const int lane = (int)(g % vpr);
+    dst[u] = nullptr;
+    val[u] = pkv_u32x4{0u, 0u, 0u, 0u};
+    if (task < n_tasks) {
+      const int kv = (int)(task & 1);
+      const int64_t rs = task >> 1;
+      const int64_t row = rs / k, slot = rs % k;
+      const int64_t i = idx[rs] + idx_offset;
+      const pkv_u32x4 *src = kv ? src_v : src_k;
+      pkv_u32x4 *d = kv ? dst_v : dst_k;
+      dst[u] = d + ((row * dst_len + dst_row0 + slot) * vpr + lane);
+      if ((uint64_t)i < (uint64_t)src_len) val[u] = src[(row * src_len + i) * vpr + lane];
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < kGatherUnroll; ++u)
+    if (dst[u]) *dst[u] = val[u];
+}
+
+// Ragged form: virtual head v owns slots [cu_topk[v], cu_topk[v+1]) of
+// idx_packed and writes rows cu_k[v] + sink_local_end + s of the packed
+// destination.  grid (ceil(max_k * vpr * 2 / 256), V).
+__global__ __launch_bounds__(kGatherThreads) void pkv_gather_packed_kernel(
+    const pkv_u32x4 *__restrict__ src_k, const pkv_u32x4 *__restrict__ src_v, int64_t src_len,
+    const int64_t *__restrict__ idx_packed, const int32_t *__restrict__ cu_topk, const int32_t *__restrict__ cu_k,
+    int64_t sink_local_end, pkv_u32x4 *__restrict__ dst_k, pkv_u32x4 *__restrict__ dst_v, int64_t total_k, int vpr) {
+  const int v = blockIdx.y;
+  const int64_t g = (int64_t)blockIdx.x * kGatherThreads + threadIdx.x;
+  const int64_t task = g / vpr;
+  const int lane = (int)(g % vpr);
+  const int kv = (int)(task & 1);
+  const int64_t s = task >> 1;
+  const int64_t begin = cu_topk[v];
+  const int64_t n = (int64_t)cu_topk[v + 1] - begin;
+  if (s >= n) return;
+  const int64_t drow = (int64_t)cu_k[v] + sink_local_end + s;
+  if (drow < 0 || drow >= total_k) return;
+  const int64_t i = idx_packed[begin + s];
+  pkv_u32x4 val = pkv_u32x4{0u, 0u, 0u, 0u};
+  if ((uint64_t)i < (uint64_t)src_len) val = (kv ? src_v : src_k)[((int64_t)v * src_len + i) * vpr + lane];
+  (kv ? dst_v : dst_k)[drow * vpr + lane] = val;
+}
+
+// Plain streaming copy of n 16-byte vectors (calibration of HBM counters, tests).
+__global__ __launch_bounds__(256) void pkv_copy_kernel(const pkv_u32x4 *__restrict__ src, pkv_u32x4 *__restrict__ dst,
+                                                       int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = src[i];
+}
+
+int check_common(const void *src_k, const void *src_v, const void *dst_k, const void *dst_v, int rows, int row_bytes) {
+  PKV_REQUIRE(src_k && src_v && dst_k && dst_v, "gather: null pointer");
+  PKV_REQUIRE(rows > 0, "gather: bad row count %d", rows);
+  PKV_REQUIRE(row_bytes > 0 && row_bytes % 16 == 0 && row_bytes <= 4096, "row_bytes must be a multiple of 16 (got %d)",
+              row_bytes);
+  PKV_REQUIRE(pkv_aligned(src_k, 16) && pkv_aligned(src_v, 16) && pkv_aligned(dst_k, 16) && pkv_aligned(dst_v, 16),
+              "gather: buffers must be 16-byte aligned");
+  return PKV_OK;
+}
+
+int device_view_of_host(const void *host, const void **dev) {
+  void *d = nullptr;
+  hipError_t e = hipHostGetDevicePointer(&d, const_cast<void *>(host), 0);
+  if (e != hipSuccess || d == nullptr) {
+    (void)hipGetLastError();
+    pkv_set_error("source is not pinned, device-mapped host memory (%s)", hipGetErrorString(e));
+    return PKV_EINVAL;
+  }
+  *dev = d;
+  return PKV_OK;
+}
+
+}  // namespace
+
+int pkv_launch_gather(const void *src_k, const void *src_v, int64_t src_len, const int64_t *idx, int64_t k,
+                      int64_t idx_offset, void *dst_k, void *dst_v, int64_t dst_len, int64_t dst_row0, int rows,
+                      int row_bytes, hipStream_t s) {
+  int rc = check_common(src_k, src_v, dst_k, dst_v, rows, row_bytes);
+  if (rc) return rc;
+  PKV_REQUIRE(idx && k > 0 && src_len > 0 && dst_row0 >= 0 && dst_row0 + k <= dst_len,
+              "gather: k=%lld src_len=%lld dst_row0=%lld dst_len=%lld", (long long)k, (long long)src_len,
+              (long long)dst_row0, (long long)dst_len);
+  const int vpr = row_bytes / 16;
+  const int64_t n_tasks = (int64_t)rows * k * 2;
+  const int64_t lanes = n_tasks * vpr;
+  const int64_t per_block = (int64_t)kGatherThreads * kGatherUnroll;
+  const int64_t blocks = (lanes + per_block - 1) / per_block;
+  PKV_REQUIRE(blocks < ((int64_t)1 << 31), "gather too large");
+  hipLaunchKernelGGL(pkv_gather_rows_kernel, dim3((unsigned)blocks), dim3(kGatherThreads), 0, s,
+                     (const pkv_u32x4 *)src_k, (const pkv_u32x4 *)src_v, src_len, idx, k, idx_offset,
+                     (pkv_u32x4 *)dst_k, (pkv_u32x4 *)dst_v, dst_len, dst_row0, n_tasks, vpr);
+  PKV_LAUNCH_CHECK("pkv_gather_rows_kernel");
+  return PKV_OK;
+}
+
+extern "C" int pkv_gather_hbm(const void *src_k, const void *src_v, int64_t src_len, const int64_t *idx, int64_t k,
+                              int64_t idx_offset, void *dst_k, void *dst_v, int64_t dst_len, int64_t dst_row0, int bs,
+                              int n_kv_heads, int row_bytes, void *stream) {
+  return pkv_launch_gather(src_k, src_v, src_len, idx, k, idx_offset, dst_k, dst_v, dst_len, dst_row0,
+                           bs * n_kv_heads, row_bytes, (hipStream_t)stream);
+}
+
+extern "C" int pkv_gather_uva(const void *src_k, const void *src_v, int64_t src_len, const int64_t *idx, int64_t k,
+                              int64_t idx_offset, void *dst_k, void *dst_v, int64_t dst_len, int64_t dst_row0, int bs,
+                              int n_kv_heads, int row_bytes, void *stream) {
+  PKV_REQUIRE(src_k && src_v, "gather: null pointer");
+  const void *dk, *dv;
+  int rc = device_view_of_host(src_k, &dk);
+  if (rc) return rc;
+  rc = device_view_of_host(src_v, &dv);
+  if (rc) return rc;
+  return pkv_launch_gather(dk, dv, src_len, idx, k, idx_offset, dst_k, dst_v, dst_len, dst_row0, bs * n_kv_heads,
+                           row_bytes, (hipStream_t)stream);
+}
+
+extern "C" int pkv_gather_uva_packed(const void *src_k, const void *src_v, int64_t src_len, const int64_t *idx_packed,
+                                     const int32_t *cu_topk, const int32_t *cu_k, int64_t sink_local_end,
+                                     int64_t max_k, void *dst_k, void *dst_v, int64_t total_k, int bs, int n_kv_heads,
+                                     int row_bytes, void *stream) {
+  int rc = check_common(src_k, src_v, dst_k, dst_v, bs * n_kv_heads, row_bytes);
+  if (rc) return rc;
+  PKV_REQUIRE(idx_packed && cu_topk && cu_k && max_k > 0 && total_k > 0 && src_len > 0 && sink_local_end >= 0,
+              "packed gather: bad arguments");
+  const void *dk = src_k, *dv = src_v;
+  hipPointerAttribute_t attr;
+  if (hipPointerGetAttributes(&attr, src_k) == hipSuccess && attr.type == hipMemoryTypeHost) {
+    rc = device_view_of_host(src_k, &dk);
+    if (rc) return rc;
+    rc = device_view_of_host(src_v, &dv);
+    if (rc) return rc;
+  } else {
+    (void)hipGetLastError();
+  }
+  const int vpr = row_bytes / 16;
+  const int64_t lanes = max_k * 2 * vpr;
+  dim3 grid((unsigned)((lanes + kGatherThreads - 1) / kGatherThreads), (unsigned)(bs * n_kv_heads));
+  hipLaunchKernelGGL(pkv_gather_packed_kernel, grid, dim3(kGatherThreads), 0, (hipStream_t)stream,
+                     (const pkv_u32x4 *)dk, (const pkv_u32x4 *)dv, src_len, idx_packed, cu_topk, cu_k, sink_local_end,
+                     (pkv_u32x4 *)dst_k, (pkv_u32x4 *)dst_v, total_k, vpr);
+  PKV_LAUNCH_CHECK("pkv_gather_packed_kernel");
+  return PKV_OK;
+}
+
+extern "C" int pkv_copy_bytes(const void *src, void *dst, size_t bytes, void *stream) {
+  PKV_REQUIRE(src && dst && bytes % 16 == 0 && pkv_aligned(src, 16) && pkv_aligned(dst, 16),
+              "pkv_copy_bytes: 16-byte aligned buffers and size required");
+  if (bytes == 0) return PKV_OK;
+  const int64_t n = (int64_t)(bytes / 16);
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  hipLaunchKernelGGL(pkv_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                     (const pkv_u32x4 *)src, (pkv_u32x4 *)dst, n);
+  PKV_LAUNCH_CHECK("pkv_copy_kernel");
+  return PKV_OK;
+}

@@ -1,0 +1,155 @@
+// One layer's retrieval for one decode step as a fixed sequence of launches on
+// the caller's stream: query prep + vote table -> collision scan (+ chunk
+// histograms) -> candidate select -> 4-bit rerank -> exact top-k -> optional
+// gather of the selected K/V rows.
+//
+// Reference: cache_hub/polar_cache.py:1126-1162 (collision_based_topk_batch),
+// :1207-1231, :1244-1304 and the gather at :1075-1095.
+#include "pkv_common.h"
+
+PKV_INTERNAL int pkv_launch_identity_fill(int64_t *out, int64_t len, int64_t k, int rows, hipStream_t s);
+
+namespace {
+
+struct WsLayout {
+  size_t qhat, qnorm, lut, cnt, hist, cand, scores, total;
+  int64_t cnt_stride;
+  int chunk_keys;
+  int64_t n_chunks;
+};
+
+WsLayout layout(int rows, int64_t n_keys, int64_t n_cand, int64_t /*k*/) {
+  WsLayout w;
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    size_t o = off;
+    off += pkv_align_up(bytes, 256);
+    return o;
+  };
+  w.chunk_keys = pkv_pick_chunk_keys(rows, n_keys);
+  w.n_chunks = (n_keys + w.chunk_keys - 1) / w.chunk_keys;
+  w.cnt_stride = (int64_t)pkv_align_up((size_t)n_keys, 16);
+  w.qhat = take((size_t)rows * 128 * sizeof(float));
+  w.qnorm = take((size_t)rows * sizeof(float));
+  w.lut = take((size_t)rows * 4096);
+  w.cnt = take((size_t)rows * (size_t)w.cnt_stride);
+  w.hist = take((size_t)rows * (size_t)w.n_chunks * 128 * sizeof(uint16_t));
+  w.cand = take((size_t)rows * (size_t)n_cand * sizeof(int64_t));
+  w.scores = take((size_t)rows * (size_t)n_cand * sizeof(float));
+  w.total = off;
+  return w;
+}
+
+bool shape_ok(int rows, int64_t n_keys, int64_t n_cand, int64_t k) {
+  return rows > 0 && rows <= 65535 && n_keys > 0 && n_keys <= PKV_MAX_KEYS_PER_ROW && n_cand > 0 &&
+         n_cand <= n_keys && k > 0 && k <= n_cand;
+}
+
+}  // namespace
+
+extern "C" size_t pkv_retrieve_ws_bytes(int rows, int64_t n_keys, int64_t n_cand, int64_t k) {
+  if (!shape_ok(rows, n_keys, n_cand, k)) return 0;
+  return layout(rows, n_keys, n_cand, k).total;
+}
+
+extern "C" int pkv_retrieve_ws_view(void *ws, int rows, int64_t n_keys, int64_t n_cand, int64_t k, const char *name,
+                                    void **ptr, size_t *bytes) {
+  PKV_REQUIRE(ws && name && ptr && bytes && shape_ok(rows, n_keys, n_cand, k), "pkv_retrieve_ws_view: bad arguments");
+  const WsLayout w = layout(rows, n_keys, n_cand, k);
+  char *base = (char *)ws;
+  if (!strcmp(name, "qhat")) {
+    *ptr = base + w.qhat, *bytes = (size_t)rows * 128 * 4;
+  } else if (!strcmp(name, "qnorm")) {
+    *ptr = base + w.qnorm, *bytes = (size_t)rows * 4;
+  } else if (!strcmp(name, "lut")) {
+    *ptr = base + w.lut, *bytes = (size_t)rows * 4096;
+  } else if (!strcmp(name, "cnt_u8")) {
+    *ptr = base + w.cnt, *bytes = (size_t)rows * (size_t)w.cnt_stride;
+  } else if (!strcmp(name, "chunk_hist")) {
+    *ptr = base + w.hist, *bytes = (size_t)rows * (size_t)w.n_chunks * 256;
+  } else if (!strcmp(name, "cand")) {
+    *ptr = base + w.cand, *bytes = (size_t)rows * (size_t)n_cand * 8;
+  } else if (!strcmp(name, "scores")) {
+    *ptr = base + w.scores, *bytes = (size_t)rows * (size_t)n_cand * 4;
+  } else {
+    pkv_set_error("unknown workspace segment '%s'", name);
+    return PKV_EINVAL;
+  }
+  return PKV_OK;
+}
+
+extern "C" int pkv_retrieve(const pkv_retrieve_args *a, void *ws, size_t ws_bytes, void *stream) {
+  PKV_REQUIRE(a != nullptr, "pkv_retrieve: null args");
+  PKV_REQUIRE(a->q && a->signs && a->centers && a->cluster_counts && a->codes && a->nib && a->weight && a->out_ids,
+              "pkv_retrieve: null pointer");
+  PKV_REQUIRE(a->dtype == PKV_DTYPE_F32 || a->dtype == PKV_DTYPE_BF16, "unknown dtype %d", a->dtype);
+  PKV_REQUIRE(a->bs > 0 && a->n_kv_heads > 0 && a->group > 0, "bad shape bs=%d kv_heads=%d group=%d", a->bs,
+              a->n_kv_heads, a->group);
+  const int rows = a->bs * a->n_kv_heads;
+  PKV_REQUIRE(shape_ok(rows, a->n_keys, a->n_cand, a->k),
+              "need 0 < k <= n_cand <= n_keys <= 2^24 (k=%lld n_cand=%lld n_keys=%lld rows=%d)", (long long)a->k,
+              (long long)a->n_cand, (long long)a->n_keys, rows);
+  PKV_REQUIRE(a->key0 >= 0 && a->key0 + a->n_keys <= a->cap, "retrieval zone [%lld,+%lld) exceeds capacity %lld",
+              (long long)a->key0, (long long)a->n_keys, (long long)a->cap);
+  PKV_REQUIRE(a->n_tiers >= 1 && a->n_tiers <= PKV_MAX_TIERS, "n_tiers must be in [1,%d]", PKV_MAX_TIERS);
+  PKV_REQUIRE(pkv_aligned(a->codes, 16) && pkv_aligned(a->nib, 16) && pkv_aligned(a->weight, 16),
+              "codes / nib / weight must be 16-byte aligned");
+  const WsLayout w = layout(rows, a->n_keys, a->n_cand, a->k);
+  if (!ws || ws_bytes < w.total || !pkv_aligned(ws, 256)) {
+    pkv_set_error("pkv_retrieve: workspace of %zu bytes (256-aligned) required, got %zu", w.total, ws_bytes);
+    return PKV_ENOMEM;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  char *base = (char *)ws;
+  float *qhat = (float *)(base + w.qhat);
+  float *qnorm = (float *)(base + w.qnorm);
+  uint8_t *lut = (uint8_t *)(base + w.lut);
+  uint8_t *cnt = (uint8_t *)(base + w.cnt);
+  uint16_t *hist = (uint16_t *)(base + w.hist);
+  int64_t *cand = (int64_t *)(base + w.cand);
+  float *scores = (float *)(base + w.scores);
+
+  PkvTiers t;
+  memset(&t, 0, sizeof t);
+  t.n = a->n_tiers;
+  for (int i = 0; i < a->n_tiers; ++i) t.t[i] = a->tier_counts[i];
+
+  const int H = a->n_kv_heads;
+  int rc = pkv_launch_query_prep_lut(a->q, a->dtype, a->bs, H, a->group, a->signs, a->cluster_counts,
+                                     (int64_t)H * 4096, 4096, t, qhat, qnorm, lut, nullptr, s);
+  if (rc) return rc;
+  const uint8_t *codes = a->codes + a->key0 * 16;
+  const uint8_t *nib = a->nib + a->key0 * 64;
+  const uint16_t *weight = a->weight + a->key0 * 16;
+  if (a->n_cand == a->n_keys) {
+    rc = pkv_launch_identity_fill(cand, a->n_keys, a->n_cand, rows, s);
+  } else {
+    rc = pkv_launch_scan(codes, (int64_t)H * a->cap * 16, a->cap * 16, 16, 1, a->bs, H, a->n_keys, lut, cnt,
+                         w.cnt_stride, nullptr, hist, w.chunk_keys, s);
+    if (rc) return rc;
+    rc = pkv_launch_select(cnt, w.cnt_stride, hist, w.chunk_keys, rows, a->n_keys, a->n_cand, cand, s);
+  }
+  if (rc) return rc;
+  rc = pkv_launch_rerank(cand, a->bs, H, a->n_cand, a->n_keys, nib, (int64_t)H * a->cap * 64, a->cap * 64, 64, 4,
+                         weight, (int64_t)H * a->cap * 16, a->cap * 16, 16, 1, qhat, qnorm, a->centers, scores,
+                         nullptr, s);
+  if (rc) return rc;
+  rc = pkv_launch_topk_f32(scores, a->n_cand, cand, a->n_cand, rows, a->n_cand, a->k, a->out_ids, a->out_scores,
+                           nullptr, 0, s);
+  if (rc) return rc;
+  if (a->src_k) {
+    PKV_REQUIRE(a->src_v && a->dst_k && a->dst_v, "pkv_retrieve: gather needs src_v, dst_k, dst_v");
+    const void *sk = a->src_k, *sv = a->src_v;
+    if (a->gather_from_host) {
+      void *dk = nullptr, *dv = nullptr;
+      rc = pkv_host_device_pointer(a->src_k, &dk);
+      if (rc) return rc;
+      rc = pkv_host_device_pointer(a->src_v, &dv);
+      if (rc) return rc;
+      sk = dk, sv = dv;
+    }
+    rc = pkv_launch_gather(sk, sv, a->src_len, a->out_ids, a->k, a->idx_offset, a->dst_k, a->dst_v, a->dst_len,
+                           a->dst_row0, rows, a->row_bytes, s);
+  }
+  return rc;
+}

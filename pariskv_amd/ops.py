@@ -1,0 +1,409 @@
+"""Tensor-level wrappers over the C ABI: pointer/stride plumbing only.
+
+Tensors use the reference's *logical* shapes (``cache_hub/polar_cache.py:288-312``):
+``codebook [bs,H,B,N] u8``, ``key_4bit [bs,H,B,N,4] u8``, ``key_block_weight
+[bs,H,B,N] bf16`` with arbitrary strides, so the same call accepts the
+reference's subspace-major tensors and key-major storage exposed as permuted
+views (see :func:`alloc_keymajor`).  PyTorch is used for device memory and
+streams only; every computation happens in ``libpariskv_hip.so``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Sequence
+
+import torch
+
+from . import _lib
+
+B_SUB, M_SUB, K_CLUSTERS, HEAD_DIM = 16, 8, 256, 128
+TIER_RATIOS = (0.05, 0.15, 0.30, 0.50, 0.75, 1.0)  # cache_hub/polar_cache.py:1221
+# cache_hub/polar_cache.py:188-193 rounded to bf16
+MAG_THRESHOLDS = (0.08447265625, 0.169921875, 0.2578125, 0.349609375, 0.44921875, 0.55859375, 0.69140625)
+MAG_CENTERS = (0.0419921875, 0.126953125, 0.212890625, 0.302734375, 0.396484375, 0.5, 0.6171875, 0.76171875)
+
+
+def _p(t: Optional[torch.Tensor]):
+    return C.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _stream(t: torch.Tensor):
+    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _dt(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return _lib.DTYPE_F32
+    if dtype == torch.bfloat16:
+        return _lib.DTYPE_BF16
+    raise RuntimeError(f"unsupported dtype {dtype}: float32 or bfloat16 expected")
+
+
+def _need(cond: bool, msg: str):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _cuda(*ts):
+    for t in ts:
+        if t is not None:
+            _need(t.is_cuda, "tensor must be on the GPU")
+
+
+def srht_signs(device, seed: int = 42) -> torch.Tensor:
+    """SRHT diagonal in {+-1}^128 as float32.  The reference draws it from the
+    device generator (``polar_cache.py:59-63``); here it is a CPU-generator draw
+    so that every machine gets the same vector."""
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randint(0, 2, (HEAD_DIM,), generator=g).to(torch.float32) * 2 - 1).to(device)
+
+
+def mag_centers(device) -> torch.Tensor:
+    return torch.tensor(MAG_CENTERS, dtype=torch.float32, device=device)
+
+
+def alloc_keymajor(bs: int, heads: int, cap: int, device):
+    """Key-major storage + reference-shaped views.
+
+    Returns ``(codes_km [bs,H,cap,16] u8, nib_km [bs,H,cap,64] u8, w_km [bs,H,cap,16] bf16,
+    codebook [bs,H,16,cap], key_4bit [bs,H,16,cap,4], key_block_weight [bs,H,16,cap])``;
+    the last three are permuted views of the first three."""
+    codes = torch.zeros(bs, heads, cap, B_SUB, dtype=torch.uint8, device=device)
+    nib = torch.zeros(bs, heads, cap, B_SUB * 4, dtype=torch.uint8, device=device)
+    w = torch.zeros(bs, heads, cap, B_SUB, dtype=torch.bfloat16, device=device)
+    return (codes, nib, w, codes.permute(0, 1, 3, 2), nib.view(bs, heads, cap, B_SUB, 4).permute(0, 1, 3, 2, 4),
+            w.permute(0, 1, 3, 2))
+
+
+# ------------------------------------------------------------------- append
+
+
+def encode_append(keys: torch.Tensor, signs: torch.Tensor, codebook: torch.Tensor,
+                  key_4bit: Optional[torch.Tensor], key_block_weight: Optional[torch.Tensor],
+                  cluster_counts: Optional[torch.Tensor]) -> None:
+    """keys [bs,H,S,128] -> writes codebook [bs,H,16,S], key_4bit [bs,H,16,S,4],
+    key_block_weight [bs,H,16,S] (any strides) and ``cluster_counts += histogram``."""
+    _cuda(keys, signs, codebook, key_4bit, key_block_weight, cluster_counts)
+    bs, H, S, D = keys.shape
+    _need(D == HEAD_DIM and keys.stride(3) == 1, "keys must be [bs,H,S,128] with a contiguous last dim")
+    _need(signs.dtype == torch.float32 and signs.numel() == HEAD_DIM and signs.is_contiguous(), "signs: float32[128]")
+    _need(codebook.dtype == torch.uint8 and tuple(codebook.shape) == (bs, H, B_SUB, S), "codebook must be u8 [bs,H,16,S]")
+    ns = (0, 0, 0, 0)
+    if key_4bit is not None:
+        _need(key_4bit.dtype == torch.uint8 and tuple(key_4bit.shape) == (bs, H, B_SUB, S, 4) and
+              key_4bit.stride(4) == 1, "key_4bit must be u8 [bs,H,16,S,4] with a contiguous last dim")
+        ns = (key_4bit.stride(0), key_4bit.stride(1), key_4bit.stride(3), key_4bit.stride(2))
+    ws = (0, 0, 0, 0)
+    if key_block_weight is not None:
+        _need(key_block_weight.dtype == torch.bfloat16 and tuple(key_block_weight.shape) == (bs, H, B_SUB, S),
+              "key_block_weight must be bf16 [bs,H,16,S]")
+        ws = (key_block_weight.stride(0), key_block_weight.stride(1), key_block_weight.stride(3),
+              key_block_weight.stride(2))
+    cc = (0, 0)
+    if cluster_counts is not None:
+        _need(cluster_counts.dtype == torch.int32 and tuple(cluster_counts.shape) == (bs, H, B_SUB, K_CLUSTERS) and
+              cluster_counts.stride(3) == 1 and cluster_counts.stride(2) == K_CLUSTERS,
+              "cluster_counts must be int32 [bs,H,16,256] with contiguous [16,256] blocks")
+        cc = (cluster_counts.stride(0), cluster_counts.stride(1))
+    _lib.check(_lib.lib().pkv_encode_append(
+        _p(keys), _dt(keys.dtype), bs, H, S, keys.stride(0), keys.stride(1), keys.stride(2), _p(signs),
+        _p(codebook), codebook.stride(0), codebook.stride(1), codebook.stride(3), codebook.stride(2),
+        _p(key_4bit), *ns, _p(key_block_weight), *ws, _p(cluster_counts), *cc, _stream(keys)))
+
+
+def count_cluster_keys(codebook: torch.Tensor, cluster_counts: torch.Tensor) -> None:
+    """cluster_counts[bs,H,16,256] += per-subspace histogram of codebook [bs,H,16,N]."""
+    _cuda(codebook, cluster_counts)
+    bs, H, Bs, N = codebook.shape
+    _need(codebook.dtype == torch.uint8 and Bs == B_SUB, "codebook must be u8 [bs,H,16,N]")
+    _need(cluster_counts.dtype == torch.int32 and tuple(cluster_counts.shape) == (bs, H, B_SUB, K_CLUSTERS) and
+          cluster_counts.stride(3) == 1 and cluster_counts.stride(2) == K_CLUSTERS, "cluster_counts: int32 [bs,H,16,256]")
+    _lib.check(_lib.lib().pkv_count_cluster_keys(
+        _p(codebook), codebook.stride(0), codebook.stride(1), codebook.stride(3), codebook.stride(2), bs, H, N,
+        _p(cluster_counts), cluster_counts.stride(0), cluster_counts.stride(1), _stream(codebook)))
+
+
+# --------------------------------------------------------------- query side
+
+
+def _tiers(tier_counts: Sequence[int]):
+    _need(1 <= len(tier_counts) <= _lib.MAX_TIERS, f"tier_num must be in [1,{_lib.MAX_TIERS}]")
+    return (C.c_uint32 * len(tier_counts))(*[int(t) for t in tier_counts]), len(tier_counts)
+
+
+def query_prep_lut(queries: torch.Tensor, n_kv_heads: int, signs: torch.Tensor, cluster_counts: torch.Tensor,
+                   tier_counts: Sequence[int], want_sorted_ids: bool = False):
+    """queries [bs,1,Hq,128] or [bs,Hq,128] -> (qhat [bs,H,128] f32, qnorm [bs,H] f32,
+    lut [bs,H,16,256] u8, sorted_ids [bs,H,16,256] i64 or None)."""
+    _cuda(queries, signs, cluster_counts)
+    q = queries.reshape(queries.shape[0], -1, HEAD_DIM) if queries.dim() == 4 else queries
+    _need(q.is_contiguous() and q.shape[-1] == HEAD_DIM, "queries must be contiguous [bs,(1,)Hq,128]")
+    bs, Hq, _ = q.shape
+    _need(Hq % n_kv_heads == 0, "num_heads must be a multiple of num_key_value_heads")
+    group = Hq // n_kv_heads
+    _need(cluster_counts.dtype == torch.int32 and tuple(cluster_counts.shape) == (bs, n_kv_heads, B_SUB, K_CLUSTERS)
+          and cluster_counts.stride(3) == 1 and cluster_counts.stride(2) == K_CLUSTERS,
+          "cluster_counts must be int32 [bs,H,16,256]")
+    dev = q.device
+    qhat = torch.empty(bs, n_kv_heads, HEAD_DIM, dtype=torch.float32, device=dev)
+    qnorm = torch.empty(bs, n_kv_heads, dtype=torch.float32, device=dev)
+    lut = torch.empty(bs, n_kv_heads, B_SUB, K_CLUSTERS, dtype=torch.uint8, device=dev)
+    sorted_ids = torch.empty(bs, n_kv_heads, B_SUB, K_CLUSTERS, dtype=torch.int64, device=dev) if want_sorted_ids else None
+    tc, nt = _tiers(tier_counts)
+    _lib.check(_lib.lib().pkv_query_prep_lut(
+        _p(q), _dt(q.dtype), bs, n_kv_heads, group, _p(signs), _p(cluster_counts), cluster_counts.stride(0),
+        cluster_counts.stride(1), tc, nt, _p(qhat), _p(qnorm), _p(lut), _p(sorted_ids), _stream(q)))
+    return qhat, qnorm, lut, sorted_ids
+
+
+def update_cache_cnt(sorted_cluster_ids: torch.Tensor, cluster_key_counts: torch.Tensor, codebook: torch.Tensor,
+                     tier_counts: Sequence[int]) -> torch.Tensor:
+    """Tiered collision vote from a caller-supplied ranking -> int32 [bs,H,N]."""
+    _cuda(sorted_cluster_ids, cluster_key_counts, codebook)
+    _need(codebook.dtype == torch.uint8, "code_book must be uint8 tensor")
+    _need(sorted_cluster_ids.dtype == torch.int64, "sorted_cluster_ids must be int64 tensor")
+    _need(cluster_key_counts.dtype == torch.int32, "cluster_key_counts must be int32 tensor")
+    _need(sorted_cluster_ids.dim() == 4 and codebook.dim() == 4 and cluster_key_counts.dim() == 4, "4-D tensors expected")
+    bs, H, Bs, K = sorted_cluster_ids.shape
+    _need(Bs == B_SUB and K == K_CLUSTERS, "only sub_spaces=16, num_clusters=256 is built")
+    _need(tuple(cluster_key_counts.shape) == (bs, H, Bs, K) and tuple(codebook.shape[:3]) == (bs, H, Bs), "shape mismatch")
+    _need(sorted_cluster_ids.stride(3) == 1 and cluster_key_counts.stride(3) == 1, "last dims must be contiguous")
+    N = codebook.shape[3]
+    cnt = torch.empty(bs, H, N, dtype=torch.int32, device=codebook.device)
+    lut_ws = torch.empty(bs * H * B_SUB * K_CLUSTERS, dtype=torch.uint8, device=codebook.device)
+    tc, nt = _tiers(tier_counts)
+    si, ck, cb = sorted_cluster_ids, cluster_key_counts, codebook
+    _lib.check(_lib.lib().pkv_update_cache_cnt(
+        _p(si), si.stride(0), si.stride(1), si.stride(2), _p(ck), ck.stride(0), ck.stride(1), ck.stride(2),
+        _p(cb), cb.stride(0), cb.stride(1), cb.stride(3), cb.stride(2), bs, H, N, tc, nt, _p(lut_ws), _p(cnt),
+        _stream(cb)))
+    return cnt
+
+
+def update_cache_cnt_legacy(sorted_cluster_ids: torch.Tensor, topk_cluster_cnt: torch.Tensor,
+                            codebook: torch.Tensor) -> torch.Tensor:
+    """Single-tier vote on the legacy int32 tensors -> int32 [bs,H,N]."""
+    _cuda(sorted_cluster_ids, topk_cluster_cnt, codebook)
+    for t, name in ((sorted_cluster_ids, "sorted_cluster_ids"), (topk_cluster_cnt, "topk_cluster_cnt"), (codebook, "codebook")):
+        _need(t.dtype == torch.int32 and t.is_contiguous(), f"{name} must be a contiguous int32 tensor")
+    bs, H, Bs, K = sorted_cluster_ids.shape
+    _need(Bs == B_SUB and K == K_CLUSTERS and tuple(topk_cluster_cnt.shape) == (bs, H, Bs) and
+          tuple(codebook.shape[:3]) == (bs, H, Bs), "shape mismatch (sub_spaces=16, num_clusters=256 only)")
+    N = codebook.shape[3]
+    cnt = torch.empty(bs, H, N, dtype=torch.int32, device=codebook.device)
+    lut_ws = torch.empty(bs * H * B_SUB * K_CLUSTERS, dtype=torch.uint8, device=codebook.device)
+    _lib.check(_lib.lib().pkv_update_cache_cnt_legacy(_p(sorted_cluster_ids), _p(topk_cluster_cnt), _p(codebook), bs, H,
+                                                      N, _p(lut_ws), _p(cnt), _stream(codebook)))
+    return cnt
+
+
+def pick_chunk_keys(rows: int, n_keys: int) -> int:
+    chunk = 2048
+    while chunk < 16384 and rows * ((n_keys + chunk - 1) // chunk) > 1024:
+        chunk *= 2
+    while chunk < 32768 and (n_keys + chunk - 1) // chunk > 512:
+        chunk *= 2
+    return chunk
+
+
+def collision_scan(codebook: torch.Tensor, lut: torch.Tensor, out_dtype=torch.int32, want_hist: bool = False):
+    """Votes per key from a ready table.  Returns (cnt [bs,H,N], chunk_hist or None, chunk_keys)."""
+    _cuda(codebook, lut)
+    bs, H, Bs, N = codebook.shape
+    _need(codebook.dtype == torch.uint8 and Bs == B_SUB, "codebook must be u8 [bs,H,16,N]")
+    _need(lut.dtype == torch.uint8 and lut.is_contiguous() and lut.numel() == bs * H * B_SUB * K_CLUSTERS, "lut: u8 [bs,H,16,256]")
+    cnt = torch.empty(bs, H, N, dtype=out_dtype, device=codebook.device)
+    chunk = pick_chunk_keys(bs * H, N)
+    hist = None
+    if want_hist:
+        hist = torch.empty(bs * H, (N + chunk - 1) // chunk, 128, dtype=torch.int16, device=codebook.device)
+    u8 = cnt if out_dtype == torch.uint8 else None
+    i32 = cnt if out_dtype == torch.int32 else None
+    _need(u8 is not None or i32 is not None, "out_dtype must be uint8 or int32")
+    _lib.check(_lib.lib().pkv_collision_scan(_p(codebook), codebook.stride(0), codebook.stride(1), codebook.stride(3),
+                                             codebook.stride(2), bs, H, N, _p(lut), _p(u8), _p(i32), _p(hist), chunk,
+                                             _stream(codebook)))
+    return cnt, hist, chunk
+
+
+# --------------------------------------------------------------- selections
+
+
+def bucket_topk(x: torch.Tensor, k: int) -> torch.Tensor:
+    """int32 [rows,L] values in [0,127] -> int64 [rows,k]."""
+    _cuda(x)
+    _need(x.dim() == 2, "input must be 2D [B, L]")
+    if x.dtype != torch.int32:
+        x = x.to(torch.int32)
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    rows, L = x.shape
+    _need(k > 0, "k must be positive")
+    _need(k <= L, "k cannot exceed sequence length")
+    out = torch.empty(rows, k, dtype=torch.int64, device=x.device)
+    nbytes = _lib.lib().pkv_bucket_topk_ws_bytes(rows, L)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    _lib.check(_lib.lib().pkv_bucket_topk(_p(x), x.stride(0), rows, L, k, _p(out), _p(ws), nbytes, _stream(x)))
+    return out
+
+
+def topk_f32(x: torch.Tensor, k: int, ids: Optional[torch.Tensor] = None, want_values: bool = False):
+    """Exact top-k of fp32 [rows,L], descending; ties -> smaller ``ids`` (position when None)."""
+    _cuda(x, ids)
+    _need(x.dim() == 2, "input must be 2D [B, L]")
+    if x.dtype != torch.float32:
+        x = x.to(torch.float32)
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    rows, L = x.shape
+    _need(k > 0, "k must be positive")
+    _need(k <= L, "k cannot exceed sequence length")
+    if ids is not None:
+        _need(ids.dtype == torch.int64 and tuple(ids.shape) == (rows, L) and ids.stride(1) == 1, "ids: int64 [rows,L]")
+    out = torch.empty(rows, k, dtype=torch.int64, device=x.device)
+    vals = torch.empty(rows, k, dtype=torch.float32, device=x.device) if want_values else None
+    _lib.check(_lib.lib().pkv_topk_f32(_p(x), x.stride(0), _p(ids), ids.stride(0) if ids is not None else 0, rows, L, k,
+                                       _p(out), _p(vals), None, 0, _stream(x)))
+    return (out, vals) if want_values else out
+
+
+def rerank4(coarse_indices: torch.Tensor, key_4bit: torch.Tensor, key_block_weight: torch.Tensor, qhat: torch.Tensor,
+            qnorm: torch.Tensor, centers: torch.Tensor, want_v4b: bool = False):
+    """fp32 scores [bs,H,C] of the candidates (and optionally the unpacked bf16 values)."""
+    _cuda(coarse_indices, key_4bit, key_block_weight, qhat, qnorm, centers)
+    _need(coarse_indices.dtype == torch.int64 and coarse_indices.is_contiguous(), "coarse_indices must be contiguous int64")
+    _need(key_4bit.dtype == torch.uint8, "key_4bit must be byte tensor")
+    _need(key_block_weight.dtype == torch.bfloat16, "key_block_weight must be bfloat16 tensor")
+    bs, H, Bs, N, nb = key_4bit.shape
+    _need(Bs == B_SUB and nb == 4, "only support B = 16, m = 8")
+    _need(key_4bit.stride(-1) == 1, "key_4bit must be contiguous in the last dimension")
+    _need(tuple(key_block_weight.shape) == (bs, H, Bs, N), "key_block_weight shape mismatch")
+    Cn = coarse_indices.shape[-1]
+    _need(tuple(coarse_indices.shape) == (bs, H, Cn), "coarse_indices must be [bs,H,C]")
+    qhat = qhat.reshape(bs, H, HEAD_DIM)
+    _need(qhat.dtype == torch.float32 and qhat.is_contiguous(), "qhat must be contiguous float32 [bs,H,128]")
+    qnorm = qnorm.reshape(bs, H)
+    _need(qnorm.dtype == torch.float32 and qnorm.is_contiguous(), "qnorm must be contiguous float32 [bs,H]")
+    _need(centers.dtype == torch.float32 and centers.numel() == 8 and centers.is_contiguous(), "centers: float32[8]")
+    scores = torch.empty(bs, H, Cn, dtype=torch.float32, device=key_4bit.device)
+    v4b = torch.empty(bs, H, Bs, Cn, M_SUB, dtype=torch.bfloat16, device=key_4bit.device) if want_v4b else None
+    k4, kw = key_4bit, key_block_weight
+    _lib.check(_lib.lib().pkv_rerank4(
+        _p(coarse_indices), bs, H, Cn, N, _p(k4), k4.stride(0), k4.stride(1), k4.stride(3), k4.stride(2),
+        _p(kw), kw.stride(0), kw.stride(1), kw.stride(3), kw.stride(2), _p(qhat), _p(qnorm), _p(centers), _p(scores),
+        _p(v4b), _stream(k4)))
+    return scores, v4b
+
+
+# ------------------------------------------------------------------ gathers
+
+
+def _gather(fn, src_k, src_v, idx, dst_k, dst_v, idx_offset, dst_row0):
+    bs, H, src_len, D = src_k.shape
+    _need(src_k.shape == src_v.shape and dst_k.shape == dst_v.shape, "K/V shape mismatch")
+    _need(src_k.dtype == src_v.dtype == dst_k.dtype == dst_v.dtype, "K/V dtype mismatch")
+    _need(idx.dtype == torch.int64 and idx.is_cuda and idx.is_contiguous() and tuple(idx.shape[:2]) == (bs, H),
+          "selected_indices must be contiguous int64 [bs,H,K] on the GPU")
+    for t in (src_k, src_v, dst_k, dst_v):
+        _need(t.is_contiguous(), "K/V buffers must be contiguous")
+    _need(dst_k.is_cuda and dst_v.is_cuda and tuple(dst_k.shape[:2]) == (bs, H) and dst_k.shape[3] == D, "dst shape mismatch")
+    k = idx.shape[2]
+    row_bytes = D * src_k.element_size()
+    _lib.check(fn(_p(src_k), _p(src_v), src_len, _p(idx), k, idx_offset, _p(dst_k), _p(dst_v), dst_k.shape[2], dst_row0,
+                  bs, H, row_bytes, _stream(dst_k)))
+
+
+def gather_uva(src_k, src_v, idx, dst_k, dst_v, idx_offset: int = 0, dst_row0: int = 0) -> None:
+    """dst[b,h,dst_row0+i,:] = src[b,h,idx[b,h,i]+idx_offset,:] with src in pinned host memory."""
+    _need(src_k.is_cpu and src_v.is_cpu and src_k.is_pinned() and src_v.is_pinned(), "src must be pinned CPU tensors")
+    _gather(_lib.lib().pkv_gather_uva, src_k, src_v, idx, dst_k, dst_v, idx_offset, dst_row0)
+
+
+def gather_hbm(src_k, src_v, idx, dst_k, dst_v, idx_offset: int = 0, dst_row0: int = 0) -> None:
+    _need(src_k.is_cuda and src_v.is_cuda, "src must be GPU tensors")
+    _gather(_lib.lib().pkv_gather_hbm, src_k, src_v, idx, dst_k, dst_v, idx_offset, dst_row0)
+
+
+def gather_uva_packed(src_k, src_v, k_packed, v_packed, indices_packed, cu_seqlens_topk, cu_seqlens_k,
+                      sink_local_end: int, global_k: int) -> None:
+    bs, H, src_len, D = src_k.shape
+    _need(k_packed.is_cuda and v_packed.is_cuda and k_packed.is_contiguous() and v_packed.is_contiguous(), "packed dst on GPU")
+    _need(indices_packed.dtype == torch.int64 and cu_seqlens_topk.dtype == torch.int32 and cu_seqlens_k.dtype == torch.int32,
+          "indices int64, cu_seqlens int32")
+    _need(cu_seqlens_topk.numel() == bs * H + 1 and cu_seqlens_k.numel() == bs * H + 1, "cu_seqlens must have V+1 entries")
+    total_k = k_packed.shape[0]
+    _lib.check(_lib.lib().pkv_gather_uva_packed(
+        _p(src_k), _p(src_v), src_len, _p(indices_packed), _p(cu_seqlens_topk), _p(cu_seqlens_k), sink_local_end,
+        max(1, global_k), _p(k_packed), _p(v_packed), total_k, bs, H, D * src_k.element_size(), _stream(k_packed)))
+
+
+def gather_cpu(src: torch.Tensor, index: torch.Tensor, out: torch.Tensor, n_threads: int = 1) -> None:
+    """Host gather [B,H,N,D] -> [B,H,K,D] (cache_hub/gather/gather_cpu.cpp contract)."""
+    _need(src.is_cpu and index.is_cpu and out.is_cpu, "src, index and out must be on CPU")
+    _need(src.dim() == 4 and index.dim() == 3 and out.dim() == 4, "src [B,H,N,D], index [B,H,K], out [B,H,K,D]")
+    _need(index.dtype == torch.int64 and index.is_contiguous(), "index must be contiguous int64")
+    _need(src.dtype == out.dtype, "src/out dtype must match")
+    Bn, H, N, D = src.shape
+    K = index.shape[2]
+    _need(tuple(index.shape[:2]) == (Bn, H) and tuple(out.shape) == (Bn, H, K, D), "shape mismatch")
+    ss = (C.c_int64 * 4)(*src.stride())
+    os_ = (C.c_int64 * 4)(*out.stride())
+    _lib.check(_lib.lib().pkv_gather_cpu(_p(src), ss, _p(index), _p(out), os_, Bn, H, N, D, K, src.element_size(), n_threads))
+
+
+# ------------------------------------------------------- fused decode step
+
+
+class RetrievePlan:
+    """Persistent workspace + argument block for :func:`pkv_retrieve` on key-major storage."""
+
+    def __init__(self, bs: int, n_kv_heads: int, group: int, cap: int, device, max_keys: int, max_cand: int, max_k: int):
+        self.bs, self.H, self.group, self.cap, self.device = bs, n_kv_heads, group, cap, device
+        self.rows = bs * n_kv_heads
+        nbytes = _lib.lib().pkv_retrieve_ws_bytes(self.rows, max_keys, max_cand, max_k)
+        _need(nbytes > 0, "bad retrieval shape")
+        # the layout depends on (n_keys, n_cand); size for the worst case of each segment
+        self.ws = torch.empty(int(nbytes) + (1 << 16), dtype=torch.uint8, device=device)
+        self.max = (max_keys, max_cand, max_k)
+
+    def run(self, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, k,
+            out_ids=None, out_scores=None, gather=None):
+        """Returns out_ids int64 [bs,H,k].  ``gather`` = dict(src_k, src_v, from_host, idx_offset, dst_k, dst_v, dst_row0)."""
+        lib = _lib.lib()
+        need = lib.pkv_retrieve_ws_bytes(self.rows, n_keys, n_cand, k)
+        _need(need > 0, "need 0 < k <= n_cand <= n_keys")
+        if need > self.ws.numel():
+            self.ws = torch.empty(int(need), dtype=torch.uint8, device=self.device)
+        q = queries.reshape(self.bs, -1, HEAD_DIM)
+        _need(q.is_contiguous() and q.shape[1] == self.H * self.group, "queries must be contiguous [bs,1,Hq,128]")
+        if out_ids is None:
+            out_ids = torch.empty(self.bs, self.H, k, dtype=torch.int64, device=self.device)
+        a = _lib.RetrieveArgs()
+        a.q, a.dtype, a.bs, a.n_kv_heads, a.group = q.data_ptr(), _dt(q.dtype), self.bs, self.H, self.group
+        a.signs, a.centers, a.cluster_counts = signs.data_ptr(), centers.data_ptr(), cluster_counts.data_ptr()
+        _need(cluster_counts.is_contiguous(), "cluster_counts must be contiguous")
+        for t in (codes_km, nib_km, w_km):
+            _need(t.is_contiguous() and t.shape[2] == self.cap, "key-major storage must be contiguous [bs,H,cap,*]")
+        a.codes, a.nib, a.weight = codes_km.data_ptr(), nib_km.data_ptr(), w_km.data_ptr()
+        a.cap, a.key0, a.n_keys = self.cap, key0, n_keys
+        for i, t in enumerate(tier_counts):
+            a.tier_counts[i] = int(t)
+        a.n_tiers, a.n_cand, a.k = len(tier_counts), n_cand, k
+        a.out_ids = out_ids.data_ptr()
+        a.out_scores = out_scores.data_ptr() if out_scores is not None else None
+        if gather is not None:
+            sk, sv, dk, dv = gather["src_k"], gather["src_v"], gather["dst_k"], gather["dst_v"]
+            a.src_k, a.src_v, a.gather_from_host = sk.data_ptr(), sv.data_ptr(), int(bool(gather["from_host"]))
+            a.src_len, a.idx_offset = sk.shape[2], int(gather.get("idx_offset", 0))
+            a.dst_k, a.dst_v, a.dst_len, a.dst_row0 = dk.data_ptr(), dv.data_ptr(), dk.shape[2], int(gather.get("dst_row0", 0))
+            a.row_bytes = sk.shape[3] * sk.element_size()
+        _lib.check(lib.pkv_retrieve(C.byref(a), _p(self.ws), self.ws.numel(), _stream(self.ws)))
+        return out_ids
+
+    def view(self, name: str, n_keys: int, n_cand: int, k: int, dtype: torch.dtype) -> torch.Tensor:
+        """An intermediate of the last :meth:`run` (qhat, qnorm, lut, cnt_u8, chunk_hist, cand, scores)."""
+        ptr, nbytes = C.c_void_p(), C.c_size_t()
+        _lib.check(_lib.lib().pkv_retrieve_ws_view(_p(self.ws), self.rows, n_keys, n_cand, k, name.encode(), C.byref(ptr),
+                                                   C.byref(nbytes)))
+        off = ptr.value - self.ws.data_ptr()
+        return self.ws[off:off + nbytes.value].view(dtype)

@@ -1,0 +1,551 @@
+"""GPU parity tests: every HIP entry point, called through the C ABI, against the
+CPU oracle on identical seeded inputs.
+
+Bar: bit-exact for codes, nibbles, weights (bf16 bits), vote counts, candidate
+lists and final top-k indices; rerank scores within 1e-5 relative of the oracle
+(they are in fact evaluated in the same order, so equality is also asserted).
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import workloads as W
+from oracle import pkv_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from pariskv_amd import ops as _ops
+
+    return _ops
+
+
+@pytest.fixture(scope="module")
+def wl_cfg1():
+    return W.cfg1()
+
+
+@pytest.fixture(scope="module")
+def wl_cfg2():
+    return W.cfg2()
+
+
+@pytest.fixture(scope="module")
+def wl_small_bf16():
+    # ragged length (not a multiple of any tile), 2 sequences
+    return W.make_workload("small", 2, 2, 4, 5000 + 37, 333, 100, O.BF16, 0.5, seed0=5)
+
+
+def _say(msg):
+    print(msg, flush=True)
+
+
+# ------------------------------------------------------------------- encode
+
+
+@pytest.mark.parametrize("dtype", [O.F32, O.BF16])
+@pytest.mark.parametrize("layout", ["keymajor", "reference"])
+def test_encode_append_bit_exact(ops, dtype, layout):
+    _say(f"encode dtype={dtype} layout={layout}")
+    bs, H, S = 2, 3, 1000 + 13
+    tdt = torch.bfloat16 if dtype == O.BF16 else torch.float32
+    signs = O.srht_signs(42)
+    keys = np.stack([O.synth_keys(S, 100 + r, bf16=dtype == O.BF16) for r in range(bs * H)]).reshape(bs, H, S, 128)
+    keys[0, 0, 5] = 0.0  # a zero key must not produce NaNs
+    tk = torch.from_numpy(keys).to(tdt).to(DEV)
+    if layout == "keymajor":
+        _, _, _, cb, k4, kw = ops.alloc_keymajor(bs, H, S, DEV)
+    else:
+        cb = torch.zeros(bs, H, 16, S, dtype=torch.uint8, device=DEV)
+        k4 = torch.zeros(bs, H, 16, S, 4, dtype=torch.uint8, device=DEV)
+        kw = torch.zeros(bs, H, 16, S, dtype=torch.bfloat16, device=DEV)
+    cc = torch.zeros(bs, H, 16, 256, dtype=torch.int32, device=DEV)
+    ops.encode_append(tk, torch.from_numpy(signs).to(DEV), cb, k4, kw, cc)
+    ops.encode_append(tk[:, :, :100], torch.from_numpy(signs).to(DEV), cb[..., :100], k4[:, :, :, :100], kw[..., :100], cc)
+    torch.cuda.synchronize()
+    for r in range(bs * H):
+        b, h = divmod(r, H)
+        codes, nib, w = O.encode(keys[b, h], signs, dtype)
+        assert np.array_equal(cb[b, h].cpu().numpy().T, codes)
+        assert np.array_equal(k4[b, h].cpu().numpy().transpose(1, 0, 2), nib)
+        assert np.array_equal(kw[b, h].float().cpu().numpy().T, w)
+        ref_cc = O.count_cluster_keys(codes)
+        ref_cc = O.count_cluster_keys(codes[:100], ref_cc)  # += semantics
+        assert np.array_equal(cc[b, h].cpu().numpy(), ref_cc)
+    # count_cluster_keys on its own
+    cc2 = torch.zeros_like(cc)
+    ops.count_cluster_keys(cb, cc2)
+    ops.count_cluster_keys(cb[..., :100], cc2)
+    assert torch.equal(cc2, cc)
+
+
+def test_encode_without_rabitq_outputs(ops):
+    S = 300
+    signs = O.srht_signs(42)
+    keys = O.synth_keys(S, 9)
+    cb = torch.zeros(1, 1, 16, S, dtype=torch.uint8, device=DEV)
+    ops.encode_append(torch.from_numpy(keys).view(1, 1, S, 128).to(DEV), torch.from_numpy(signs).to(DEV), cb, None, None, None)
+    assert np.array_equal(cb[0, 0].cpu().numpy().T, O.encode(keys, signs, O.F32)[0])
+
+
+# --------------------------------------------------------------- query side
+
+
+@pytest.mark.parametrize("wl_name", ["wl_cfg1", "wl_small_bf16"])
+def test_query_prep_lut_bit_exact(ops, request, wl_name):
+    w = request.getfixturevalue(wl_name)
+    _say(f"query_prep_lut {w.name}")
+    d = W.to_device(w, DEV, torch)
+    qhat, qnorm, lut, ids = ops.query_prep_lut(d["queries"], w.H, d["signs"], d["cluster_counts"], w.tiers, want_sorted_ids=True)
+    torch.cuda.synchronize()
+    for r in range(w.R):
+        st = W.oracle_stages(w, r)
+        b, h = divmod(r, w.H)
+        assert np.array_equal(qhat[b, h].cpu().numpy().view(np.uint32), st["qhat"].view(np.uint32))
+        assert np.float32(qnorm[b, h].item()) == np.float32(st["qnorm"])
+        assert np.array_equal(ids[b, h].cpu().numpy(), st["sorted_ids"])
+        assert np.array_equal(lut[b, h].cpu().numpy(), st["lut"])
+
+
+def test_query_prep_single_tier_and_group1(ops, wl_cfg1):
+    w = wl_cfg1
+    d = W.to_device(w, DEV, torch)
+    q1 = d["queries"].view(w.bs, w.H, w.G, 128)[:, :, 0].contiguous()  # group size 1
+    qhat, qnorm, lut, ids = ops.query_prep_lut(q1.view(w.bs, w.H, 128), w.H, d["signs"], d["cluster_counts"], [500], True)
+    torch.cuda.synchronize()
+    for r in range(w.R):
+        qh, qn = O.query_prep(w.queries[0, r * w.G:r * w.G + 1], w.signs, w.dtype)
+        lut_ref = O.tier_lut(O.rank_centroids(qh, w.dtype), w.cluster_counts[r], [500])
+        assert np.array_equal(lut[0, r].cpu().numpy(), lut_ref) and lut_ref.max() == 1
+
+
+def _collision_recipe(bs, kv_heads, kv_len, seed=42):
+    """Input recipe of the reference's collision self-test (collision_fused/collision_test.py:16-53)."""
+    torch.manual_seed(seed)
+    ids = torch.stack([torch.stack([torch.stack([torch.randperm(256) for _ in range(16)])
+                                    for _ in range(kv_heads)]) for _ in range(bs)]).to(torch.int64)
+    counts = torch.randint(1, max(2, kv_len // 2), (bs, kv_heads, 16, 256), dtype=torch.int32)
+    codebook = torch.randint(0, 256, (bs, kv_heads, 16, kv_len), dtype=torch.int32).to(torch.uint8)
+    return ids, counts, codebook
+
+
+@pytest.mark.parametrize("kv_len,ratio,ntier", [(2048, 0.2, 6), (4999, 0.5, 6), (2048, 0.3, 1), (70001, 0.2, 6)])
+@pytest.mark.parametrize("layout", ["reference", "keymajor"])
+def test_update_cache_cnt_interface(ops, kv_len, ratio, ntier, layout):
+    from pariskv_amd.cache_hub.collision_fused import update_cache_cnt_cuda_interface
+
+    _say(f"update_cache_cnt kv_len={kv_len} ntier={ntier} layout={layout}")
+    bs, H = 2, 3
+    ids, counts, codebook = _collision_recipe(bs, H, kv_len)
+    ratios = list(O.TIER_RATIOS) if ntier == 6 else [1.0]
+    tiers = O.tier_counts(kv_len, ratio, ratios)
+    cb = codebook.to(DEV)
+    if layout == "keymajor":
+        cb = cb.permute(0, 1, 3, 2).contiguous().permute(0, 1, 3, 2)  # same logical tensor, key-major memory
+    cnt = update_cache_cnt_cuda_interface(ids.to(DEV), counts.to(DEV), cb, tiers)
+    torch.cuda.synchronize()
+    assert cnt.dtype == torch.int32 and tuple(cnt.shape) == (bs, H, kv_len)
+    for b in range(bs):
+        for h in range(H):
+            lut = O.tier_lut(ids[b, h].numpy(), counts[b, h].numpy(), tiers)
+            ref = O.collision_count(np.ascontiguousarray(codebook[b, h].numpy().T), lut)
+            assert np.array_equal(cnt[b, h].cpu().numpy(), ref)
+
+
+def test_update_cache_cnt_sliced_views(ops):
+    """The cache passes slices [.., start:end] of larger tensors (polar_cache.py:1051-1055)."""
+    from pariskv_amd.cache_hub.collision_fused import update_cache_cnt_cuda_interface
+
+    bs, H, cap, s, e = 1, 2, 3000, 129, 2777
+    ids, counts, codebook = _collision_recipe(bs, H, cap)
+    tiers = O.tier_counts(e - s, 0.5)
+    for layout in ("reference", "keymajor"):
+        cb = codebook.to(DEV)
+        if layout == "keymajor":
+            cb = cb.permute(0, 1, 3, 2).contiguous().permute(0, 1, 3, 2)
+        cnt = update_cache_cnt_cuda_interface(ids.to(DEV), counts.to(DEV), cb[:, :, :, s:e], tiers)
+        for h in range(H):
+            lut = O.tier_lut(ids[0, h].numpy(), counts[0, h].numpy(), tiers)
+            ref = O.collision_count(np.ascontiguousarray(codebook[0, h, :, s:e].numpy().T), lut)
+            assert np.array_equal(cnt[0, h].cpu().numpy(), ref)
+
+
+def test_update_cache_cnt_legacy(ops):
+    from pariskv_amd.cache_hub.collision.collision import update_cache_cnt_cuda
+
+    bs, H, N = 1, 4, 3001
+    torch.manual_seed(42)  # recipe of collision/collision.py:11-26
+    ids = torch.stack([torch.stack([torch.stack([torch.randperm(256) for _ in range(16)]) for _ in range(H)])
+                       for _ in range(bs)]).to(torch.int32)
+    topk_cnt = torch.randint(1, 256, (bs, H, 16), dtype=torch.int32)
+    codebook = torch.randint(0, 256, (bs, H, 16, N), dtype=torch.int32)
+    cnt = update_cache_cnt_cuda(ids.to(DEV), topk_cnt.to(DEV), codebook.to(DEV)).cpu()
+    # membership form of collision/collision.py:29-45
+    for h in range(H):
+        ref = np.zeros(N, np.int32)
+        for b in range(16):
+            sel = set(ids[0, h, b, :int(topk_cnt[0, h, b])].tolist())
+            ref += np.isin(codebook[0, h, b].numpy(), list(sel)).astype(np.int32)
+        assert np.array_equal(cnt[0, h].numpy(), ref)
+
+
+def test_interface_errors(ops):
+    from pariskv_amd.cache_hub.collision_fused import update_cache_cnt_cuda_interface
+    from pariskv_amd.cache_hub.topk import load_radix_topk_ext
+
+    ids, counts, codebook = _collision_recipe(1, 1, 512)
+    with pytest.raises(RuntimeError, match="uint8"):
+        update_cache_cnt_cuda_interface(ids.to(DEV), counts.to(DEV), codebook.to(torch.int32).to(DEV), [10])
+    with pytest.raises(RuntimeError, match="int64"):
+        update_cache_cnt_cuda_interface(ids.to(torch.int32).to(DEV), counts.to(DEV), codebook.to(DEV), [10])
+    with pytest.raises(RuntimeError, match="tier_num"):
+        update_cache_cnt_cuda_interface(ids.to(DEV), counts.to(DEV), codebook.to(DEV), [])
+    ext = load_radix_topk_ext()
+    x = torch.zeros(2, 100, dtype=torch.int32, device=DEV)
+    with pytest.raises(RuntimeError, match="exceed"):
+        ext.bucket_topk(x, 101)
+    with pytest.raises(RuntimeError, match="positive"):
+        ext.radix_topk(x.float(), 0)
+    with pytest.raises(RuntimeError, match="3D"):
+        ext.radix_topk_3d(x, 5)
+
+
+# --------------------------------------------------------------- selections
+
+
+@pytest.mark.parametrize("rows,L,k", [(8, 8192, 1024), (3, 5037, 333), (2, 2048, 2048), (4, 100000, 5000), (1, 300, 1),
+                                      (2, 4096, 4095)])
+def test_bucket_and_radix_topk_on_counts(ops, rows, L, k):
+    from pariskv_amd.cache_hub.topk import load_radix_topk_ext
+
+    _say(f"bucket_topk rows={rows} L={L} k={k}")
+    ext = load_radix_topk_ext()
+    rng = np.random.default_rng(L + k)
+    x = rng.binomial(96, 0.1, size=(rows, L)).astype(np.int32)
+    tx = torch.from_numpy(x).to(DEV)
+    out_b = ext.bucket_topk(tx, k).cpu().numpy()
+    out_r = ext.radix_topk_3d(tx.view(1, rows, L), k).cpu().numpy()[0]  # hot call of polar_cache.py:1241
+    assert out_b.dtype == np.int64
+    for r in range(rows):
+        ref, _ = O.select_candidates(x[r], k)
+        assert np.array_equal(out_b[r], ref)
+        assert np.array_equal(out_r[r], ref)
+        tv = torch.topk(torch.from_numpy(x[r]), k).values.numpy()  # the reference's own check: same value multiset
+        assert np.array_equal(np.sort(x[r][out_b[r]]), np.sort(tv))
+
+
+def test_bucket_topk_all_equal_and_clamp(ops):
+    x = torch.full((2, 3000), 7, dtype=torch.int32, device=DEV)
+    assert torch.equal(ops.bucket_topk(x, 50).cpu(), torch.arange(50).expand(2, 50))
+    y = torch.tensor([[500, -3, 4, 127, 128, 0, 9, 9]], dtype=torch.int32, device=DEV)
+    assert ops.bucket_topk(y, 3).cpu().tolist() == [[0, 3, 4]]  # values clamp to [0,127]: 500,127,128 tie at 127
+
+
+@pytest.mark.parametrize("rows,L,k", [(32, 4096, 1024), (8, 1024, 256), (3, 777, 100), (2, 8192, 8192), (4, 20000, 2048),
+                                      (2, 105000, 2048), (1, 9000, 1)])
+def test_topk_f32_exact(ops, rows, L, k):
+    _say(f"topk_f32 rows={rows} L={L} k={k}")
+    rng = np.random.default_rng(L * 7 + k)
+    x = rng.standard_normal((rows, L)).astype(np.float32)
+    x[:, ::5] = np.round(x[:, ::5], 1)  # exact ties
+    ids = np.stack([rng.permutation(4 * L)[:L] for _ in range(rows)]).astype(np.int64)
+    tx, tid = torch.from_numpy(x).to(DEV), torch.from_numpy(ids).to(DEV)
+    out, vals = ops.topk_f32(tx, k, tid, want_values=True)
+    out_pos = ops.topk_f32(tx, k)
+    torch.cuda.synchronize()
+    for r in range(rows):
+        ref_ids, ref_pos = O.topk_f32(x[r], ids[r], k)
+        assert np.array_equal(out[r].cpu().numpy(), ref_ids)
+        assert np.array_equal(vals[r].cpu().numpy(), x[r][ref_pos])
+        assert np.array_equal(out_pos[r].cpu().numpy(), O.topk_f32(x[r], None, k)[1])
+    tv = torch.topk(tx, k, dim=-1).values  # same values, same order as torch.topk
+    assert torch.equal(vals, tv)
+
+
+def test_radix_topk_float_api(ops):
+    from pariskv_amd.cache_hub.topk import radix_topk, fast_topk, fast_topk_with_ratio
+
+    g = torch.Generator().manual_seed(0)
+    x = torch.rand(4, 3000, generator=g) * 96
+    out = radix_topk(x.to(DEV), 64).cpu()
+    assert torch.equal(torch.gather(x, 1, out), torch.topk(x, 64).values)
+    xi = (x * 1).to(torch.int32)
+    assert fast_topk(xi.to(DEV), 64).shape == (4, 64)
+    assert fast_topk_with_ratio(xi.to(DEV).view(2, 2, 3000), 0.05).shape == (2, 2, 150)
+
+
+# ------------------------------------------------------------------- rerank
+
+
+@pytest.mark.parametrize("layout", ["keymajor", "reference"])
+def test_partial_rerank_parity(ops, wl_small_bf16, layout):
+    from pariskv_amd.cache_hub.rerank.rerank import partial_rerank_cuda
+
+    w = wl_small_bf16
+    _say(f"rerank layout={layout}")
+    d = W.to_device(w, DEV, torch)
+    k4 = d["nib_km"].view(w.bs, w.H, w.N, 16, 4).permute(0, 1, 3, 2, 4)
+    kw = d["w_km"].permute(0, 1, 3, 2)
+    if layout == "reference":
+        k4, kw = k4.contiguous(), kw.contiguous()
+    rng = np.random.default_rng(1)
+    cand = np.stack([rng.permutation(w.N)[:w.C] for _ in range(w.R)]).astype(np.int64).reshape(w.bs, w.H, w.C)
+    stages = [W.oracle_stages(w, r) for r in range(w.R)]
+    q_blocks = torch.from_numpy(np.stack([s["qhat"] for s in stages])).view(w.bs, w.H, 16, 8).to(torch.bfloat16).to(DEV)
+    q_norm = torch.tensor([s["qnorm"] for s in stages]).view(w.bs, w.H, 1).to(torch.bfloat16).to(DEV)
+    centers = torch.tensor(ops.MAG_CENTERS, dtype=torch.bfloat16, device=DEV)
+    scores, v4b = partial_rerank_cuda(torch.from_numpy(cand).to(DEV), k4, kw, q_blocks, q_norm, centers, 16, 8)
+    torch.cuda.synchronize()
+    assert scores.dtype == torch.float32 and tuple(v4b.shape) == (w.bs, w.H, 16, w.C, 8)
+    th, ce = O.mag_constants()
+    for r in range(w.R):
+        b, h = divmod(r, w.H)
+        ref = O.rerank(cand[b, h], w.nib[r], w.weight[r], stages[r]["qhat"], stages[r]["qnorm"])
+        got = scores[b, h].cpu().numpy()
+        np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-5 * np.abs(ref).max())  # the stated tolerance
+        assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))                 # and in fact identical
+        # unpacked values (reference's second output): +-centers by nibble
+        nibs = w.nib[r][cand[b, h]]  # [C,16,4]
+        v = np.stack([nibs & 0x0F, nibs >> 4], axis=-1).reshape(w.C, 16, 8)
+        ref_v = np.where(v & 8, 1.0, -1.0).astype(np.float32) * ce[v & 7]
+        assert np.array_equal(v4b[b, h].float().cpu().numpy(), ref_v.transpose(1, 0, 2))
+
+
+def test_rerank_out_of_range_candidate_is_masked(ops, wl_small_bf16):
+    w = wl_small_bf16
+    d = W.to_device(w, DEV, torch)
+    k4 = d["nib_km"].view(w.bs, w.H, w.N, 16, 4).permute(0, 1, 3, 2, 4)
+    kw = d["w_km"].permute(0, 1, 3, 2)
+    cand = torch.tensor([0, w.N - 1, w.N, -1, 5], dtype=torch.int64, device=DEV).expand(w.bs, w.H, 5).contiguous()
+    qhat = torch.zeros(w.bs, w.H, 128, device=DEV)
+    scores, _ = ops.rerank4(cand, k4, kw, qhat, torch.ones(w.bs, w.H, device=DEV), ops.mag_centers(DEV))
+    s = scores[0, 0].cpu()
+    assert torch.isinf(s[2]) and torch.isinf(s[3]) and s[0] == 0 and s[1] == 0 and s[4] == 0
+
+
+# ------------------------------------------------------------------ gathers
+
+
+def test_h2d_gather_kv_matches_index_select(ops):
+    from pariskv_amd.cache_hub.gather_trans import h2d_gather_kv
+
+    bs, heads, kv_len, topk, max_topk = 2, 8, 32 * 1024, 100, 160  # shape of trans_h2d.py:108-120
+    g = torch.Generator().manual_seed(0)
+    src_k = torch.randn(bs, heads, kv_len, 128, generator=g).to(torch.bfloat16).pin_memory()
+    src_v = torch.randn(bs, heads, kv_len, 128, generator=g).to(torch.bfloat16).pin_memory()
+    idx = torch.randint(0, kv_len, (bs, heads, topk), generator=g)
+    dst_k = torch.zeros(bs, heads, max_topk, 128, dtype=torch.bfloat16, device=DEV)
+    dst_v = torch.zeros_like(dst_k)
+    h2d_gather_kv(src_k, src_v, idx.to(DEV), dst_k, dst_v)
+    torch.cuda.synchronize()
+    ek = torch.gather(src_k, 2, idx.unsqueeze(-1).expand(-1, -1, -1, 128))
+    ev = torch.gather(src_v, 2, idx.unsqueeze(-1).expand(-1, -1, -1, 128))
+    assert torch.equal(dst_k[:, :, :topk].cpu().view(torch.int16), ek.view(torch.int16))
+    assert torch.equal(dst_v[:, :, :topk].cpu().view(torch.int16), ev.view(torch.int16))
+    assert not dst_k[:, :, topk:].any()  # rows beyond topk untouched
+    # oracle gather on one row
+    ref = O.gather_rows(src_k[1, 3].view(torch.int16).numpy(), idx[1, 3].numpy())
+    assert np.array_equal(dst_k[1, 3, :topk].cpu().view(torch.int16).numpy(), ref)
+    with pytest.raises(AssertionError):
+        h2d_gather_kv(src_k.clone(), src_v, idx.to(DEV), dst_k, dst_v)  # unpinned source
+
+
+def test_gather_hbm_with_offset_and_bounds(ops):
+    bs, H, n, k = 1, 2, 500, 40
+    g = torch.Generator().manual_seed(1)
+    sk = torch.randn(bs, H, n, 128, generator=g).to(torch.bfloat16).to(DEV)
+    sv = torch.randn(bs, H, n, 128, generator=g).to(torch.bfloat16).to(DEV)
+    idx = torch.randint(0, n - 20, (bs, H, k), generator=g)
+    idx[0, 0, 0] = n  # out of range after the offset -> zero row, no fault
+    dk = torch.ones(bs, H, 64, 128, dtype=torch.bfloat16, device=DEV)
+    dv = torch.ones_like(dk)
+    ops.gather_hbm(sk, sv, idx.to(DEV), dk, dv, idx_offset=20, dst_row0=8)
+    torch.cuda.synchronize()
+    exp = torch.gather(sk.cpu(), 2, (idx + 20).clamp(max=n - 1).unsqueeze(-1).expand(-1, -1, -1, 128))
+    exp[0, 0, 0] = 0
+    assert torch.equal(dk[:, :, 8:8 + k].cpu(), exp) and (dk[:, :, :8] == 1).all() and (dk[:, :, 8 + k:] == 1).all()
+
+
+def test_gather_uva_packed_layout(ops):
+    """Ragged gather contract of polar_cache_adaptivek_varlen.py:1573-1644."""
+    bs, H, n, sl_end = 2, 2, 1000, 6
+    V = bs * H
+    g = torch.Generator().manual_seed(2)
+    ks = torch.tensor([5, 0, 17, 9])
+    src_k = torch.randn(bs, H, n, 128, generator=g).to(torch.bfloat16).pin_memory()
+    src_v = torch.randn(bs, H, n, 128, generator=g).to(torch.bfloat16).pin_memory()
+    idx_packed = torch.randint(0, n, (int(ks.sum()),), generator=g)
+    cu_topk = torch.zeros(V + 1, dtype=torch.int32)
+    cu_topk[1:] = torch.cumsum(ks, 0)
+    cu_k = torch.zeros(V + 1, dtype=torch.int32)
+    cu_k[1:] = torch.cumsum(ks + sl_end, 0)
+    total = int(cu_k[-1])
+    kp = torch.zeros(total, 128, dtype=torch.bfloat16, device=DEV)
+    vp = torch.zeros_like(kp)
+    ops.gather_uva_packed(src_k, src_v, kp, vp, idx_packed.to(DEV), cu_topk.to(DEV), cu_k.to(DEV), sl_end, int(ks.max()))
+    torch.cuda.synchronize()
+    exp_k = torch.zeros(total, 128, dtype=torch.bfloat16)
+    exp_v = torch.zeros_like(exp_k)
+    for v in range(V):
+        b, h = divmod(v, H)
+        for s in range(int(ks[v])):
+            src = int(idx_packed[int(cu_topk[v]) + s])
+            exp_k[int(cu_k[v]) + sl_end + s] = src_k[b, h, src]
+            exp_v[int(cu_k[v]) + sl_end + s] = src_v[b, h, src]
+    assert torch.equal(kp.cpu(), exp_k) and torch.equal(vp.cpu(), exp_v)
+
+
+# ------------------------------------------------------- fused decode step
+
+
+def _run_fused(ops, w, gather_host=False):
+    d = W.to_device(w, DEV, torch)
+    plan = ops.RetrievePlan(w.bs, w.H, w.G, w.N, DEV, w.N, w.C, w.K)
+    scores = torch.empty(w.bs, w.H, w.K, dtype=torch.float32, device=DEV)
+    out = plan.run(d["queries"], d["signs"], d["centers"], d["cluster_counts"], d["codes_km"], d["nib_km"], d["w_km"], 0,
+                   w.N, w.tiers, w.C, w.K, out_scores=scores)
+    torch.cuda.synchronize()
+    return plan, out, scores
+
+
+@pytest.mark.parametrize("wl_name", ["wl_cfg1", "wl_cfg2", "wl_small_bf16"])
+def test_retrieve_fused_matches_oracle(ops, request, wl_name):
+    w = request.getfixturevalue(wl_name)
+    _say(f"retrieve {w.name}: R={w.R} N={w.N} C={w.C} K={w.K}")
+    plan, out, scores = _run_fused(ops, w)
+    cnt_stride = (w.N + 15) // 16 * 16
+    cnt = plan.view("cnt_u8", w.N, w.C, w.K, torch.uint8).view(w.R, cnt_stride)[:, :w.N].cpu().numpy()
+    cand = plan.view("cand", w.N, w.C, w.K, torch.int64).view(w.R, w.C).cpu().numpy()
+    sc = plan.view("scores", w.N, w.C, w.K, torch.float32).view(w.R, w.C).cpu().numpy()
+    hist = plan.view("chunk_hist", w.N, w.C, w.K, torch.int16).view(w.R, -1, 128).cpu().numpy().astype(np.int64) & 0xFFFF
+    for r in range(w.R):
+        b, h = divmod(r, w.H)
+        st = W.oracle_stages(w, r)
+        assert np.array_equal(cnt[r], st["cnt"].astype(np.uint8)), f"vote counts differ in row {r}"
+        assert np.array_equal(hist[r].sum(axis=0), np.bincount(st["cnt"], minlength=128)), f"histogram row {r}"
+        assert np.array_equal(cand[r], st["cand"]), f"candidate list differs in row {r}"
+        np.testing.assert_allclose(sc[r], st["scores"], rtol=1e-5, atol=1e-5 * np.abs(st["scores"]).max())
+        assert np.array_equal(out[b, h].cpu().numpy(), st["final"]), f"final top-k differs in row {r}"
+        assert np.array_equal(scores[b, h].cpu().numpy(), st["final_scores"])
+        # whole-row oracle entry point agrees as well
+        q = w.queries[b, h * w.G:(h + 1) * w.G]
+        whole = O.retrieve_row(q, w.signs, w.dtype, w.codes[r], w.nib[r], w.weight[r], w.cluster_counts[r], w.tiers, w.C, w.K)
+        assert np.array_equal(out[b, h].cpu().numpy(), whole)
+
+
+def test_retrieve_subrange_and_candidates_equal_keys(ops, wl_small_bf16):
+    """Retrieval zone = [key0, key0+n) of a larger capacity; and C == N (identity candidates)."""
+    w = wl_small_bf16
+    d = W.to_device(w, DEV, torch)
+    key0, n = 64, 2000
+    plan = ops.RetrievePlan(w.bs, w.H, w.G, w.N, DEV, w.N, w.N, 64)
+    tiers = O.tier_counts(n, 0.5)
+    out = plan.run(d["queries"], d["signs"], d["centers"], d["cluster_counts"], d["codes_km"], d["nib_km"], d["w_km"], key0,
+                   n, tiers, 200, 64)
+    out_all = plan.run(d["queries"], d["signs"], d["centers"], d["cluster_counts"], d["codes_km"], d["nib_km"], d["w_km"],
+                       key0, n, tiers, n, 64)
+    torch.cuda.synchronize()
+    for r in range(w.R):
+        b, h = divmod(r, w.H)
+        q = w.queries[b, h * w.G:(h + 1) * w.G]
+        sl = slice(key0, key0 + n)
+        ref = O.retrieve_row(q, w.signs, w.dtype, w.codes[r][sl], w.nib[r][sl], w.weight[r][sl], w.cluster_counts[r], tiers, 200, 64)
+        assert np.array_equal(out[b, h].cpu().numpy(), ref)
+        qhat, qn = O.query_prep(q, w.signs, w.dtype)
+        s_all = O.rerank(np.arange(n), w.nib[r][sl], w.weight[r][sl], qhat, qn)
+        assert np.array_equal(out_all[b, h].cpu().numpy(), O.topk_f32(s_all, None, 64)[0])
+
+
+def test_retrieve_with_uva_gather(ops, wl_small_bf16):
+    w = wl_small_bf16
+    d = W.to_device(w, DEV, torch)
+    kcpu = torch.from_numpy(w.keys.reshape(w.bs, w.H, w.N, 128)).to(torch.bfloat16).pin_memory()
+    vcpu = torch.from_numpy(w.values.reshape(w.bs, w.H, w.N, 128)).to(torch.bfloat16).pin_memory()
+    dk = torch.zeros(w.bs, w.H, w.K + 3, 128, dtype=torch.bfloat16, device=DEV)
+    dv = torch.zeros_like(dk)
+    plan = ops.RetrievePlan(w.bs, w.H, w.G, w.N, DEV, w.N, w.C, w.K)
+    out = plan.run(d["queries"], d["signs"], d["centers"], d["cluster_counts"], d["codes_km"], d["nib_km"], d["w_km"], 0,
+                   w.N, w.tiers, w.C, w.K,
+                   gather=dict(src_k=kcpu, src_v=vcpu, from_host=True, dst_k=dk, dst_v=dv, dst_row0=3))
+    torch.cuda.synchronize()
+    idx = out.cpu().unsqueeze(-1).expand(-1, -1, -1, 128)
+    assert torch.equal(dk[:, :, 3:].cpu(), torch.gather(kcpu, 2, idx))
+    assert torch.equal(dv[:, :, 3:].cpu(), torch.gather(vcpu, 2, idx))
+    for r in range(w.R):
+        b, h = divmod(r, w.H)
+        assert np.array_equal(out[b, h].cpu().numpy(), W.oracle_stages(w, r)["final"])
+
+
+def test_retrieve_argument_errors(ops, wl_small_bf16):
+    w = wl_small_bf16
+    d = W.to_device(w, DEV, torch)
+    plan = ops.RetrievePlan(w.bs, w.H, w.G, w.N, DEV, w.N, w.C, w.K)
+    args = (d["queries"], d["signs"], d["centers"], d["cluster_counts"], d["codes_km"], d["nib_km"], d["w_km"])
+    with pytest.raises(RuntimeError):
+        plan.run(*args, 0, w.N, w.tiers, w.C, w.C + 1)        # k > n_cand
+    with pytest.raises(RuntimeError):
+        plan.run(*args, 10, w.N, w.tiers, w.C, w.K)           # zone exceeds capacity
+    with pytest.raises(RuntimeError):
+        plan.run(*args, 0, w.N, w.tiers, w.N + 1, w.K)        # n_cand > n_keys
+
+
+# ------------------------------------------------ full-size property checks
+
+
+@pytest.mark.parametrize("N,R,C,K", [(131072, 32, 4096, 1024)])
+def test_full_size_properties(ops, N, R, C, K):
+    """BASELINE config 3 shape on GPU-generated inputs: size-independent properties plus a
+    sampled-row comparison with the oracle (GPU-encoded index copied back to the host)."""
+    _say(f"full-size N={N} R={R} C={C} K={K}")
+    bs, H, G = 4, 8, 4
+    g = torch.Generator(device=DEV).manual_seed(0)
+    keys = torch.randn(bs, H, N, 128, generator=g, device=DEV, dtype=torch.float32)
+    keys[..., [7, 31, 64, 101]] *= 10
+    keys = keys.to(torch.bfloat16)
+    q = (keys.float().mean(dim=2, keepdim=True) + 0.5 * torch.randn(bs, H, G, 128, generator=g, device=DEV)).to(torch.bfloat16)
+    q = q.view(bs, 1, H * G, 128).contiguous()
+    signs = ops.srht_signs(DEV)
+    codes_km, nib_km, w_km, cb, k4, kw = ops.alloc_keymajor(bs, H, N, DEV)
+    cc = torch.zeros(bs, H, 16, 256, dtype=torch.int32, device=DEV)
+    ops.encode_append(keys, signs, cb, k4, kw, cc)
+    assert int(cc.sum()) == R * N * 16 and bool((cc.sum(dim=-1) == N).all())  # every key lands in one cluster per subspace
+    tiers = O.tier_counts(N, 0.2)
+    plan = ops.RetrievePlan(bs, H, G, N, DEV, N, C, K)
+    sc = torch.empty(bs, H, K, device=DEV)
+    out1 = plan.run(q, signs, ops.mag_centers(DEV), cc, codes_km, nib_km, w_km, 0, N, tiers, C, K, out_scores=sc).clone()
+    cand = plan.view("cand", N, C, K, torch.int64).view(R, C).clone()
+    cnt = plan.view("cnt_u8", N, C, K, torch.uint8).view(R, N).clone()
+    out2 = plan.run(q, signs, ops.mag_centers(DEV), cc, codes_km, nib_km, w_km, 0, N, tiers, C, K)
+    torch.cuda.synchronize()
+    assert torch.equal(out1, out2)                                   # deterministic / idempotent
+    assert bool((sc[..., :-1] >= sc[..., 1:]).all())                 # descending scores
+    assert bool((out1 >= 0).all()) and bool((out1 < N).all())
+    srt = out1.sort(dim=-1).values
+    assert bool((srt[..., 1:] != srt[..., :-1]).all())               # no duplicates
+    # candidates: distinct, and every non-candidate has a count <= every candidate's
+    cs = cand.sort(dim=-1).values
+    assert bool((cs[:, 1:] != cs[:, :-1]).all())
+    cand_cnt = torch.gather(cnt, 1, cand)
+    mask = torch.ones_like(cnt, dtype=torch.bool).scatter_(1, cand, False)
+    rest_max = torch.where(mask, cnt, torch.zeros_like(cnt)).max(dim=1).values
+    assert bool((cand_cnt.min(dim=1).values >= rest_max).all())
+    # final ids are a subset of the candidates
+    assert bool(torch.isin(out1.view(R, K), cand).all())
+    # sampled rows against the oracle, using the GPU-encoded index
+    for r in (0, 13, 31):
+        b, h = divmod(r, H)
+        ref = O.retrieve_row(q.view(bs, H, G, 128)[b, h].float().cpu().numpy(), signs.cpu().numpy(), O.BF16,
+                             codes_km[b, h].cpu().numpy(), nib_km[b, h].cpu().numpy().reshape(N, 16, 4),
+                             w_km[b, h].float().cpu().numpy(), cc[b, h].cpu().numpy(), tiers, C, K)
+        assert np.array_equal(out1[b, h].cpu().numpy(), ref)
+        # and the GPU encode of that row equals the oracle's encode
+        codes, nib, wt = O.encode(keys[b, h].float().cpu().numpy(), signs.cpu().numpy(), O.BF16)
+        assert np.array_equal(codes_km[b, h].cpu().numpy(), codes)
+        assert np.array_equal(nib_km[b, h].cpu().numpy().reshape(N, 16, 4), nib)
+        assert np.array_equal(w_km[b, h].float().cpu().numpy(), wt)
