@@ -1,0 +1,259 @@
+#!/usr/bin/env python3
+"""Benchmark of the retrieval hot path on one MI355X.
+
+A "step" is one layer's retrieval for one decode step: query prep + vote table ->
+collision scan -> candidate select -> 4-bit rerank -> exact top-k -> UVA gather
+of the selected K/V rows out of pinned host memory.  The workload is
+BASELINE.json's config 3 (the one the metric is quoted on): batch 4 x 8 KV heads
+(32 q heads, head_dim 128), 131072 cached keys per head, 4096 candidates, top-k
+1024, bf16, full-precision KV in pinned host memory.
+
+Steps rotate over LAYERS distinct layer indexes (448 MiB each) so that no
+layer's codes are still in the 256 MB last-level cache when it is scanned again,
+as in a real decode step, which walks all layers of the model.
+
+Prints ONE JSON line (see README / DESIGN.md for the field meanings).
+"""
+import argparse
+import ctypes as C
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "tests")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
+TIER_RATIOS = (0.05, 0.15, 0.30, 0.50, 0.75, 1.0)
+
+# HBM bytes moved by one collision-scan launch at this workload, from the two
+# rocprofv3 --pmc runs summarised in profiles/ (None until measured).
+SCAN_TRAFFIC_BYTES = 72676000  # profiles/scan_cfg3_hbm_traffic.md
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--layers", type=int, default=8, help="distinct layer indexes rotated through")
+    ap.add_argument("--context", type=int, default=131072)
+    ap.add_argument("--batch", type=int, default=4)
+    ap.add_argument("--candidates", type=int, default=4096)
+    ap.add_argument("--topk", type=int, default=1024)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", choices=["scan", "copy"], default=None,
+                    help="profiling aid: launch only the collision scan (or the calibration copy) --steps times")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (rows would shard across GPUs by (batch, kv-head), "
+              "see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from pariskv_amd import _lib, ops
+
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    bs, H, G, D = args.batch, 8, 4, 128
+    N, Cn, K, L = args.context, args.candidates, args.topk, args.layers
+    R = bs * H
+    lib = _lib.lib()
+
+    # ---------------------------------------------------------------- inputs
+    signs = ops.srht_signs(dev)
+    centers = ops.mag_centers(dev)
+    tiers = [int(math.ceil(N * 0.2 * r)) for r in TIER_RATIOS]  # collision_ratio 0.2 for >= 30K keys
+    layers = []
+    kcpu = torch.empty(bs, H, N, D, dtype=torch.bfloat16, pin_memory=True)
+    vcpu = torch.empty(bs, H, N, D, dtype=torch.bfloat16, pin_memory=True)
+    for l in range(L):
+        codes_km, nib_km, w_km, cb, k4, kw = ops.alloc_keymajor(bs, H, N, dev)
+        cc = torch.zeros(bs, H, 16, 256, dtype=torch.int32, device=dev)
+        q = torch.empty(bs, 1, H * G, D, dtype=torch.bfloat16, device=dev)
+        for b in range(bs):  # independent seed per sequence (and per layer)
+            g = torch.Generator(device=dev).manual_seed(1000 * l + b)
+            keys = torch.randn(1, H, N, D, generator=g, device=dev, dtype=torch.float32)
+            keys[..., [7, 31, 64, 101]] *= 10.0  # four fixed outlier channels
+            kb = keys.to(torch.bfloat16)
+            qq = keys.mean(dim=2, keepdim=True) + 0.5 * torch.randn(1, H, G, D, generator=g, device=dev)
+            q[b, 0] = qq.view(H * G, D).to(torch.bfloat16)
+            ops.encode_append(kb, signs, cb[b:b + 1], k4[b:b + 1], kw[b:b + 1], cc[b:b + 1])
+            if l == 0:
+                kcpu[b].copy_(kb[0])
+                vcpu[b].copy_(torch.randn(H, N, D, generator=g, device=dev).to(torch.bfloat16))
+            del keys, kb
+        layers.append(dict(codes=codes_km, nib=nib_km, w=w_km, cc=cc, q=q))
+    dst_k = torch.empty(bs, H, K, D, dtype=torch.bfloat16, device=dev)
+    dst_v = torch.empty_like(dst_k)
+    out_ids = torch.empty(bs, H, K, dtype=torch.int64, device=dev)
+    plan = ops.RetrievePlan(bs, H, G, N, dev, N, Cn, K)
+    gather = dict(src_k=kcpu, src_v=vcpu, from_host=True, dst_k=dst_k, dst_v=dst_v)
+    torch.cuda.synchronize()
+
+    def step(i, with_gather=True):
+        ly = layers[i % L]
+        plan.run(ly["q"], signs, centers, ly["cc"], ly["codes"], ly["nib"], ly["w"], 0, N, tiers, Cn, K, out_ids=out_ids,
+                 gather=gather if with_gather else None)
+
+    def timed(fn, n):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for i in range(n):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1000.0 / n  # us per call
+
+    # ------------------------------------------------ profiling-only modes
+    chunk = ops.pick_chunk_keys(R, N)
+    n_chunks = (N + chunk - 1) // chunk
+    cnt_stride = (N + 15) // 16 * 16
+    cnt_ws = torch.empty(R, cnt_stride, dtype=torch.uint8, device=dev)
+    hist_ws = torch.empty(R, n_chunks, 128, dtype=torch.int16, device=dev)
+    luts = []
+    for ly in layers:
+        _, _, lut, _ = ops.query_prep_lut(ly["q"], H, signs, ly["cc"], tiers)
+        luts.append(lut)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def scan_only(i):
+        ly = layers[i % L]
+        _lib.check(lib.pkv_collision_scan(ly["codes"].data_ptr(), H * N * 16, N * 16, 16, 1, bs, H, N,
+                                          luts[i % L].data_ptr(), cnt_ws.data_ptr(), None, hist_ws.data_ptr(), chunk,
+                                          stream))
+
+    if args.only == "scan":
+        for i in range(args.warmup + args.steps):
+            scan_only(i)
+        torch.cuda.synchronize()
+        print(json.dumps({"only": "scan", "launches": args.warmup + args.steps, "bytes_per_launch": R * N * 17}))
+        return
+    if args.only == "copy":
+        nbytes = R * N * 16
+        a = layers[0]["codes"]
+        b2 = torch.empty_like(a)
+        for i in range(args.warmup + args.steps):
+            _lib.check(lib.pkv_copy_bytes(layers[i % L]["codes"].data_ptr(), b2.data_ptr(), nbytes, stream))
+        torch.cuda.synchronize()
+        print(json.dumps({"only": "copy", "launches": args.warmup + args.steps, "read_bytes": nbytes, "write_bytes": nbytes}))
+        return
+
+    # ------------------------------------------------------------- timing
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t_wall0 = time.perf_counter()
+    us_step = timed(step, args.steps)                       # full retrieval incl. UVA gather  (the metric)
+    t_wall = time.perf_counter() - t_wall0
+    us_gpu = timed(lambda i: step(i, False), args.steps)    # on-GPU stages only
+
+    def gather_only(i):
+        ops.gather_uva(kcpu, vcpu, out_ids, dst_k, dst_v)
+
+    step(0)
+    us_gather = timed(gather_only, max(8, args.steps // 4))
+
+    # dominant kernel: the collision scan, timed by its own begin/end timestamps
+    kus = C.c_float()
+    scan_us = []
+    for i in range(args.warmup + args.steps):
+        ly = layers[i % L]
+        _lib.check(lib.pkv_collision_scan_timed(ly["codes"].data_ptr(), H * N * 16, N * 16, 16, 1, bs, H, N,
+                                                luts[i % L].data_ptr(), cnt_ws.data_ptr(), cnt_stride,
+                                                hist_ws.data_ptr(), chunk, C.byref(kus), stream))
+        if i >= args.warmup:
+            scan_us.append(kus.value)
+    scan_avg_us = sum(scan_us) / len(scan_us)
+    scan_bytes = R * N * (16 + 1)                     # 16 B of codes read + 1 B vote count written per key
+    achieved = scan_bytes / (scan_avg_us * 1e-6) / 1e9
+
+    a_hbm = R * (16 * N + 96 * Cn + 8 * K + 512 * K)  # algorithmic HBM bytes of the whole on-GPU pipeline
+    a_pcie = R * 512 * K
+
+    result = {
+        "metric": "retrieval us/layer/decode-step at 128K ctx; achieved HBM GB/s vs peak",
+        "value": round(us_step, 2),
+        "unit": "us/layer/decode-step",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(us_step / 1000.0, 5),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u8 votes / f32 rerank (bf16 keys)",
+        "data": "synthetic",
+        "config": {"workload": f"BASELINE config 3: batch {bs} x {H} KV heads (GQA {G}), head_dim {D}, {N} keys/head, "
+                               f"collision -> {Cn} candidates, 4-bit rerank -> top-{K}, KV in pinned host memory "
+                               f"(UVA gather), {L} rotating layers",
+                   "rows": R, "keys_per_row": N, "candidates": Cn, "topk": K, "collision_ratio": 0.2},
+        "stages_us": {"full_retrieval_with_uva_gather": round(us_step, 2), "on_gpu_stages": round(us_gpu, 2),
+                      "uva_gather_alone": round(us_gather, 2)},
+        "hbm_fraction_on_gpu_stages": round(a_hbm / (us_gpu * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+        "algorithmic_bytes": {"hbm_per_step": a_hbm, "pcie_per_step": a_pcie},
+        "pcie_GBps_gather": round(a_pcie / (us_gather * 1e-6) / 1e9, 2),
+        "roofline": {"kernel": "pkv_scan_keymajor_kernel", "bound": "hbm", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": SCAN_TRAFFIC_BYTES, "bytes_per_launch": scan_bytes,
+                     "avg_launch_us": round(scan_avg_us, 2)},
+        "wall_s_timed_region": round(t_wall, 4),
+    }
+
+    # ------------------------------------------------------- CPU baseline
+    if not args.no_cpu_baseline:
+        import numpy as np
+
+        from oracle import pkv_oracle as O  # the checker, timed here as the reported CPU baseline only
+
+        O.build()
+        ly = layers[0]
+        rows = list(range(R))
+        host = []
+        for r in rows:
+            b, h = divmod(r, H)
+            host.append(dict(
+                q=ly["q"].view(bs, H, G, D)[b, h].float().cpu().numpy(),
+                codes=ly["codes"][b, h].cpu().numpy(), nib=ly["nib"][b, h].cpu().numpy().reshape(N, 16, 4),
+                w=ly["w"][b, h].float().cpu().numpy(), cc=ly["cc"][b, h].cpu().numpy(),
+                k=kcpu[b, h].view(torch.int16).numpy(), v=vcpu[b, h].view(torch.int16).numpy()))
+        sg = signs.cpu().numpy()
+
+        def cpu_layer_step():
+            outs = []
+            for hst in host:
+                ids = O.retrieve_row(hst["q"], sg, O.BF16, hst["codes"], hst["nib"], hst["w"], hst["cc"], tiers, Cn, K)
+                O.gather_rows(hst["k"], ids)
+                O.gather_rows(hst["v"], ids)
+                outs.append(ids)
+            return outs
+
+        ref_ids = cpu_layer_step()  # warm-up, and a parity check of the benchmarked GPU path on the real workload
+        step(0)
+        torch.cuda.synchronize()
+        gpu_ids = out_ids.view(R, K).cpu().numpy()
+        parity = all(np.array_equal(gpu_ids[r], ref_ids[r]) for r in rows)
+        times = []
+        t_end = time.perf_counter() + 25.0
+        while len(times) < 20 and (time.perf_counter() < t_end or len(times) < 3):
+            t0 = time.perf_counter()
+            cpu_layer_step()
+            times.append(time.perf_counter() - t0)
+        times.sort()
+        med = times[len(times) // 2]
+        result["cpu_baseline"] = {"value": round(med * 1e6, 1), "unit": "us/layer/decode-step", "cores": 1, "kind": "port",
+                                  "sample": f"all {R} rows of one layer at the full workload (C oracle, single thread, "
+                                            f"host gather included), median of {len(times)} repetitions",
+                                  "host_cpus": os.cpu_count()}
+        result["parity_vs_oracle_on_bench_workload"] = bool(parity)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
