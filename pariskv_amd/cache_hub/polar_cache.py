@@ -1,0 +1,383 @@
+"""PolarANN KV cache with collision retrieval + 4-bit rerank, on the HIP kernels.
+
+Same constructor and methods as the reference's ``cache_hub/polar_cache.py``
+(``polar_cache.__init__`` :103-128, ``prefill_update_kv_cache`` :379,
+``decode_update_kv_cache`` :827, ``compute`` :1002, ``sync`` :1310) so it drops in
+under ``attn_hub/polar_attn.py``.  What differs inside:
+
+* metadata is stored key-major (``ops.alloc_keymajor``); ``codebook_gpu``,
+  ``key_4bit_packed_gpu`` and ``key_block_weight_gpu`` are reference-shaped views of it;
+* one decode step's retrieval is a single ``pkv_retrieve`` call (6 launches) that
+  also gathers the selected K/V rows straight behind the dense prefix, so no
+  ``torch.cat`` / ``torch.gather`` of K/V happens per step;
+* zone counters are per layer (see ``zones.py``);
+* the offload copy is ordered by stream events, not a host-blocking synchronize.
+"""
+from __future__ import annotations
+
+import json
+import math
+import os
+from typing import Optional
+
+import torch
+import torch.nn.functional as F
+
+from .. import ops
+from .cache import KV_Cache
+from .zones import LayerZones
+
+USE_RABITQ_RERANK = True
+DEFAULT_SRHT_ROUNDS = 1
+
+
+def _sign_codebook_ok(path: Optional[str], d: int):
+    """Read the codebook config (polar_cache.py:152-160) and make sure it is the sign enumeration."""
+    if path is None:
+        return 8, 1, 256
+    try:
+        with open(path, "r") as f:
+            cb = json.load(f)
+        cfg = cb["config"]
+        m, k_r, k_omega = cfg["m"], cfg["K_r"], cfg["K_omega"]
+    except (FileNotFoundError, KeyError, json.JSONDecodeError) as e:
+        raise ValueError(f"Cannot read codebook parameters: {e}")
+    if cfg.get("d", d) != d or m != 8 or k_r != 1 or k_omega != 256:
+        raise ValueError(f"Codebook parameter mismatch! only d=128, m=8, K_r=1, K_omega=256 is built; got {cfg}")
+    signs = cb.get("angular_signs")
+    if signs is not None:
+        for c in (0, 1, 2, 77, 128, 255):
+            if [1 if (c >> j) & 1 else -1 for j in range(8)] != [1 if v >= 0 else -1 for v in signs[c]]:
+                raise ValueError("only the sign-enumeration codebook (centroid id = sign bit pattern) is supported")
+    return m, k_r, k_omega
+
+
+class polar_cache(KV_Cache):
+
+    def __init__(self, valid_start, layer_num: int, batch_size: int, max_length: int, num_key_value_heads: int,
+                 num_heads: int, head_dim: int, dtype: torch.dtype, layer_mapping: dict, max_new_length: int,
+                 sink_size: int, local_size: int, core: int = 0, nprobe: int = 0, cache_unit_size: int = 0,
+                 cache_cluster_num: int = 0, num_gpus: int = 1, model_size: int = 0,
+                 codebook_path: Optional[str] = None, final_topk: int = 100, dynamic_update_interval: int = 512,
+                 full_attention_threshold: int = 2000, enable_offload: bool = True,
+                 collision_ratio: Optional[float] = None, candidate_ratio: Optional[float] = None) -> None:
+        super().__init__(layer_num, batch_size, max_length, num_key_value_heads, num_heads, head_dim, dtype,
+                         layer_mapping, num_gpus, model_size)
+        if head_dim != ops.HEAD_DIM:
+            raise ValueError("head_dim must be 128")
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError("dtype must be bfloat16 or float32")
+        self.valid_start = valid_start
+        self.sink_size = sink_size
+        self.local_size = local_size
+        self.steady_size = sink_size + local_size
+        self.dynamic_update_interval = dynamic_update_interval if dynamic_update_interval is not None else local_size
+        self.group_size = self.num_heads // self.kv_head
+        self.batch_groups = self.batch_size * self.kv_head
+        self.max_new_length = max_new_length
+        self.input_length = self.max_length - max_new_length
+        self.FULL_ATTENTION_THRESHOLD = full_attention_threshold
+        self.current_seq_len = [0] * layer_num
+        self.final_topk = final_topk
+        self.enable_offload = enable_offload
+        self._collision_ratio = collision_ratio
+        self._candidate_ratio = candidate_ratio
+        if codebook_path is not None and not os.path.isabs(codebook_path):
+            codebook_path = os.path.abspath(codebook_path)
+        self.codebook_path = codebook_path
+        self.polar_m, self.polar_K_r, self.polar_K_omega = _sign_codebook_ok(codebook_path, head_dim)
+        self.polar_B = head_dim // self.polar_m
+
+        self.device = torch.device(list(layer_mapping.values())[0] if layer_mapping else "cuda:0")
+        if self.device.type != "cuda":
+            raise RuntimeError("GPU required")  # polar_cache.py:40-41
+        dev, bs, H, D, I = self.device, batch_size, self.kv_head, head_dim, self.dynamic_update_interval
+        self._srht_signs = ops.srht_signs(dev, seed=42)
+        self._mag_centers = ops.mag_centers(dev)
+        self.unified_kv_capacity = self.input_length + self.max_new_length
+        self._zones = [LayerZones(sink_size, local_size, I, enable_offload) for _ in range(layer_num)]
+
+        if enable_offload:
+            # GPU rows: [sink | local | update buffer | gathered top-k (transient)]
+            self.gpu_kv_capacity = sink_size + local_size + I
+            rows = self.gpu_kv_capacity + final_topk
+            self.cpu_kv_capacity = max(1, self.unified_kv_capacity - sink_size - local_size)
+            self._copy_stream = torch.cuda.Stream(device=dev)
+            self._copy_events = [torch.cuda.Event() for _ in range(layer_num)]
+            self._offload_inflight = [False] * layer_num
+            self.unified_keys_cpu = [torch.zeros((bs, H, self.cpu_kv_capacity, D), dtype=dtype, pin_memory=True)
+                                     for _ in range(layer_num)]
+            self.unified_values_cpu = [torch.zeros((bs, H, self.cpu_kv_capacity, D), dtype=dtype, pin_memory=True)
+                                       for _ in range(layer_num)]
+            self.cpu_valid_end = [0] * layer_num
+            self._offload_keys_buffer = [torch.empty((bs, H, I, D), dtype=dtype, device=dev) for _ in range(layer_num)]
+            self._offload_values_buffer = [torch.empty((bs, H, I, D), dtype=dtype, device=dev) for _ in range(layer_num)]
+        else:
+            # GPU rows: every token at its absolute position; a separate buffer holds the attended set
+            self.gpu_kv_capacity = self.unified_kv_capacity
+            rows = self.unified_kv_capacity
+            self.unified_keys_cpu = None
+            self.unified_values_cpu = None
+            self.cpu_valid_end = None
+            att_rows = sink_size + final_topk + local_size + I
+            self._attn_k = torch.zeros((bs, H, att_rows, D), dtype=dtype, device=dev)
+            self._attn_v = torch.zeros((bs, H, att_rows, D), dtype=dtype, device=dev)
+        self.unified_keys_gpu = [torch.zeros((bs, H, rows, D), dtype=dtype, device=dev) for _ in range(layer_num)]
+        self.unified_values_gpu = [torch.zeros((bs, H, rows, D), dtype=dtype, device=dev) for _ in range(layer_num)]
+
+        # index metadata, addressed by absolute position (polar_cache.py:283-312)
+        self.retrieval_zone_capacity = self.unified_kv_capacity
+        cap = self.retrieval_zone_capacity
+        self._codes_km, self._nib_km, self._w_km = [], [], []
+        self.codebook_gpu, self.key_4bit_packed_gpu, self.key_block_weight_gpu = [], [], []
+        for _ in range(layer_num):
+            c, n, w, cb, k4, kw = ops.alloc_keymajor(bs, H, cap, dev)
+            self._codes_km.append(c), self._nib_km.append(n), self._w_km.append(w)
+            self.codebook_gpu.append(cb), self.key_4bit_packed_gpu.append(k4), self.key_block_weight_gpu.append(kw)
+        self.cluster_key_counts_gpu = [torch.zeros((bs, H, self.polar_B, self.polar_K_omega), dtype=torch.int32, device=dev)
+                                       for _ in range(layer_num)]
+        self.context = 0
+        self._hadamard_scale = 1.0 / math.sqrt(head_dim)
+        max_keys = max(1, cap - sink_size)
+        max_cand = max(1, math.ceil(max_keys * 0.5))
+        self._plan = ops.RetrievePlan(bs, H, self.group_size, cap, dev, max_keys, max_cand, max(1, min(final_topk, max_cand)))
+        self._out_ids = torch.empty((bs, H, max(1, final_topk)), dtype=torch.int64, device=dev)
+        self.last_topk_indices = None  # [bs, H, K] of the most recent retrieval (zone-relative), for inspection
+
+    # ------------------------------------------------------------- helpers
+    @property
+    def _actual_retrieval_length(self):
+        return self._zones[0].encoded
+
+    def _vs(self, batch_idx=0) -> int:
+        vs = self.valid_start
+        if isinstance(vs, (list, tuple)) or hasattr(vs, "__len__"):
+            return int(vs[batch_idx])
+        return int(vs)
+
+    def _get_adaptive_ratios(self, retrieval_len):
+        """(candidate_ratio, collision_ratio) by retrieval-zone length (polar_cache.py:1113-1124)."""
+        if retrieval_len < 5000:
+            cand, coll = 0.5, 0.5
+        elif retrieval_len < 10000:
+            cand, coll = 0.25, 0.3
+        elif retrieval_len < 30000:
+            cand, coll = 0.2, 0.25
+        else:
+            cand, coll = 0.1, 0.2
+        if self._candidate_ratio is not None:
+            cand = self._candidate_ratio
+        if self._collision_ratio is not None:
+            coll = self._collision_ratio
+        return cand, coll
+
+    def _wait_offload(self, layer_idx: int) -> None:
+        """Order the current stream after the layer's last host copy (GPU-side wait, no host block)."""
+        if self.enable_offload and self._offload_inflight[layer_idx]:
+            torch.cuda.current_stream(self.device).wait_event(self._copy_events[layer_idx])
+            self._offload_inflight[layer_idx] = False
+
+    def _offload_rows(self, layer_idx: int, b0: int, b1: int, src_k: torch.Tensor, src_v: torch.Tensor, cpu_row0: int):
+        """Async D2H of [b1-b0, H, n, D] staging tensors into the pinned host zone (polar_cache.py:457-471, 778-799)."""
+        n = src_k.shape[2]
+        ready = torch.cuda.Event()
+        ready.record(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(self._copy_stream):
+            self._copy_stream.wait_event(ready)
+            self.unified_keys_cpu[layer_idx][b0:b1, :, cpu_row0:cpu_row0 + n].copy_(src_k, non_blocking=True)
+            self.unified_values_cpu[layer_idx][b0:b1, :, cpu_row0:cpu_row0 + n].copy_(src_v, non_blocking=True)
+            self._copy_events[layer_idx].record(self._copy_stream)
+        src_k.record_stream(self._copy_stream)
+        src_v.record_stream(self._copy_stream)
+        self._offload_inflight[layer_idx] = True
+
+    def _encode(self, layer_idx: int, keys_bhsd: torch.Tensor, b0: int, b1: int, abs0: int) -> None:
+        """Encode keys [b1-b0, H, n, D] (any strides) into metadata positions [abs0, abs0+n) and add to the cluster sizes."""
+        n = keys_bhsd.shape[2]
+        if n == 0:
+            return
+        sl = slice(abs0, abs0 + n)
+        ops.encode_append(keys_bhsd, self._srht_signs, self.codebook_gpu[layer_idx][b0:b1, :, :, sl],
+                          self.key_4bit_packed_gpu[layer_idx][b0:b1, :, :, sl], self.key_block_weight_gpu[layer_idx][b0:b1, :, :, sl],
+                          self.cluster_key_counts_gpu[layer_idx][b0:b1])
+
+    # ------------------------------------------------------------- prefill
+    def prefill_update_kv_cache(self, query_states, key_states, value_states, layer_idx, batch_idx):
+        """key/value_states [bsz, S, Hkv, D].  bsz == 1: sample ``batch_idx``; bsz == batch_size: lockstep
+        (uniform valid_start).  Returns the states from valid_start on, like the reference (:379-387, :504, :611)."""
+        bsz, seq_len, _, _ = key_states.shape
+        if bsz == 1:
+            b0, vs = int(batch_idx), self._vs(batch_idx)
+        else:
+            assert bsz == self.batch_size, f"bsz({bsz}) must equal cache batch_size({self.batch_size}) for lockstep mode."
+            vs = self._vs(0)
+            if hasattr(self.valid_start, "__len__"):
+                assert all(int(v) == vs for v in list(self.valid_start)[:bsz]), "lockstep multi-batch requires same valid_start"
+            if batch_idx != 0:
+                return key_states[:, vs:], value_states[:, vs:]
+            b0 = 0
+        b1 = b0 + bsz
+        assert seq_len <= self.input_length
+        z = self._zones[layer_idx]
+        n_tok = seq_len - vs
+        retrieval, local_len = z.prefill(n_tok)
+        self.current_seq_len[layer_idx] = n_tok
+        k = key_states[:, vs:].permute(0, 2, 1, 3)   # [bsz, H, n_tok, D] view of the model's layout
+        v = value_states[:, vs:].permute(0, 2, 1, 3)
+        kg, vg = self.unified_keys_gpu[layer_idx], self.unified_values_gpu[layer_idx]
+        last = (layer_idx == self.layer_num - 1) and (b1 == self.batch_size)
+        if retrieval == 0:  # short prompt: everything stays dense on the GPU (:430-440)
+            n = min(n_tok, self.gpu_kv_capacity)
+            kg[b0:b1, :, :n] = k[:, :, :n].to(self.dtype)
+            vg[b0:b1, :, :n] = v[:, :, :n].to(self.dtype)
+            if last:
+                self.context += n
+            return key_states[:, vs:], value_states[:, vs:]
+        S0, r_end = self.sink_size, self.sink_size + retrieval
+        if self.enable_offload:
+            kg[b0:b1, :, :S0] = k[:, :, :S0].to(self.dtype)
+            vg[b0:b1, :, :S0] = v[:, :, :S0].to(self.dtype)
+            kg[b0:b1, :, S0:S0 + local_len] = k[:, :, r_end:].to(self.dtype)
+            vg[b0:b1, :, S0:S0 + local_len] = v[:, :, r_end:].to(self.dtype)
+            stage_k = k[:, :, S0:r_end].to(self.dtype).contiguous()
+            stage_v = v[:, :, S0:r_end].to(self.dtype).contiguous()
+            self._wait_offload(layer_idx)
+            self._offload_rows(layer_idx, b0, b1, stage_k, stage_v, 0)
+            self.cpu_valid_end[layer_idx] = retrieval
+            enc_src = stage_k
+        else:
+            kg[b0:b1, :, :n_tok] = k.to(self.dtype)
+            vg[b0:b1, :, :n_tok] = v.to(self.dtype)
+            enc_src = kg[b0:b1, :, S0:r_end]
+        self.cluster_key_counts_gpu[layer_idx][b0:b1].zero_()  # prefill assigns, refresh accumulates (:493, :775)
+        self._encode(layer_idx, enc_src, b0, b1, S0)
+        if last:
+            self.context += n_tok
+        return key_states[:, vs:], value_states[:, vs:]
+
+    # -------------------------------------------------------------- decode
+    def decode_update_kv_cache(self, key_states, value_states, layer_idx):
+        """Append one token ([bs,1,Hkv,D]); refresh the index when this layer's update buffer fills (:827-881)."""
+        z = self._zones[layer_idx]
+        slot = z.append_slot()
+        self.unified_keys_gpu[layer_idx][:, :, slot, :] = key_states[:, 0]
+        self.unified_values_gpu[layer_idx][:, :, slot, :] = value_states[:, 0]
+        refresh = z.appended()
+        self.current_seq_len[layer_idx] = z.seq_len
+        if layer_idx == 0:
+            self.context += 1
+        if refresh is not None:
+            self._update_polar_index(layer_idx, refresh)
+        return None, None
+
+    def _update_polar_index(self, layer_idx: int, r) -> None:
+        """Move the oldest ``interval`` tokens of local ++ buffer into the retrieval zone (:743-821)."""
+        kg, vg = self.unified_keys_gpu[layer_idx], self.unified_values_gpu[layer_idx]
+        n, S0 = r.n_new, self.sink_size
+        bs = self.batch_size
+        self._encode(layer_idx, kg[:, :, r.gpu_row0:r.gpu_row0 + n], 0, bs, r.encode_abs0)
+        if not self.enable_offload:
+            return
+        self._wait_offload(layer_idx)  # staging buffers are free again
+        sk, sv = self._offload_keys_buffer[layer_idx][:, :, :n], self._offload_values_buffer[layer_idx][:, :, :n]
+        sk.copy_(kg[:, :, S0:S0 + n])
+        sv.copy_(vg[:, :, S0:S0 + n])
+        self._offload_rows(layer_idx, 0, bs, sk, sv, r.cpu_row0)
+        self.cpu_valid_end[layer_idx] = r.cpu_row0 + n
+        # slide the window: rows [sink+n, sink+local+n) -> [sink, sink+local)
+        L = self.local_size
+        if n < L:
+            kg[:, :, S0:S0 + L] = kg[:, :, S0 + n:S0 + n + L].clone()
+            vg[:, :, S0:S0 + L] = vg[:, :, S0 + n:S0 + n + L].clone()
+        else:
+            kg[:, :, S0:S0 + L] = kg[:, :, S0 + n:S0 + n + L]
+            vg[:, :, S0:S0 + L] = vg[:, :, S0 + n:S0 + n + L]
+
+    # -------------------------------------------------------------- compute
+    def get_region_indices(self, layer_idx, device=None):
+        """Region summary (reference :645-684), from the per-layer counters."""
+        z = self._zones[layer_idx]
+        device = device or self.device
+        sink_n = min(self.sink_size, z.seq_len)
+        return {
+            "sink_indices": torch.arange(0, sink_n, device=device, dtype=torch.long),
+            "local_indices": torch.arange(z.local_start, z.seq_len, device=device, dtype=torch.long),
+            "retrieval_start": self.sink_size,
+            "retrieval_length": z.encoded,
+            "total_len": z.seq_len,
+            "local_len": z.dense_tail_len,
+        }
+
+    def _compute_local_start(self, layer_idx=0):
+        return self._zones[layer_idx].local_start
+
+    def _attend(self, queries, k, v):
+        """softmax(q k^T / sqrt(D)) v over the gathered set; q [bs,1,Hq,D], k/v [bs,Hkv,S,D] (:1097-1105)."""
+        q = queries.transpose(1, 2)  # [bs, Hq, 1, D]
+        out = F.scaled_dot_product_attention(q, k, v, is_causal=False, enable_gqa=self.group_size > 1)
+        return out.transpose(1, 2).contiguous()
+
+    def _full_kv(self, layer_idx):
+        """Dense fallback: every stored token (reference _get_full_kv_for_attention :701-737)."""
+        z = self._zones[layer_idx]
+        kg, vg = self.unified_keys_gpu[layer_idx], self.unified_values_gpu[layer_idx]
+        if not self.enable_offload:
+            return kg[:, :, :z.seq_len], vg[:, :, :z.seq_len]
+        n = z.gpu_prefix_rows
+        if z.encoded == 0:
+            return kg[:, :, :n], vg[:, :, :n]
+        self._copy_stream.synchronize()  # the host reads below must see what the copy stream wrote (:707)
+        self._offload_inflight[layer_idx] = False
+        rk = self.unified_keys_cpu[layer_idx][:, :, :z.encoded].to(self.device, non_blocking=True)
+        rv = self.unified_values_cpu[layer_idx][:, :, :z.encoded].to(self.device, non_blocking=True)
+        return torch.cat([kg[:, :, :n], rk], dim=2), torch.cat([vg[:, :, :n], rv], dim=2)
+
+    def retrieval_shape(self, layer_idx):
+        """(n_keys, n_cand, k, tier_counts) the next retrieval of this layer will use."""
+        z = self._zones[layer_idx]
+        n_keys = self.cpu_valid_end[layer_idx] if self.enable_offload else z.encoded
+        cand_ratio, coll_ratio = self._get_adaptive_ratios(n_keys)
+        n_cand = min(n_keys, max(1, int(math.ceil(n_keys * cand_ratio))))        # :1239-1240
+        k = min(self.final_topk, n_cand)                                          # :1300
+        tiers = [int(math.ceil(n_keys * coll_ratio * r)) for r in ops.TIER_RATIOS]  # :1221-1222
+        return n_keys, n_cand, k, tiers
+
+    def compute(self, queries, layer_idx):
+        """Decode attention for one token: [bs,1,Hq,D] -> [bs,1,Hq,D] (:1002-1107)."""
+        z = self._zones[layer_idx]
+        total = z.seq_len
+        n_keys = (self.cpu_valid_end[layer_idx] if self.enable_offload else z.encoded)
+        min_total = max(self.FULL_ATTENTION_THRESHOLD, self.sink_size + self.local_size + self.final_topk * 2)
+        if total < min_total or n_keys <= 0:
+            k, v = self._full_kv(layer_idx)
+            return self._attend(queries, k, v)
+        n_keys, n_cand, topk, tiers = self.retrieval_shape(layer_idx)
+        kg, vg = self.unified_keys_gpu[layer_idx], self.unified_values_gpu[layer_idx]
+        q = queries.contiguous()
+        if self.enable_offload:
+            self._wait_offload(layer_idx)
+            prefix = z.gpu_prefix_rows
+            gather = dict(src_k=self.unified_keys_cpu[layer_idx], src_v=self.unified_values_cpu[layer_idx], from_host=True,
+                          idx_offset=0, dst_k=kg, dst_v=vg, dst_row0=prefix)
+            att_k, att_v = kg[:, :, :prefix + topk], vg[:, :, :prefix + topk]
+        else:
+            S0, tail = self.sink_size, z.dense_tail_len
+            ak, av = self._attn_k, self._attn_v
+            ak[:, :, :S0] = kg[:, :, :S0]
+            av[:, :, :S0] = vg[:, :, :S0]
+            ak[:, :, S0 + topk:S0 + topk + tail] = kg[:, :, z.local_start:total]
+            av[:, :, S0 + topk:S0 + topk + tail] = vg[:, :, z.local_start:total]
+            gather = dict(src_k=kg, src_v=vg, from_host=False, idx_offset=self.sink_size, dst_k=ak, dst_v=av, dst_row0=S0)
+            att_k, att_v = ak[:, :, :S0 + topk + tail], av[:, :, :S0 + topk + tail]
+        out_ids = self._out_ids[:, :, :topk]
+        if not out_ids.is_contiguous():
+            out_ids = torch.empty((self.batch_size, self.kv_head, topk), dtype=torch.int64, device=self.device)
+        self._plan.run(q, self._srht_signs, self._mag_centers, self.cluster_key_counts_gpu[layer_idx], self._codes_km[layer_idx],
+                       self._nib_km[layer_idx], self._w_km[layer_idx], self.sink_size, n_keys, tiers, n_cand, topk,
+                       out_ids=out_ids, gather=gather)
+        self.last_topk_indices = out_ids
+        return self._attend(q, att_k, att_v)
+
+    def sync(self, layer_idx, batch_idx):
+        """No-op, as in the reference (:1310-1312)."""
+        pass

@@ -1,0 +1,166 @@
+"""End-to-end tests of the polar_cache drop-in on the GPU: prefill, decode appends with index
+refreshes and host offload, retrieval and attention, for several layers.
+
+Checked per step: (1) the retrieved indices equal the CPU oracle's on the cache's own index
+(bit-exact); (2) the attention output equals an fp32 torch softmax attention over
+sink ++ selected ++ dense tail taken from the test's own record of every K/V it fed
+(bf16 tolerance 2e-2 abs)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import pkv_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _make_cache(offload, bs, Hkv, Hq, layers, S, max_new, sink, local, interval, final_topk, thr=100, **kw):
+    from pariskv_amd.cache_hub.polar_cache import polar_cache
+
+    return polar_cache(valid_start=[0] * bs, layer_num=layers, batch_size=bs, max_length=S + max_new,
+                       num_key_value_heads=Hkv, num_heads=Hq, head_dim=128, dtype=torch.bfloat16,
+                       layer_mapping={i: DEV for i in range(layers)}, max_new_length=max_new, sink_size=sink,
+                       local_size=local, core=1, nprobe=1, cache_unit_size=1, cache_cluster_num=1, num_gpus=1, model_size=7,
+                       final_topk=final_topk, dynamic_update_interval=interval, full_attention_threshold=thr,
+                       enable_offload=offload, **kw)
+
+
+def _ref_attention(q, K, V, G):
+    """fp32 softmax(q k^T / sqrt(D)) v.  q [Hq,D], K/V [Hkv,S,D] -> [Hq,D]."""
+    Hq, D = q.shape
+    out = torch.empty(Hq, D)
+    for hq in range(Hq):
+        h = hq // G
+        s = (K[h].float() @ q[hq].float()) / math.sqrt(D)
+        out[hq] = torch.softmax(s, dim=0) @ V[h].float()
+    return out
+
+
+def _synth_kv(gen, bs, S, Hkv):
+    k = torch.randn(bs, S, Hkv, 128, generator=gen)
+    k[..., [7, 31, 64, 101]] *= 10.0
+    v = torch.randn(bs, S, Hkv, 128, generator=gen)
+    return k.to(torch.bfloat16), v.to(torch.bfloat16)
+
+
+@pytest.mark.parametrize("offload", [True, False])
+def test_decode_loop_matches_oracle_and_dense_reference(offload):
+    from pariskv_amd.attn_hub import polar_decode_attn
+
+    print(f"polar_cache decode loop offload={offload}", flush=True)
+    bs, Hkv, Hq, layers, S, steps = 2, 2, 8, 2, 3000, 70
+    sink, local, I, topk = 4, 64, 32, 200
+    G = Hq // Hkv
+    cache = _make_cache(offload, bs, Hkv, Hq, layers, S, steps + 10, sink, local, I, topk)
+    gen = torch.Generator().manual_seed(0)
+    hist_k = [None] * layers
+    hist_v = [None] * layers
+    for l in range(layers):
+        k, v = _synth_kv(gen, bs, S, Hkv)
+        hist_k[l], hist_v[l] = k, v
+        ko, vo = cache.prefill_update_kv_cache(None, k.to(DEV), v.to(DEV), l, 0)
+        assert ko.shape == k.shape
+    assert cache.current_seq_len == [S] * layers and cache.context == S
+    signs = O.srht_signs(42)
+    checked = 0
+    for step in range(steps):
+        for l in range(layers):
+            k1, v1 = _synth_kv(gen, bs, 1, Hkv)
+            q = (hist_k[l].float().mean(dim=1).repeat_interleave(G, dim=1) + 0.5 * torch.randn(bs, Hq, 128, generator=gen))
+            q = q.to(torch.bfloat16).view(bs, 1, Hq, 128)
+            hist_k[l] = torch.cat([hist_k[l], k1], dim=1)
+            hist_v[l] = torch.cat([hist_v[l], v1], dim=1)
+            assert cache.decode_update_kv_cache(k1.to(DEV), v1.to(DEV), l) == (None, None)
+            out = polar_decode_attn(q.to(DEV), None, None, l, cache)
+            assert out.shape == (bs, 1, Hq, 128)
+            if step % 9 != 0 and step not in (I - 1, I, 2 * I - 1, 2 * I):
+                continue
+            torch.cuda.synchronize()
+            total = S + step + 1
+            z = cache._zones[l]
+            assert z.seq_len == total
+            n_keys, n_cand, kk, tiers = cache.retrieval_shape(l)
+            assert n_keys == z.encoded == (S - sink - local) + I * ((step + 1) // I)
+            got_ids = cache.last_topk_indices.cpu().numpy()
+            codes = cache._codes_km[l].cpu().numpy()
+            nib = cache._nib_km[l].cpu().numpy()
+            w = cache._w_km[l].float().cpu().numpy()
+            cc = cache.cluster_key_counts_gpu[l].cpu().numpy()
+            for b in range(bs):
+                for h in range(Hkv):
+                    sl = slice(sink, sink + n_keys)
+                    # the cache's index over the retrieval zone equals the oracle's encoding of the true keys
+                    if step == 0:
+                        ec, en, ew = O.encode(hist_k[l][b, sink:sink + n_keys, h].float().numpy(), signs, O.BF16)
+                        assert np.array_equal(codes[b, h][sl], ec) and np.array_equal(nib[b, h][sl].reshape(-1, 16, 4), en)
+                        assert np.array_equal(w[b, h][sl], ew)
+                        assert np.array_equal(cc[b, h], O.count_cluster_keys(ec))
+                    ref_ids = O.retrieve_row(q[b, 0, h * G:(h + 1) * G].float().numpy(), signs, O.BF16, codes[b, h][sl],
+                                             nib[b, h][sl].reshape(-1, 16, 4), w[b, h][sl], cc[b, h], tiers, n_cand, kk)
+                    assert np.array_equal(got_ids[b, h], ref_ids), f"step {step} layer {l} row {(b, h)}"
+                # fp32 reference attention over sink ++ selected ++ dense tail
+                K = hist_k[l][b].permute(1, 0, 2)  # [Hkv, total, D]
+                V = hist_v[l][b].permute(1, 0, 2)
+                ref = torch.empty(Hq, 128)
+                for h in range(Hkv):
+                    sel = torch.cat([torch.arange(sink), torch.from_numpy(got_ids[b, h]) + sink,
+                                     torch.arange(sink + n_keys, total)])
+                    assert len(sel) == sink + kk + (total - sink - n_keys)
+                    ref[h * G:(h + 1) * G] = _ref_attention(q[b, 0, h * G:(h + 1) * G], K[h:h + 1, sel], V[h:h + 1, sel], G=G * 10)
+                err = (out[b, 0].float().cpu() - ref).abs().max().item()
+                assert err < 2e-2, f"attention differs by {err} at step {step} layer {l}"
+            checked += 1
+    assert checked >= 10
+    assert cache.context == S + steps
+
+
+@pytest.mark.parametrize("offload", [True, False])
+def test_short_sequences_use_dense_attention(offload):
+    """Below the retrieval threshold the cache attends to every token (polar_cache.py:1033-1045), whether the
+    tokens sit in the GPU window or already in the (host) retrieval zone; and a prompt shorter than
+    sink+local fills the dense rows first."""
+    bs, Hkv, Hq, S, steps = 1, 2, 4, 300, 40
+    G = Hq // Hkv
+    for S in (300, 20):
+        cache = _make_cache(offload, bs, Hkv, Hq, 1, S, steps + 5, 4, 32, 16, 50, thr=2000)
+        gen = torch.Generator().manual_seed(1)
+        k, v = _synth_kv(gen, bs, S, Hkv)
+        cache.prefill_update_kv_cache(None, k.to(DEV), v.to(DEV), 0, 0)
+        for step in range(steps):
+            k1, v1 = _synth_kv(gen, bs, 1, Hkv)
+            k, v = torch.cat([k, k1], 1), torch.cat([v, v1], 1)
+            q = torch.randn(bs, 1, Hq, 128, generator=gen).to(torch.bfloat16)
+            cache.decode_update_kv_cache(k1.to(DEV), v1.to(DEV), 0)
+            out = cache.compute(q.to(DEV), 0)
+            ref = _ref_attention(q[0, 0], k[0].permute(1, 0, 2), v[0].permute(1, 0, 2), G)
+            err = (out[0, 0].float().cpu() - ref).abs().max().item()
+            assert err < 2e-2, (S, step, err)
+        cache._zones[0].check()
+
+
+def test_single_sample_prefill_and_constructor_errors():
+    from pariskv_amd.cache_hub.polar_cache import polar_cache
+
+    bs, Hkv, Hq, S = 3, 2, 4, 600
+    cache = _make_cache(True, bs, Hkv, Hq, 1, S, 8, 4, 32, 16, 40)
+    gen = torch.Generator().manual_seed(2)
+    ks = []
+    for b in range(bs):  # one sample at a time (reference _prefill_single_sample)
+        k, v = _synth_kv(gen, 1, S, Hkv)
+        ks.append(k)
+        cache.prefill_update_kv_cache(None, k.to(DEV), v.to(DEV), 0, b)
+    torch.cuda.synchronize()
+    signs = O.srht_signs(42)
+    n = S - 36
+    for b in range(bs):
+        ec, _, _ = O.encode(ks[b][0, 4:4 + n, 1].float().numpy(), signs, O.BF16)
+        assert np.array_equal(cache._codes_km[0][b, 1, 4:4 + n].cpu().numpy(), ec)
+        assert torch.equal(cache.unified_keys_cpu[0][b, :, :n], ks[b][0, 4:4 + n].permute(1, 0, 2))
+    assert cache.context == S and cache.codebook_gpu[0].shape == (bs, Hkv, 16, S + 8)
+    with pytest.raises(ValueError):
+        _make_cache(True, 1, 2, 4, 1, 100, 8, 4, 32, 16, 40, codebook_path="/nonexistent.json")
+    with pytest.raises(ValueError):
+        polar_cache([0], 1, 1, 100, 2, 4, 64, torch.bfloat16, {0: DEV}, 8, 4, 32)
