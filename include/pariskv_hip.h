@@ -234,6 +234,31 @@ int pkv_host_free(void *host_ptr);
 /* Device-visible address of a pinned host pointer (PKV_EINVAL if not pinned). */
 int pkv_host_device_pointer(const void *host_ptr, void **dev_ptr);
 
+/* -------------------------------------------------------------- adaptive-k */
+
+/* Replaces adaptive_topk (cache_hub/adaptive_k_fused/adaptive_topk.cu:272-309;
+ * python adaptive_topk.py:331-405; semantics adaptive_topk_ref :255-313) and the
+ * v2 form whose source is absent from the reference (call site
+ * cache_hub/polar_cache_adaptivek_varlen.py:1741-1753).
+ * sl_logits/sl_vnorm float [rows][sl] (row strides given) are the exact, already
+ * scaled logits and value norms of the dense (sink/local/buffer) tokens.
+ * Candidate logit = float(cand_scores[row][i]) * cand_scale with cand_scores
+ * [rows][n_cand] of cand_dtype (PKV_DTYPE_F32 with cand_scale 1 for prescaled
+ * logits; PKV_DTYPE_BF16 with the attention scale for raw rerank scores).
+ * Candidate value norm = cand_vnorm[row][i], or, when cand_vnorm is NULL,
+ * value_norm[row*vn_stride + cand_ids[row][i] + vn_offset].
+ * benefit = exp(logit - max) * ||v||; adaptive_k[row] = smallest k <= k_out with
+ * dense_benefit + sum of the k largest candidate benefits >= threshold * total
+ * (k_out if never, 1 if total <= 0); topk_ids int64 [rows][k_out] = cand_ids in
+ * descending benefit order (ties: candidate position ascending).
+ * ws: pkv_adaptive_topk_ws_bytes(rows, n_cand, k_out) bytes. */
+size_t pkv_adaptive_topk_ws_bytes(int rows, int64_t n_cand, int64_t k_out);
+int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, const float *sl_vnorm, int64_t slv_stride,
+                      int64_t sl, const void *cand_scores, int cand_dtype, float cand_scale,
+                      const float *cand_vnorm, const float *value_norm, int64_t vn_stride, int64_t vn_offset,
+                      const int64_t *cand_ids, int64_t n_cand, float threshold, int64_t k_out, int rows,
+                      int64_t *adaptive_k, int64_t *topk_ids, void *ws, size_t ws_bytes, void *stream);
+
 /* ------------------------------------------------------- fused decode step */
 
 /* One layer's retrieval for one decode step, key-major storage:

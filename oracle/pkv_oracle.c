@@ -327,18 +327,19 @@ float pkv_o_expf(float x) {
   return y * u2f((uint32_t)(e + 127) << 23);
 }
 
-/* Sum in a fixed parallel-friendly order: 256 strided partial sums (element i
- * goes to lane i mod 256, accumulated in increasing i), then a pairwise tree
- * over the 256 lanes (stride 1, 2, 4, ...). */
-static float sum256(const float *x, int64_t n) {
-  float lane[256];
-  for (int t = 0; t < 256; ++t) {
+/* Sum in a fixed parallel-friendly order: 1024 strided partial sums (element i
+ * goes to lane i mod 1024, accumulated in increasing i), then a pairwise tree
+ * over the 1024 lanes (stride 1, 2, 4, ...). */
+#define PKV_O_SUM_LANES 1024
+static float sum_lanes(const float *x, int64_t n) {
+  float lane[PKV_O_SUM_LANES];
+  for (int t = 0; t < PKV_O_SUM_LANES; ++t) {
     float acc = 0.0f;
-    for (int64_t i = t; i < n; i += 256) acc = acc + x[i];
+    for (int64_t i = t; i < n; i += PKV_O_SUM_LANES) acc = acc + x[i];
     lane[t] = acc;
   }
-  for (int h = 1; h < 256; h <<= 1)
-    for (int i = 0; i < 256; i += 2 * h) lane[i] = lane[i] + lane[i + h];
+  for (int h = 1; h < PKV_O_SUM_LANES; h <<= 1)
+    for (int i = 0; i < PKV_O_SUM_LANES; i += 2 * h) lane[i] = lane[i] + lane[i + h];
   return lane[0];
 }
 
@@ -354,8 +355,8 @@ int64_t pkv_o_adaptive_topk(const float *sl_logits, const float *sl_vnorm, int64
   float *ben = (float *)malloc((size_t)(n_cand > 0 ? n_cand : 1) * sizeof(float));
   for (int64_t i = 0; i < sl; ++i) ben_sl[i] = pkv_o_expf(sl_logits[i] - g) * sl_vnorm[i];
   for (int64_t i = 0; i < n_cand; ++i) ben[i] = pkv_o_expf(cand_logits[i] - g) * cand_vnorm[i];
-  float sl_benefit = sum256(ben_sl, sl);        /* :289 */
-  float total = sl_benefit + sum256(ben, n_cand); /* :299 */
+  float sl_benefit = sum_lanes(ben_sl, sl);        /* :289 */
+  float total = sl_benefit + sum_lanes(ben, n_cand); /* :299 */
   /* :293-296 top-K_out by benefit, descending; ties by candidate position */
   int64_t *pos = (int64_t *)malloc((size_t)(k_out > 0 ? k_out : 1) * sizeof(int64_t));
   pkv_o_topk_f32(ben, NULL, n_cand, k_out, NULL, pos);

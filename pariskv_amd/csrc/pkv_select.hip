@@ -260,6 +260,173 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_radix_kernel(const floa
   emit_topk(s_keys, k, out_ids + (int64_t)row * k, out_vals ? out_vals + (int64_t)row * k : nullptr);
 }
 
+// ------------------------------------------------------------------ adaptive-k
+//
+// Reference: cache_hub/adaptive_k_fused/adaptive_topk.cu:108-266 (one 512-thread
+// block per row, 31 one-bit radix passes, atomic compaction, bitonic sort, serial
+// cumsum) with the semantics of adaptive_topk_ref (adaptive_topk.py:255-313).
+// Here: eight 8-bit passes over a 64-bit (benefit, position) key, so ties are
+// resolved by candidate position and the result is reproducible; sums run in a
+// fixed lane/tree order; exp() is a fixed fp32 sequence shared with the CPU checker.
+
+__device__ __forceinline__ float pkv_expf(float x) {
+  if (!(x >= -87.0f)) return (x != x) ? x : 0.0f;
+  if (x > 88.0f) return __uint_as_float(0x7f800000u);
+  const float n = rintf(x * 1.44269504f);
+  float r = x - n * 0.693359375f;
+  r = r - n * (-2.12194440e-4f);
+  float p = 1.9875691500e-4f;
+  p = p * r + 1.3981999507e-3f;
+  p = p * r + 8.3334519073e-3f;
+  p = p * r + 4.1665795894e-2f;
+  p = p * r + 1.6666665459e-1f;
+  p = p * r + 5.0000001201e-1f;
+  const float z = r * r;
+  float y = p * z + r;
+  y = y + 1.0f;
+  return y * __uint_as_float((uint32_t)((int)n + 127) << 23);
+}
+
+// Sum over the workgroup's 1024 lanes as a pairwise tree (stride 1, 2, 4, ...): xor butterflies
+// inside each wave, then the 16 wave sums.  Every thread returns the same value.
+__device__ __forceinline__ float block_tree_sum_1024(float v, float *s_part) {
+#pragma unroll
+  for (int m = 1; m < PKV_WAVE; m <<= 1) v = v + __shfl_xor(v, m, PKV_WAVE);
+  __syncthreads();
+  if (pkv_lane() == 0) s_part[threadIdx.x / PKV_WAVE] = v;
+  __syncthreads();
+  float w[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) w[i] = s_part[i];
+#pragma unroll
+  for (int h = 1; h < 16; h <<= 1)
+#pragma unroll
+    for (int i = 0; i < 16; i += 2 * h) w[i] = w[i] + w[i + h];
+  return w[0];
+}
+
+__device__ __forceinline__ float block_max_1024(float v, float *s_part) {
+#pragma unroll
+  for (int m = 1; m < PKV_WAVE; m <<= 1) v = fmaxf(v, __shfl_xor(v, m, PKV_WAVE));
+  __syncthreads();
+  if (pkv_lane() == 0) s_part[threadIdx.x / PKV_WAVE] = v;
+  __syncthreads();
+  float r = s_part[0];
+#pragma unroll
+  for (int i = 1; i < 16; ++i) r = fmaxf(r, s_part[i]);
+  return r;
+}
+
+__device__ __forceinline__ float cand_logit(const void *__restrict__ scores, int dtype, float scale, int64_t i) {
+  const float x = (dtype == PKV_DTYPE_BF16) ? pkv_bf16_bits_to_f32(((const uint16_t *)scores)[i])
+                                            : ((const float *)scores)[i];
+  return x * scale;
+}
+
+// One workgroup of 1024 threads per row; dynamic LDS P*8 bytes (P = pow2 >= k_out).
+__global__ __launch_bounds__(kTopkThreads) void pkv_adaptive_topk_kernel(
+    const float *__restrict__ sl_logits, int64_t sl_stride, const float *__restrict__ sl_vnorm, int64_t slv_stride,
+    int64_t sl, const void *__restrict__ cand_scores, int cand_dtype, float cand_scale,
+    const float *__restrict__ cand_vnorm, const float *__restrict__ value_norm, int64_t vn_stride, int64_t vn_offset,
+    const int64_t *__restrict__ cand_ids, int64_t n_cand, float threshold, int64_t k_out, int P,
+    int64_t *__restrict__ adaptive_k, int64_t *__restrict__ topk_ids, float *__restrict__ ws_ben) {
+  extern __shared__ uint64_t s_keys[];
+  __shared__ float s_part[16];
+  __shared__ uint32_t s_hist[257];
+  __shared__ uint32_t s_digit, s_need, s_counter;
+  const int row = blockIdx.x;
+  const int tid = threadIdx.x;
+  const float *sll = sl_logits + (int64_t)row * sl_stride;
+  const float *slv = sl_vnorm + (int64_t)row * slv_stride;
+  const char *cs = (const char *)cand_scores + (int64_t)row * n_cand * (cand_dtype == PKV_DTYPE_BF16 ? 2 : 4);
+  const int64_t *ci = cand_ids + (int64_t)row * n_cand;
+  const float *cv = cand_vnorm ? cand_vnorm + (int64_t)row * n_cand : nullptr;
+  const float *vn = value_norm ? value_norm + (int64_t)row * vn_stride : nullptr;
+  float *ben = ws_ben + (int64_t)row * n_cand;
+
+  // joint max of the dense (sink/local) logits and the candidate logits
+  float m = -__uint_as_float(0x7f800000u);
+  for (int64_t i = tid; i < sl; i += kTopkThreads) m = fmaxf(m, sll[i]);
+  for (int64_t i = tid; i < n_cand; i += kTopkThreads) m = fmaxf(m, cand_logit(cs, cand_dtype, cand_scale, i));
+  const float g = block_max_1024(m, s_part);
+
+  float acc = 0.f;
+  for (int64_t i = tid; i < sl; i += kTopkThreads) acc = acc + pkv_expf(sll[i] - g) * slv[i];
+  const float sl_benefit = block_tree_sum_1024(acc, s_part);
+  acc = 0.f;
+  for (int64_t i = tid; i < n_cand; i += kTopkThreads) {
+    const float vnorm = cv ? cv[i] : vn[ci[i] + vn_offset];
+    const float b = pkv_expf(cand_logit(cs, cand_dtype, cand_scale, i) - g) * vnorm;
+    ben[i] = b;
+    acc = acc + b;
+  }
+  const float total = sl_benefit + block_tree_sum_1024(acc, s_part);
+  __syncthreads();  // ben[] of this row is complete (written and read by this workgroup only)
+
+  // k_out-th largest (benefit, ~position) key
+  uint64_t prefix = 0;
+  uint32_t need = (uint32_t)k_out;
+  for (int pass = 0; pass < 8; ++pass) {
+    const int shift = 56 - 8 * pass;
+    if (tid < 257) s_hist[tid] = 0;
+    __syncthreads();
+    for (int64_t i = tid; i < n_cand; i += kTopkThreads) {
+      const uint64_t key = make_key(ben, nullptr, i);
+      if (pass == 0 || (key >> (shift + 8)) == (prefix >> (shift + 8)))
+        atomicAdd(&s_hist[(uint32_t)(key >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    uint32_t suf = 0, suf_next = 0;
+    if (tid < 256) {
+      for (int d = tid + 1; d < 256; ++d) suf_next += s_hist[d];
+      suf = suf_next + s_hist[tid];
+    }
+    __syncthreads();
+    if (tid < 256 && suf >= need && suf_next < need) {
+      s_digit = (uint32_t)tid;
+      s_need = need - suf_next;
+    }
+    __syncthreads();
+    prefix |= (uint64_t)s_digit << shift;
+    need = s_need;
+  }
+  if (tid == 0) s_counter = 0;
+  for (int i = tid; i < P; i += kTopkThreads) s_keys[i] = 0ull;
+  __syncthreads();
+  for (int64_t i = tid; i < n_cand; i += kTopkThreads) {
+    const uint64_t key = make_key(ben, nullptr, i);
+    if (key >= prefix) {
+      const uint32_t slot = atomicAdd(&s_counter, 1u);
+      if (slot < (uint32_t)k_out) s_keys[slot] = key;
+    }
+  }
+  __syncthreads();
+  bitonic_sort_desc(s_keys, P);
+
+  // smallest k with sl_benefit + cumsum_k >= threshold * total (sequential fp32 cumsum)
+  if (tid == 0) {
+    int64_t k = k_out;
+    if (total <= 0.f) {
+      k = 1;
+    } else {
+      float csum = 0.f;
+      const float tgt = threshold * total;
+      for (int64_t i = 0; i < k_out; ++i) {
+        csum = csum + pkv_from_ordered_u32((uint32_t)(s_keys[i] >> 32));
+        if (sl_benefit + csum >= tgt) {
+          k = i + 1;
+          break;
+        }
+      }
+    }
+    adaptive_k[row] = k;
+  }
+  for (int64_t i = tid; i < k_out; i += kTopkThreads) {
+    const uint32_t pos = ~(uint32_t)s_keys[i];
+    topk_ids[(int64_t)row * k_out + i] = (pos < (uint64_t)n_cand) ? ci[pos] : 0;
+  }
+}
+
 static int pow2_ceil(int64_t v) {
   int p = 1;
   while (p < v) p <<= 1;
@@ -367,4 +534,35 @@ extern "C" int pkv_topk_f32(const float *x, int64_t x_stride, const int64_t *ids
                             void *stream) {
   return pkv_launch_topk_f32(x, x_stride, ids, ids_stride, rows, len, k, out_ids, out_vals, ws, ws_bytes,
                              (hipStream_t)stream);
+}
+
+extern "C" size_t pkv_adaptive_topk_ws_bytes(int rows, int64_t n_cand, int64_t) {
+  if (rows <= 0 || n_cand <= 0) return 256;
+  return pkv_align_up((size_t)rows * (size_t)n_cand * sizeof(float), 256);
+}
+
+extern "C" int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, const float *sl_vnorm, int64_t slv_stride,
+                                 int64_t sl, const void *cand_scores, int cand_dtype, float cand_scale,
+                                 const float *cand_vnorm, const float *value_norm, int64_t vn_stride, int64_t vn_offset,
+                                 const int64_t *cand_ids, int64_t n_cand, float threshold, int64_t k_out, int rows,
+                                 int64_t *adaptive_k, int64_t *topk_ids, void *ws, size_t ws_bytes, void *stream) {
+  PKV_REQUIRE(cand_scores && cand_ids && adaptive_k && topk_ids && (cand_vnorm || value_norm),
+              "pkv_adaptive_topk: null pointer");
+  PKV_REQUIRE(sl >= 0 && (sl == 0 || (sl_logits && sl_vnorm)), "pkv_adaptive_topk: dense logits missing");
+  PKV_REQUIRE(cand_dtype == PKV_DTYPE_F32 || cand_dtype == PKV_DTYPE_BF16, "unknown candidate score dtype %d", cand_dtype);
+  PKV_REQUIRE(rows > 0 && n_cand > 0 && n_cand < ((int64_t)1 << 31) && k_out > 0 && k_out <= n_cand,
+              "need 0 < k_out <= n_cand (k_out=%lld n_cand=%lld rows=%d)", (long long)k_out, (long long)n_cand, rows);
+  PKV_REQUIRE(k_out <= kTopkMaxSort, "k_out up to %d supported (got %lld)", kTopkMaxSort, (long long)k_out);
+  const size_t need = pkv_adaptive_topk_ws_bytes(rows, n_cand, k_out);
+  if (!ws || ws_bytes < need || !pkv_aligned(ws, 16)) {
+    pkv_set_error("pkv_adaptive_topk: workspace of %zu bytes required, got %zu", need, ws_bytes);
+    return PKV_ENOMEM;
+  }
+  const int P = pow2_ceil(k_out);
+  hipLaunchKernelGGL(pkv_adaptive_topk_kernel, dim3((unsigned)rows), dim3(kTopkThreads), (size_t)P * 8,
+                     (hipStream_t)stream, sl_logits, sl_stride, sl_vnorm, slv_stride, sl, cand_scores, cand_dtype,
+                     cand_scale, cand_vnorm, value_norm, vn_stride, vn_offset, cand_ids, n_cand, threshold, k_out, P,
+                     adaptive_k, topk_ids, (float *)ws);
+  PKV_LAUNCH_CHECK("pkv_adaptive_topk_kernel");
+  return PKV_OK;
 }

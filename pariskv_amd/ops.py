@@ -295,6 +295,46 @@ def rerank4(coarse_indices: torch.Tensor, key_4bit: torch.Tensor, key_block_weig
     return scores, v4b
 
 
+def adaptive_topk(sl_logits: torch.Tensor, sl_vnorm: torch.Tensor, cand_scores: torch.Tensor, cand_scale: float,
+                  cand_ids: torch.Tensor, threshold: float, k_out: int, cand_vnorm: Optional[torch.Tensor] = None,
+                  value_norm: Optional[torch.Tensor] = None, vn_offset: int = 0):
+    """Adaptive top-k by value-weighted attention mass.
+
+    sl_logits / sl_vnorm fp32 [bs,H,sl] (last dim contiguous); cand_scores fp32 or bf16 [bs,H,C] contiguous
+    (logit = score * cand_scale); cand_ids int64 [bs,H,C]; candidate value norms either ``cand_vnorm`` fp32 [bs,H,C]
+    or gathered from ``value_norm`` fp32 [bs,H,cap] at ``cand_ids + vn_offset``.
+    Returns (adaptive_k int64 [bs,H], topk_ids int64 [bs,H,k_out])."""
+    _cuda(sl_logits, sl_vnorm, cand_scores, cand_ids, cand_vnorm, value_norm)
+    bs, H, Cn = cand_scores.shape
+    rows = bs * H
+    _need(cand_scores.is_contiguous() and cand_ids.is_contiguous() and cand_ids.dtype == torch.int64 and
+          tuple(cand_ids.shape) == (bs, H, Cn), "cand_scores / cand_ids must be contiguous [bs,H,C]")
+    sl = sl_logits.shape[-1]
+    for t in (sl_logits, sl_vnorm):
+        _need(t.dtype == torch.float32 and tuple(t.shape) == (bs, H, sl) and (sl == 0 or t.stride(2) == 1) and
+              (H == 1 or t.stride(0) == H * t.stride(1)), "dense logits / value norms must be fp32 [bs,H,sl] with uniform row stride")
+    _need(0 < k_out <= Cn, "topk_cap must be in (0, cand_len]")
+    if cand_vnorm is not None:
+        _need(cand_vnorm.dtype == torch.float32 and cand_vnorm.is_contiguous() and tuple(cand_vnorm.shape) == (bs, H, Cn),
+              "cand_vnorm must be contiguous fp32 [bs,H,C]")
+        vn_stride = 0
+    else:
+        _need(value_norm is not None and value_norm.dtype == torch.float32 and value_norm.is_contiguous() and
+              tuple(value_norm.shape[:2]) == (bs, H), "value_norm must be contiguous fp32 [bs,H,cap]")
+        vn_stride = value_norm.shape[2]
+    dev = cand_scores.device
+    ak = torch.empty(bs, H, dtype=torch.int64, device=dev)
+    ids = torch.empty(bs, H, k_out, dtype=torch.int64, device=dev)
+    nbytes = _lib.lib().pkv_adaptive_topk_ws_bytes(rows, Cn, k_out)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    row_stride = lambda t: t.stride(1) if H > 1 else (t.stride(0) if bs > 1 else max(1, sl))
+    _lib.check(_lib.lib().pkv_adaptive_topk(
+        _p(sl_logits), row_stride(sl_logits), _p(sl_vnorm), row_stride(sl_vnorm), sl, _p(cand_scores),
+        _dt(cand_scores.dtype), float(cand_scale), _p(cand_vnorm), _p(value_norm), vn_stride, vn_offset, _p(cand_ids), Cn,
+        float(threshold), k_out, rows, _p(ak), _p(ids), _p(ws), nbytes, _stream(cand_scores)))
+    return ak, ids
+
+
 # ------------------------------------------------------------------ gathers
 
 

@@ -549,3 +549,78 @@ def test_full_size_properties(ops, N, R, C, K):
         assert np.array_equal(codes_km[b, h].cpu().numpy(), codes)
         assert np.array_equal(nib_km[b, h].cpu().numpy().reshape(N, 16, 4), nib)
         assert np.array_equal(w_km[b, h].float().cpu().numpy(), wt)
+
+
+# --------------------------------------------------------------- adaptive-k
+
+
+def _adaptive_recipe(bs, kv_heads, sl_len, cand_len, seed, head_dim=128):
+    """Seeded input recipe of the reference's adaptive-k self-test (adaptive_topk.py:178-249), on the CPU."""
+    torch.manual_seed(seed)
+    q = (torch.randn(bs, kv_heads, head_dim) * 0.1).to(torch.bfloat16)
+    slk = (torch.randn(bs, kv_heads, sl_len, head_dim) * 0.1).to(torch.bfloat16)
+    sl_vnorm = torch.rand(bs, kv_heads, sl_len) + 0.5
+    base = math.sqrt(head_dim)
+    cs = torch.randn(bs, kv_heads, cand_len) * (0.3 * base)
+    rng = torch.Generator().manual_seed(seed)
+    heavy = torch.randint(16, 1025, (bs, kv_heads), generator=rng).tolist()
+    for b in range(bs):
+        for h in range(kv_heads):
+            n = min(heavy[b][h], cand_len)
+            cs[b, h, :n] += torch.rand(n) * 5.0 * base + 3.0 * base
+    ci = torch.stack([torch.stack([torch.randperm(cand_len) for _ in range(kv_heads)]) for _ in range(bs)])
+    cv = torch.rand(bs, kv_heads, cand_len) + 0.5
+    return q, slk, sl_vnorm, cs.to(torch.bfloat16), ci, cv, 1.0 / base
+
+
+@pytest.mark.parametrize("cfg", [dict(bs=1, kv_heads=8, sl_len=320, cand_len=12500, topk_cap=2048, threshold=0.95, seed=42),
+                                 dict(bs=1, kv_heads=8, sl_len=832, cand_len=5000, topk_cap=2048, threshold=0.95, seed=7),
+                                 dict(bs=2, kv_heads=8, sl_len=576, cand_len=8000, topk_cap=2048, threshold=0.85, seed=123),
+                                 dict(bs=1, kv_heads=16, sl_len=320, cand_len=15000, topk_cap=2048, threshold=0.95, seed=99),
+                                 dict(bs=1, kv_heads=2, sl_len=64, cand_len=700, topk_cap=2048, threshold=0.95, seed=5),
+                                 dict(bs=1, kv_heads=2, sl_len=320, cand_len=104858, topk_cap=2048, threshold=0.95, seed=6)])
+def test_adaptive_topk_matches_oracle(ops, cfg):
+    """The reference's four seeded shapes (adaptive_topk.py:492-497) + a short and a 1M-context-sized one.
+    Its acceptance rule is `k exact, first-k index sets equal`; with the fixed tie rule the whole list is compared."""
+    from pariskv_amd.cache_hub.adaptive_k_fused import adaptive_topk_cuda
+
+    _say(f"adaptive_topk {cfg}")
+    q, slk, slv, cs, ci, cv, scale = _adaptive_recipe(cfg["bs"], cfg["kv_heads"], cfg["sl_len"], cfg["cand_len"], cfg["seed"])
+    ak, ids = adaptive_topk_cuda(q.to(DEV), slk.to(DEV), slv.to(DEV), cs.to(DEV), ci.to(DEV), cv.to(DEV), scale,
+                                 cfg["threshold"], cfg["topk_cap"])
+    torch.cuda.synchronize()
+    k_out = min(cfg["topk_cap"], cfg["cand_len"])
+    assert tuple(ids.shape) == (cfg["bs"], cfg["kv_heads"], k_out) and ak.dtype == torch.int64
+    # same dense logits expression as the call under test, evaluated by torch on the GPU
+    sl_logits = (torch.einsum("bhd,bhkd->bhk", q.to(DEV), slk.to(DEV)).to(torch.float32) * scale).cpu().numpy()
+    for b in range(cfg["bs"]):
+        for h in range(cfg["kv_heads"]):
+            lc = (cs[b, h].float() * np.float32(scale)).numpy()
+            k_ref, ids_ref = O.adaptive_topk(sl_logits[b, h], slv[b, h].numpy(), lc, cv[b, h].numpy(), ci[b, h].numpy(),
+                                             cfg["threshold"], k_out)
+            assert int(ak[b, h]) == k_ref, (b, h, int(ak[b, h]), k_ref)
+            assert np.array_equal(ids[b, h].cpu().numpy(), ids_ref)
+    assert int(ak.min()) >= 1 and int(ak.max()) <= k_out
+
+
+def test_adaptive_topk_value_norm_gather_and_edges(ops):
+    """v2 form: bf16 scores scaled in the kernel, ||v|| gathered at cand_idx + sink (varlen call site :1741-1753);
+    plus total <= 0 -> 1 and never reached -> k_out."""
+    bs, H, sl, Cn, cap, sink = 1, 3, 100, 3000, 5000, 64
+    q, slk, slv, cs, ci, cv, scale = _adaptive_recipe(bs, H, sl, Cn, 11)
+    vn = torch.rand(bs, H, cap) + 0.5
+    sl_logits = (torch.einsum("bhd,bhkd->bhk", q, slk).float() * scale)
+    ak, ids = ops.adaptive_topk(sl_logits.to(DEV), slv.to(DEV), cs.to(DEV), scale, ci.to(DEV), 0.9, 1024,
+                                value_norm=vn.to(DEV), vn_offset=sink)
+    for h in range(H):
+        cvn = vn[0, h][ci[0, h] + sink]
+        k_ref, ids_ref = O.adaptive_topk(sl_logits[0, h].numpy(), slv[0, h].numpy(), (cs[0, h].float() * np.float32(scale)).numpy(),
+                                         cvn.numpy(), ci[0, h].numpy(), 0.9, 1024)
+        assert int(ak[0, h]) == k_ref and np.array_equal(ids[0, h].cpu().numpy(), ids_ref)
+    z = torch.zeros(1, 1, 50, device=DEV)
+    ak, _ = ops.adaptive_topk(z[..., :5], z[..., :5], z, 1.0, torch.arange(50, device=DEV).view(1, 1, 50), 0.95, 10, cand_vnorm=z)
+    assert int(ak) == 1
+    one = torch.ones(1, 1, 50, device=DEV)
+    ak, ids = ops.adaptive_topk(z[..., :1], one[..., :1], z, 1.0, torch.arange(50, device=DEV).flip(0).view(1, 1, 50).contiguous(),
+                                0.95, 10, cand_vnorm=one)
+    assert int(ak) == 10 and ids[0, 0].cpu().tolist() == list(range(49, 39, -1))
