@@ -624,3 +624,92 @@ def test_adaptive_topk_value_norm_gather_and_edges(ops):
     ak, ids = ops.adaptive_topk(z[..., :1], one[..., :1], z, 1.0, torch.arange(50, device=DEV).flip(0).view(1, 1, 50).contiguous(),
                                 0.95, 10, cand_vnorm=one)
     assert int(ak) == 10 and ids[0, 0].cpu().tolist() == list(range(49, 39, -1))
+
+
+# ---------------------------------- BASELINE config 4: 1M keys, adaptive-k, packed gather
+
+
+def test_million_key_adaptive_pipeline(ops):
+    """Llama-3-8B head shape, batch 1, 1M cached keys per head with a slowly drifting key mean (0.5 degrees per 1K
+    tokens), bucket top-k over 1M vote counts, rerank of all candidates, adaptive-k (k clamped to [256, 2048], mass
+    0.95), packed UVA gather.  Every stage of two sampled rows is compared with the oracle; the rest by properties."""
+    from pariskv_amd.cache_hub.topk import load_radix_topk_ext
+
+    _say("cfg4: N=2^20")
+    bs, H, G, N = 1, 8, 4, 1 << 20
+    sink, sl = 64, 64 + 512
+    Cn = int(math.ceil(N * 0.05))
+    cap_k, min_k, thr = 2048, 256, 0.95
+    g = torch.Generator(device=DEV).manual_seed(4)
+    keys = torch.randn(bs, H, N, 128, generator=g, device=DEV)
+    keys[..., [7, 31, 64, 101]] *= 10.0
+    ang = torch.arange(N, device=DEV, dtype=torch.float32) * (0.5 / 1000.0) * (math.pi / 180.0)
+    keys[..., 0] += 3.0 * torch.cos(ang)
+    keys[..., 1] += 3.0 * torch.sin(ang)
+    keys = keys.to(torch.bfloat16)
+    q = (keys[:, :, -4096:].float().mean(dim=2, keepdim=True) + 0.5 * torch.randn(bs, H, G, 128, generator=g, device=DEV))
+    q = q.to(torch.bfloat16).view(bs, 1, H * G, 128).contiguous()
+    signs = ops.srht_signs(DEV)
+    codes_km, nib_km, w_km, cb, k4, kw = ops.alloc_keymajor(bs, H, N, DEV)
+    cc = torch.zeros(bs, H, 16, 256, dtype=torch.int32, device=DEV)
+    ops.encode_append(keys, signs, cb, k4, kw, cc)
+    tiers = O.tier_counts(N, 0.2)
+    assert tiers == [10486, 31458, 62915, 104858, 157287, 209716]
+    qhat, qnorm, lut, _ = ops.query_prep_lut(q, H, signs, cc, tiers)
+    cnt, _, _ = ops.collision_scan(cb, lut, out_dtype=torch.int32)
+    cand = load_radix_topk_ext().radix_topk_3d(cnt, Cn)          # "radix top-k over 1M scores" (polar_cache.py:1241)
+    scores, _ = ops.rerank4(cand, k4, kw, qhat, qnorm, ops.mag_centers(DEV))
+    # dense side of adaptive-k: logits and value norms of sink + local tokens, ||v|| of every cached token
+    sl_logits = torch.randn(bs, H, sl, generator=g, device=DEV) * 0.5
+    sl_vnorm = torch.rand(bs, H, sl, generator=g, device=DEV) + 0.5
+    value_norm = torch.rand(bs, H, N + sink, generator=g, device=DEV) + 0.5
+    scale = 1.0 / math.sqrt(128)
+    k_out = min(cap_k, Cn)
+    ak, ids = ops.adaptive_topk(sl_logits, sl_vnorm, scores, scale, cand, thr, k_out, value_norm=value_norm, vn_offset=sink)
+    ak = ak.clamp(min=max(1, min_k), max=max(1, cap_k))           # polar_cache_adaptivek_varlen.py:1759
+    torch.cuda.synchronize()
+    sg = signs.cpu().numpy()
+    for r in (1, 6):
+        codes = codes_km[0, r].cpu().numpy()
+        ec, en, ew = O.encode(keys[0, r].float().cpu().numpy(), sg, O.BF16)
+        assert np.array_equal(codes, ec) and np.array_equal(nib_km[0, r].cpu().numpy().reshape(N, 16, 4), en)
+        assert np.array_equal(w_km[0, r].float().cpu().numpy(), ew)
+        assert np.array_equal(cc[0, r].cpu().numpy(), O.count_cluster_keys(ec))
+        qh, qn = O.query_prep(q.view(bs, H, G, 128)[0, r].float().cpu().numpy(), sg, O.BF16)
+        lut_ref = O.tier_lut(O.rank_centroids(qh, O.BF16), cc[0, r].cpu().numpy(), tiers)
+        cnt_ref = O.collision_count(ec, lut_ref)
+        assert np.array_equal(cnt[0, r].cpu().numpy(), cnt_ref)
+        cand_ref, _ = O.select_candidates(cnt_ref, Cn)
+        assert np.array_equal(cand[0, r].cpu().numpy(), cand_ref)
+        sc_ref = O.rerank(cand_ref, en, ew, qh, qn)
+        got = scores[0, r].cpu().numpy()
+        np.testing.assert_allclose(got, sc_ref, rtol=1e-5, atol=1e-5 * np.abs(sc_ref).max())
+        vn = value_norm[0, r].cpu().numpy()[cand_ref + sink]
+        k_ref, ids_ref = O.adaptive_topk(sl_logits[0, r].cpu().numpy(), sl_vnorm[0, r].cpu().numpy(), got * np.float32(scale), vn,
+                                         cand_ref, thr, k_out)
+        assert int(ak[0, r]) == min(max(k_ref, min_k), cap_k)
+        assert np.array_equal(ids[0, r].cpu().numpy(), ids_ref)
+    assert int(ak.min()) >= min_k and int(ak.max()) <= cap_k
+    # pack the per-head prefixes (polar_cache_adaptivek_varlen.py:1817-1832) and gather them raggedly out of host memory
+    V = bs * H
+    mask = torch.arange(k_out, device=DEV).unsqueeze(0) < ak.view(V, 1)
+    packed = ids.view(V, k_out)[mask].contiguous()
+    cu_topk = torch.zeros(V + 1, dtype=torch.int32, device=DEV)
+    cu_topk[1:] = torch.cumsum(ak.view(V), 0)
+    cu_k = torch.zeros(V + 1, dtype=torch.int32, device=DEV)
+    cu_k[1:] = torch.cumsum(ak.view(V) + sl, 0)
+    total = int(cu_k[-1])
+    kcpu = torch.empty(bs, H, N, 128, dtype=torch.bfloat16, pin_memory=True)
+    vcpu = torch.empty(bs, H, N, 128, dtype=torch.bfloat16, pin_memory=True)
+    kcpu.copy_(keys)
+    vcpu.copy_(-keys)
+    kp = torch.zeros(total, 128, dtype=torch.bfloat16, device=DEV)
+    vp = torch.zeros_like(kp)
+    ops.gather_uva_packed(kcpu, vcpu, kp, vp, packed, cu_topk, cu_k, sl, int(ak.max()))
+    torch.cuda.synchronize()
+    for v in range(V):
+        n = int(ak.view(V)[v])
+        sel = ids.view(V, k_out)[v, :n]
+        base = int(cu_k[v]) + sl
+        assert torch.equal(kp[base:base + n], keys[0, v][sel]) and torch.equal(vp[base:base + n], -keys[0, v][sel])
+        assert not kp[int(cu_k[v]):base].any()   # the sink/local slots are the caller's to fill
