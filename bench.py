@@ -117,6 +117,7 @@ def main():
     cnt_stride = (N + 15) // 16 * 16
     cnt_ws = torch.empty(R, cnt_stride, dtype=torch.uint8, device=dev)
     hist_ws = torch.empty(R, n_chunks, 128, dtype=torch.int16, device=dev)
+    rowsuf_ws = torch.zeros(R, 128, dtype=torch.int32, device=dev)
     luts = []
     for ly in layers:
         _, _, lut, _ = ops.query_prep_lut(ly["q"], H, signs, ly["cc"], tiers)
@@ -126,8 +127,8 @@ def main():
     def scan_only(i):
         ly = layers[i % L]
         _lib.check(lib.pkv_collision_scan(ly["codes"].data_ptr(), H * N * 16, N * 16, 16, 1, bs, H, N,
-                                          luts[i % L].data_ptr(), cnt_ws.data_ptr(), None, hist_ws.data_ptr(), chunk,
-                                          stream))
+                                          luts[i % L].data_ptr(), cnt_ws.data_ptr(), None, rowsuf_ws.data_ptr(),
+                                          hist_ws.data_ptr(), chunk, stream))
 
     if args.only == "scan":
         for i in range(args.warmup + args.steps):
@@ -167,7 +168,7 @@ def main():
         ly = layers[i % L]
         _lib.check(lib.pkv_collision_scan_timed(ly["codes"].data_ptr(), H * N * 16, N * 16, 16, 1, bs, H, N,
                                                 luts[i % L].data_ptr(), cnt_ws.data_ptr(), cnt_stride,
-                                                hist_ws.data_ptr(), chunk, C.byref(kus), stream))
+                                                rowsuf_ws.data_ptr(), hist_ws.data_ptr(), chunk, C.byref(kus), stream))
         if i >= args.warmup:
             scan_us.append(kus.value)
     scan_avg_us = sum(scan_us) / len(scan_us)

@@ -121,14 +121,17 @@ int pkv_update_cache_cnt_legacy(const int32_t *sorted_ids, const int32_t *topk_c
 
 /* The scan stage of the fused pipeline: votes per key from a ready LUT
  * (the per-key loop of cache_hub/collision_fused/collision.cu:204-228).
- * cnt_u8 [R][n_keys] and/or cnt_i32 [R][n_keys] (either may be NULL, not both);
- * chunk_hist uint16 [R][n_chunks][128] (NULL to skip) receives the histogram of
- * each `chunk_keys`-key chunk, n_chunks = ceil(n_keys / chunk_keys);
+ * cnt_u8 [R][n_keys] and/or cnt_i32 [R][n_keys] (either may be NULL, not both).
+ * When chunk_suf is non-NULL the pass also leaves the histograms the candidate
+ * select needs, in suffix form (suf[t] = number of keys with count >= t):
+ * chunk_suf uint16 [R][n_chunks][128] for each `chunk_keys`-key chunk
+ * (n_chunks = ceil(n_keys / chunk_keys)) and row_suf uint32 [R][128], which is
+ * ADDED to with atomics and must be zero on entry.
  * chunk_keys must be a multiple of 2048 and at most 32768. */
 int pkv_collision_scan(const uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t cs_key, int64_t cs_sub,
                        int bs, int n_kv_heads, int64_t n_keys, const uint8_t *lut,
-                       uint8_t *cnt_u8, int32_t *cnt_i32, uint16_t *chunk_hist, int chunk_keys,
-                       void *stream);
+                       uint8_t *cnt_u8, int32_t *cnt_i32, uint32_t *row_suf, uint16_t *chunk_suf,
+                       int chunk_keys, void *stream);
 
 /* pkv_collision_scan (u8 counts, row stride cnt_u8_stride) as ONE launch whose
  * own begin/end timestamps are returned in *kernel_us: the call blocks until
@@ -136,8 +139,8 @@ int pkv_collision_scan(const uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t
  * no counterpart in the reference. */
 int pkv_collision_scan_timed(const uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t cs_key, int64_t cs_sub,
                              int bs, int n_kv_heads, int64_t n_keys, const uint8_t *lut,
-                             uint8_t *cnt_u8, int64_t cnt_u8_stride, uint16_t *chunk_hist, int chunk_keys,
-                             float *kernel_us, void *stream);
+                             uint8_t *cnt_u8, int64_t cnt_u8_stride, uint32_t *row_suf, uint16_t *chunk_suf,
+                             int chunk_keys, float *kernel_us, void *stream);
 
 /* ------------------------------------------------------------- selections */
 
@@ -305,8 +308,8 @@ size_t pkv_retrieve_ws_bytes(int rows, int64_t n_keys, int64_t n_cand, int64_t k
 int pkv_retrieve(const pkv_retrieve_args *args, void *ws, size_t ws_bytes, void *stream);
 
 /* Names and device pointers of the intermediates inside a pkv_retrieve
- * workspace (for tests and profiling): qhat, qnorm, lut, cnt_u8, chunk_hist,
- * cand, scores.  Returns PKV_EINVAL for an unknown name. */
+ * workspace (for tests and profiling): qhat, qnorm, lut, cnt_u8,
+ * chunk_suffix_hist, row_suffix_hist, cand, scores.  Returns PKV_EINVAL for an unknown name. */
 int pkv_retrieve_ws_view(void *ws, int rows, int64_t n_keys, int64_t n_cand, int64_t k,
                          const char *name, void **ptr, size_t *bytes);
 

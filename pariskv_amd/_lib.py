@@ -52,8 +52,8 @@ PROTOTYPES = {
     "pkv_update_cache_cnt": (_i, [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64,
                                   _i, _i, _i64, _vp, _i, _vp, _vp, _vp]),
     "pkv_update_cache_cnt_legacy": (_i, [_vp, _vp, _vp, _i, _i, _i64, _vp, _vp, _vp]),
-    "pkv_collision_scan": (_i, [_vp, _i64, _i64, _i64, _i64, _i, _i, _i64, _vp, _vp, _vp, _vp, _i, _vp]),
-    "pkv_collision_scan_timed": (_i, [_vp, _i64, _i64, _i64, _i64, _i, _i, _i64, _vp, _vp, _i64, _vp, _i,
+    "pkv_collision_scan": (_i, [_vp, _i64, _i64, _i64, _i64, _i, _i, _i64, _vp, _vp, _vp, _vp, _vp, _i, _vp]),
+    "pkv_collision_scan_timed": (_i, [_vp, _i64, _i64, _i64, _i64, _i, _i, _i64, _vp, _vp, _i64, _vp, _vp, _i,
                                       C.POINTER(C.c_float), _vp]),
     "pkv_copy_bytes": (_i, [_vp, _vp, _sz, _vp]),
     "pkv_bucket_topk_ws_bytes": (_sz, [_i, _i64]),

@@ -39,14 +39,14 @@ __device__ __forceinline__ void load_lut(uint32_t *s_lut, const uint8_t *__restr
 __global__ __launch_bounds__(kScanThreads) void pkv_scan_keymajor_kernel(
     const uint8_t *__restrict__ codes, int64_t cs_b, int64_t cs_h, int n_kv_heads, int64_t n_keys,
     const uint8_t *__restrict__ lut, uint8_t *__restrict__ cnt_u8, int64_t cnt_u8_stride,
-    int32_t *__restrict__ cnt_i32, uint16_t *__restrict__ chunk_hist, int chunk_keys) {
+    int32_t *__restrict__ cnt_i32, uint32_t *__restrict__ row_suf, uint16_t *__restrict__ chunk_suf, int chunk_keys) {
   const int row = blockIdx.y;
   const int chunk = blockIdx.x;
   const int b = row / n_kv_heads, h = row % n_kv_heads;
   const int tid = threadIdx.x;
 
   __shared__ uint32_t s_lut[1024];
-  __shared__ uint32_t s_hist[128 * kHistCopies];
+  __shared__ uint32_t s_hist[128 * kHistCopies];  // also reused for the compacted histogram
   load_lut(s_lut, lut, row);
   for (int i = tid; i < 128 * kHistCopies; i += kScanThreads) s_hist[i] = 0;
   __syncthreads();
@@ -73,18 +73,22 @@ __global__ __launch_bounds__(kScanThreads) void pkv_scan_keymajor_kernel(
         const int c = lut_sum16(l8, v[u]);
         if (out8) out8[i] = (uint8_t)c;
         if (out32) out32[i] = c;
-        if (chunk_hist) atomicAdd(&s_hist[c * kHistCopies + copy], 1u);
+        if (chunk_suf) atomicAdd(&s_hist[c * kHistCopies + copy], 1u);
       }
     }
   }
-  if (chunk_hist) {
+  if (chunk_suf) {
     __syncthreads();
+    uint32_t sum = 0;
     if (tid < 128) {
-      uint32_t s = 0;
 #pragma unroll
-      for (int c = 0; c < kHistCopies; ++c) s += s_hist[tid * kHistCopies + c];
-      chunk_hist[((int64_t)row * gridDim.x + chunk) * 128 + tid] = (uint16_t)s;
+      for (int c = 0; c < kHistCopies; ++c) sum += s_hist[tid * kHistCopies + c];
     }
+    __syncthreads();
+    if (tid < 128) s_hist[tid] = sum;  // compacted histogram in the first 128 words
+    __syncthreads();
+    pkv_store_suffix_hist(s_hist, &s_hist[128], row_suf + (int64_t)row * 128,
+                          chunk_suf + ((int64_t)row * gridDim.x + chunk) * 128);
   }
 }
 
@@ -92,14 +96,14 @@ __global__ __launch_bounds__(kScanThreads) void pkv_scan_keymajor_kernel(
 __global__ __launch_bounds__(kScanThreads) void pkv_scan_strided_kernel(
     const uint8_t *__restrict__ codes, int64_t cs_b, int64_t cs_h, int64_t cs_key, int64_t cs_sub, int n_kv_heads,
     int64_t n_keys, const uint8_t *__restrict__ lut, uint8_t *__restrict__ cnt_u8, int64_t cnt_u8_stride,
-    int32_t *__restrict__ cnt_i32, uint16_t *__restrict__ chunk_hist, int chunk_keys) {
+    int32_t *__restrict__ cnt_i32, uint32_t *__restrict__ row_suf, uint16_t *__restrict__ chunk_suf, int chunk_keys) {
   const int row = blockIdx.y;
   const int chunk = blockIdx.x;
   const int b = row / n_kv_heads, h = row % n_kv_heads;
   const int tid = threadIdx.x;
 
   __shared__ uint32_t s_lut[1024];
-  __shared__ uint32_t s_hist[128 * kHistCopies];
+  __shared__ uint32_t s_hist[128 * kHistCopies];  // also reused for the compacted histogram
   load_lut(s_lut, lut, row);
   for (int i = tid; i < 128 * kHistCopies; i += kScanThreads) s_hist[i] = 0;
   __syncthreads();
@@ -118,16 +122,20 @@ __global__ __launch_bounds__(kScanThreads) void pkv_scan_strided_kernel(
     for (int s = 0; s < 16; ++s) c += l8[s * 256 + base[i * cs_key + s * cs_sub]];
     if (out8) out8[i] = (uint8_t)c;
     if (out32) out32[i] = c;
-    if (chunk_hist) atomicAdd(&s_hist[c * kHistCopies + copy], 1u);
+    if (chunk_suf) atomicAdd(&s_hist[c * kHistCopies + copy], 1u);
   }
-  if (chunk_hist) {
+  if (chunk_suf) {
     __syncthreads();
+    uint32_t sum = 0;
     if (tid < 128) {
-      uint32_t s = 0;
 #pragma unroll
-      for (int c = 0; c < kHistCopies; ++c) s += s_hist[tid * kHistCopies + c];
-      chunk_hist[((int64_t)row * gridDim.x + chunk) * 128 + tid] = (uint16_t)s;
+      for (int c = 0; c < kHistCopies; ++c) sum += s_hist[tid * kHistCopies + c];
     }
+    __syncthreads();
+    if (tid < 128) s_hist[tid] = sum;  // compacted histogram in the first 128 words
+    __syncthreads();
+    pkv_store_suffix_hist(s_hist, &s_hist[128], row_suf + (int64_t)row * 128,
+                          chunk_suf + ((int64_t)row * gridDim.x + chunk) * 128);
   }
 }
 
@@ -157,8 +165,8 @@ __global__ __launch_bounds__(kScanThreads) void pkv_scan_i32_codes_kernel(const 
 
 static int launch_scan_impl(const uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t cs_key, int64_t cs_sub, int bs,
                             int n_kv_heads, int64_t n_keys, const uint8_t *lut, uint8_t *cnt_u8,
-                            int64_t cnt_u8_stride, int32_t *cnt_i32, uint16_t *chunk_hist, int chunk_keys,
-                            hipStream_t s, hipEvent_t ev_start, hipEvent_t ev_stop) {
+                            int64_t cnt_u8_stride, int32_t *cnt_i32, uint32_t *row_suf, uint16_t *chunk_suf,
+                            int chunk_keys, hipStream_t s, hipEvent_t ev_start, hipEvent_t ev_stop) {
   PKV_REQUIRE(chunk_keys >= 2048 && chunk_keys % 2048 == 0 && chunk_keys <= 32768,
               "chunk_keys must be a multiple of 2048 in [2048,32768], got %d", chunk_keys);
   const int64_t n_chunks = (n_keys + chunk_keys - 1) / chunk_keys;
@@ -169,12 +177,12 @@ static int launch_scan_impl(const uint8_t *codes, int64_t cs_b, int64_t cs_h, in
   if (keymajor) {
     // the ext launch ties the two events to this dispatch's own begin/end timestamps
     hipExtLaunchKernelGGL(pkv_scan_keymajor_kernel, grid, dim3(kScanThreads), 0, s, ev_start, ev_stop, 0, codes, cs_b,
-                          cs_h, n_kv_heads, n_keys, lut, cnt_u8, cnt_u8_stride, cnt_i32, chunk_hist, chunk_keys);
+                          cs_h, n_kv_heads, n_keys, lut, cnt_u8, cnt_u8_stride, cnt_i32, row_suf, chunk_suf, chunk_keys);
     PKV_LAUNCH_CHECK("pkv_scan_keymajor_kernel");
   } else {
     hipExtLaunchKernelGGL(pkv_scan_strided_kernel, grid, dim3(kScanThreads), 0, s, ev_start, ev_stop, 0, codes, cs_b,
-                          cs_h, cs_key, cs_sub, n_kv_heads, n_keys, lut, cnt_u8, cnt_u8_stride, cnt_i32, chunk_hist,
-                          chunk_keys);
+                          cs_h, cs_key, cs_sub, n_kv_heads, n_keys, lut, cnt_u8, cnt_u8_stride, cnt_i32, row_suf,
+                          chunk_suf, chunk_keys);
     PKV_LAUNCH_CHECK("pkv_scan_strided_kernel");
   }
   return PKV_OK;
@@ -182,9 +190,9 @@ static int launch_scan_impl(const uint8_t *codes, int64_t cs_b, int64_t cs_h, in
 
 int pkv_launch_scan(const uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t cs_key, int64_t cs_sub, int bs,
                     int n_kv_heads, int64_t n_keys, const uint8_t *lut, uint8_t *cnt_u8, int64_t cnt_u8_stride,
-                    int32_t *cnt_i32, uint16_t *chunk_hist, int chunk_keys, hipStream_t s) {
+                    int32_t *cnt_i32, uint32_t *row_suf, uint16_t *chunk_suf, int chunk_keys, hipStream_t s) {
   return launch_scan_impl(codes, cs_b, cs_h, cs_key, cs_sub, bs, n_kv_heads, n_keys, lut, cnt_u8, cnt_u8_stride, cnt_i32,
-                          chunk_hist, chunk_keys, s, nullptr, nullptr);
+                          row_suf, chunk_suf, chunk_keys, s, nullptr, nullptr);
 }
 
 int pkv_launch_scan_i32_codes(const int32_t *codebook, int rows, int64_t n_keys, const uint8_t *lut, int32_t *cnt,
@@ -197,19 +205,21 @@ int pkv_launch_scan_i32_codes(const int32_t *codebook, int rows, int64_t n_keys,
 
 extern "C" int pkv_collision_scan(const uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t cs_key, int64_t cs_sub,
                                   int bs, int n_kv_heads, int64_t n_keys, const uint8_t *lut, uint8_t *cnt_u8,
-                                  int32_t *cnt_i32, uint16_t *chunk_hist, int chunk_keys, void *stream) {
+                                  int32_t *cnt_i32, uint32_t *row_suf, uint16_t *chunk_suf, int chunk_keys,
+                                  void *stream) {
   PKV_REQUIRE(codes && lut && (cnt_u8 || cnt_i32), "pkv_collision_scan: null pointer");
   PKV_REQUIRE(bs > 0 && n_kv_heads > 0 && (int64_t)bs * n_kv_heads <= 65535 && n_keys > 0 &&
                   n_keys <= PKV_MAX_KEYS_PER_ROW,
               "bad shape bs=%d kv_heads=%d n_keys=%lld", bs, n_kv_heads, (long long)n_keys);
+  PKV_REQUIRE((row_suf == nullptr) == (chunk_suf == nullptr), "row_suf and chunk_suf go together");
   return pkv_launch_scan(codes, cs_b, cs_h, cs_key, cs_sub, bs, n_kv_heads, n_keys, lut, cnt_u8, n_keys, cnt_i32,
-                         chunk_hist, chunk_keys, (hipStream_t)stream);
+                         row_suf, chunk_suf, chunk_keys, (hipStream_t)stream);
 }
 
 extern "C" int pkv_collision_scan_timed(const uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t cs_key,
                                         int64_t cs_sub, int bs, int n_kv_heads, int64_t n_keys, const uint8_t *lut,
-                                        uint8_t *cnt_u8, int64_t cnt_u8_stride, uint16_t *chunk_hist, int chunk_keys,
-                                        float *kernel_us, void *stream) {
+                                        uint8_t *cnt_u8, int64_t cnt_u8_stride, uint32_t *row_suf, uint16_t *chunk_suf,
+                                        int chunk_keys, float *kernel_us, void *stream) {
   PKV_REQUIRE(codes && lut && cnt_u8 && kernel_us, "pkv_collision_scan_timed: null pointer");
   PKV_REQUIRE(bs > 0 && n_kv_heads > 0 && (int64_t)bs * n_kv_heads <= 65535 && n_keys > 0 &&
                   n_keys <= PKV_MAX_KEYS_PER_ROW && cnt_u8_stride >= n_keys,
@@ -218,7 +228,7 @@ extern "C" int pkv_collision_scan_timed(const uint8_t *codes, int64_t cs_b, int6
   PKV_HIP(hipEventCreate(&e0));
   PKV_HIP(hipEventCreate(&e1));
   int rc = launch_scan_impl(codes, cs_b, cs_h, cs_key, cs_sub, bs, n_kv_heads, n_keys, lut, cnt_u8, cnt_u8_stride,
-                            nullptr, chunk_hist, chunk_keys, (hipStream_t)stream, e0, e1);
+                            nullptr, row_suf, chunk_suf, chunk_keys, (hipStream_t)stream, e0, e1);
   if (rc == PKV_OK) {
     float ms = 0.f;
     hipError_t e = hipEventSynchronize(e1);

@@ -50,12 +50,12 @@ struct PkvTiers {
 };
 
 // Keys per workgroup-chunk of the collision scan / candidate select, chosen so
-// that rows * n_chunks is about a thousand workgroups (4 per CU) while the
+// that rows * n_chunks is about two thousand workgroups (8 per CU) while the
 // per-row chunk histograms (uint16 [n_chunks][128]) stay small.  Always a
 // multiple of 2048 and at most 32768 (a chunk's histogram bins are uint16).
 static inline int pkv_pick_chunk_keys(int rows, int64_t n_keys) {
   int64_t chunk = 2048;
-  while (chunk < 16384 && (int64_t)rows * ((n_keys + chunk - 1) / chunk) > 1024) chunk *= 2;
+  while (chunk < 16384 && (int64_t)rows * ((n_keys + chunk - 1) / chunk) > 2048) chunk *= 2;
   while (chunk < 32768 && (n_keys + chunk - 1) / chunk > 512) chunk *= 2;
   return (int)chunk;
 }
@@ -67,14 +67,19 @@ static inline int pkv_pick_chunk_keys(int rows, int64_t n_keys) {
 PKV_INTERNAL int pkv_launch_query_prep_lut(const void *q, int dtype, int bs, int n_kv_heads, int group,
                                            const float *signs, const int32_t *cc, int64_t cc_b, int64_t cc_h,
                                            const PkvTiers &tiers, float *qhat, float *qnorm, uint8_t *lut,
-                                           int64_t *sorted_ids, hipStream_t s);
+                                           int64_t *sorted_ids, uint32_t *row_suf_to_zero, hipStream_t s);
 PKV_INTERNAL int pkv_launch_scan(const uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t cs_key, int64_t cs_sub,
                                  int bs, int n_kv_heads, int64_t n_keys, const uint8_t *lut, uint8_t *cnt_u8,
-                                 int64_t cnt_u8_stride, int32_t *cnt_i32, uint16_t *chunk_hist, int chunk_keys,
-                                 hipStream_t s);
-PKV_INTERNAL int pkv_launch_select(const uint8_t *cnt_u8, int64_t cnt_stride, const uint16_t *chunk_hist,
-                                   int chunk_keys, int rows, int64_t n_keys, int64_t k, int64_t *out,
-                                   hipStream_t s);
+                                 int64_t cnt_u8_stride, int32_t *cnt_i32, uint32_t *row_suf, uint16_t *chunk_suf,
+                                 int chunk_keys, hipStream_t s);
+PKV_INTERNAL int pkv_launch_select(const uint8_t *cnt_u8, int64_t cnt_stride, const uint32_t *row_suf,
+                                   const uint16_t *chunk_suf, int chunk_keys, int rows, int64_t n_keys, int64_t k,
+                                   int64_t *out, hipStream_t s);
+PKV_INTERNAL int pkv_launch_select_rerank(const uint8_t *cnt_u8, int64_t cnt_stride, const uint32_t *row_suf,
+                                          const uint16_t *chunk_suf, int chunk_keys, int bs, int n_kv_heads, int64_t n_keys, int64_t k,
+                                          const uint8_t *nib, int64_t ns_b, int64_t ns_h, const uint16_t *weight,
+                                          int64_t ws_b, int64_t ws_h, const float *qhat, const float *qnorm,
+                                          const float *centers, int64_t *cand, float *scores, hipStream_t s);
 PKV_INTERNAL int pkv_launch_rerank(const int64_t *cand, int bs, int n_kv_heads, int64_t n_cand, int64_t n_keys,
                                    const uint8_t *nib, int64_t ns_b, int64_t ns_h, int64_t ns_key, int64_t ns_sub,
                                    const uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key,
@@ -137,6 +142,130 @@ __device__ __forceinline__ int pkv_wave_incl_scan(int v) {
     if (lane >= d) v += o;
   }
   return v;
+}
+
+// Normalise and SRHT-rotate one 128-vector spread over 16 lanes: lane s (= lane id & 15) holds
+// dims 8s..8s+7 in x[] (and the matching SRHT signs in sg[]).  On return y[] holds the rotated unit
+// vector's dims 8s..8s+7 and the norm is returned (both rounded to `dtype` where the reference's
+// tensors are).  Operation order: sum of squares sequential inside the 8 dims, then a pairwise tree
+// over the 16 lanes; natural-order Walsh-Hadamard butterflies h = 1..64 (three in-lane stages, four
+// lane-xor stages); then * 1/sqrt(128).  All 16 lanes of the group must be active.
+__device__ __forceinline__ float pkv_normalize_rotate_16(const float (&x)[8], const float (&sg)[8], int s, int dtype,
+                                                         float (&y)[8]) {
+  float acc = x[0] * x[0];
+#pragma unroll
+  for (int j = 1; j < 8; ++j) acc = acc + x[j] * x[j];
+#pragma unroll
+  for (int m = 1; m < 16; m <<= 1) acc = acc + __shfl_xor(acc, m, PKV_WAVE);
+  const float n = pkv_rdt(sqrtf(acc), dtype);
+  const float den = n < 1e-8f ? 1e-8f : n;
+  float t[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) t[j] = pkv_rdt(x[j] / den, dtype) * sg[j];
+#pragma unroll
+  for (int hh = 1; hh < 8; hh <<= 1) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if ((i & hh) == 0) {
+        const float a = t[i], c = t[i + hh];
+        t[i] = a + c;
+        t[i + hh] = a - c;
+      }
+    }
+  }
+#pragma unroll
+  for (int m = 1; m < 16; m <<= 1) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float o = __shfl_xor(t[j], m, PKV_WAVE);
+      t[j] = (s & m) ? (o - t[j]) : (t[j] + o);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) y[j] = pkv_rdt(t[j] * PKV_HADAMARD_SCALE, dtype);
+  return n;
+}
+
+// ---- 4-bit rerank core (shared by the stand-alone rerank and the fused select+rerank kernels) ----
+// s_prod[d][v] = qhat[d] * value(v) for the 16 possible 4-bit codes v (bit 3 = sign, set = positive;
+// bits 0-2 = magnitude centre): the product of the reference's expression is looked up instead of
+// recomputed (same single rounding), one conflict-free LDS read per dim.
+template <int NT>
+__device__ __forceinline__ void pkv_build_prod_table(float *s_prod, const float *__restrict__ qhat_row,
+                                                     const float *__restrict__ centers) {
+#pragma unroll
+  for (int u = 0; u < 128 * 16 / NT; ++u) {
+    const int e = threadIdx.x + u * NT;
+    const float a = centers[e & 7];
+    s_prod[e] = qhat_row[e >> 4] * ((e & 8) ? a : -a);
+  }
+}
+
+typedef const __attribute__((address_space(3))) float *pkv_lds_cfloat_ptr;
+
+__device__ __forceinline__ float pkv_block_dot(const float *__restrict__ s_prod, int blk, uint32_t word) {
+  // the table always lives in LDS: say so, or the 128 reads become flat loads with 64-bit addresses
+  const pkv_lds_cfloat_ptr lp = (pkv_lds_cfloat_ptr)s_prod;
+  float t = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float prod = lp[(8 * blk + j) * 16 + ((word >> (4 * j)) & 15u)];
+    t = (j == 0) ? prod : t + prod;
+  }
+  return t;
+}
+
+// Score of one key stored key-major: 64 B of nibbles at np, 16 bf16 weights at wp (both 16-byte aligned).
+// Order: dims 0..7 inside a block, blocks 0..15, then * ||q||; multiply and add rounded separately.
+// The four 16-byte groups are walked by a rolled loop that rotates the data registers, so that only one
+// group's 32 table reads are in flight at a time (fully unrolled, the scheduler hoists all 128 reads and
+// the kernel needs ~170 registers).
+__device__ __forceinline__ float pkv_rerank_keymajor(const float *__restrict__ s_prod, const pkv_u32x4 *__restrict__ np,
+                                                     const pkv_u32x4 *__restrict__ wp, float qnorm) {
+  pkv_u32x4 n0 = np[0], n1 = np[1], n2 = np[2], n3 = np[3];
+  pkv_u32x4 w0 = wp[0], w1 = wp[1];
+  const pkv_lds_cfloat_ptr lp = (pkv_lds_cfloat_ptr)s_prod;
+  float s = 0.f;
+#pragma unroll 1
+  for (int u = 0; u < 4; ++u) {
+    const uint32_t words[4] = {n0.x, n0.y, n0.z, n0.w};
+    const uint32_t wpair[2] = {w0.x, w0.y};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float t = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float prod = lp[(32 * u + 8 * i + j) * 16 + ((words[i] >> (4 * j)) & 15u)];
+        t = (j == 0) ? prod : t + prod;
+      }
+      const uint32_t wb = (i & 1) ? (wpair[i >> 1] >> 16) : (wpair[i >> 1] & 0xffffu);
+      const float tw = t * pkv_bf16_bits_to_f32(wb);
+      s = (u == 0 && i == 0) ? tw : s + tw;
+    }
+    n0 = n1, n1 = n2, n2 = n3;
+    w0 = pkv_u32x4{w0.z, w0.w, w1.x, w1.y};
+    w1 = pkv_u32x4{w1.z, w1.w, 0u, 0u};
+  }
+  return s * qnorm;
+}
+
+// Turn a 128-bin histogram in LDS (s_hist) into its suffix sums suf[t] = sum_{t' >= t} hist[t'],
+// store them as the chunk's uint16 suffix histogram and add them to the row's uint32 suffix totals.
+// Called by all threads of a workgroup with >= 128 threads; contains barriers.  s_w0: one LDS word.
+__device__ __forceinline__ void pkv_store_suffix_hist(const uint32_t *s_hist, uint32_t *s_w0,
+                                                      uint32_t *__restrict__ row_suf, uint16_t *__restrict__ chunk_suf) {
+  const int tid = threadIdx.x;
+  int incl = 0;
+  if (tid < 128) {  // thread t owns bin 127 - t: an inclusive scan over t is the suffix sum over bins
+    incl = pkv_wave_incl_scan((int)s_hist[127 - tid]);
+    if (tid == PKV_WAVE - 1) *s_w0 = (uint32_t)incl;
+  }
+  __syncthreads();
+  if (tid < 128) {
+    if (tid >= PKV_WAVE) incl += (int)*s_w0;
+    chunk_suf[127 - tid] = (uint16_t)incl;
+    if (incl) atomicAdd(&row_suf[127 - tid], (uint32_t)incl);
+  }
 }
 
 // Exclusive scan across a workgroup of NT threads (NT multiple of 64, <= 1024).

@@ -69,40 +69,8 @@ __global__ __launch_bounds__(kEncThreads) void pkv_encode_kernel(
       const float4 c = *(const float4 *)((const float *)keys + off + 4);
       x[0] = a.x, x[1] = a.y, x[2] = a.z, x[3] = a.w, x[4] = c.x, x[5] = c.y, x[6] = c.z, x[7] = c.w;
     }
-    // ||k||
-    float acc = x[0] * x[0];
-#pragma unroll
-    for (int j = 1; j < 8; ++j) acc = acc + x[j] * x[j];
-#pragma unroll
-    for (int m = 1; m < 16; m <<= 1) acc = acc + __shfl_xor(acc, m, PKV_WAVE);
-    const float n = pkv_rdt(sqrtf(acc), dtype);
-    const float den = n < 1e-8f ? 1e-8f : n;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) x[j] = pkv_rdt(x[j] / den, dtype) * sg[j];
-    // Walsh-Hadamard, natural order: in-lane h = 1, 2, 4
-#pragma unroll
-    for (int hh = 1; hh < 8; hh <<= 1) {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        if ((i & hh) == 0) {
-          const float a = x[i], c = x[i + hh];
-          x[i] = a + c;
-          x[i + hh] = a - c;
-        }
-      }
-    }
-    // cross-lane h = 8, 16, 32, 64  <->  lane xor 1, 2, 4, 8
-#pragma unroll
-    for (int m = 1; m < 16; m <<= 1) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float o = __shfl_xor(x[j], m, PKV_WAVE);
-        x[j] = (s & m) ? (o - x[j]) : (x[j] + o);
-      }
-    }
     float y[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) y[j] = pkv_rdt(x[j] * PKV_HADAMARD_SCALE, dtype);
+    const float n = pkv_normalize_rotate_16(x, sg, s, dtype, y);
 
     uint32_t code = 0;
 #pragma unroll

@@ -22,71 +22,69 @@ __device__ __forceinline__ int tier_weight_from_rank(int my_count, const PkvTier
   return w;
 }
 
-// grid (16 subspaces, R rows), 256 threads.
+// grid (16 subspaces, R rows), 256 threads.  The rotation runs in the first wave only (16 lanes per
+// vector, shuffles, no barriers); the 256 threads then score, rank and weigh the 256 centroids.
 __global__ __launch_bounds__(256) void pkv_query_prep_lut_kernel(
     const void *__restrict__ q, int dtype, int n_kv_heads, int group, const float *__restrict__ signs,
     const int32_t *__restrict__ cc, int64_t cc_b, int64_t cc_h, PkvTiers tiers, float *__restrict__ qhat,
-    float *__restrict__ qnorm, uint8_t *__restrict__ lut, int64_t *__restrict__ sorted_ids) {
+    float *__restrict__ qnorm, uint8_t *__restrict__ lut, int64_t *__restrict__ sorted_ids,
+    uint32_t *__restrict__ row_suf_to_zero) {
   const int sub = blockIdx.x;
   const int row = blockIdx.y;
   const int b = row / n_kv_heads, h = row % n_kv_heads;
   const int tid = threadIdx.x;
 
-  __shared__ float x[128];
-  __shared__ float blk[16];
-  __shared__ float s_norm;
-  __shared__ uint32_t s_key[256];
+  // the collision scan that follows accumulates the row's suffix histogram with atomics
+  if (row_suf_to_zero && sub == 1 && tid < 128) row_suf_to_zero[(int64_t)row * 128 + tid] = 0u;
+
+  __shared__ float s_y[128];
+  __shared__ __attribute__((aligned(16))) uint32_t s_key[256];
   __shared__ int s_id[256];
-  __shared__ int s_cnt[256];
+  __shared__ int s_cc[256];
+  __shared__ int s_part[128];
   __shared__ int s_wave_tot[4];
 
-  // group mean (polar_cache.py:1029-1030), sequential over the G heads
-  if (tid < 128) {
-    const int64_t base = ((int64_t)b * n_kv_heads * group + (int64_t)h * group) * 128 + tid;
-    float acc = 0.f;
-    for (int g = 0; g < group; ++g) {
-      float v = (dtype == PKV_DTYPE_BF16)
-                    ? pkv_bf16_bits_to_f32(((const uint16_t *)q)[base + (int64_t)g * 128])
-                    : ((const float *)q)[base + (int64_t)g * 128];
-      acc = (g == 0) ? v : acc + v;
-    }
-    x[tid] = pkv_rdt(acc / (float)group, dtype);
-  }
-  __syncthreads();
-  // ||q||: sequential inside each 8-block, pairwise tree over the 16 blocks
-  if (tid < 16) {
-    float acc = x[8 * tid] * x[8 * tid];
+  // cluster sizes by centroid id; issued first so that the latency overlaps the rotation
+  s_cc[tid] = cc[(int64_t)b * cc_b + (int64_t)h * cc_h + sub * 256 + tid];
+
+  if (tid < PKV_WAVE) {
+    const int s = tid & 15;
+    const int64_t base = ((int64_t)b * n_kv_heads * group + (int64_t)h * group) * 128 + 8 * s;
+    float acc[8], sg[8];
 #pragma unroll
-    for (int j = 1; j < 8; ++j) acc = acc + x[8 * tid + j] * x[8 * tid + j];
-    blk[tid] = acc;
-  }
-  __syncthreads();
-  if (tid == 0) {
-    for (int hh = 1; hh < 16; hh <<= 1)
-      for (int i = 0; i < 16; i += 2 * hh) blk[i] = blk[i] + blk[i + hh];
-    s_norm = pkv_rdt(sqrtf(blk[0]), dtype);
-  }
-  __syncthreads();
-  const float n = s_norm;
-  const float den = n < 1e-8f ? 1e-8f : n;
-  if (tid < 128) x[tid] = pkv_rdt(x[tid] / den, dtype) * signs[tid];
-  __syncthreads();
-  // natural-order Walsh-Hadamard butterflies, h = 1..64
-  for (int hh = 1; hh < 128; hh <<= 1) {
-    if (tid < 64) {
-      const int i = ((tid & ~(hh - 1)) << 1) | (tid & (hh - 1));
-      const float a = x[i], c = x[i + hh];
-      x[i] = a + c;
-      x[i + hh] = a - c;
+    for (int j = 0; j < 8; ++j) sg[j] = signs[8 * s + j];
+    // group mean (polar_cache.py:1029-1030), sequential over the G heads
+    for (int g = 0; g < group; ++g) {
+      float v[8];
+      if (dtype == PKV_DTYPE_BF16) {
+        const pkv_u32x4 w = *(const pkv_u32x4 *)((const uint16_t *)q + base + (int64_t)g * 128);
+        const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+          v[2 * p] = __uint_as_float(ww[p] << 16);
+          v[2 * p + 1] = __uint_as_float(ww[p] & 0xffff0000u);
+        }
+      } else {
+        const float4 a = *(const float4 *)((const float *)q + base + (int64_t)g * 128);
+        const float4 c = *(const float4 *)((const float *)q + base + (int64_t)g * 128 + 4);
+        v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = c.x, v[5] = c.y, v[6] = c.z, v[7] = c.w;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j] = (g == 0) ? v[j] : acc[j] + v[j];
     }
-    __syncthreads();
+    float x[8], y[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[j] = pkv_rdt(acc[j] / (float)group, dtype);
+    const float n = pkv_normalize_rotate_16(x, sg, s, dtype, y);
+    if (tid < 16) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        s_y[8 * s + j] = y[j];
+        if (sub == 0) qhat[(int64_t)row * 128 + 8 * s + j] = y[j];
+      }
+      if (sub == 0 && tid == 0) qnorm[row] = n;
+    }
   }
-  if (tid < 128) {
-    const float y = pkv_rdt(x[tid] * PKV_HADAMARD_SCALE, dtype);
-    x[tid] = y;
-    if (sub == 0) qhat[(int64_t)row * 128 + tid] = y;
-  }
-  if (sub == 0 && tid == 0) qnorm[row] = n;
   __syncthreads();
 
   // score of centroid c = tid: sum_j (+-) qhat_sub[j], sequential j
@@ -94,29 +92,53 @@ __global__ __launch_bounds__(256) void pkv_query_prep_lut_kernel(
     float acc = 0.f;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const float v = x[8 * sub + j];
+      const float v = s_y[8 * sub + j];
       const float t = ((tid >> j) & 1) ? v : -v;
       acc = (j == 0) ? t : acc + t;
     }
     acc = pkv_rdt(acc + 0.0f, dtype);
-    s_key[tid] = pkv_ordered_u32(acc);
+    uint32_t key = pkv_ordered_u32(acc);
+    // bf16 scores occupy the top 16 bits: fold the tie rule (smaller id first) into one 32-bit key
+    if (dtype == PKV_DTYPE_BF16) key = ((key >> 16) << 8) | (uint32_t)(255 - tid);
+    s_key[tid] = key;
   }
   __syncthreads();
-  // rank = number of centroids ahead of this one under (score desc, id asc)
+  // rank = number of centroids ahead of this one under (score desc, id asc).  The sign codebook is
+  // antipodal (score[255-c] == -score[c] exactly), hence rank[255-c] = 255 - rank[c]: thread t counts,
+  // for centroid c = t & 127, over half (t >> 7) of the keys; the two partial counts are added.
   {
-    const uint32_t mine = s_key[tid];
-    int rank = 0;
+    const int c = tid & 127, half = tid >> 7;
+    const uint32_t mine = s_key[c];
+    int part = 0;
+    const pkv_u32x4 *k4 = (const pkv_u32x4 *)s_key + half * 32;
+    if (dtype == PKV_DTYPE_BF16) {
 #pragma unroll 8
-    for (int c = 0; c < 256; ++c) {
-      const uint32_t k = s_key[c];
-      rank += (k > mine || (k == mine && c < tid)) ? 1 : 0;
+      for (int c4 = 0; c4 < 32; ++c4) {
+        const pkv_u32x4 k = k4[c4];
+        part += (k.x > mine) + (k.y > mine) + (k.z > mine) + (k.w > mine);
+      }
+    } else {
+#pragma unroll 8
+      for (int c4 = 0; c4 < 32; ++c4) {
+        const pkv_u32x4 k = k4[c4];
+        const int o = half * 128 + 4 * c4;
+        part += (k.x > mine || (k.x == mine && o + 0 < c)) ? 1 : 0;
+        part += (k.y > mine || (k.y == mine && o + 1 < c)) ? 1 : 0;
+        part += (k.z > mine || (k.z == mine && o + 2 < c)) ? 1 : 0;
+        part += (k.w > mine || (k.w == mine && o + 3 < c)) ? 1 : 0;
+      }
     }
-    s_id[rank] = tid;
-    s_cnt[rank] = cc[(int64_t)b * cc_b + (int64_t)h * cc_h + sub * 256 + tid];
+    if (half) s_part[c] = part;
+    __syncthreads();
+    if (!half) {
+      const int rank = part + s_part[c];
+      s_id[rank] = c;
+      s_id[255 - rank] = 255 - c;
+    }
   }
   __syncthreads();
-  const int w = tier_weight_from_rank(s_cnt[tid], tiers, s_wave_tot);
   const int id = s_id[tid];
+  const int w = tier_weight_from_rank(s_cc[id], tiers, s_wave_tot);
   lut[((int64_t)row * 16 + sub) * 256 + id] = (uint8_t)w;
   if (sorted_ids) sorted_ids[((int64_t)row * 16 + sub) * 256 + tid] = id;
 }
@@ -153,10 +175,11 @@ __global__ __launch_bounds__(256) void pkv_lut_from_sorted_kernel(
 
 int pkv_launch_query_prep_lut(const void *q, int dtype, int bs, int n_kv_heads, int group, const float *signs,
                               const int32_t *cc, int64_t cc_b, int64_t cc_h, const PkvTiers &tiers, float *qhat,
-                              float *qnorm, uint8_t *lut, int64_t *sorted_ids, hipStream_t s) {
+                              float *qnorm, uint8_t *lut, int64_t *sorted_ids, uint32_t *row_suf_to_zero,
+                              hipStream_t s) {
   dim3 grid(16, (unsigned)(bs * n_kv_heads));
   hipLaunchKernelGGL(pkv_query_prep_lut_kernel, grid, dim3(256), 0, s, q, dtype, n_kv_heads, group, signs, cc,
-                     cc_b, cc_h, tiers, qhat, qnorm, lut, sorted_ids);
+                     cc_b, cc_h, tiers, qhat, qnorm, lut, sorted_ids, row_suf_to_zero);
   PKV_LAUNCH_CHECK("pkv_query_prep_lut_kernel");
   return PKV_OK;
 }
@@ -175,6 +198,7 @@ extern "C" int pkv_query_prep_lut(const void *q, int dtype, int bs, int n_kv_hea
                                   const uint32_t *tier_counts, int n_tiers, float *qhat, float *qnorm,
                                   uint8_t *lut, int64_t *sorted_ids, void *stream) {
   PKV_REQUIRE(q && signs && cluster_counts && qhat && qnorm && lut, "pkv_query_prep_lut: null pointer");
+  PKV_REQUIRE(pkv_aligned(q, 16), "queries must be 16-byte aligned");
   PKV_REQUIRE(dtype == PKV_DTYPE_F32 || dtype == PKV_DTYPE_BF16, "unknown dtype %d", dtype);
   PKV_REQUIRE(bs > 0 && n_kv_heads > 0 && group > 0 && (int64_t)bs * n_kv_heads <= 65535,
               "bad shape bs=%d kv_heads=%d group=%d", bs, n_kv_heads, group);
@@ -182,7 +206,7 @@ extern "C" int pkv_query_prep_lut(const void *q, int dtype, int bs, int n_kv_hea
   int rc = make_tiers(tier_counts, n_tiers, t);
   if (rc) return rc;
   return pkv_launch_query_prep_lut(q, dtype, bs, n_kv_heads, group, signs, cluster_counts, cc_b, cc_h, t, qhat,
-                                   qnorm, lut, sorted_ids, (hipStream_t)stream);
+                                   qnorm, lut, sorted_ids, nullptr, (hipStream_t)stream);
 }
 
 extern "C" int pkv_update_cache_cnt(const int64_t *sorted_ids, int64_t si_b, int64_t si_h, int64_t si_sub,
@@ -204,7 +228,7 @@ extern "C" int pkv_update_cache_cnt(const int64_t *sorted_ids, int64_t si_b, int
                      cluster_counts, cc_b, cc_h, cc_sub, (const int32_t *)nullptr, n_kv_heads, t, lut_ws);
   PKV_LAUNCH_CHECK("pkv_lut_from_sorted_kernel");
   return pkv_launch_scan(codes, cs_b, cs_h, cs_key, cs_sub, bs, n_kv_heads, n_keys, lut_ws, nullptr, 0, cnt,
-                         nullptr, pkv_pick_chunk_keys(bs * n_kv_heads, n_keys), s);
+                         nullptr, nullptr, pkv_pick_chunk_keys(bs * n_kv_heads, n_keys), s);
 }
 
 PKV_INTERNAL int pkv_launch_scan_i32_codes(const int32_t *codebook, int rows, int64_t n_keys, const uint8_t *lut,

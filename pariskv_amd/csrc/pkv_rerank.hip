@@ -15,20 +15,8 @@ namespace {
 
 constexpr int kRerankThreads = 256;
 
-__device__ __forceinline__ float block_dot(const float *__restrict__ s_q, const float *__restrict__ s_val, int blk,
-                                           uint32_t word) {
-  float t = 0.f;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const float prod = s_q[8 * blk + j] * s_val[(word >> (4 * j)) & 15u];
-    t = (j == 0) ? prod : t + prod;
-  }
-  return t;
-}
-
 __device__ __forceinline__ void store_v4b(uint16_t *__restrict__ v4b, int64_t row, int64_t n_cand, int64_t i, int blk,
                                           const float *__restrict__ s_val, uint32_t word) {
-  if (!v4b) return;
   pkv_u32x4 o;
   uint32_t h[8];
 #pragma unroll
@@ -52,13 +40,13 @@ __global__ __launch_bounds__(kRerankThreads) void pkv_rerank_kernel(
   const int row = blockIdx.y;
   const int b = row / n_kv_heads, h = row % n_kv_heads;
   const int tid = threadIdx.x;
-  __shared__ float s_q[128];
+  __shared__ float s_prod[128 * 16];
   __shared__ float s_val[16];
-  if (tid < 128) s_q[tid] = qhat[(int64_t)row * 128 + tid];
   if (tid < 16) {
     const float a = centers[tid & 7];
     s_val[tid] = (tid & 8) ? a : -a;  // sign bit set = positive (rerank.cu:107-119)
   }
+  pkv_build_prod_table<kRerankThreads>(s_prod, qhat + (int64_t)row * 128, centers);
   __syncthreads();
   const int64_t i = (int64_t)blockIdx.x * kRerankThreads + tid;
   if (i >= n_cand) return;
@@ -84,7 +72,7 @@ __global__ __launch_bounds__(kRerankThreads) void pkv_rerank_kernel(
     const uint32_t wpair[8] = {wv[0].x, wv[0].y, wv[0].z, wv[0].w, wv[1].x, wv[1].y, wv[1].z, wv[1].w};
 #pragma unroll
     for (int blk = 0; blk < 16; ++blk) {
-      const float t = block_dot(s_q, s_val, blk, words[blk]);
+      const float t = pkv_block_dot(s_prod, blk, words[blk]);
       const uint32_t wb = (blk & 1) ? (wpair[blk >> 1] >> 16) : (wpair[blk >> 1] & 0xffffu);
       const float tw = t * pkv_bf16_bits_to_f32(wb);
       s = (blk == 0) ? tw : s + tw;
@@ -94,7 +82,7 @@ __global__ __launch_bounds__(kRerankThreads) void pkv_rerank_kernel(
 #pragma unroll 4
     for (int blk = 0; blk < 16; ++blk) {
       const uint32_t word = *(const uint32_t *)(nrow + key * ns_key + (int64_t)blk * ns_sub);
-      const float t = block_dot(s_q, s_val, blk, word);
+      const float t = pkv_block_dot(s_prod, blk, word);
       const float tw = t * pkv_bf16_bits_to_f32(wrow[key * ws_key + (int64_t)blk * ws_sub]);
       s = (blk == 0) ? tw : s + tw;
       if (V4B) store_v4b(v4b, row, n_cand, i, blk, s_val, word);

@@ -1,7 +1,7 @@
 // One layer's retrieval for one decode step as a fixed sequence of launches on
 // the caller's stream: query prep + vote table -> collision scan (+ chunk
-// histograms) -> candidate select -> 4-bit rerank -> exact top-k -> optional
-// gather of the selected K/V rows.
+// histograms) -> candidate select fused with the 4-bit rerank -> exact top-k ->
+// optional gather of the selected K/V rows (5 launches).
 //
 // Reference: cache_hub/polar_cache.py:1126-1162 (collision_based_topk_batch),
 // :1207-1231, :1244-1304 and the gather at :1075-1095.
@@ -12,7 +12,7 @@ PKV_INTERNAL int pkv_launch_identity_fill(int64_t *out, int64_t len, int64_t k, 
 namespace {
 
 struct WsLayout {
-  size_t qhat, qnorm, lut, cnt, hist, cand, scores, total;
+  size_t qhat, qnorm, lut, cnt, hist, rowsuf, cand, scores, total;
   int64_t cnt_stride;
   int chunk_keys;
   int64_t n_chunks;
@@ -34,6 +34,7 @@ WsLayout layout(int rows, int64_t n_keys, int64_t n_cand, int64_t /*k*/) {
   w.lut = take((size_t)rows * 4096);
   w.cnt = take((size_t)rows * (size_t)w.cnt_stride);
   w.hist = take((size_t)rows * (size_t)w.n_chunks * 128 * sizeof(uint16_t));
+  w.rowsuf = take((size_t)rows * 128 * sizeof(uint32_t));
   w.cand = take((size_t)rows * (size_t)n_cand * sizeof(int64_t));
   w.scores = take((size_t)rows * (size_t)n_cand * sizeof(float));
   w.total = off;
@@ -65,8 +66,10 @@ extern "C" int pkv_retrieve_ws_view(void *ws, int rows, int64_t n_keys, int64_t 
     *ptr = base + w.lut, *bytes = (size_t)rows * 4096;
   } else if (!strcmp(name, "cnt_u8")) {
     *ptr = base + w.cnt, *bytes = (size_t)rows * (size_t)w.cnt_stride;
-  } else if (!strcmp(name, "chunk_hist")) {
+  } else if (!strcmp(name, "chunk_suffix_hist")) {
     *ptr = base + w.hist, *bytes = (size_t)rows * (size_t)w.n_chunks * 256;
+  } else if (!strcmp(name, "row_suffix_hist")) {
+    *ptr = base + w.rowsuf, *bytes = (size_t)rows * 512;
   } else if (!strcmp(name, "cand")) {
     *ptr = base + w.cand, *bytes = (size_t)rows * (size_t)n_cand * 8;
   } else if (!strcmp(name, "scores")) {
@@ -92,8 +95,9 @@ extern "C" int pkv_retrieve(const pkv_retrieve_args *a, void *ws, size_t ws_byte
   PKV_REQUIRE(a->key0 >= 0 && a->key0 + a->n_keys <= a->cap, "retrieval zone [%lld,+%lld) exceeds capacity %lld",
               (long long)a->key0, (long long)a->n_keys, (long long)a->cap);
   PKV_REQUIRE(a->n_tiers >= 1 && a->n_tiers <= PKV_MAX_TIERS, "n_tiers must be in [1,%d]", PKV_MAX_TIERS);
-  PKV_REQUIRE(pkv_aligned(a->codes, 16) && pkv_aligned(a->nib, 16) && pkv_aligned(a->weight, 16),
-              "codes / nib / weight must be 16-byte aligned");
+  PKV_REQUIRE(pkv_aligned(a->codes, 16) && pkv_aligned(a->nib, 16) && pkv_aligned(a->weight, 16) &&
+                  pkv_aligned(a->q, 16),
+              "queries / codes / nib / weight must be 16-byte aligned");
   const WsLayout w = layout(rows, a->n_keys, a->n_cand, a->k);
   if (!ws || ws_bytes < w.total || !pkv_aligned(ws, 256)) {
     pkv_set_error("pkv_retrieve: workspace of %zu bytes (256-aligned) required, got %zu", w.total, ws_bytes);
@@ -106,6 +110,7 @@ extern "C" int pkv_retrieve(const pkv_retrieve_args *a, void *ws, size_t ws_byte
   uint8_t *lut = (uint8_t *)(base + w.lut);
   uint8_t *cnt = (uint8_t *)(base + w.cnt);
   uint16_t *hist = (uint16_t *)(base + w.hist);
+  uint32_t *rowsuf = (uint32_t *)(base + w.rowsuf);
   int64_t *cand = (int64_t *)(base + w.cand);
   float *scores = (float *)(base + w.scores);
 
@@ -116,23 +121,25 @@ extern "C" int pkv_retrieve(const pkv_retrieve_args *a, void *ws, size_t ws_byte
 
   const int H = a->n_kv_heads;
   int rc = pkv_launch_query_prep_lut(a->q, a->dtype, a->bs, H, a->group, a->signs, a->cluster_counts,
-                                     (int64_t)H * 4096, 4096, t, qhat, qnorm, lut, nullptr, s);
+                                     (int64_t)H * 4096, 4096, t, qhat, qnorm, lut, nullptr, rowsuf, s);
   if (rc) return rc;
   const uint8_t *codes = a->codes + a->key0 * 16;
   const uint8_t *nib = a->nib + a->key0 * 64;
   const uint16_t *weight = a->weight + a->key0 * 16;
   if (a->n_cand == a->n_keys) {
     rc = pkv_launch_identity_fill(cand, a->n_keys, a->n_cand, rows, s);
+    if (rc) return rc;
+    rc = pkv_launch_rerank(cand, a->bs, H, a->n_cand, a->n_keys, nib, (int64_t)H * a->cap * 64, a->cap * 64, 64, 4,
+                           weight, (int64_t)H * a->cap * 16, a->cap * 16, 16, 1, qhat, qnorm, a->centers, scores,
+                           nullptr, s);
   } else {
     rc = pkv_launch_scan(codes, (int64_t)H * a->cap * 16, a->cap * 16, 16, 1, a->bs, H, a->n_keys, lut, cnt,
-                         w.cnt_stride, nullptr, hist, w.chunk_keys, s);
+                         w.cnt_stride, nullptr, rowsuf, hist, w.chunk_keys, s);
     if (rc) return rc;
-    rc = pkv_launch_select(cnt, w.cnt_stride, hist, w.chunk_keys, rows, a->n_keys, a->n_cand, cand, s);
+    rc = pkv_launch_select_rerank(cnt, w.cnt_stride, rowsuf, hist, w.chunk_keys, a->bs, H, a->n_keys, a->n_cand, nib,
+                                  (int64_t)H * a->cap * 64, a->cap * 64, weight, (int64_t)H * a->cap * 16, a->cap * 16,
+                                  qhat, qnorm, a->centers, cand, scores, s);
   }
-  if (rc) return rc;
-  rc = pkv_launch_rerank(cand, a->bs, H, a->n_cand, a->n_keys, nib, (int64_t)H * a->cap * 64, a->cap * 64, 64, 4,
-                         weight, (int64_t)H * a->cap * 16, a->cap * 16, 16, 1, qhat, qnorm, a->centers, scores,
-                         nullptr, s);
   if (rc) return rc;
   rc = pkv_launch_topk_f32(scores, a->n_cand, cand, a->n_cand, rows, a->n_cand, a->k, a->out_ids, a->out_scores,
                            nullptr, 0, s);

@@ -20,64 +20,75 @@ constexpr int kSelThreads = 256;
 constexpr int kSelKeysPerThread = 8;
 constexpr int kSelKeysPerIter = kSelThreads * kSelKeysPerThread;  // 2048
 
+// Threshold and output offsets of one workgroup from the suffix histograms the collision scan leaves
+// behind: row_suf[row][t] = keys of the row with count >= t (summed over chunks with atomics),
+// chunk_suf[row][c][t] = the same for chunk c alone.  theta = largest t with row_suf[t] >= k;
+// base_gt = keys above theta in earlier chunks; base_eq = (keys above theta in the row) + keys at
+// theta in earlier chunks.  Two dependent loads, no loops over bins.
+__device__ __forceinline__ void select_prologue(const uint32_t *__restrict__ row_suf,
+                                                const uint16_t *__restrict__ chunk_suf, int row, int chunk,
+                                                int n_chunks, int64_t k, uint32_t &theta, int64_t &base_gt,
+                                                int64_t &base_eq) {
+  __shared__ uint32_t s_rs[129];
+  __shared__ uint32_t s_theta, s_ngt;
+  __shared__ uint32_t s_red[2][kSelThreads / PKV_WAVE];
+  const int tid = threadIdx.x;
+  if (tid < 128) s_rs[tid] = row_suf[(int64_t)row * 128 + tid];
+  if (tid == 128) {
+    s_rs[128] = 0;
+    s_theta = 0;
+    s_ngt = 0;
+  }
+  __syncthreads();
+  if (tid < 128 && (int64_t)s_rs[tid] >= k && (int64_t)s_rs[tid + 1] < k) {
+    s_theta = (uint32_t)tid;
+    s_ngt = s_rs[tid + 1];
+  }
+  __syncthreads();
+  theta = s_theta;
+  uint32_t gt = 0, eq = 0;
+  const uint16_t *cs = chunk_suf + (int64_t)row * n_chunks * 128;
+  for (int c = tid; c < chunk; c += kSelThreads) {
+    const uint32_t ge = cs[(int64_t)c * 128 + theta];
+    const uint32_t g = theta < 127 ? cs[(int64_t)c * 128 + theta + 1] : 0u;
+    gt += g;
+    eq += ge - g;
+  }
+#pragma unroll
+  for (int m = 1; m < PKV_WAVE; m <<= 1) {
+    gt += __shfl_xor(gt, m, PKV_WAVE);
+    eq += __shfl_xor(eq, m, PKV_WAVE);
+  }
+  if (pkv_lane() == 0) {
+    s_red[0][tid / PKV_WAVE] = gt;
+    s_red[1][tid / PKV_WAVE] = eq;
+  }
+  __syncthreads();
+  gt = eq = 0;
+#pragma unroll
+  for (int w = 0; w < kSelThreads / PKV_WAVE; ++w) {
+    gt += s_red[0][w];
+    eq += s_red[1][w];
+  }
+  base_gt = gt;
+  base_eq = (int64_t)s_ngt + eq;
+}
+
 // grid (n_chunks, rows).  cnt rows are padded to a multiple of 16 bytes and
 // 16-byte aligned, so every thread's 8 counts are one aligned 64-bit load.
 __global__ __launch_bounds__(kSelThreads) void pkv_select_kernel(const uint8_t *__restrict__ cnt,
                                                                  int64_t cnt_stride,
-                                                                 const uint16_t *__restrict__ chunk_hist,
+                                                                 const uint32_t *__restrict__ row_suf,
+                                                                 const uint16_t *__restrict__ chunk_suf,
                                                                  int chunk_keys, int64_t n_keys, int64_t k,
                                                                  int64_t *__restrict__ out) {
   const int row = blockIdx.y;
   const int chunk = blockIdx.x;
-  const int n_chunks = gridDim.x;
   const int tid = threadIdx.x;
-
-  __shared__ uint32_t s_tot[129], s_bef[129], s_stot[129], s_sbef[129];
-  __shared__ int s_theta;
-  __shared__ uint32_t s_ngt, s_gtb, s_eqb;
   __shared__ int s_scan[2][kSelThreads / PKV_WAVE];
-
-  if (tid < 128) {
-    const uint16_t *hp = chunk_hist + (int64_t)row * n_chunks * 128 + tid;
-    uint32_t tot = 0, bef = 0;
-    for (int c = 0; c < n_chunks; ++c) {
-      const uint32_t v = hp[(int64_t)c * 128];
-      tot += v;
-      if (c < chunk) bef += v;
-    }
-    s_tot[tid] = tot;
-    s_bef[tid] = bef;
-  } else if (tid == 128) {
-    s_tot[128] = 0;
-    s_bef[128] = 0;
-    s_stot[128] = 0;
-    s_sbef[128] = 0;
-    s_theta = 0;
-    s_ngt = 0;
-    s_gtb = 0;
-    s_eqb = 0;
-  }
-  __syncthreads();
-  if (tid < 128) {  // suffix sums over bins >= tid
-    uint32_t st = 0, sb = 0;
-    for (int t = tid; t < 128; ++t) {
-      st += s_tot[t];
-      sb += s_bef[t];
-    }
-    s_stot[tid] = st;
-    s_sbef[tid] = sb;
-  }
-  __syncthreads();
-  if (tid < 128 && (int64_t)s_stot[tid] >= k && (int64_t)s_stot[tid + 1] < k) {
-    s_theta = tid;             // k-th largest count
-    s_ngt = s_stot[tid + 1];   // keys strictly above it, whole row
-    s_gtb = s_sbef[tid + 1];   // ... of those, in earlier chunks
-    s_eqb = s_bef[tid];        // keys equal to it in earlier chunks
-  }
-  __syncthreads();
-  const uint32_t theta = (uint32_t)s_theta;
-  int64_t base_gt = s_gtb;
-  int64_t base_eq = (int64_t)s_ngt + s_eqb;
+  uint32_t theta;
+  int64_t base_gt, base_eq;
+  select_prologue(row_suf, chunk_suf, row, chunk, gridDim.x, k, theta, base_gt, base_eq);
   int64_t *orow = out + (int64_t)row * k;
   const uint8_t *crow = cnt + (int64_t)row * cnt_stride;
 
@@ -118,6 +129,90 @@ __global__ __launch_bounds__(kSelThreads) void pkv_select_kernel(const uint8_t *
   }
 }
 
+// Candidate select fused with the 4-bit rerank (key-major storage): every workgroup finds the
+// candidates of its chunk as above, parks them in LDS and scores them right away, so the candidate
+// list is never re-read and one launch disappears from the decode step.
+// out/scores: [rows][k]; position p of a row holds the candidate's key index and its score.
+__global__ __launch_bounds__(kSelThreads) void pkv_select_rerank_kernel(
+    const uint8_t *__restrict__ cnt, int64_t cnt_stride, const uint32_t *__restrict__ row_suf,
+    const uint16_t *__restrict__ chunk_suf, int chunk_keys, int n_kv_heads, int64_t n_keys, int64_t k,
+    const uint8_t *__restrict__ nib, int64_t ns_b, int64_t ns_h, const uint16_t *__restrict__ weight, int64_t ws_b,
+    int64_t ws_h, const float *__restrict__ qhat, const float *__restrict__ qnorm, const float *__restrict__ centers,
+    int64_t *__restrict__ out, float *__restrict__ scores) {
+  const int row = blockIdx.y;
+  const int chunk = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int b = row / n_kv_heads, h = row % n_kv_heads;
+
+  __shared__ int s_scan[2][kSelThreads / PKV_WAVE];
+  __shared__ float s_prod[128 * 16];
+  __shared__ uint16_t s_list_key[kSelKeysPerIter];  // offset of the key inside the iteration's 2048-key block
+  __shared__ int32_t s_list_pos[kSelKeysPerIter];   // output position, -1 = dropped tie
+
+  pkv_build_prod_table<kSelThreads>(s_prod, qhat + (int64_t)row * 128, centers);
+  const float qn = qnorm[row];
+  uint32_t theta;
+  int64_t base_gt, base_eq;
+  select_prologue(row_suf, chunk_suf, row, chunk, gridDim.x, k, theta, base_gt, base_eq);
+  int64_t *orow = out + (int64_t)row * k;
+  float *srow = scores + (int64_t)row * k;
+  const uint8_t *crow = cnt + (int64_t)row * cnt_stride;
+  const uint8_t *nrow = nib + (int64_t)b * ns_b + (int64_t)h * ns_h;
+  const uint16_t *wrow = weight + (int64_t)b * ws_b + (int64_t)h * ws_h;
+
+  const int64_t chunk_begin = (int64_t)chunk * chunk_keys;
+  const int64_t chunk_end = (chunk_begin + chunk_keys < n_keys) ? chunk_begin + chunk_keys : n_keys;
+  int it = 0;
+  for (int64_t blk0 = chunk_begin; blk0 < chunk_end; blk0 += kSelKeysPerIter, ++it) {
+    const int64_t i0 = blk0 + (int64_t)tid * kSelKeysPerThread;
+    uint32_t gt_mask = 0, eq_mask = 0;
+    if (i0 < chunk_end) {
+      const pkv_u32x2 w = *(const pkv_u32x2 *)(crow + i0);
+      const uint32_t ww[2] = {w.x, w.y};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const uint32_t v = (ww[j >> 2] >> (8 * (j & 3))) & 0xffu;
+        const bool valid = i0 + j < chunk_end;
+        gt_mask |= (valid && v > theta) ? (1u << j) : 0u;
+        eq_mask |= (valid && v == theta) ? (1u << j) : 0u;
+      }
+    }
+    const int packed = __popc(gt_mask) | (__popc(eq_mask) << 16);
+    int total;
+    const int excl = pkv_block_excl_scan<kSelThreads>(packed, s_scan[it & 1], total);
+    const int n_gt_it = total & 0xffff, n_sel_it = n_gt_it + (total >> 16);
+    int64_t pg = base_gt + (excl & 0xffff);
+    int64_t pe = base_eq + (excl >> 16);
+    int lg = excl & 0xffff;            // slot in this iteration's LDS list: strictly-above keys first,
+    int le = n_gt_it + (excl >> 16);   // then the keys at the threshold
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (gt_mask & (1u << j)) {
+        s_list_key[lg] = (uint16_t)(tid * kSelKeysPerThread + j);
+        s_list_pos[lg] = pg < k ? (int32_t)pg : -1;
+        ++lg, ++pg;
+      } else if (eq_mask & (1u << j)) {
+        s_list_key[le] = (uint16_t)(tid * kSelKeysPerThread + j);
+        s_list_pos[le] = pe < k ? (int32_t)pe : -1;
+        ++le, ++pe;
+      }
+    }
+    base_gt += n_gt_it;
+    base_eq += total >> 16;
+    __syncthreads();
+#pragma unroll 1
+    for (int j = tid; j < n_sel_it; j += kSelThreads) {
+      const int32_t pos = s_list_pos[j];
+      if (pos >= 0) {
+        const int64_t key = blk0 + s_list_key[j];
+        orow[pos] = key;
+        srow[pos] = pkv_rerank_keymajor(s_prod, (const pkv_u32x4 *)(nrow + key * 64), (const pkv_u32x4 *)(wrow + key * 16), qn);
+      }
+    }
+    __syncthreads();  // the list is rewritten by the next iteration
+  }
+}
+
 // out[row][i] = i (i < len) else 0: the reference's `length <= k` branch
 // (radix_topk.cu:154-159).
 __global__ void pkv_identity_fill_kernel(int64_t *__restrict__ out, int64_t len, int64_t k, int rows) {
@@ -127,13 +222,14 @@ __global__ void pkv_identity_fill_kernel(int64_t *__restrict__ out, int64_t len,
   out[g] = i < len ? i : 0;
 }
 
-// int32 counts -> clamped u8 counts (padded rows) + per-chunk histograms.
+// int32 counts -> clamped u8 counts (padded rows) + per-chunk suffix histograms + row suffix totals.
 __global__ __launch_bounds__(256) void pkv_counts_to_u8_kernel(const int32_t *__restrict__ x, int64_t x_stride,
                                                                int64_t len, uint8_t *__restrict__ cnt,
-                                                               int64_t cnt_stride, uint16_t *__restrict__ chunk_hist,
-                                                               int chunk_keys) {
+                                                               int64_t cnt_stride, uint32_t *__restrict__ row_suf,
+                                                               uint16_t *__restrict__ chunk_suf, int chunk_keys) {
   const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
   __shared__ uint32_t s_hist[128];
+  __shared__ uint32_t s_w0;
   if (tid < 128) s_hist[tid] = 0;
   __syncthreads();
   const int64_t k0 = (int64_t)chunk * chunk_keys;
@@ -145,7 +241,13 @@ __global__ __launch_bounds__(256) void pkv_counts_to_u8_kernel(const int32_t *__
     atomicAdd(&s_hist[v], 1u);
   }
   __syncthreads();
-  if (tid < 128) chunk_hist[((int64_t)row * gridDim.x + chunk) * 128 + tid] = (uint16_t)s_hist[tid];
+  pkv_store_suffix_hist(s_hist, &s_w0, row_suf + (int64_t)row * 128,
+                        chunk_suf + ((int64_t)row * gridDim.x + chunk) * 128);
+}
+
+__global__ void pkv_zero_u32_kernel(uint32_t *__restrict__ p, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0u;
 }
 
 // ------------------------------------------------------------ exact fp32 top-k
@@ -159,35 +261,95 @@ __device__ __forceinline__ uint64_t make_key(const float *__restrict__ x, const 
   return ((uint64_t)pkv_ordered_u32(x[i]) << 32) | (uint64_t)(~id);
 }
 
-// Descending bitonic sort of P (power of two) 64-bit keys in LDS.
-__device__ __forceinline__ void bitonic_sort_desc(uint64_t *s, int P) {
+__device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int mask) {
+  const uint32_t lo = __shfl_xor((uint32_t)v, mask, PKV_WAVE);
+  const uint32_t hi = __shfl_xor((uint32_t)(v >> 32), mask, PKV_WAVE);
+  return ((uint64_t)hi << 32) | lo;
+}
+
+// Descending bitonic sort of 1024*E 64-bit keys held E per thread (thread t owns sorted positions
+// t*E .. t*E+E-1).  Strides below E are exchanged inside the thread, strides below 64*E between the
+// lanes of a wave (no barrier), only the remaining strides go through LDS (`s_buf`, 1024*E keys,
+// laid out [e][thread] so that a wave touches consecutive addresses).  For 4096 keys that is 10
+// barrier-separated exchanges instead of 78.
+template <int E>
+__device__ __forceinline__ void bitonic_sort_desc_regs(uint64_t (&v)[E], uint64_t *s_buf) {
+  constexpr int P = kTopkThreads * E;
+  const int tid = threadIdx.x;
+#pragma unroll
   for (int size = 2; size <= P; size <<= 1) {
+#pragma unroll
     for (int stride = size >> 1; stride > 0; stride >>= 1) {
-      for (int t = threadIdx.x; t < P / 2; t += kTopkThreads) {
-        const int lo = ((t & ~(stride - 1)) << 1) | (t & (stride - 1));
-        const int hi = lo + stride;
-        const bool desc = (lo & size) == 0;
-        const uint64_t a = s[lo], b = s[hi];
-        if (desc ? (a < b) : (a > b)) {
-          s[lo] = b;
-          s[hi] = a;
+      if (stride < E) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          if ((e & stride) == 0) {
+            const bool desc = ((tid * E + e) & size) == 0;
+            const uint64_t a = v[e], b = v[e | stride];
+            const bool sw = desc ? (a < b) : (a > b);
+            v[e] = sw ? b : a;
+            v[e | stride] = sw ? a : b;
+          }
+        }
+      } else if (stride < PKV_WAVE * E) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          const int i = tid * E + e;
+          const uint64_t o = shfl_xor_u64(v[e], stride / E);
+          const bool want_max = ((i & stride) == 0) == ((i & size) == 0);
+          v[e] = want_max ? (v[e] > o ? v[e] : o) : (v[e] < o ? v[e] : o);
+        }
+      } else {
+        __syncthreads();  // earlier readers of s_buf are done
+#pragma unroll
+        for (int e = 0; e < E; ++e) s_buf[e * kTopkThreads + tid] = v[e];
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          const int i = tid * E + e;
+          const uint64_t o = s_buf[e * kTopkThreads + (tid ^ (stride / E))];
+          const bool want_max = ((i & stride) == 0) == ((i & size) == 0);
+          v[e] = want_max ? (v[e] > o ? v[e] : o) : (v[e] < o ? v[e] : o);
         }
       }
-      __syncthreads();
     }
   }
 }
 
-__device__ __forceinline__ void emit_topk(const uint64_t *s, int64_t k, int64_t *__restrict__ out_ids,
-                                          float *__restrict__ out_vals) {
-  for (int64_t i = threadIdx.x; i < k; i += kTopkThreads) {
-    const uint64_t key = s[i];
-    out_ids[i] = (int64_t)(uint32_t)(~(uint32_t)key);
-    if (out_vals) out_vals[i] = pkv_from_ordered_u32((uint32_t)(key >> 32));
+// Sort the n_valid (<= 1024*E) keys in s_keys[0 .. 1024*E) (zero padded) and emit the first k.
+template <int E>
+__device__ __forceinline__ void sort_lds_keys_and_emit(uint64_t *s_keys, int64_t k, int64_t *__restrict__ out_ids,
+                                                       float *__restrict__ out_vals, uint64_t *sorted_copy) {
+  uint64_t v[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) v[e] = s_keys[threadIdx.x * E + e];
+  __syncthreads();
+  bitonic_sort_desc_regs<E>(v, s_keys);
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const int64_t i = (int64_t)threadIdx.x * E + e;
+    if (i < k) {
+      out_ids[i] = (int64_t)(uint32_t)(~(uint32_t)v[e]);
+      if (out_vals) out_vals[i] = pkv_from_ordered_u32((uint32_t)(v[e] >> 32));
+    }
+  }
+  if (sorted_copy) {  // the caller wants the sorted keys back in LDS
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < E; ++e) sorted_copy[threadIdx.x * E + e] = v[e];
+    __syncthreads();
   }
 }
 
-// len <= 8192: sort everything.  One workgroup per row, dynamic LDS P*8 bytes.
+#define PKV_DISPATCH_E(P, CALL)            \
+  do {                                     \
+    if ((P) <= 1024) { CALL(1); }          \
+    else if ((P) == 2048) { CALL(2); }     \
+    else if ((P) == 4096) { CALL(4); }     \
+    else { CALL(8); }                      \
+  } while (0)
+
+// len <= 8192: sort everything.  One workgroup per row, dynamic LDS max(P,1024)*8 bytes.
 __global__ __launch_bounds__(kTopkThreads) void pkv_topk_sort_kernel(const float *__restrict__ x, int64_t x_stride,
                                                                      const int64_t *__restrict__ ids,
                                                                      int64_t ids_stride, int len, int P, int64_t k,
@@ -197,10 +359,120 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_sort_kernel(const float
   const int row = blockIdx.x;
   const float *xr = x + (int64_t)row * x_stride;
   const int64_t *ir = ids ? ids + (int64_t)row * ids_stride : nullptr;
-  for (int i = threadIdx.x; i < P; i += kTopkThreads) s_keys[i] = i < len ? make_key(xr, ir, i) : 0ull;
+  int64_t *oi = out_ids + (int64_t)row * k;
+  float *ov = out_vals ? out_vals + (int64_t)row * k : nullptr;
+#define PKV_SORT_ALL(E)                                                            \
+  {                                                                                \
+    uint64_t v[E];                                                                 \
+    _Pragma("unroll") for (int e = 0; e < E; ++e) {                                \
+      const int i = threadIdx.x * E + e;                                           \
+      v[e] = i < len ? make_key(xr, ir, i) : 0ull;                                 \
+    }                                                                              \
+    bitonic_sort_desc_regs<E>(v, s_keys);                                          \
+    _Pragma("unroll") for (int e = 0; e < E; ++e) {                                \
+      const int64_t i = (int64_t)threadIdx.x * E + e;                              \
+      if (i < k) {                                                                 \
+        oi[i] = (int64_t)(uint32_t)(~(uint32_t)v[e]);                              \
+        if (ov) ov[i] = pkv_from_ordered_u32((uint32_t)(v[e] >> 32));              \
+      }                                                                            \
+    }                                                                              \
+  }
+  PKV_DISPATCH_E(P, PKV_SORT_ALL);
+#undef PKV_SORT_ALL
+}
+
+// Inclusive scan of one value per thread over the first 256 threads of a 1024-thread workgroup
+// (all 1024 threads must call it: it contains a barrier).  s_tot: 4 ints.
+__device__ __forceinline__ int scan256_in_1024(int v, int *s_tot) {
+  const int tid = threadIdx.x;
+  int incl = 0;
+  if (tid < 256) {
+    incl = pkv_wave_incl_scan(v);
+    if (pkv_lane() == PKV_WAVE - 1) s_tot[tid / PKV_WAVE] = incl;
+  }
   __syncthreads();
-  bitonic_sort_desc(s_keys, P);
-  emit_topk(s_keys, k, out_ids + (int64_t)row * k, out_vals ? out_vals + (int64_t)row * k : nullptr);
+  if (tid < 256) {
+    const int w = tid / PKV_WAVE;
+    for (int i = 0; i < w; ++i) incl += s_tot[i];
+  }
+  return incl;
+}
+
+// MSB-first 8-bit radix select of the k-th largest of the 64-bit keys held EIN per thread.
+// Returns the threshold prefix and the shift at which it became exact: the k winners are the keys
+// with (key >> shift) >= (prefix >> shift).  Stops as soon as the threshold bucket is taken whole.
+template <int EIN>
+__device__ __forceinline__ void radix_select_regs(const uint64_t (&v)[EIN], uint32_t k, uint32_t *s_hist, int *s_tot,
+                                                  uint32_t *s_bcast, uint64_t &prefix_out, int &shift_out) {
+  const int tid = threadIdx.x;
+  uint64_t prefix = 0;
+  uint32_t need = k;
+  int shift = 56;
+  for (int pass = 0; pass < 8; ++pass, shift -= 8) {
+    if (tid < 256) s_hist[tid] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < EIN; ++e)
+      if (pass == 0 || (v[e] >> (shift + 8)) == (prefix >> (shift + 8)))
+        atomicAdd(&s_hist[(uint32_t)(v[e] >> shift) & 255u], 1u);
+    __syncthreads();
+    // thread t < 256 owns digit d = 255 - t, so an inclusive scan over t is the suffix sum over digits >= d
+    const uint32_t val = (tid < 256) ? s_hist[255 - tid] : 0u;
+    const uint32_t suf = (uint32_t)scan256_in_1024((int)val, s_tot);
+    if (tid < 256 && suf >= need && suf - val < need) {
+      s_bcast[0] = 255u - (uint32_t)tid;        // threshold digit
+      s_bcast[1] = need - (suf - val);          // still needed inside that bucket
+      s_bcast[2] = (val == need - (suf - val));  // bucket taken whole -> done
+    }
+    __syncthreads();
+    prefix |= (uint64_t)s_bcast[0] << shift;
+    need = s_bcast[1];
+    const bool done = s_bcast[2] != 0;
+    __syncthreads();  // s_bcast / s_hist are rewritten by the next pass
+    if (done || pass == 7) break;
+  }
+  prefix_out = prefix;
+  shift_out = shift;
+}
+
+// len <= 8192 and k well below len: select the k winners exactly, then sort only those.
+template <int EIN>
+__global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
+    const float *__restrict__ x, int64_t x_stride, const int64_t *__restrict__ ids, int64_t ids_stride, int len, int P,
+    int64_t k, int64_t *__restrict__ out_ids, float *__restrict__ out_vals) {
+  extern __shared__ uint64_t s_keys[];
+  __shared__ uint32_t s_hist[256];
+  __shared__ int s_tot[4];
+  __shared__ uint32_t s_bcast[3];
+  __shared__ uint32_t s_counter;
+  const int row = blockIdx.x;
+  const int tid = threadIdx.x;
+  const float *xr = x + (int64_t)row * x_stride;
+  const int64_t *ir = ids ? ids + (int64_t)row * ids_stride : nullptr;
+  uint64_t v[EIN];
+#pragma unroll
+  for (int e = 0; e < EIN; ++e) {
+    const int i = tid + e * kTopkThreads;
+    v[e] = i < len ? make_key(xr, ir, i) : 0ull;
+  }
+  if (tid == 0) s_counter = 0;
+  for (int i = tid; i < (P < 1024 ? 1024 : P); i += kTopkThreads) s_keys[i] = 0ull;
+  uint64_t prefix;
+  int shift;
+  radix_select_regs<EIN>(v, (uint32_t)k, s_hist, s_tot, s_bcast, prefix, shift);
+#pragma unroll
+  for (int e = 0; e < EIN; ++e) {
+    if ((v[e] >> shift) >= (prefix >> shift) && v[e] != 0ull) {
+      const uint32_t slot = atomicAdd(&s_counter, 1u);
+      if (slot < (uint32_t)k) s_keys[slot] = v[e];
+    }
+  }
+  __syncthreads();
+  int64_t *oi = out_ids + (int64_t)row * k;
+  float *ov = out_vals ? out_vals + (int64_t)row * k : nullptr;
+#define PKV_SORT_K(E) sort_lds_keys_and_emit<E>(s_keys, k, oi, ov, nullptr)
+  PKV_DISPATCH_E(P, PKV_SORT_K);
+#undef PKV_SORT_K
 }
 
 // len > 8192, k <= 8192: eight 8-bit MSB-first radix passes find the k-th
@@ -246,7 +518,7 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_radix_kernel(const floa
   }
   // prefix is now the k-th largest key
   if (tid == 0) s_counter = 0;
-  for (int i = tid; i < P; i += kTopkThreads) s_keys[i] = 0ull;
+  for (int i = tid; i < (P < 1024 ? 1024 : P); i += kTopkThreads) s_keys[i] = 0ull;
   __syncthreads();
   for (int64_t i = tid; i < len; i += kTopkThreads) {
     const uint64_t key = make_key(xr, ir, i);
@@ -256,8 +528,11 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_radix_kernel(const floa
     }
   }
   __syncthreads();
-  bitonic_sort_desc(s_keys, P);
-  emit_topk(s_keys, k, out_ids + (int64_t)row * k, out_vals ? out_vals + (int64_t)row * k : nullptr);
+  int64_t *oi = out_ids + (int64_t)row * k;
+  float *ov = out_vals ? out_vals + (int64_t)row * k : nullptr;
+#define PKV_SORT_K(E) sort_lds_keys_and_emit<E>(s_keys, k, oi, ov, nullptr)
+  PKV_DISPATCH_E(P, PKV_SORT_K);
+#undef PKV_SORT_K
 }
 
 // ------------------------------------------------------------------ adaptive-k
@@ -391,7 +666,7 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adaptive_topk_kernel(
     need = s_need;
   }
   if (tid == 0) s_counter = 0;
-  for (int i = tid; i < P; i += kTopkThreads) s_keys[i] = 0ull;
+  for (int i = tid; i < (P < 1024 ? 1024 : P); i += kTopkThreads) s_keys[i] = 0ull;
   __syncthreads();
   for (int64_t i = tid; i < n_cand; i += kTopkThreads) {
     const uint64_t key = make_key(ben, nullptr, i);
@@ -401,7 +676,9 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adaptive_topk_kernel(
     }
   }
   __syncthreads();
-  bitonic_sort_desc(s_keys, P);
+#define PKV_SORT_K(E) sort_lds_keys_and_emit<E>(s_keys, 0, nullptr, nullptr, s_keys)
+  PKV_DISPATCH_E(P, PKV_SORT_K);
+#undef PKV_SORT_K
 
   // smallest k with sl_benefit + cumsum_k >= threshold * total (sequential fp32 cumsum)
   if (tid == 0) {
@@ -427,6 +704,8 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adaptive_topk_kernel(
   }
 }
 
+static size_t lds_bytes(int P) { return (size_t)(P < 1024 ? 1024 : P) * 8; }
+
 static int pow2_ceil(int64_t v) {
   int p = 1;
   while (p < v) p <<= 1;
@@ -435,7 +714,8 @@ static int pow2_ceil(int64_t v) {
 
 }  // namespace
 
-int pkv_launch_select(const uint8_t *cnt_u8, int64_t cnt_stride, const uint16_t *chunk_hist, int chunk_keys, int rows,
+int pkv_launch_select(const uint8_t *cnt_u8, int64_t cnt_stride, const uint32_t *row_suf, const uint16_t *chunk_suf,
+                      int chunk_keys, int rows,
                       int64_t n_keys, int64_t k, int64_t *out, hipStream_t s) {
   PKV_REQUIRE(k >= 1 && k < n_keys, "select needs 1 <= k < n_keys (k=%lld n=%lld)", (long long)k,
               (long long)n_keys);
@@ -443,9 +723,30 @@ int pkv_launch_select(const uint8_t *cnt_u8, int64_t cnt_stride, const uint16_t 
               "count rows must be 16-byte aligned and padded");
   const int64_t n_chunks = (n_keys + chunk_keys - 1) / chunk_keys;
   dim3 grid((unsigned)n_chunks, (unsigned)rows);
-  hipLaunchKernelGGL(pkv_select_kernel, grid, dim3(kSelThreads), 0, s, cnt_u8, cnt_stride, chunk_hist, chunk_keys,
+  hipLaunchKernelGGL(pkv_select_kernel, grid, dim3(kSelThreads), 0, s, cnt_u8, cnt_stride, row_suf, chunk_suf, chunk_keys,
                      n_keys, k, out);
   PKV_LAUNCH_CHECK("pkv_select_kernel");
+  return PKV_OK;
+}
+
+int pkv_launch_select_rerank(const uint8_t *cnt_u8, int64_t cnt_stride, const uint32_t *row_suf,
+                             const uint16_t *chunk_suf, int chunk_keys, int bs,
+                             int n_kv_heads, int64_t n_keys, int64_t k, const uint8_t *nib, int64_t ns_b, int64_t ns_h,
+                             const uint16_t *weight, int64_t ws_b, int64_t ws_h, const float *qhat, const float *qnorm,
+                             const float *centers, int64_t *cand, float *scores, hipStream_t s) {
+  PKV_REQUIRE(k >= 1 && k < n_keys && k < ((int64_t)1 << 31), "select needs 1 <= k < n_keys (k=%lld n=%lld)", (long long)k,
+              (long long)n_keys);
+  PKV_REQUIRE(cnt_stride % 16 == 0 && cnt_stride >= n_keys && pkv_aligned(cnt_u8, 16),
+              "count rows must be 16-byte aligned and padded");
+  PKV_REQUIRE(pkv_aligned(nib, 16) && pkv_aligned(weight, 16) && ns_b % 16 == 0 && ns_h % 16 == 0 && ws_b % 8 == 0 &&
+                  ws_h % 8 == 0,
+              "key-major nibbles / weights must be 16-byte aligned");
+  const int64_t n_chunks = (n_keys + chunk_keys - 1) / chunk_keys;
+  dim3 grid((unsigned)n_chunks, (unsigned)(bs * n_kv_heads));
+  hipLaunchKernelGGL(pkv_select_rerank_kernel, grid, dim3(kSelThreads), 0, s, cnt_u8, cnt_stride, row_suf, chunk_suf,
+                     chunk_keys,
+                     n_kv_heads, n_keys, k, nib, ns_b, ns_h, weight, ws_b, ws_h, qhat, qnorm, centers, cand, scores);
+  PKV_LAUNCH_CHECK("pkv_select_rerank_kernel");
   return PKV_OK;
 }
 
@@ -458,20 +759,21 @@ PKV_INTERNAL int pkv_launch_identity_fill(int64_t *out, int64_t len, int64_t k, 
 }
 
 static void bucket_ws_layout(int rows, int64_t len, int &chunk_keys, int64_t &cnt_stride, size_t &off_hist,
-                             size_t &total) {
+                             size_t &off_row, size_t &total) {
   chunk_keys = pkv_pick_chunk_keys(rows, len);
   cnt_stride = (int64_t)pkv_align_up((size_t)len, 16);
   const int64_t n_chunks = (len + chunk_keys - 1) / chunk_keys;
   off_hist = pkv_align_up((size_t)rows * (size_t)cnt_stride, 256);
-  total = off_hist + pkv_align_up((size_t)rows * (size_t)n_chunks * 128 * sizeof(uint16_t), 256);
+  off_row = off_hist + pkv_align_up((size_t)rows * (size_t)n_chunks * 128 * sizeof(uint16_t), 256);
+  total = off_row + pkv_align_up((size_t)rows * 128 * sizeof(uint32_t), 256);
 }
 
 extern "C" size_t pkv_bucket_topk_ws_bytes(int rows, int64_t len) {
   if (rows <= 0 || len <= 0) return 256;
   int ck;
   int64_t cs;
-  size_t oh, tot;
-  bucket_ws_layout(rows, len, ck, cs, oh, tot);
+  size_t oh, orow, tot;
+  bucket_ws_layout(rows, len, ck, cs, oh, orow, tot);
   return tot;
 }
 
@@ -486,19 +788,23 @@ extern "C" int pkv_bucket_topk(const int32_t *x, int64_t x_stride, int rows, int
   if (len == k) return pkv_launch_identity_fill(out, len, k, rows, s);
   int ck;
   int64_t cs;
-  size_t oh, tot;
-  bucket_ws_layout(rows, len, ck, cs, oh, tot);
+  size_t oh, orow, tot;
+  bucket_ws_layout(rows, len, ck, cs, oh, orow, tot);
   if (!ws || ws_bytes < tot || !pkv_aligned(ws, 256)) {
     pkv_set_error("pkv_bucket_topk: workspace of %zu bytes (256-aligned) required, got %zu", tot, ws_bytes);
     return PKV_ENOMEM;
   }
   uint8_t *cnt = (uint8_t *)ws;
   uint16_t *hist = (uint16_t *)((char *)ws + oh);
+  uint32_t *row_suf = (uint32_t *)((char *)ws + orow);
   const int64_t n_chunks = (len + ck - 1) / ck;
+  hipLaunchKernelGGL(pkv_zero_u32_kernel, dim3((unsigned)((rows * 128 + 255) / 256)), dim3(256), 0, s, row_suf,
+                     (int64_t)rows * 128);
+  PKV_LAUNCH_CHECK("pkv_zero_u32_kernel");
   hipLaunchKernelGGL(pkv_counts_to_u8_kernel, dim3((unsigned)n_chunks, (unsigned)rows), dim3(256), 0, s, x, x_stride,
-                     len, cnt, cs, hist, ck);
+                     len, cnt, cs, row_suf, hist, ck);
   PKV_LAUNCH_CHECK("pkv_counts_to_u8_kernel");
-  return pkv_launch_select(cnt, cs, hist, ck, rows, len, k, out, s);
+  return pkv_launch_select(cnt, cs, row_suf, hist, ck, rows, len, k, out, s);
 }
 
 size_t pkv_topk_ws_bytes_impl(int, int64_t, int64_t) { return 256; }
@@ -513,16 +819,25 @@ int pkv_launch_topk_f32(const float *x, int64_t x_stride, const int64_t *ids, in
   PKV_REQUIRE(k > 0, "k must be positive");
   PKV_REQUIRE(k <= len, "k cannot exceed sequence length");
   PKV_REQUIRE(rows > 0 && len < ((int64_t)1 << 31), "bad shape rows=%d len=%lld", rows, (long long)len);
-  if (len <= kTopkMaxSort) {
+  if (len <= kTopkMaxSort && pow2_ceil(k) * 2 <= pow2_ceil(len) && pow2_ceil(len) >= 2048) {
+    const int P = pow2_ceil(k);
+    const int ein = pow2_ceil(len) / kTopkThreads;
+#define PKV_SEL(EIN)                                                                                              \
+  hipLaunchKernelGGL((pkv_topk_select_sort_kernel<EIN>), dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes(P), s, \
+                     x, x_stride, ids, ids_stride, (int)len, P, k, out_ids, out_vals)
+    if (ein <= 2) PKV_SEL(2); else if (ein == 4) PKV_SEL(4); else PKV_SEL(8);
+#undef PKV_SEL
+    PKV_LAUNCH_CHECK("pkv_topk_select_sort_kernel");
+  } else if (len <= kTopkMaxSort) {
     const int P = pow2_ceil(len);
-    hipLaunchKernelGGL(pkv_topk_sort_kernel, dim3((unsigned)rows), dim3(kTopkThreads), (size_t)P * 8, s, x, x_stride,
+    hipLaunchKernelGGL(pkv_topk_sort_kernel, dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes(P), s, x, x_stride,
                        ids, ids_stride, (int)len, P, k, out_ids, out_vals);
     PKV_LAUNCH_CHECK("pkv_topk_sort_kernel");
   } else {
     PKV_REQUIRE(k <= kTopkMaxSort, "k up to %d supported when len > %d (got %lld)", kTopkMaxSort, kTopkMaxSort,
                 (long long)k);
     const int P = pow2_ceil(k);
-    hipLaunchKernelGGL(pkv_topk_radix_kernel, dim3((unsigned)rows), dim3(kTopkThreads), (size_t)P * 8, s, x,
+    hipLaunchKernelGGL(pkv_topk_radix_kernel, dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes(P), s, x,
                        x_stride, ids, ids_stride, len, P, k, out_ids, out_vals);
     PKV_LAUNCH_CHECK("pkv_topk_radix_kernel");
   }
@@ -559,7 +874,7 @@ extern "C" int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, cons
     return PKV_ENOMEM;
   }
   const int P = pow2_ceil(k_out);
-  hipLaunchKernelGGL(pkv_adaptive_topk_kernel, dim3((unsigned)rows), dim3(kTopkThreads), (size_t)P * 8,
+  hipLaunchKernelGGL(pkv_adaptive_topk_kernel, dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes(P),
                      (hipStream_t)stream, sl_logits, sl_stride, sl_vnorm, slv_stride, sl, cand_scores, cand_dtype,
                      cand_scale, cand_vnorm, value_norm, vn_stride, vn_offset, cand_ids, n_cand, threshold, k_out, P,
                      adaptive_k, topk_ids, (float *)ws);

@@ -199,7 +199,7 @@ def update_cache_cnt_legacy(sorted_cluster_ids: torch.Tensor, topk_cluster_cnt: 
 
 def pick_chunk_keys(rows: int, n_keys: int) -> int:
     chunk = 2048
-    while chunk < 16384 and rows * ((n_keys + chunk - 1) // chunk) > 1024:
+    while chunk < 16384 and rows * ((n_keys + chunk - 1) // chunk) > 2048:
         chunk *= 2
     while chunk < 32768 and (n_keys + chunk - 1) // chunk > 512:
         chunk *= 2
@@ -207,23 +207,25 @@ def pick_chunk_keys(rows: int, n_keys: int) -> int:
 
 
 def collision_scan(codebook: torch.Tensor, lut: torch.Tensor, out_dtype=torch.int32, want_hist: bool = False):
-    """Votes per key from a ready table.  Returns (cnt [bs,H,N], chunk_hist or None, chunk_keys)."""
+    """Votes per key from a ready table.  Returns (cnt [bs,H,N], (row_suf, chunk_suf) or None, chunk_keys);
+    the suffix histograms count keys with a vote count >= t, per row and per chunk."""
     _cuda(codebook, lut)
     bs, H, Bs, N = codebook.shape
     _need(codebook.dtype == torch.uint8 and Bs == B_SUB, "codebook must be u8 [bs,H,16,N]")
     _need(lut.dtype == torch.uint8 and lut.is_contiguous() and lut.numel() == bs * H * B_SUB * K_CLUSTERS, "lut: u8 [bs,H,16,256]")
     cnt = torch.empty(bs, H, N, dtype=out_dtype, device=codebook.device)
     chunk = pick_chunk_keys(bs * H, N)
-    hist = None
+    hist = row_suf = None
     if want_hist:
         hist = torch.empty(bs * H, (N + chunk - 1) // chunk, 128, dtype=torch.int16, device=codebook.device)
+        row_suf = torch.zeros(bs * H, 128, dtype=torch.int32, device=codebook.device)
     u8 = cnt if out_dtype == torch.uint8 else None
     i32 = cnt if out_dtype == torch.int32 else None
     _need(u8 is not None or i32 is not None, "out_dtype must be uint8 or int32")
     _lib.check(_lib.lib().pkv_collision_scan(_p(codebook), codebook.stride(0), codebook.stride(1), codebook.stride(3),
-                                             codebook.stride(2), bs, H, N, _p(lut), _p(u8), _p(i32), _p(hist), chunk,
-                                             _stream(codebook)))
-    return cnt, hist, chunk
+                                             codebook.stride(2), bs, H, N, _p(lut), _p(u8), _p(i32), _p(row_suf), _p(hist),
+                                             chunk, _stream(codebook)))
+    return cnt, ((row_suf, hist) if want_hist else None), chunk
 
 
 # --------------------------------------------------------------- selections

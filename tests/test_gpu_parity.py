@@ -423,12 +423,14 @@ def test_retrieve_fused_matches_oracle(ops, request, wl_name):
     cnt = plan.view("cnt_u8", w.N, w.C, w.K, torch.uint8).view(w.R, cnt_stride)[:, :w.N].cpu().numpy()
     cand = plan.view("cand", w.N, w.C, w.K, torch.int64).view(w.R, w.C).cpu().numpy()
     sc = plan.view("scores", w.N, w.C, w.K, torch.float32).view(w.R, w.C).cpu().numpy()
-    hist = plan.view("chunk_hist", w.N, w.C, w.K, torch.int16).view(w.R, -1, 128).cpu().numpy().astype(np.int64) & 0xFFFF
+    suf = plan.view("chunk_suffix_hist", w.N, w.C, w.K, torch.int16).view(w.R, -1, 128).cpu().numpy().astype(np.int64) & 0xFFFF
+    row_suf = plan.view("row_suffix_hist", w.N, w.C, w.K, torch.int32).view(w.R, 128).cpu().numpy().astype(np.int64)
     for r in range(w.R):
         b, h = divmod(r, w.H)
         st = W.oracle_stages(w, r)
         assert np.array_equal(cnt[r], st["cnt"].astype(np.uint8)), f"vote counts differ in row {r}"
-        assert np.array_equal(hist[r].sum(axis=0), np.bincount(st["cnt"], minlength=128)), f"histogram row {r}"
+        ref_suf = np.cumsum(np.bincount(st["cnt"], minlength=128)[::-1])[::-1]  # keys with count >= t
+        assert np.array_equal(suf[r].sum(axis=0), ref_suf) and np.array_equal(row_suf[r], ref_suf), f"histogram row {r}"
         assert np.array_equal(cand[r], st["cand"]), f"candidate list differs in row {r}"
         np.testing.assert_allclose(sc[r], st["scores"], rtol=1e-5, atol=1e-5 * np.abs(st["scores"]).max())
         assert np.array_equal(out[b, h].cpu().numpy(), st["final"]), f"final top-k differs in row {r}"
