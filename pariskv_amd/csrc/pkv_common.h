@@ -5,6 +5,7 @@
 #include <hip/hip_ext.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "../../include/pariskv_hip.h"
@@ -50,12 +51,12 @@ struct PkvTiers {
 };
 
 // Keys per workgroup-chunk of the collision scan / candidate select, chosen so
-// that rows * n_chunks is about two thousand workgroups (8 per CU) while the
-// per-row chunk histograms (uint16 [n_chunks][128]) stay small.  Always a
+// that rows * n_chunks is about a thousand workgroups (4 per CU, the measured
+// optimum at 32 rows x 128K keys) while the per-row chunk histograms (uint16 [n_chunks][128]) stay small.  Always a
 // multiple of 2048 and at most 32768 (a chunk's histogram bins are uint16).
 static inline int pkv_pick_chunk_keys(int rows, int64_t n_keys) {
   int64_t chunk = 2048;
-  while (chunk < 16384 && (int64_t)rows * ((n_keys + chunk - 1) / chunk) > 2048) chunk *= 2;
+  while (chunk < 16384 && (int64_t)rows * ((n_keys + chunk - 1) / chunk) > 1024) chunk *= 2;
   while (chunk < 32768 && (n_keys + chunk - 1) / chunk > 512) chunk *= 2;
   return (int)chunk;
 }

@@ -199,7 +199,7 @@ def update_cache_cnt_legacy(sorted_cluster_ids: torch.Tensor, topk_cluster_cnt: 
 
 def pick_chunk_keys(rows: int, n_keys: int) -> int:
     chunk = 2048
-    while chunk < 16384 and rows * ((n_keys + chunk - 1) // chunk) > 2048:
+    while chunk < 16384 and rows * ((n_keys + chunk - 1) // chunk) > 1024:
         chunk *= 2
     while chunk < 32768 and (n_keys + chunk - 1) // chunk > 512:
         chunk *= 2
