@@ -134,14 +134,39 @@ __device__ __forceinline__ float pkv_from_ordered_u32(uint32_t k) {
 
 __device__ __forceinline__ int pkv_lane() { return (int)(threadIdx.x & (PKV_WAVE - 1)); }
 
-// Inclusive scan over the 64 lanes of a wave.
-__device__ __forceinline__ int pkv_wave_incl_scan(int v) {
-  const int lane = pkv_lane();
-#pragma unroll
-  for (int d = 1; d < PKV_WAVE; d <<= 1) {
-    int o = __shfl_up(v, d, PKV_WAVE);
-    if (lane >= d) v += o;
+// Value of lane (lane ^ M).  M = 1, 2, 4, 8 are data-parallel-primitive moves inside a row of 16 lanes
+// (no trip through the LDS crossbar); 16 and 32 use the generic lane permute.
+template <int M>
+__device__ __forceinline__ uint32_t pkv_lane_xor(uint32_t v) {
+  const int x = (int)v;
+  if (M == 1) return (uint32_t)__builtin_amdgcn_mov_dpp(x, 0xB1, 0xf, 0xf, false);   // quad_perm [1,0,3,2]
+  if (M == 2) return (uint32_t)__builtin_amdgcn_mov_dpp(x, 0x4E, 0xf, 0xf, false);   // quad_perm [2,3,0,1]
+  if (M == 4) {
+    int r = __builtin_amdgcn_update_dpp(x, x, 0x104, 0xf, 0x5, false);  // banks 0,2 read lane + 4 (row_shl:4)
+    r = __builtin_amdgcn_update_dpp(r, x, 0x114, 0xf, 0xa, false);      // banks 1,3 read lane - 4 (row_shr:4)
+    return (uint32_t)r;
   }
+  if (M == 8) return (uint32_t)__builtin_amdgcn_mov_dpp(x, 0x128, 0xf, 0xf, false);  // row_ror:8
+  return (uint32_t)__shfl_xor(x, M, PKV_WAVE);
+}
+template <int M>
+__device__ __forceinline__ float pkv_lane_xor_f(float v) {
+  return __uint_as_float(pkv_lane_xor<M>(__float_as_uint(v)));
+}
+template <int M>
+__device__ __forceinline__ uint64_t pkv_lane_xor64(uint64_t v) {
+  return ((uint64_t)pkv_lane_xor<M>((uint32_t)(v >> 32)) << 32) | pkv_lane_xor<M>((uint32_t)v);
+}
+
+// Inclusive scan over the 64 lanes of a wave: four row_shr steps inside each row of 16 lanes, then the
+// row totals travel with row_bcast:15 (rows 1, 3) and row_bcast:31 (rows 2, 3).
+__device__ __forceinline__ int pkv_wave_incl_scan(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, true);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, true);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, true);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, true);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);
   return v;
 }
 
@@ -156,8 +181,10 @@ __device__ __forceinline__ float pkv_normalize_rotate_16(const float (&x)[8], co
   float acc = x[0] * x[0];
 #pragma unroll
   for (int j = 1; j < 8; ++j) acc = acc + x[j] * x[j];
-#pragma unroll
-  for (int m = 1; m < 16; m <<= 1) acc = acc + __shfl_xor(acc, m, PKV_WAVE);
+  acc = acc + pkv_lane_xor_f<1>(acc);
+  acc = acc + pkv_lane_xor_f<2>(acc);
+  acc = acc + pkv_lane_xor_f<4>(acc);
+  acc = acc + pkv_lane_xor_f<8>(acc);
   const float n = pkv_rdt(sqrtf(acc), dtype);
   const float den = n < 1e-8f ? 1e-8f : n;
   float t[8];
@@ -174,17 +201,85 @@ __device__ __forceinline__ float pkv_normalize_rotate_16(const float (&x)[8], co
       }
     }
   }
-#pragma unroll
-  for (int m = 1; m < 16; m <<= 1) {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float o = __shfl_xor(t[j], m, PKV_WAVE);
-      t[j] = (s & m) ? (o - t[j]) : (t[j] + o);
-    }
+#define PKV_FWHT_LANE_STAGE(M)                              \
+  _Pragma("unroll") for (int j = 0; j < 8; ++j) {           \
+    const float o = pkv_lane_xor_f<M>(t[j]);                \
+    t[j] = (s & M) ? (o - t[j]) : (t[j] + o);               \
   }
+  PKV_FWHT_LANE_STAGE(1)
+  PKV_FWHT_LANE_STAGE(2)
+  PKV_FWHT_LANE_STAGE(4)
+  PKV_FWHT_LANE_STAGE(8)
+#undef PKV_FWHT_LANE_STAGE
 #pragma unroll
   for (int j = 0; j < 8; ++j) y[j] = pkv_rdt(t[j] * PKV_HADAMARD_SCALE, dtype);
   return n;
+}
+
+// Group mean of the G query heads of row (b, h), normalised and SRHT-rotated (polar_cache.py:1027-1031,
+// 905-922).  Called by all 64 lanes of ONE wave: 16 lanes per copy of the vector, four identical copies;
+// lane l gets dims 8(l & 15) .. +7 of the rotated unit vector in y[] and the norm of the mean as result.
+// The G heads are added in order; their loads are all issued before the first add (8 at a time, with no
+// branch between them, so that they are in flight together).
+template <bool BF16>
+__device__ __forceinline__ float pkv_query_mean_rotate_t(const void *__restrict__ q, int b, int h, int n_kv_heads,
+                                                         int group, const float *__restrict__ signs, float (&y)[8]) {
+  constexpr int dtype = BF16 ? PKV_DTYPE_BF16 : PKV_DTYPE_F32;
+  const int s = pkv_lane() & 15;
+  const int64_t base = ((int64_t)b * n_kv_heads * group + (int64_t)h * group) * 128 + 8 * s;
+  float acc[8], sg[8];
+  const float4 s0 = *(const float4 *)(signs + 8 * s), s1 = *(const float4 *)(signs + 8 * s + 4);
+  sg[0] = s0.x, sg[1] = s0.y, sg[2] = s0.z, sg[3] = s0.w, sg[4] = s1.x, sg[5] = s1.y, sg[6] = s1.z, sg[7] = s1.w;
+  for (int g0 = 0; g0 < group; g0 += 8) {
+    pkv_u32x4 raw[8][BF16 ? 1 : 2];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int g = g0 + u < group ? g0 + u : group - 1;
+      if (BF16) {
+        raw[u][0] = *(const pkv_u32x4 *)((const uint16_t *)q + base + (int64_t)g * 128);
+      } else {
+        raw[u][0] = *(const pkv_u32x4 *)((const float *)q + base + (int64_t)g * 128);
+        raw[u][BF16 ? 0 : 1] = *(const pkv_u32x4 *)((const float *)q + base + (int64_t)g * 128 + 4);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      float v[8];
+      if (BF16) {
+        const uint32_t ww[4] = {raw[u][0].x, raw[u][0].y, raw[u][0].z, raw[u][0].w};
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+          v[2 * p] = __uint_as_float(ww[p] << 16);
+          v[2 * p + 1] = __uint_as_float(ww[p] & 0xffff0000u);
+        }
+      } else {
+        const pkv_u32x4 lo = raw[u][0], hi = raw[u][BF16 ? 0 : 1];
+        v[0] = __uint_as_float(lo.x), v[1] = __uint_as_float(lo.y), v[2] = __uint_as_float(lo.z);
+        v[3] = __uint_as_float(lo.w), v[4] = __uint_as_float(hi.x), v[5] = __uint_as_float(hi.y);
+        v[6] = __uint_as_float(hi.z), v[7] = __uint_as_float(hi.w);
+      }
+      const bool first = g0 + u == 0, live = g0 + u < group;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j] = first ? v[j] : (live ? acc[j] + v[j] : acc[j]);
+    }
+  }
+  float x[8];
+  if ((group & (group - 1)) == 0) {  // power of two: multiplying by the reciprocal is the same division, exactly
+    const float inv = 1.0f / (float)group;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[j] = pkv_rdt(acc[j] * inv, dtype);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[j] = pkv_rdt(acc[j] / (float)group, dtype);
+  }
+  return pkv_normalize_rotate_16(x, sg, s, dtype, y);
+}
+
+__device__ __forceinline__ float pkv_query_mean_rotate(const void *__restrict__ q, int dtype, int b, int h,
+                                                       int n_kv_heads, int group, const float *__restrict__ signs,
+                                                       float (&y)[8]) {
+  return dtype == PKV_DTYPE_BF16 ? pkv_query_mean_rotate_t<true>(q, b, h, n_kv_heads, group, signs, y)
+                                 : pkv_query_mean_rotate_t<false>(q, b, h, n_kv_heads, group, signs, y);
 }
 
 // ---- 4-bit rerank core (shared by the stand-alone rerank and the fused select+rerank kernels) ----
@@ -251,7 +346,8 @@ __device__ __forceinline__ float pkv_rerank_keymajor(const float *__restrict__ s
 }
 
 // Turn a 128-bin histogram in LDS (s_hist) into its suffix sums suf[t] = sum_{t' >= t} hist[t'],
-// store them as the chunk's uint16 suffix histogram and add them to the row's uint32 suffix totals.
+// store them as the chunk's uint16 suffix histogram and add them to the row's uint32 suffix totals
+// (row_suf may be null).
 // Called by all threads of a workgroup with >= 128 threads; contains barriers.  s_w0: one LDS word.
 __device__ __forceinline__ void pkv_store_suffix_hist(const uint32_t *s_hist, uint32_t *s_w0,
                                                       uint32_t *__restrict__ row_suf, uint16_t *__restrict__ chunk_suf) {
@@ -265,7 +361,7 @@ __device__ __forceinline__ void pkv_store_suffix_hist(const uint32_t *s_hist, ui
   if (tid < 128) {
     if (tid >= PKV_WAVE) incl += (int)*s_w0;
     chunk_suf[127 - tid] = (uint16_t)incl;
-    if (incl) atomicAdd(&row_suf[127 - tid], (uint32_t)incl);
+    if (row_suf && incl) atomicAdd(&row_suf[127 - tid], (uint32_t)incl);
   }
 }
 

@@ -49,33 +49,8 @@ __global__ __launch_bounds__(256) void pkv_query_prep_lut_kernel(
 
   if (tid < PKV_WAVE) {
     const int s = tid & 15;
-    const int64_t base = ((int64_t)b * n_kv_heads * group + (int64_t)h * group) * 128 + 8 * s;
-    float acc[8], sg[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) sg[j] = signs[8 * s + j];
-    // group mean (polar_cache.py:1029-1030), sequential over the G heads
-    for (int g = 0; g < group; ++g) {
-      float v[8];
-      if (dtype == PKV_DTYPE_BF16) {
-        const pkv_u32x4 w = *(const pkv_u32x4 *)((const uint16_t *)q + base + (int64_t)g * 128);
-        const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-          v[2 * p] = __uint_as_float(ww[p] << 16);
-          v[2 * p + 1] = __uint_as_float(ww[p] & 0xffff0000u);
-        }
-      } else {
-        const float4 a = *(const float4 *)((const float *)q + base + (int64_t)g * 128);
-        const float4 c = *(const float4 *)((const float *)q + base + (int64_t)g * 128 + 4);
-        v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = c.x, v[5] = c.y, v[6] = c.z, v[7] = c.w;
-      }
-#pragma unroll
-      for (int j = 0; j < 8; ++j) acc[j] = (g == 0) ? v[j] : acc[j] + v[j];
-    }
-    float x[8], y[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) x[j] = pkv_rdt(acc[j] / (float)group, dtype);
-    const float n = pkv_normalize_rotate_16(x, sg, s, dtype, y);
+    float y[8];
+    const float n = pkv_query_mean_rotate(q, dtype, b, h, n_kv_heads, group, signs, y);
     if (tid < 16) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) {

@@ -261,10 +261,45 @@ __device__ __forceinline__ uint64_t make_key(const float *__restrict__ x, const 
   return ((uint64_t)pkv_ordered_u32(x[i]) << 32) | (uint64_t)(~id);
 }
 
+// Key of lane (lane ^ mask); mask is a constant once the callers' loops are unrolled, so the switch folds.
 __device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int mask) {
-  const uint32_t lo = __shfl_xor((uint32_t)v, mask, PKV_WAVE);
-  const uint32_t hi = __shfl_xor((uint32_t)(v >> 32), mask, PKV_WAVE);
-  return ((uint64_t)hi << 32) | lo;
+  switch (mask) {
+    case 1: return pkv_lane_xor64<1>(v);
+    case 2: return pkv_lane_xor64<2>(v);
+    case 4: return pkv_lane_xor64<4>(v);
+    case 8: return pkv_lane_xor64<8>(v);
+    case 16: return pkv_lane_xor64<16>(v);
+    default: return pkv_lane_xor64<32>(v);
+  }
+}
+
+// hist[d] += 1 for every active lane.  Lanes of a wave that share the leading lane's digit are added
+// with one atomic (two rounds), which is what keeps the first radix passes, where nearly all keys
+// fall into one or two buckets, from serialising on a single LDS address.
+__device__ __forceinline__ void wave_hist_add(uint32_t *hist, uint32_t d, bool active) {
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    const uint64_t act = __ballot(active);
+    if (act == 0) return;
+    const int leader = __ffsll((long long)act) - 1;
+    const uint32_t dl = (uint32_t)__builtin_amdgcn_readlane((int)d, leader);
+    const uint64_t same = __ballot(active && d == dl);
+    if (pkv_lane() == leader) atomicAdd(&hist[dl], (uint32_t)__popcll((long long)same));
+    if (d == dl) active = false;
+  }
+  if (active) atomicAdd(&hist[d], 1u);
+}
+
+// Slot for every lane with `take` set, out of a workgroup-wide counter: one atomic per wave.
+__device__ __forceinline__ uint32_t wave_take_slots(uint32_t *counter, bool take) {
+  const uint64_t m = __ballot(take);
+  if (m == 0) return 0u;
+  const int leader = __ffsll((long long)m) - 1;
+  uint32_t base = 0;
+  if (pkv_lane() == leader) base = atomicAdd(counter, (uint32_t)__popcll((long long)m));
+  base = (uint32_t)__builtin_amdgcn_readlane((int)base, leader);
+  const uint64_t below = m & (((uint64_t)1 << pkv_lane()) - 1);
+  return base + (uint32_t)__popcll((long long)below);
 }
 
 // Descending bitonic sort of 1024*E 64-bit keys held E per thread (thread t owns sorted positions
@@ -381,58 +416,106 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_sort_kernel(const float
 #undef PKV_SORT_ALL
 }
 
-// Inclusive scan of one value per thread over the first 256 threads of a 1024-thread workgroup
-// (all 1024 threads must call it: it contains a barrier).  s_tot: 4 ints.
-__device__ __forceinline__ int scan256_in_1024(int v, int *s_tot) {
+// Second half of a radix-select pass, called by all 1024 threads after their histogram atomics: the
+// first wave scans the pass's 256 bins (lane l owns digits 255 - 4l .. 252 - 4l, descending, so an
+// inclusive scan over lanes is the suffix sum over digits) and leaves in s_bcast[(pass & 1) * 4 ..]:
+// the threshold digit, the keys still needed inside that bucket, and whether the bucket is taken whole.
+// Meanwhile the other histogram buffer is cleared for the next pass.  Two barriers.
+__device__ __forceinline__ void radix_pass_decide(uint32_t *s_hist, uint32_t *s_bcast, int pass, uint32_t need) {
   const int tid = threadIdx.x;
-  int incl = 0;
-  if (tid < 256) {
-    incl = pkv_wave_incl_scan(v);
-    if (pkv_lane() == PKV_WAVE - 1) s_tot[tid / PKV_WAVE] = incl;
+  const uint32_t *hist = s_hist + (pass & 1) * 256;
+  uint32_t *res = s_bcast + (pass & 1) * 4;
+  __syncthreads();
+  if (tid < PKV_WAVE) {
+    uint32_t h[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) h[j] = hist[255 - 4 * tid - j];
+    const uint32_t mine = h[0] + h[1] + h[2] + h[3];
+    uint32_t above = (uint32_t)pkv_wave_incl_scan((int)mine) - mine;  // keys in digits above this lane's four
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (above < need && above + h[j] >= need) {
+        res[0] = (uint32_t)(255 - 4 * tid - j);
+        res[1] = need - above;
+        res[2] = (h[j] == need - above);
+      }
+      above += h[j];
+    }
+  } else if (tid < PKV_WAVE + 256) {
+    s_hist[((pass + 1) & 1) * 256 + tid - PKV_WAVE] = 0;
   }
   __syncthreads();
-  if (tid < 256) {
-    const int w = tid / PKV_WAVE;
-    for (int i = 0; i < w; ++i) incl += s_tot[i];
-  }
-  return incl;
 }
 
 // MSB-first 8-bit radix select of the k-th largest of the 64-bit keys held EIN per thread.
 // Returns the threshold prefix and the shift at which it became exact: the k winners are the keys
 // with (key >> shift) >= (prefix >> shift).  Stops as soon as the threshold bucket is taken whole.
+// s_hist: 512 words (two alternating histograms), s_bcast: 8 words.
 template <int EIN>
-__device__ __forceinline__ void radix_select_regs(const uint64_t (&v)[EIN], uint32_t k, uint32_t *s_hist, int *s_tot,
+__device__ __forceinline__ void radix_select_regs(const uint64_t (&v)[EIN], uint32_t k, uint32_t *s_hist,
                                                   uint32_t *s_bcast, uint64_t &prefix_out, int &shift_out) {
   const int tid = threadIdx.x;
   uint64_t prefix = 0;
   uint32_t need = k;
   int shift = 56;
+  if (tid < 512) s_hist[tid] = 0;
+  __syncthreads();
   for (int pass = 0; pass < 8; ++pass, shift -= 8) {
-    if (tid < 256) s_hist[tid] = 0;
-    __syncthreads();
+    uint32_t *hist = s_hist + (pass & 1) * 256;
+    uint32_t *res = s_bcast + (pass & 1) * 4;
 #pragma unroll
     for (int e = 0; e < EIN; ++e)
-      if (pass == 0 || (v[e] >> (shift + 8)) == (prefix >> (shift + 8)))
-        atomicAdd(&s_hist[(uint32_t)(v[e] >> shift) & 255u], 1u);
-    __syncthreads();
-    // thread t < 256 owns digit d = 255 - t, so an inclusive scan over t is the suffix sum over digits >= d
-    const uint32_t val = (tid < 256) ? s_hist[255 - tid] : 0u;
-    const uint32_t suf = (uint32_t)scan256_in_1024((int)val, s_tot);
-    if (tid < 256 && suf >= need && suf - val < need) {
-      s_bcast[0] = 255u - (uint32_t)tid;        // threshold digit
-      s_bcast[1] = need - (suf - val);          // still needed inside that bucket
-      s_bcast[2] = (val == need - (suf - val));  // bucket taken whole -> done
-    }
-    __syncthreads();
-    prefix |= (uint64_t)s_bcast[0] << shift;
-    need = s_bcast[1];
-    const bool done = s_bcast[2] != 0;
-    __syncthreads();  // s_bcast / s_hist are rewritten by the next pass
-    if (done || pass == 7) break;
+      wave_hist_add(hist, (uint32_t)(v[e] >> shift) & 255u,
+                    pass == 0 || (v[e] >> (shift + 8)) == (prefix >> (shift + 8)));
+    radix_pass_decide(s_hist, s_bcast, pass, need);
+    prefix |= (uint64_t)res[0] << shift;
+    need = res[1];
+    if (res[2] != 0 || pass == 7) break;
   }
   prefix_out = prefix;
   shift_out = shift;
+}
+
+// The same selection over keys that do not fit the registers: key_of(i), i < len, is evaluated again
+// in every pass.
+template <typename KeyFn>
+__device__ __forceinline__ void radix_select_streamed(KeyFn key_of, int64_t len, uint32_t k, uint32_t *s_hist,
+                                                      uint32_t *s_bcast, uint64_t &prefix_out, int &shift_out) {
+  const int tid = threadIdx.x;
+  uint64_t prefix = 0;
+  uint32_t need = k;
+  int shift = 56;
+  if (tid < 512) s_hist[tid] = 0;
+  __syncthreads();
+  for (int pass = 0; pass < 8; ++pass, shift -= 8) {
+    uint32_t *hist = s_hist + (pass & 1) * 256;
+    const uint32_t *res = s_bcast + (pass & 1) * 4;
+    for (int64_t i0 = 0; i0 < len; i0 += kTopkThreads) {  // whole waves stay in the loop: it uses ballots
+      const int64_t i = i0 + tid;
+      const uint64_t key = i < len ? key_of(i) : 0ull;
+      wave_hist_add(hist, (uint32_t)(key >> shift) & 255u,
+                    i < len && (pass == 0 || (key >> (shift + 8)) == (prefix >> (shift + 8))));
+    }
+    radix_pass_decide(s_hist, s_bcast, pass, need);
+    prefix |= (uint64_t)res[0] << shift;
+    need = res[1];
+    if (res[2] != 0 || pass == 7) break;
+  }
+  prefix_out = prefix;
+  shift_out = shift;
+}
+
+// Winners of a streamed selection into s_keys[0 .. k) (any order); s_counter must be 0.
+template <typename KeyFn>
+__device__ __forceinline__ void collect_winners_streamed(KeyFn key_of, int64_t len, uint32_t k, uint64_t prefix,
+                                                         int shift, uint32_t *s_counter, uint64_t *s_keys) {
+  for (int64_t i0 = 0; i0 < len; i0 += kTopkThreads) {
+    const int64_t i = i0 + threadIdx.x;
+    const uint64_t key = i < len ? key_of(i) : 0ull;
+    const bool win = i < len && (key >> shift) >= (prefix >> shift);
+    const uint32_t slot = wave_take_slots(s_counter, win);
+    if (win && slot < k) s_keys[slot] = key;
+  }
 }
 
 // len <= 8192 and k well below len: select the k winners exactly, then sort only those.
@@ -441,9 +524,8 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
     const float *__restrict__ x, int64_t x_stride, const int64_t *__restrict__ ids, int64_t ids_stride, int len, int P,
     int64_t k, int64_t *__restrict__ out_ids, float *__restrict__ out_vals) {
   extern __shared__ uint64_t s_keys[];
-  __shared__ uint32_t s_hist[256];
-  __shared__ int s_tot[4];
-  __shared__ uint32_t s_bcast[3];
+  __shared__ uint32_t s_hist[512];
+  __shared__ uint32_t s_bcast[8];
   __shared__ uint32_t s_counter;
   const int row = blockIdx.x;
   const int tid = threadIdx.x;
@@ -459,13 +541,12 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
   for (int i = tid; i < (P < 1024 ? 1024 : P); i += kTopkThreads) s_keys[i] = 0ull;
   uint64_t prefix;
   int shift;
-  radix_select_regs<EIN>(v, (uint32_t)k, s_hist, s_tot, s_bcast, prefix, shift);
+  radix_select_regs<EIN>(v, (uint32_t)k, s_hist, s_bcast, prefix, shift);
 #pragma unroll
   for (int e = 0; e < EIN; ++e) {
-    if ((v[e] >> shift) >= (prefix >> shift) && v[e] != 0ull) {
-      const uint32_t slot = atomicAdd(&s_counter, 1u);
-      if (slot < (uint32_t)k) s_keys[slot] = v[e];
-    }
+    const bool win = (v[e] >> shift) >= (prefix >> shift) && v[e] != 0ull;
+    const uint32_t slot = wave_take_slots(&s_counter, win);
+    if (win && slot < (uint32_t)k) s_keys[slot] = v[e];
   }
   __syncthreads();
   int64_t *oi = out_ids + (int64_t)row * k;
@@ -475,58 +556,29 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
 #undef PKV_SORT_K
 }
 
-// len > 8192, k <= 8192: eight 8-bit MSB-first radix passes find the k-th
-// largest 64-bit key exactly, the k winners are collected into LDS and sorted.
+// len > 8192, k <= 8192: 8-bit MSB-first radix passes over the row find the k winners
+// exactly; they are collected into LDS and sorted.
 __global__ __launch_bounds__(kTopkThreads) void pkv_topk_radix_kernel(const float *__restrict__ x, int64_t x_stride,
                                                                       const int64_t *__restrict__ ids,
                                                                       int64_t ids_stride, int64_t len, int P,
                                                                       int64_t k, int64_t *__restrict__ out_ids,
                                                                       float *__restrict__ out_vals) {
   extern __shared__ uint64_t s_keys[];
-  __shared__ uint32_t s_hist[257];
-  __shared__ uint32_t s_digit, s_need, s_counter;
+  __shared__ uint32_t s_hist[512];
+  __shared__ uint32_t s_bcast[8];
+  __shared__ uint32_t s_counter;
   const int row = blockIdx.x;
   const int tid = threadIdx.x;
   const float *xr = x + (int64_t)row * x_stride;
   const int64_t *ir = ids ? ids + (int64_t)row * ids_stride : nullptr;
+  auto key_of = [&](int64_t i) { return make_key(xr, ir, i); };
 
-  uint64_t prefix = 0;
-  uint32_t need = (uint32_t)k;
-  for (int pass = 0; pass < 8; ++pass) {
-    const int shift = 56 - 8 * pass;
-    if (tid < 257) s_hist[tid] = 0;
-    __syncthreads();
-    for (int64_t i = tid; i < len; i += kTopkThreads) {
-      const uint64_t key = make_key(xr, ir, i);
-      if (pass == 0 || (key >> (shift + 8)) == (prefix >> (shift + 8)))
-        atomicAdd(&s_hist[(uint32_t)(key >> shift) & 255u], 1u);
-    }
-    __syncthreads();
-    uint32_t suf = 0, suf_next = 0;
-    if (tid < 256) {
-      for (int d = tid + 1; d < 256; ++d) suf_next += s_hist[d];
-      suf = suf_next + s_hist[tid];
-    }
-    __syncthreads();
-    if (tid < 256 && suf >= need && suf_next < need) {
-      s_digit = (uint32_t)tid;
-      s_need = need - suf_next;
-    }
-    __syncthreads();
-    prefix |= (uint64_t)s_digit << shift;
-    need = s_need;
-  }
-  // prefix is now the k-th largest key
   if (tid == 0) s_counter = 0;
   for (int i = tid; i < (P < 1024 ? 1024 : P); i += kTopkThreads) s_keys[i] = 0ull;
-  __syncthreads();
-  for (int64_t i = tid; i < len; i += kTopkThreads) {
-    const uint64_t key = make_key(xr, ir, i);
-    if (key >= prefix) {
-      const uint32_t slot = atomicAdd(&s_counter, 1u);
-      if (slot < (uint32_t)k) s_keys[slot] = key;
-    }
-  }
+  uint64_t prefix;
+  int shift;
+  radix_select_streamed(key_of, len, (uint32_t)k, s_hist, s_bcast, prefix, shift);
+  collect_winners_streamed(key_of, len, (uint32_t)k, prefix, shift, &s_counter, s_keys);
   __syncthreads();
   int64_t *oi = out_ids + (int64_t)row * k;
   float *ov = out_vals ? out_vals + (int64_t)row * k : nullptr;
@@ -607,8 +659,9 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adaptive_topk_kernel(
     int64_t *__restrict__ adaptive_k, int64_t *__restrict__ topk_ids, float *__restrict__ ws_ben) {
   extern __shared__ uint64_t s_keys[];
   __shared__ float s_part[16];
-  __shared__ uint32_t s_hist[257];
-  __shared__ uint32_t s_digit, s_need, s_counter;
+  __shared__ uint32_t s_hist[512];
+  __shared__ uint32_t s_bcast[8];
+  __shared__ uint32_t s_counter;
   const int row = blockIdx.x;
   const int tid = threadIdx.x;
   const float *sll = sl_logits + (int64_t)row * sl_stride;
@@ -638,43 +691,14 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adaptive_topk_kernel(
   const float total = sl_benefit + block_tree_sum_1024(acc, s_part);
   __syncthreads();  // ben[] of this row is complete (written and read by this workgroup only)
 
-  // k_out-th largest (benefit, ~position) key
-  uint64_t prefix = 0;
-  uint32_t need = (uint32_t)k_out;
-  for (int pass = 0; pass < 8; ++pass) {
-    const int shift = 56 - 8 * pass;
-    if (tid < 257) s_hist[tid] = 0;
-    __syncthreads();
-    for (int64_t i = tid; i < n_cand; i += kTopkThreads) {
-      const uint64_t key = make_key(ben, nullptr, i);
-      if (pass == 0 || (key >> (shift + 8)) == (prefix >> (shift + 8)))
-        atomicAdd(&s_hist[(uint32_t)(key >> shift) & 255u], 1u);
-    }
-    __syncthreads();
-    uint32_t suf = 0, suf_next = 0;
-    if (tid < 256) {
-      for (int d = tid + 1; d < 256; ++d) suf_next += s_hist[d];
-      suf = suf_next + s_hist[tid];
-    }
-    __syncthreads();
-    if (tid < 256 && suf >= need && suf_next < need) {
-      s_digit = (uint32_t)tid;
-      s_need = need - suf_next;
-    }
-    __syncthreads();
-    prefix |= (uint64_t)s_digit << shift;
-    need = s_need;
-  }
+  // the k_out largest (benefit, ~position) keys
+  auto key_of = [&](int64_t i) { return make_key(ben, nullptr, i); };
   if (tid == 0) s_counter = 0;
   for (int i = tid; i < (P < 1024 ? 1024 : P); i += kTopkThreads) s_keys[i] = 0ull;
-  __syncthreads();
-  for (int64_t i = tid; i < n_cand; i += kTopkThreads) {
-    const uint64_t key = make_key(ben, nullptr, i);
-    if (key >= prefix) {
-      const uint32_t slot = atomicAdd(&s_counter, 1u);
-      if (slot < (uint32_t)k_out) s_keys[slot] = key;
-    }
-  }
+  uint64_t prefix;
+  int shift;
+  radix_select_streamed(key_of, n_cand, (uint32_t)k_out, s_hist, s_bcast, prefix, shift);
+  collect_winners_streamed(key_of, n_cand, (uint32_t)k_out, prefix, shift, &s_counter, s_keys);
   __syncthreads();
 #define PKV_SORT_K(E) sort_lds_keys_and_emit<E>(s_keys, 0, nullptr, nullptr, s_keys)
   PKV_DISPATCH_E(P, PKV_SORT_K);

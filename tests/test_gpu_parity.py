@@ -176,6 +176,32 @@ def test_update_cache_cnt_sliced_views(ops):
             assert np.array_equal(cnt[0, h].cpu().numpy(), ref)
 
 
+@pytest.mark.parametrize("layout", ["reference", "keymajor"])
+def test_collision_scan_histograms(ops, layout):
+    """Stand-alone scan from a ready table: u8 counts plus the per-chunk and per-row suffix histograms."""
+    bs, H, N = 2, 2, 9001
+    ids, counts, codebook = _collision_recipe(bs, H, N)
+    tiers = O.tier_counts(N, 0.3)
+    lut = np.stack([np.stack([O.tier_lut(ids[b, h].numpy(), counts[b, h].numpy(), tiers) for h in range(H)])
+                    for b in range(bs)])
+    cb = codebook.to(DEV)
+    if layout == "keymajor":
+        cb = cb.permute(0, 1, 3, 2).contiguous().permute(0, 1, 3, 2)
+    cnt, (row_suf, chunk_suf), chunk = ops.collision_scan(cb, torch.from_numpy(lut).to(DEV), torch.uint8, want_hist=True)
+    torch.cuda.synchronize()
+    n_chunks = (N + chunk - 1) // chunk
+    for b in range(bs):
+        for h in range(H):
+            r = b * H + h
+            ref = O.collision_count(np.ascontiguousarray(codebook[b, h].numpy().T), lut[b, h])
+            assert np.array_equal(cnt[b, h].cpu().numpy(), ref.astype(np.uint8))
+            suf = lambda x: np.cumsum(np.bincount(x, minlength=128)[::-1])[::-1]
+            assert np.array_equal(row_suf[r].cpu().numpy(), suf(ref))
+            got = chunk_suf[r].cpu().numpy().astype(np.int64) & 0xFFFF
+            for c in range(n_chunks):
+                assert np.array_equal(got[c], suf(ref[c * chunk:(c + 1) * chunk]))
+
+
 def test_update_cache_cnt_legacy(ops):
     from pariskv_amd.cache_hub.collision.collision import update_cache_cnt_cuda
 
