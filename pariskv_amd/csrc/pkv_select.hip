@@ -17,8 +17,32 @@
 namespace {
 
 constexpr int kSelThreads = 256;
-constexpr int kSelKeysPerThread = 8;
-constexpr int kSelKeysPerIter = kSelThreads * kSelKeysPerThread;  // 2048
+constexpr int kSelKeysPerThread = 16;                                  // one 128-bit load of counts
+constexpr int kSelKeysPerIter = kSelThreads * kSelKeysPerThread;  // 4096
+
+// 16 one-byte counts (all <= 127) against the threshold, four at a time: adding 127 - theta
+// (128 - theta) to a byte sets its top bit exactly when the count is above (at or above) theta, and no
+// byte overflows into its neighbour.  Bit 8b + 7 of gt[d] / eq[d] stands for key 4d + b; only the
+// first n_valid keys count.
+__device__ __forceinline__ void count_masks16(const pkv_u32x4 w, uint32_t theta, int64_t n_valid, uint32_t (&gt)[4],
+                                              uint32_t (&eq)[4]) {
+  const uint32_t kgt = (127u - theta) * 0x01010101u, kge = (128u - theta) * 0x01010101u;
+  const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const int64_t left = n_valid - 4 * d;
+    const uint32_t vm = left >= 4 ? 0x80808080u : (left <= 0 ? 0u : (0x80808080u >> (8 * (4 - (int)left))));
+    const uint32_t v7 = ww[d] & 0x7f7f7f7fu;
+    const uint32_t g = (v7 + kgt) & vm;
+    const uint32_t ge = (v7 + kge) & vm;
+    gt[d] = g;
+    eq[d] = ge & ~g;
+  }
+}
+
+__device__ __forceinline__ int popc4(const uint32_t (&m)[4]) {
+  return __popc(m[0]) + __popc(m[1]) + __popc(m[2]) + __popc(m[3]);
+}
 
 // Threshold and output offsets of one workgroup from the suffix histograms the collision scan leaves
 // behind: row_suf[row][t] = keys of the row with count >= t (summed over chunks with atomics),
@@ -74,8 +98,8 @@ __device__ __forceinline__ void select_prologue(const uint32_t *__restrict__ row
   base_eq = (int64_t)s_ngt + eq;
 }
 
-// grid (n_chunks, rows).  cnt rows are padded to a multiple of 16 bytes and
-// 16-byte aligned, so every thread's 8 counts are one aligned 64-bit load.
+// grid (n_chunks, rows).  cnt rows are padded to a multiple of 16 bytes and 16-byte aligned, so every
+// thread's 16 counts are one aligned 128-bit load (issued before the threshold is known).
 __global__ __launch_bounds__(kSelThreads) void pkv_select_kernel(const uint8_t *__restrict__ cnt,
                                                                  int64_t cnt_stride,
                                                                  const uint32_t *__restrict__ row_suf,
@@ -86,41 +110,43 @@ __global__ __launch_bounds__(kSelThreads) void pkv_select_kernel(const uint8_t *
   const int chunk = blockIdx.x;
   const int tid = threadIdx.x;
   __shared__ int s_scan[2][kSelThreads / PKV_WAVE];
+  const uint8_t *crow = cnt + (int64_t)row * cnt_stride;
+  const int64_t chunk_begin = (int64_t)chunk * chunk_keys;
+  const int64_t chunk_end = (chunk_begin + chunk_keys < n_keys) ? chunk_begin + chunk_keys : n_keys;
+  const pkv_u32x4 zero4 = {0u, 0u, 0u, 0u};
+  int64_t i0 = chunk_begin + (int64_t)tid * kSelKeysPerThread;
+  pkv_u32x4 w = i0 < chunk_end ? *(const pkv_u32x4 *)(crow + i0) : zero4;  // padded rows: always in bounds
+
   uint32_t theta;
   int64_t base_gt, base_eq;
   select_prologue(row_suf, chunk_suf, row, chunk, gridDim.x, k, theta, base_gt, base_eq);
   int64_t *orow = out + (int64_t)row * k;
-  const uint8_t *crow = cnt + (int64_t)row * cnt_stride;
 
-  const int64_t chunk_begin = (int64_t)chunk * chunk_keys;
-  const int64_t chunk_end = (chunk_begin + chunk_keys < n_keys) ? chunk_begin + chunk_keys : n_keys;
   int it = 0;
   for (int64_t blk0 = chunk_begin; blk0 < chunk_end; blk0 += kSelKeysPerIter, ++it) {
-    const int64_t i0 = blk0 + (int64_t)tid * kSelKeysPerThread;
-    uint32_t gt_mask = 0, eq_mask = 0;
-    if (i0 < chunk_end) {
-      const pkv_u32x2 w = *(const pkv_u32x2 *)(crow + i0);  // padded rows: always in bounds
-      const uint32_t ww[2] = {w.x, w.y};
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const uint32_t v = (ww[j >> 2] >> (8 * (j & 3))) & 0xffu;
-        const bool valid = i0 + j < chunk_end;
-        gt_mask |= (valid && v > theta) ? (1u << j) : 0u;
-        eq_mask |= (valid && v == theta) ? (1u << j) : 0u;
-      }
-    }
-    const int packed = __popc(gt_mask) | (__popc(eq_mask) << 16);
+    uint32_t gt[4], eq[4];
+    count_masks16(w, theta, chunk_end - i0, gt, eq);
+    const int64_t i_cur = i0;
+    i0 += kSelKeysPerIter;
+    if (blk0 + kSelKeysPerIter < chunk_end) w = i0 < chunk_end ? *(const pkv_u32x4 *)(crow + i0) : zero4;
+    const int packed = popc4(gt) | (popc4(eq) << 16);
     int total;
     const int excl = pkv_block_excl_scan<kSelThreads>(packed, s_scan[it & 1], total);
     int64_t pg = base_gt + (excl & 0xffff);
     int64_t pe = base_eq + (excl >> 16);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      if (gt_mask & (1u << j)) {
-        if (pg < k) orow[pg] = i0 + j;
+    for (int d = 0; d < 4; ++d) {
+      uint32_t g = gt[d], e = eq[d];
+      while (g) {
+        const int bit = __ffs((int)g) - 1;
+        g &= g - 1;
+        if (pg < k) orow[pg] = i_cur + 4 * d + (bit >> 3);
         ++pg;
-      } else if (eq_mask & (1u << j)) {
-        if (pe < k) orow[pe] = i0 + j;
+      }
+      while (e) {
+        const int bit = __ffs((int)e) - 1;
+        e &= e - 1;
+        if (pe < k) orow[pe] = i_cur + 4 * d + (bit >> 3);
         ++pe;
       }
     }
@@ -146,8 +172,15 @@ __global__ __launch_bounds__(kSelThreads) void pkv_select_rerank_kernel(
 
   __shared__ int s_scan[2][kSelThreads / PKV_WAVE];
   __shared__ float s_prod[128 * 16];
-  __shared__ uint16_t s_list_key[kSelKeysPerIter];  // offset of the key inside the iteration's 2048-key block
+  __shared__ uint16_t s_list_key[kSelKeysPerIter];  // offset of the key inside the iteration's 4096-key block
   __shared__ int32_t s_list_pos[kSelKeysPerIter];   // output position, -1 = dropped tie
+
+  const uint8_t *crow = cnt + (int64_t)row * cnt_stride;
+  const int64_t chunk_begin = (int64_t)chunk * chunk_keys;
+  const int64_t chunk_end = (chunk_begin + chunk_keys < n_keys) ? chunk_begin + chunk_keys : n_keys;
+  const pkv_u32x4 zero4 = {0u, 0u, 0u, 0u};
+  int64_t i0 = chunk_begin + (int64_t)tid * kSelKeysPerThread;
+  pkv_u32x4 w = i0 < chunk_end ? *(const pkv_u32x4 *)(crow + i0) : zero4;  // before the threshold is known
 
   pkv_build_prod_table<kSelThreads>(s_prod, qhat + (int64_t)row * 128, centers);
   const float qn = qnorm[row];
@@ -156,28 +189,16 @@ __global__ __launch_bounds__(kSelThreads) void pkv_select_rerank_kernel(
   select_prologue(row_suf, chunk_suf, row, chunk, gridDim.x, k, theta, base_gt, base_eq);
   int64_t *orow = out + (int64_t)row * k;
   float *srow = scores + (int64_t)row * k;
-  const uint8_t *crow = cnt + (int64_t)row * cnt_stride;
   const uint8_t *nrow = nib + (int64_t)b * ns_b + (int64_t)h * ns_h;
   const uint16_t *wrow = weight + (int64_t)b * ws_b + (int64_t)h * ws_h;
 
-  const int64_t chunk_begin = (int64_t)chunk * chunk_keys;
-  const int64_t chunk_end = (chunk_begin + chunk_keys < n_keys) ? chunk_begin + chunk_keys : n_keys;
   int it = 0;
   for (int64_t blk0 = chunk_begin; blk0 < chunk_end; blk0 += kSelKeysPerIter, ++it) {
-    const int64_t i0 = blk0 + (int64_t)tid * kSelKeysPerThread;
-    uint32_t gt_mask = 0, eq_mask = 0;
-    if (i0 < chunk_end) {
-      const pkv_u32x2 w = *(const pkv_u32x2 *)(crow + i0);
-      const uint32_t ww[2] = {w.x, w.y};
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const uint32_t v = (ww[j >> 2] >> (8 * (j & 3))) & 0xffu;
-        const bool valid = i0 + j < chunk_end;
-        gt_mask |= (valid && v > theta) ? (1u << j) : 0u;
-        eq_mask |= (valid && v == theta) ? (1u << j) : 0u;
-      }
-    }
-    const int packed = __popc(gt_mask) | (__popc(eq_mask) << 16);
+    uint32_t gt[4], eq[4];
+    count_masks16(w, theta, chunk_end - i0, gt, eq);
+    i0 += kSelKeysPerIter;
+    if (blk0 + kSelKeysPerIter < chunk_end) w = i0 < chunk_end ? *(const pkv_u32x4 *)(crow + i0) : zero4;
+    const int packed = popc4(gt) | (popc4(eq) << 16);
     int total;
     const int excl = pkv_block_excl_scan<kSelThreads>(packed, s_scan[it & 1], total);
     const int n_gt_it = total & 0xffff, n_sel_it = n_gt_it + (total >> 16);
@@ -186,13 +207,19 @@ __global__ __launch_bounds__(kSelThreads) void pkv_select_rerank_kernel(
     int lg = excl & 0xffff;            // slot in this iteration's LDS list: strictly-above keys first,
     int le = n_gt_it + (excl >> 16);   // then the keys at the threshold
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      if (gt_mask & (1u << j)) {
-        s_list_key[lg] = (uint16_t)(tid * kSelKeysPerThread + j);
+    for (int d = 0; d < 4; ++d) {
+      uint32_t g = gt[d], e = eq[d];
+      while (g) {
+        const int bit = __ffs((int)g) - 1;
+        g &= g - 1;
+        s_list_key[lg] = (uint16_t)(tid * kSelKeysPerThread + 4 * d + (bit >> 3));
         s_list_pos[lg] = pg < k ? (int32_t)pg : -1;
         ++lg, ++pg;
-      } else if (eq_mask & (1u << j)) {
-        s_list_key[le] = (uint16_t)(tid * kSelKeysPerThread + j);
+      }
+      while (e) {
+        const int bit = __ffs((int)e) - 1;
+        e &= e - 1;
+        s_list_key[le] = (uint16_t)(tid * kSelKeysPerThread + 4 * d + (bit >> 3));
         s_list_pos[le] = pe < k ? (int32_t)pe : -1;
         ++le, ++pe;
       }
@@ -273,12 +300,11 @@ __device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int mask) {
   }
 }
 
-// hist[d] += 1 for every active lane.  Lanes of a wave that share the leading lane's digit are added
-// with one atomic (two rounds), which is what keeps the first radix passes, where nearly all keys
-// fall into one or two buckets, from serialising on a single LDS address.
-__device__ __forceinline__ void wave_hist_add(uint32_t *hist, uint32_t d, bool active) {
-#pragma unroll
-  for (int r = 0; r < 2; ++r) {
+// hist[d] += 1 for every active lane.  In each of `rounds` rounds the lanes of a wave that share the
+// leading lane's digit are added with one atomic, which is what keeps the first radix passes, where
+// nearly all keys fall into one or two buckets, from serialising on a single LDS address.
+__device__ __forceinline__ void wave_hist_add(uint32_t *hist, uint32_t d, bool active, int rounds) {
+  for (int r = 0; r < rounds; ++r) {
     const uint64_t act = __ballot(active);
     if (act == 0) return;
     const int leader = __ffsll((long long)act) - 1;
@@ -302,86 +328,101 @@ __device__ __forceinline__ uint32_t wave_take_slots(uint32_t *counter, bool take
   return base + (uint32_t)__popcll((long long)below);
 }
 
-// Descending bitonic sort of 1024*E 64-bit keys held E per thread (thread t owns sorted positions
-// t*E .. t*E+E-1).  Strides below E are exchanged inside the thread, strides below 64*E between the
-// lanes of a wave (no barrier), only the remaining strides go through LDS (`s_buf`, 1024*E keys,
-// laid out [e][thread] so that a wave touches consecutive addresses).  For 4096 keys that is 10
-// barrier-separated exchanges instead of 78.
-template <int E>
+// Descending bitonic sort of NT*E 64-bit keys held E per thread by the first NT threads of the
+// 1024-thread workgroup (thread t owns sorted positions t*E .. t*E+E-1); ALL 1024 threads must call it,
+// the others only take part in the barriers.  Strides below E are exchanged inside the thread, strides
+// below 64*E between the lanes of a wave (no barrier), only the remaining strides go through LDS
+// (`s_buf`, NT*E keys, laid out [e][thread] so that a wave touches consecutive addresses).
+template <int NT, int E>
 __device__ __forceinline__ void bitonic_sort_desc_regs(uint64_t (&v)[E], uint64_t *s_buf) {
-  constexpr int P = kTopkThreads * E;
+  constexpr int P = NT * E;
   const int tid = threadIdx.x;
+  const bool active = tid < NT;
 #pragma unroll
   for (int size = 2; size <= P; size <<= 1) {
 #pragma unroll
     for (int stride = size >> 1; stride > 0; stride >>= 1) {
       if (stride < E) {
+        if (active) {
 #pragma unroll
-        for (int e = 0; e < E; ++e) {
-          if ((e & stride) == 0) {
-            const bool desc = ((tid * E + e) & size) == 0;
-            const uint64_t a = v[e], b = v[e | stride];
-            const bool sw = desc ? (a < b) : (a > b);
-            v[e] = sw ? b : a;
-            v[e | stride] = sw ? a : b;
+          for (int e = 0; e < E; ++e) {
+            if ((e & stride) == 0) {
+              const bool desc = ((tid * E + e) & size) == 0;
+              const uint64_t a = v[e], b = v[e | stride];
+              const bool sw = desc ? (a < b) : (a > b);
+              v[e] = sw ? b : a;
+              v[e | stride] = sw ? a : b;
+            }
           }
         }
       } else if (stride < PKV_WAVE * E) {
+        if (active) {  // whole waves: NT is a multiple of 64
 #pragma unroll
-        for (int e = 0; e < E; ++e) {
-          const int i = tid * E + e;
-          const uint64_t o = shfl_xor_u64(v[e], stride / E);
-          const bool want_max = ((i & stride) == 0) == ((i & size) == 0);
-          v[e] = want_max ? (v[e] > o ? v[e] : o) : (v[e] < o ? v[e] : o);
+          for (int e = 0; e < E; ++e) {
+            const int i = tid * E + e;
+            const uint64_t o = shfl_xor_u64(v[e], stride / E);
+            const bool want_max = ((i & stride) == 0) == ((i & size) == 0);
+            v[e] = ((v[e] > o) == want_max) ? v[e] : o;  // keys are distinct (or both zero padding)
+          }
         }
       } else {
         __syncthreads();  // earlier readers of s_buf are done
+        if (active) {
 #pragma unroll
-        for (int e = 0; e < E; ++e) s_buf[e * kTopkThreads + tid] = v[e];
+          for (int e = 0; e < E; ++e) s_buf[e * NT + tid] = v[e];
+        }
         __syncthreads();
+        if (active) {
 #pragma unroll
-        for (int e = 0; e < E; ++e) {
-          const int i = tid * E + e;
-          const uint64_t o = s_buf[e * kTopkThreads + (tid ^ (stride / E))];
-          const bool want_max = ((i & stride) == 0) == ((i & size) == 0);
-          v[e] = want_max ? (v[e] > o ? v[e] : o) : (v[e] < o ? v[e] : o);
+          for (int e = 0; e < E; ++e) {
+            const int i = tid * E + e;
+            const uint64_t o = s_buf[e * NT + (tid ^ (stride / E))];
+            const bool want_max = ((i & stride) == 0) == ((i & size) == 0);
+            v[e] = ((v[e] > o) == want_max) ? v[e] : o;
+          }
         }
       }
     }
   }
 }
 
-// Sort the n_valid (<= 1024*E) keys in s_keys[0 .. 1024*E) (zero padded) and emit the first k.
-template <int E>
+// Sort the keys in s_keys[0 .. NT*E) (zero padded) and emit the first k.  Called by all 1024 threads.
+template <int NT, int E>
 __device__ __forceinline__ void sort_lds_keys_and_emit(uint64_t *s_keys, int64_t k, int64_t *__restrict__ out_ids,
                                                        float *__restrict__ out_vals, uint64_t *sorted_copy) {
+  const bool active = threadIdx.x < NT;
   uint64_t v[E];
 #pragma unroll
-  for (int e = 0; e < E; ++e) v[e] = s_keys[threadIdx.x * E + e];
+  for (int e = 0; e < E; ++e) v[e] = active ? s_keys[threadIdx.x * E + e] : 0ull;
   __syncthreads();
-  bitonic_sort_desc_regs<E>(v, s_keys);
+  bitonic_sort_desc_regs<NT, E>(v, s_keys);
 #pragma unroll
   for (int e = 0; e < E; ++e) {
     const int64_t i = (int64_t)threadIdx.x * E + e;
-    if (i < k) {
+    if (active && i < k) {
       out_ids[i] = (int64_t)(uint32_t)(~(uint32_t)v[e]);
       if (out_vals) out_vals[i] = pkv_from_ordered_u32((uint32_t)(v[e] >> 32));
     }
   }
   if (sorted_copy) {  // the caller wants the sorted keys back in LDS
     __syncthreads();
+    if (active) {
 #pragma unroll
-    for (int e = 0; e < E; ++e) sorted_copy[threadIdx.x * E + e] = v[e];
+      for (int e = 0; e < E; ++e) sorted_copy[threadIdx.x * E + e] = v[e];
+    }
     __syncthreads();
   }
 }
 
-#define PKV_DISPATCH_E(P, CALL)            \
-  do {                                     \
-    if ((P) <= 1024) { CALL(1); }          \
-    else if ((P) == 2048) { CALL(2); }     \
-    else if ((P) == 4096) { CALL(4); }     \
-    else { CALL(8); }                      \
+// P keys (a power of two, at least 1024 slots in LDS): threads x keys per thread.  All 1024 threads
+// with few keys each measured faster than fewer threads with more (1024 keys: 11.9 us per launch on
+// 1024 threads, 12.3 on 512, 13.5 on 256): the compare-exchanges are issue-bound on the one CU.
+#define PKV_DISPATCH_E(P, CALL)               \
+  do {                                        \
+    if ((P) <= 1024) { CALL(1024, 1); }       \
+    else if ((P) == 2048) { CALL(1024, 2); }  \
+    else if ((P) == 4096) { CALL(1024, 4); }  \
+    else { CALL(1024, 8); }                   \
   } while (0)
 
 // len <= 8192: sort everything.  One workgroup per row, dynamic LDS max(P,1024)*8 bytes.
@@ -396,17 +437,17 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_sort_kernel(const float
   const int64_t *ir = ids ? ids + (int64_t)row * ids_stride : nullptr;
   int64_t *oi = out_ids + (int64_t)row * k;
   float *ov = out_vals ? out_vals + (int64_t)row * k : nullptr;
-#define PKV_SORT_ALL(E)                                                            \
+#define PKV_SORT_ALL(NT, E)                                                        \
   {                                                                                \
     uint64_t v[E];                                                                 \
     _Pragma("unroll") for (int e = 0; e < E; ++e) {                                \
       const int i = threadIdx.x * E + e;                                           \
-      v[e] = i < len ? make_key(xr, ir, i) : 0ull;                                 \
+      v[e] = (threadIdx.x < NT && i < len) ? make_key(xr, ir, i) : 0ull;           \
     }                                                                              \
-    bitonic_sort_desc_regs<E>(v, s_keys);                                          \
+    bitonic_sort_desc_regs<NT, E>(v, s_keys);                                      \
     _Pragma("unroll") for (int e = 0; e < E; ++e) {                                \
       const int64_t i = (int64_t)threadIdx.x * E + e;                              \
-      if (i < k) {                                                                 \
+      if (threadIdx.x < NT && i < k) {                                             \
         oi[i] = (int64_t)(uint32_t)(~(uint32_t)v[e]);                              \
         if (ov) ov[i] = pkv_from_ordered_u32((uint32_t)(v[e] >> 32));              \
       }                                                                            \
@@ -414,6 +455,21 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_sort_kernel(const float
   }
   PKV_DISPATCH_E(P, PKV_SORT_ALL);
 #undef PKV_SORT_ALL
+}
+
+// Digit of `key` in radix pass `pass` (8 bits, most significant first) and whether the key still
+// matches the prefix found by the earlier passes; works on the 32-bit halves of the key.
+__device__ __forceinline__ void radix_digit(uint64_t key, uint64_t prefix, int pass, uint32_t &digit, bool &match) {
+  const uint32_t hi = (uint32_t)(key >> 32), lo = (uint32_t)key;
+  const uint32_t phi = (uint32_t)(prefix >> 32), plo = (uint32_t)prefix;
+  const int sh = 24 - 8 * (pass & 3);
+  if (pass < 4) {
+    digit = (hi >> sh) & 255u;
+    match = pass == 0 || (hi >> (sh + 8)) == (phi >> (sh + 8));
+  } else {
+    digit = (lo >> sh) & 255u;
+    match = hi == phi && (pass == 4 || (lo >> (sh + 8)) == (plo >> (sh + 8)));
+  }
 }
 
 // Second half of a radix-select pass, called by all 1024 threads after their histogram atomics: the
@@ -464,9 +520,12 @@ __device__ __forceinline__ void radix_select_regs(const uint64_t (&v)[EIN], uint
     uint32_t *hist = s_hist + (pass & 1) * 256;
     uint32_t *res = s_bcast + (pass & 1) * 4;
 #pragma unroll
-    for (int e = 0; e < EIN; ++e)
-      wave_hist_add(hist, (uint32_t)(v[e] >> shift) & 255u,
-                    pass == 0 || (v[e] >> (shift + 8)) == (prefix >> (shift + 8)));
+    for (int e = 0; e < EIN; ++e) {
+      uint32_t digit;
+      bool match;
+      radix_digit(v[e], prefix, pass, digit, match);
+      wave_hist_add(hist, digit, match, pass < 2 ? 2 : 0);
+    }
     radix_pass_decide(s_hist, s_bcast, pass, need);
     prefix |= (uint64_t)res[0] << shift;
     need = res[1];
@@ -493,8 +552,10 @@ __device__ __forceinline__ void radix_select_streamed(KeyFn key_of, int64_t len,
     for (int64_t i0 = 0; i0 < len; i0 += kTopkThreads) {  // whole waves stay in the loop: it uses ballots
       const int64_t i = i0 + tid;
       const uint64_t key = i < len ? key_of(i) : 0ull;
-      wave_hist_add(hist, (uint32_t)(key >> shift) & 255u,
-                    i < len && (pass == 0 || (key >> (shift + 8)) == (prefix >> (shift + 8))));
+      uint32_t digit;
+      bool match;
+      radix_digit(key, prefix, pass, digit, match);
+      wave_hist_add(hist, digit, i < len && match, pass < 2 ? 2 : 0);
     }
     radix_pass_decide(s_hist, s_bcast, pass, need);
     prefix |= (uint64_t)res[0] << shift;
@@ -551,7 +612,7 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
   __syncthreads();
   int64_t *oi = out_ids + (int64_t)row * k;
   float *ov = out_vals ? out_vals + (int64_t)row * k : nullptr;
-#define PKV_SORT_K(E) sort_lds_keys_and_emit<E>(s_keys, k, oi, ov, nullptr)
+#define PKV_SORT_K(NT, E) sort_lds_keys_and_emit<NT, E>(s_keys, k, oi, ov, nullptr)
   PKV_DISPATCH_E(P, PKV_SORT_K);
 #undef PKV_SORT_K
 }
@@ -582,7 +643,7 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_radix_kernel(const floa
   __syncthreads();
   int64_t *oi = out_ids + (int64_t)row * k;
   float *ov = out_vals ? out_vals + (int64_t)row * k : nullptr;
-#define PKV_SORT_K(E) sort_lds_keys_and_emit<E>(s_keys, k, oi, ov, nullptr)
+#define PKV_SORT_K(NT, E) sort_lds_keys_and_emit<NT, E>(s_keys, k, oi, ov, nullptr)
   PKV_DISPATCH_E(P, PKV_SORT_K);
 #undef PKV_SORT_K
 }
@@ -700,7 +761,7 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adaptive_topk_kernel(
   radix_select_streamed(key_of, n_cand, (uint32_t)k_out, s_hist, s_bcast, prefix, shift);
   collect_winners_streamed(key_of, n_cand, (uint32_t)k_out, prefix, shift, &s_counter, s_keys);
   __syncthreads();
-#define PKV_SORT_K(E) sort_lds_keys_and_emit<E>(s_keys, 0, nullptr, nullptr, s_keys)
+#define PKV_SORT_K(NT, E) sort_lds_keys_and_emit<NT, E>(s_keys, 0, nullptr, nullptr, s_keys)
   PKV_DISPATCH_E(P, PKV_SORT_K);
 #undef PKV_SORT_K
 
