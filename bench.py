@@ -32,7 +32,7 @@ TIER_RATIOS = (0.05, 0.15, 0.30, 0.50, 0.75, 1.0)
 
 # HBM bytes moved by one collision-scan launch at this workload, from the two
 # rocprofv3 --pmc runs summarised in profiles/ (None until measured).
-SCAN_TRAFFIC_BYTES = 72676000  # profiles/scan_cfg3_hbm_traffic.md
+SCAN_TRAFFIC_BYTES = 72834000  # profiles/scan_cfg3_hbm_traffic.md
 
 
 def main():
