@@ -161,6 +161,15 @@ def main():
     step(0)
     us_gather = timed(gather_only, max(8, args.steps // 4))
 
+    # the attention that consumes the gathered rows (reported beside the metric, not part of it):
+    # sink 64 + local 512 dense rows in HBM plus the K gathered rows, GQA 4, one query token
+    dense_k = torch.randn(bs, H, 576, D, device=dev).to(torch.bfloat16)
+    dense_v = torch.randn(bs, H, 576, D, device=dev).to(torch.bfloat16)
+    att = ops.DecodeAttention(bs, H, G, 576 + K, dev)
+    att_out = torch.empty(bs, 1, H * G, D, dtype=torch.bfloat16, device=dev)
+    att_segs = [(dense_k, dense_v, 0, 64), (dst_k, dst_v, 0, K), (dense_k, dense_v, 64, 512)]
+    us_attn = timed(lambda i: att.run(layers[i % L]["q"], att_segs, out=att_out), args.steps)
+
     # dominant kernel: the collision scan, timed by its own begin/end timestamps
     kus = C.c_float()
     scan_us = []
@@ -196,7 +205,8 @@ def main():
                                f"(UVA gather), {L} rotating layers",
                    "rows": R, "keys_per_row": N, "candidates": Cn, "topk": K, "collision_ratio": 0.2},
         "stages_us": {"full_retrieval_with_uva_gather": round(us_step, 2), "on_gpu_stages": round(us_gpu, 2),
-                      "uva_gather_alone": round(us_gather, 2)},
+                      "uva_gather_alone": round(us_gather, 2),
+                      "decode_attention_over_gathered_set": round(us_attn, 2)},
         "hbm_fraction_on_gpu_stages": round(a_hbm / (us_gpu * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
         "algorithmic_bytes": {"hbm_per_step": a_hbm, "pcie_per_step": a_pcie},
         "pcie_GBps_gather": round(a_pcie / (us_gather * 1e-6) / 1e9, 2),

@@ -262,6 +262,31 @@ int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, const float *sl
                       const int64_t *cand_ids, int64_t n_cand, float threshold, int64_t k_out, int rows,
                       int64_t *adaptive_k, int64_t *topk_ids, void *ws, size_t ws_bytes, void *stream);
 
+/* --------------------------------------------------------- decode attention */
+
+#define PKV_ATTN_MAX_SEGMENTS 4
+
+/* One run of consecutive K/V rows (head_dim 128, rows contiguous: 128 elements
+ * apart) inside tensors laid out [bs][n_kv_heads][rows][128]; strides in
+ * elements.  Rows row0 .. row0+n_rows-1 of every (b, h) take part. */
+typedef struct pkv_attn_segment {
+  const void *k, *v;
+  int64_t stride_b, stride_h;
+  int64_t row0, n_rows;
+} pkv_attn_segment;
+
+/* Replaces the torch.cat of sink / top-k / local K and V followed by
+ * flash_attn_func (cache_hub/polar_cache.py:1084-1105): softmax(q k^T * scale) v
+ * for one query token per sequence, non-causal, over the concatenation of up to
+ * PKV_ATTN_MAX_SEGMENTS segments read in place.  q, out: [bs][n_kv_heads*group][128]
+ * in `dtype` (query head h*group+g attends with KV head h); 1 <= group <= 8.
+ * ws: pkv_decode_attention_ws_bytes(...) bytes of device memory for the
+ * per-split partial results.  fp32 accumulation; result rounded to `dtype`. */
+size_t pkv_decode_attention_ws_bytes(int bs, int n_kv_heads, int group, int64_t total_keys);
+int pkv_decode_attention(const void *q, int dtype, int bs, int n_kv_heads, int group,
+                         const pkv_attn_segment *segments, int n_segments, float scale,
+                         void *out, void *ws, size_t ws_bytes, void *stream);
+
 /* ------------------------------------------------------- fused decode step */
 
 /* One layer's retrieval for one decode step, key-major storage:

@@ -306,6 +306,31 @@ void pkv_o_gather_rows(const void *src, const int64_t *idx, int64_t k, int64_t r
     memcpy((char *)dst + i * row_bytes, (const char *)src + idx[i] * row_bytes, (size_t)row_bytes);
 }
 
+/* --------------------------------------------------------- dense attention */
+
+void pkv_o_attention(const float *q, int g_heads, const float *k, const float *v, int64_t s,
+                     float scale, float *out) {
+  double *logit = (double *)malloc(sizeof(double) * (size_t)(s > 0 ? s : 1));
+  for (int g = 0; g < g_heads; ++g) {
+    double mx = -INFINITY;
+    for (int64_t i = 0; i < s; ++i) {
+      double acc = 0.0;
+      for (int d = 0; d < PKV_O_D; ++d) acc += (double)q[g * PKV_O_D + d] * (double)k[i * PKV_O_D + d];
+      logit[i] = acc * (double)scale;
+      if (logit[i] > mx) mx = logit[i];
+    }
+    double den = 0.0, o[PKV_O_D];
+    for (int d = 0; d < PKV_O_D; ++d) o[d] = 0.0;
+    for (int64_t i = 0; i < s; ++i) {
+      const double p = exp(logit[i] - mx);
+      den += p;
+      for (int d = 0; d < PKV_O_D; ++d) o[d] += p * (double)v[i * PKV_O_D + d];
+    }
+    for (int d = 0; d < PKV_O_D; ++d) out[g * PKV_O_D + d] = (float)(o[d] / den);
+  }
+  free(logit);
+}
+
 /* --------------------------------------------------------------- adaptive-k */
 
 float pkv_o_expf(float x) {

@@ -104,6 +104,15 @@ void pkv_o_topk_f32(const float *scores, const int64_t *ids, int64_t n,
 
 /* gather_trans/trans_h2d.cu:38-74: dst[i][:] = src[idx[i]][:], rows of
  * row_bytes bytes. */
+/* Dense attention of one KV head on the gathered key set, polar_cache.py:1084-1105
+ * (flash_attn_func on the concatenated sink / top-k / local rows, non-causal,
+ * softmax scale 1/sqrt(128) by default): out[g] = softmax(q[g] . K^T * scale) V
+ * for the G query heads of the KV head.  q [G][128], k, v [S][128] fp32 (bf16
+ * inputs are passed as their exact fp32 values); accumulated in double; out [G][128]
+ * fp32, not rounded.  Pinned against torch's scaled_dot_product_attention. */
+void pkv_o_attention(const float *q, int g_heads, const float *k, const float *v, int64_t s,
+                     float scale, float *out);
+
 void pkv_o_gather_rows(const void *src, const int64_t *idx, int64_t k,
                        int64_t row_bytes, void *dst);
 

@@ -189,6 +189,16 @@ def gather_rows(src, idx):
     return dst
 
 
+def attention(q, k, v, scale=None):
+    """q [G,128], k, v [S,128] -> [G,128] fp32 (softmax(q k^T * scale) v, double accumulation)."""
+    q, k, v = _f32(q), _f32(k), _f32(v)
+    if scale is None:
+        scale = 1.0 / np.sqrt(128.0)
+    out = np.empty_like(q)
+    lib().pkv_o_attention(_p(q), C.c_int(q.shape[0]), _p(k), _p(v), C.c_int64(k.shape[0]), C.c_float(scale), _p(out))
+    return out
+
+
 def expf(x):
     x = _f32(x)
     out = np.empty_like(x)

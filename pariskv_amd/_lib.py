@@ -20,6 +20,12 @@ MAX_TIERS = 8
 _vp, _i, _i64, _sz = C.c_void_p, C.c_int, C.c_int64, C.c_size_t
 
 
+class AttnSegment(C.Structure):
+    """Mirror of ``pkv_attn_segment``."""
+
+    _fields_ = [("k", _vp), ("v", _vp), ("stride_b", _i64), ("stride_h", _i64), ("row0", _i64), ("n_rows", _i64)]
+
+
 class RetrieveArgs(C.Structure):
     """Mirror of ``pkv_retrieve_args``."""
 
@@ -72,6 +78,8 @@ PROTOTYPES = {
     "pkv_adaptive_topk_ws_bytes": (_sz, [_i, _i64, _i64]),
     "pkv_adaptive_topk": (_i, [_vp, _i64, _vp, _i64, _i64, _vp, _i, C.c_float, _vp, _vp, _i64, _i64, _vp, _i64,
                                C.c_float, _i64, _i, _vp, _vp, _vp, _sz, _vp]),
+    "pkv_decode_attention_ws_bytes": (_sz, [_i, _i, _i, _i64]),
+    "pkv_decode_attention": (_i, [_vp, _i, _i, _i, _i, C.POINTER(AttnSegment), _i, C.c_float, _vp, _vp, _sz, _vp]),
     "pkv_retrieve_ws_bytes": (_sz, [_i, _i64, _i64, _i64]),
     "pkv_retrieve": (_i, [C.POINTER(RetrieveArgs), _vp, _sz, _vp]),
     "pkv_retrieve_ws_view": (_i, [_vp, _i, _i64, _i64, _i64, C.c_char_p, C.POINTER(_vp), C.POINTER(_sz)]),

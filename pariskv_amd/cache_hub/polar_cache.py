@@ -21,7 +21,6 @@ import os
 from typing import Optional
 
 import torch
-import torch.nn.functional as F
 
 from .. import ops
 from .cache import KV_Cache
@@ -119,7 +118,7 @@ class polar_cache(KV_Cache):
             self.unified_keys_cpu = None
             self.unified_values_cpu = None
             self.cpu_valid_end = None
-            att_rows = sink_size + final_topk + local_size + I
+            att_rows = max(1, final_topk)  # the gathered top-k rows; sink and local window are attended in place
             self._attn_k = torch.zeros((bs, H, att_rows, D), dtype=dtype, device=dev)
             self._attn_v = torch.zeros((bs, H, att_rows, D), dtype=dtype, device=dev)
         self.unified_keys_gpu = [torch.zeros((bs, H, rows, D), dtype=dtype, device=dev) for _ in range(layer_num)]
@@ -142,6 +141,7 @@ class polar_cache(KV_Cache):
         max_cand = max(1, math.ceil(max_keys * 0.5))
         self._plan = ops.RetrievePlan(bs, H, self.group_size, cap, dev, max_keys, max_cand, max(1, min(final_topk, max_cand)))
         self._out_ids = torch.empty((bs, H, max(1, final_topk)), dtype=torch.int64, device=dev)
+        self._attention = ops.DecodeAttention(bs, H, self.group_size, self.unified_kv_capacity, dev)
         self.last_topk_indices = None  # [bs, H, K] of the most recent retrieval (zone-relative), for inspection
 
     # ------------------------------------------------------------- helpers
@@ -311,11 +311,10 @@ class polar_cache(KV_Cache):
     def _compute_local_start(self, layer_idx=0):
         return self._zones[layer_idx].local_start
 
-    def _attend(self, queries, k, v):
-        """softmax(q k^T / sqrt(D)) v over the gathered set; q [bs,1,Hq,D], k/v [bs,Hkv,S,D] (:1097-1105)."""
-        q = queries.transpose(1, 2)  # [bs, Hq, 1, D]
-        out = F.scaled_dot_product_attention(q, k, v, is_causal=False, enable_gqa=self.group_size > 1)
-        return out.transpose(1, 2).contiguous()
+    def _attend(self, queries, segments):
+        """softmax(q k^T / sqrt(D)) v over the attended set (:1097-1105).  queries [bs,1,Hq,D]; segments: list of
+        (k, v, row0, n_rows) runs of [bs,Hkv,rows,D] tensors, read in place by the HIP decode-attention kernel."""
+        return self._attention.run(queries, [s for s in segments if s[3] > 0])
 
     def _full_kv(self, layer_idx):
         """Dense fallback: every stored token (reference _get_full_kv_for_attention :701-737)."""
@@ -350,7 +349,9 @@ class polar_cache(KV_Cache):
         min_total = max(self.FULL_ATTENTION_THRESHOLD, self.sink_size + self.local_size + self.final_topk * 2)
         if total < min_total or n_keys <= 0:
             k, v = self._full_kv(layer_idx)
-            return self._attend(queries, k, v)
+            if not (k.stride(3) == 1 and k.stride(2) == self.head_dim and v.stride() == k.stride()):
+                k, v = k.contiguous(), v.contiguous()
+            return self._attend(queries.contiguous(), [(k, v, 0, k.shape[2])])
         n_keys, n_cand, topk, tiers = self.retrieval_shape(layer_idx)
         kg, vg = self.unified_keys_gpu[layer_idx], self.unified_values_gpu[layer_idx]
         q = queries.contiguous()
@@ -359,16 +360,11 @@ class polar_cache(KV_Cache):
             prefix = z.gpu_prefix_rows
             gather = dict(src_k=self.unified_keys_cpu[layer_idx], src_v=self.unified_values_cpu[layer_idx], from_host=True,
                           idx_offset=0, dst_k=kg, dst_v=vg, dst_row0=prefix)
-            att_k, att_v = kg[:, :, :prefix + topk], vg[:, :, :prefix + topk]
+            segments = [(kg, vg, 0, prefix + topk)]  # [sink | local + buffer | gathered top-k], one run
         else:
-            S0, tail = self.sink_size, z.dense_tail_len
             ak, av = self._attn_k, self._attn_v
-            ak[:, :, :S0] = kg[:, :, :S0]
-            av[:, :, :S0] = vg[:, :, :S0]
-            ak[:, :, S0 + topk:S0 + topk + tail] = kg[:, :, z.local_start:total]
-            av[:, :, S0 + topk:S0 + topk + tail] = vg[:, :, z.local_start:total]
-            gather = dict(src_k=kg, src_v=vg, from_host=False, idx_offset=self.sink_size, dst_k=ak, dst_v=av, dst_row0=S0)
-            att_k, att_v = ak[:, :, :S0 + topk + tail], av[:, :, :S0 + topk + tail]
+            gather = dict(src_k=kg, src_v=vg, from_host=False, idx_offset=self.sink_size, dst_k=ak, dst_v=av, dst_row0=0)
+            segments = [(kg, vg, 0, self.sink_size), (ak, av, 0, topk), (kg, vg, z.local_start, z.dense_tail_len)]
         out_ids = self._out_ids[:, :, :topk]
         if not out_ids.is_contiguous():
             out_ids = torch.empty((self.batch_size, self.kv_head, topk), dtype=torch.int64, device=self.device)
@@ -376,7 +372,7 @@ class polar_cache(KV_Cache):
                        self._nib_km[layer_idx], self._w_km[layer_idx], self.sink_size, n_keys, tiers, n_cand, topk,
                        out_ids=out_ids, gather=gather)
         self.last_topk_indices = out_ids
-        return self._attend(q, att_k, att_v)
+        return self._attend(q, segments)
 
     def sync(self, layer_idx, batch_idx):
         """No-op, as in the reference (:1310-1312)."""

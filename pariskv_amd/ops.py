@@ -12,6 +12,8 @@ from __future__ import annotations
 import ctypes as C
 from typing import Optional, Sequence
 
+import math
+
 import torch
 
 from . import _lib
@@ -377,6 +379,48 @@ def gather_uva_packed(src_k, src_v, k_packed, v_packed, indices_packed, cu_seqle
     _lib.check(_lib.lib().pkv_gather_uva_packed(
         _p(src_k), _p(src_v), src_len, _p(indices_packed), _p(cu_seqlens_topk), _p(cu_seqlens_k), sink_local_end,
         max(1, global_k), _p(k_packed), _p(v_packed), total_k, bs, H, D * src_k.element_size(), _stream(k_packed)))
+
+
+# --------------------------------------------------------- decode attention
+
+
+class DecodeAttention:
+    """softmax(q k^T * scale) v for one query token per sequence over up to four row segments of
+    [bs, Hkv, rows, 128] K/V tensors, read in place (cache_hub/polar_cache.py:1084-1105)."""
+
+    def __init__(self, bs: int, n_kv_heads: int, group: int, max_keys: int, device):
+        self.bs, self.H, self.G = bs, n_kv_heads, group
+        self.max_keys = max_keys
+        nbytes = _lib.lib().pkv_decode_attention_ws_bytes(bs, n_kv_heads, group, max(1, max_keys))
+        # the split count never exceeds 64, whatever the key count: size for that
+        nbytes = max(nbytes, bs * n_kv_heads * 64 * group * 130 * 4)
+        self.ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+    def run(self, queries: torch.Tensor, segments, scale: float = None, out: torch.Tensor = None) -> torch.Tensor:
+        """queries [bs,1,Hq,128] (or [bs,Hq,128]); segments: list of (k, v, row0, n_rows) with k, v
+        [bs,Hkv,rows,128] tensors whose rows are contiguous.  Returns a tensor shaped like `queries`."""
+        q = queries if queries.is_contiguous() else queries.contiguous()
+        _cuda(q)
+        _need(q.shape[-1] == HEAD_DIM and q.numel() == self.bs * self.H * self.G * HEAD_DIM, "queries: [bs,1,Hq,128]")
+        _need(1 <= len(segments) <= 4, "1..4 key segments")
+        segs = (_lib.AttnSegment * len(segments))()
+        for i, (k, v, row0, n_rows) in enumerate(segments):
+            _cuda(k, v)
+            _need(k.dtype == q.dtype and v.dtype == q.dtype, "q, k, v must share a dtype")
+            _need(k.dim() == 4 and k.shape == v.shape and k.stride() == v.stride() and k.shape[3] == HEAD_DIM and
+                  k.stride(3) == 1 and k.stride(2) == HEAD_DIM and tuple(k.shape[:2]) == (self.bs, self.H),
+                  "k, v: [bs,Hkv,rows,128] with contiguous rows")
+            _need(0 <= row0 and row0 + n_rows <= k.shape[2], "segment rows out of range")
+            segs[i].k, segs[i].v = _p(k), _p(v)
+            segs[i].stride_b, segs[i].stride_h = k.stride(0), k.stride(1)
+            segs[i].row0, segs[i].n_rows = row0, n_rows
+        if out is None:
+            out = torch.empty_like(q)
+        if scale is None:
+            scale = 1.0 / math.sqrt(HEAD_DIM)
+        _lib.check(_lib.lib().pkv_decode_attention(_p(q), _dt(q.dtype), self.bs, self.H, self.G, segs, len(segments),
+                                                   float(scale), _p(out), _p(self.ws), self.ws.numel(), _stream(q)))
+        return out
 
 
 def gather_cpu(src: torch.Tensor, index: torch.Tensor, out: torch.Tensor, n_threads: int = 1) -> None:

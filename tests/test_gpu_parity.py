@@ -741,3 +741,64 @@ def test_million_key_adaptive_pipeline(ops):
         base = int(cu_k[v]) + sl
         assert torch.equal(kp[base:base + n], keys[0, v][sel]) and torch.equal(vp[base:base + n], -keys[0, v][sel])
         assert not kp[int(cu_k[v]):base].any()   # the sink/local slots are the caller's to fill
+
+
+# ------------------------------------------------------- decode attention
+
+
+@pytest.mark.parametrize("dtype,group,lens", [
+    (torch.bfloat16, 4, (64, 1024, 512)),          # sink | gathered top-k | local window
+    (torch.bfloat16, 4, (64, 300, 1000, 37)),      # four ragged segments
+    (torch.bfloat16, 1, (5,)),                     # fewer keys than one workgroup step
+    (torch.bfloat16, 8, (2000,)),
+    (torch.float32, 2, (129, 64)),
+    (torch.bfloat16, 7, (64, 500)),                # 28 query / 4 KV heads
+])
+def test_decode_attention_segments_vs_oracle(ops, dtype, group, lens):
+    """softmax(q k^T / sqrt(128)) v over row segments read in place, against the double-precision
+    CPU oracle on the same (bf16-exact) inputs.  Tolerance 2e-2 absolute in bf16, 1e-4 in fp32."""
+    bs, H = 2, 3
+    _say(f"decode attention dtype={dtype} G={group} segments={lens}")
+    g = torch.Generator(device=DEV).manual_seed(11)
+    q = (torch.randn(bs, 1, H * group, 128, generator=g, device=DEV) * 1.5).to(dtype)
+    segs, ks, vs = [], [], []
+    for i, n in enumerate(lens):
+        cap = n + 17 + i
+        row0 = 3 + i
+        k = torch.randn(bs, H, cap, 128, generator=g, device=DEV).to(dtype)
+        v = torch.randn(bs, H, cap, 128, generator=g, device=DEV).to(dtype)
+        if i == 1:  # a sliced parent tensor: batch/head strides larger than rows * 128
+            big_k = torch.randn(bs, H + 1, cap + 5, 128, generator=g, device=DEV).to(dtype)
+            big_v = torch.randn(bs, H + 1, cap + 5, 128, generator=g, device=DEV).to(dtype)
+            k, v = big_k[:, :H, :cap], big_v[:, :H, :cap]
+        segs.append((k, v, row0, n))
+        ks.append(k[:, :, row0:row0 + n])
+        vs.append(v[:, :, row0:row0 + n])
+    att = ops.DecodeAttention(bs, H, group, sum(lens), DEV)
+    out = att.run(q, segs)
+    torch.cuda.synchronize()
+    assert out.shape == q.shape and out.dtype == dtype
+    kc = torch.cat(ks, dim=2).float().cpu().numpy()
+    vc = torch.cat(vs, dim=2).float().cpu().numpy()
+    qc = q.float().cpu().numpy().reshape(bs, H, group, 128)
+    got = out.float().cpu().numpy().reshape(bs, H, group, 128)
+    tol = 2e-2 if dtype == torch.bfloat16 else 1e-4
+    for b in range(bs):
+        for h in range(H):
+            ref = O.attention(qc[b, h], kc[b, h], vc[b, h])
+            assert np.abs(got[b, h] - ref).max() <= tol, (b, h, np.abs(got[b, h] - ref).max())
+
+
+def test_decode_attention_argument_errors(ops):
+    att = ops.DecodeAttention(1, 2, 4, 64, DEV)
+    q = torch.zeros(1, 1, 8, 128, dtype=torch.bfloat16, device=DEV)
+    k = torch.zeros(1, 2, 64, 128, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError, match="out of range"):
+        att.run(q, [(k, k, 10, 60)])
+    with pytest.raises(RuntimeError, match="share a dtype"):
+        att.run(q, [(k.float(), k.float(), 0, 8)])
+    with pytest.raises(RuntimeError, match="no keys"):
+        att.run(q, [(k, k, 0, 0)])
+    bad = ops.DecodeAttention(1, 2, 9, 64, DEV)
+    with pytest.raises(RuntimeError, match="group must be"):
+        bad.run(torch.zeros(1, 1, 18, 128, dtype=torch.bfloat16, device=DEV), [(k, k, 0, 8)])

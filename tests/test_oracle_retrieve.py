@@ -237,3 +237,33 @@ def test_retrieve_row_composes_the_stages(oracle, signs):
     # retrieval quality: most of the true top-K inner products are recovered
     true = np.argsort(-(keys @ q.mean(axis=0)))[:K]
     assert len(set(true.tolist()) & set(out.tolist())) > 0.6 * K
+
+
+def test_attention_matches_torch_sdpa_and_closed_forms(oracle):
+    """pkv_o_attention against the library routine (fp32 scaled_dot_product_attention, GQA group 4) and
+    two closed forms: identical keys give the mean of the values; one dominant key gives its value row."""
+    import torch
+    import torch.nn.functional as F
+
+    O = oracle
+    g = torch.Generator().manual_seed(5)
+    G, S = 4, 777
+    q = torch.randn(G, 128, generator=g)
+    k = torch.randn(S, 128, generator=g)
+    v = torch.randn(S, 128, generator=g)
+    ref = F.scaled_dot_product_attention(q.view(1, G, 1, 128), k.view(1, 1, S, 128).expand(1, G, S, 128),
+                                         v.view(1, 1, S, 128).expand(1, G, S, 128)).view(G, 128)
+    got = O.attention(q.numpy(), k.numpy(), v.numpy())
+    np.testing.assert_allclose(got, ref.numpy(), rtol=0, atol=2e-6)
+    # a non-default scale
+    ref2 = F.scaled_dot_product_attention(q.view(1, G, 1, 128), k.view(1, 1, S, 128).expand(1, G, S, 128),
+                                          v.view(1, 1, S, 128).expand(1, G, S, 128), scale=0.3).view(G, 128)
+    np.testing.assert_allclose(O.attention(q.numpy(), k.numpy(), v.numpy(), 0.3), ref2.numpy(), rtol=0, atol=2e-6)
+    # identical keys: uniform weights
+    same = np.tile(k[:1].numpy(), (S, 1))
+    np.testing.assert_allclose(O.attention(q.numpy(), same, v.numpy()), np.tile(v.numpy().mean(0), (G, 1)), atol=1e-6)
+    # one key aligned with the query and far larger than the rest
+    kk = 0.01 * k.numpy()
+    kk[123] = 50.0 * q[2].numpy()
+    out = O.attention(q[2:3].numpy(), kk, v.numpy())
+    np.testing.assert_allclose(out[0], v[123].numpy(), atol=1e-5)
