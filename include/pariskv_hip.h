@@ -280,11 +280,17 @@ typedef struct pkv_attn_segment {
  * for one query token per sequence, non-causal, over the concatenation of up to
  * PKV_ATTN_MAX_SEGMENTS segments read in place.  q, out: [bs][n_kv_heads*group][128]
  * in `dtype` (query head h*group+g attends with KV head h); 1 <= group <= 8.
+ * row_keys (device int32 [bs*n_kv_heads], or NULL): number of keys row (b, h)
+ * attends to, counted in the concatenated order - at most the total of the
+ * segments; lets the last segment be ragged (per-head adaptive k; the
+ * reference packs such rows for flash_attn_varlen_func,
+ * cache_hub/polar_cache_adaptivek_varlen.py:1597-1670).
  * ws: pkv_decode_attention_ws_bytes(...) bytes of device memory for the
  * per-split partial results.  fp32 accumulation; result rounded to `dtype`. */
 size_t pkv_decode_attention_ws_bytes(int bs, int n_kv_heads, int group, int64_t total_keys);
 int pkv_decode_attention(const void *q, int dtype, int bs, int n_kv_heads, int group,
-                         const pkv_attn_segment *segments, int n_segments, float scale,
+                         const pkv_attn_segment *segments, int n_segments,
+                         const int32_t *row_keys, float scale,
                          void *out, void *ws, size_t ws_bytes, void *stream);
 
 /* ------------------------------------------------------- fused decode step */
@@ -300,6 +306,10 @@ int pkv_decode_attention(const void *q, int dtype, int bs, int n_kv_heads, int g
  * out_ids int64 [R][k] (indices relative to key0, descending score).
  * If src_k != NULL the selected rows are gathered into dst_k/dst_v
  * (gather_from_host selects pkv_gather_uva vs pkv_gather_hbm semantics).
+ * out_ids == NULL stops after the rerank (the adaptive-k caller,
+ * cache_hub/polar_cache_adaptivek_varlen.py:1494-1496): the candidate ids
+ * int64 [R][n_cand] and their scores float [R][n_cand] are then read from the
+ * workspace segments "cand" and "scores" (pkv_retrieve_ws_view).
  * ws: pkv_retrieve_ws_bytes(R, n_keys, n_cand, k) bytes of device memory. */
 typedef struct pkv_retrieve_args {
   const void *q;            /* [bs][n_kv_heads*group][128] */
@@ -318,7 +328,7 @@ typedef struct pkv_retrieve_args {
   int n_tiers;
   int64_t n_cand;           /* C */
   int64_t k;                /* K (<= C) */
-  int64_t *out_ids;         /* [R][k] */
+  int64_t *out_ids;         /* [R][k], or NULL for candidates only */
   float *out_scores;        /* [R][k] or NULL */
   /* optional gather */
   const void *src_k, *src_v;

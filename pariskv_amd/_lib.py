@@ -79,7 +79,7 @@ PROTOTYPES = {
     "pkv_adaptive_topk": (_i, [_vp, _i64, _vp, _i64, _i64, _vp, _i, C.c_float, _vp, _vp, _i64, _i64, _vp, _i64,
                                C.c_float, _i64, _i, _vp, _vp, _vp, _sz, _vp]),
     "pkv_decode_attention_ws_bytes": (_sz, [_i, _i, _i, _i64]),
-    "pkv_decode_attention": (_i, [_vp, _i, _i, _i, _i, C.POINTER(AttnSegment), _i, C.c_float, _vp, _vp, _sz, _vp]),
+    "pkv_decode_attention": (_i, [_vp, _i, _i, _i, _i, C.POINTER(AttnSegment), _i, _vp, C.c_float, _vp, _vp, _sz, _vp]),
     "pkv_retrieve_ws_bytes": (_sz, [_i, _i64, _i64, _i64]),
     "pkv_retrieve": (_i, [C.POINTER(RetrieveArgs), _vp, _sz, _vp]),
     "pkv_retrieve_ws_view": (_i, [_vp, _i, _i64, _i64, _i64, C.c_char_p, C.POINTER(_vp), C.POINTER(_sz)]),

@@ -230,6 +230,7 @@ class polar_cache(KV_Cache):
             n = min(n_tok, self.gpu_kv_capacity)
             kg[b0:b1, :, :n] = k[:, :, :n].to(self.dtype)
             vg[b0:b1, :, :n] = v[:, :, :n].to(self.dtype)
+            self._on_prefill(layer_idx, b0, b1, v, 0, n)
             if last:
                 self.context += n
             return key_states[:, vs:], value_states[:, vs:]
@@ -251,6 +252,7 @@ class polar_cache(KV_Cache):
             enc_src = kg[b0:b1, :, S0:r_end]
         self.cluster_key_counts_gpu[layer_idx][b0:b1].zero_()  # prefill assigns, refresh accumulates (:493, :775)
         self._encode(layer_idx, enc_src, b0, b1, S0)
+        self._on_prefill(layer_idx, b0, b1, v, retrieval, local_len)
         if last:
             self.context += n_tok
         return key_states[:, vs:], value_states[:, vs:]
@@ -262,6 +264,7 @@ class polar_cache(KV_Cache):
         slot = z.append_slot()
         self.unified_keys_gpu[layer_idx][:, :, slot, :] = key_states[:, 0]
         self.unified_values_gpu[layer_idx][:, :, slot, :] = value_states[:, 0]
+        self._on_decode_write(layer_idx, slot, value_states)
         refresh = z.appended()
         self.current_seq_len[layer_idx] = z.seq_len
         if layer_idx == 0:
@@ -276,6 +279,7 @@ class polar_cache(KV_Cache):
         n, S0 = r.n_new, self.sink_size
         bs = self.batch_size
         self._encode(layer_idx, kg[:, :, r.gpu_row0:r.gpu_row0 + n], 0, bs, r.encode_abs0)
+        self._on_refresh(layer_idx, r)
         if not self.enable_offload:
             return
         self._wait_offload(layer_idx)  # staging buffers are free again
@@ -292,6 +296,16 @@ class polar_cache(KV_Cache):
         else:
             kg[:, :, S0:S0 + L] = kg[:, :, S0 + n:S0 + n + L]
             vg[:, :, S0:S0 + L] = vg[:, :, S0 + n:S0 + n + L]
+
+    # hooks for subclasses that keep more per-token state (value norms of the adaptive-k variant)
+    def _on_prefill(self, layer_idx, b0, b1, values_bhsd, retrieval, local_len):
+        pass
+
+    def _on_decode_write(self, layer_idx, slot, value_states):
+        pass
+
+    def _on_refresh(self, layer_idx, r):
+        pass
 
     # -------------------------------------------------------------- compute
     def get_region_indices(self, layer_idx, device=None):

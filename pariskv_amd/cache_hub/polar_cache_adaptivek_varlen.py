@@ -1,0 +1,164 @@
+"""Adaptive-k variant of the retrieval cache (reference: ``cache_hub/polar_cache_adaptivek_varlen.py``).
+
+Every decode step the number of retrieved tokens is chosen per (batch, kv-head) row: candidates are ranked by
+``exp(logit) * ||v||`` and the smallest k whose mass, together with the dense sink/local tokens, reaches
+``adaptive_topk_threshold`` of the total is kept (clamped to [min_k, max_k]).  Only ``sum(k)`` K/V rows cross PCIe.
+
+What differs from :class:`polar_cache`:
+
+* two value-norm caches, kept in step with the key/value slots (reference ``:450-483``, ``:1075-1078``,
+  ``:1130-1133``, ``:1179``): ``_sl_vnorm_cache [bs,H,gpu_rows]`` for the dense GPU rows and ``value_norm_gpu
+  [bs,H,capacity]`` by absolute position for the retrieval zone;
+* ``compute`` stops the retrieval after the rerank (all candidates with their scores), runs the adaptive-k
+  kernel, gathers the ragged selection with the packed UVA gather and attends over ``[sink | local | buffer]`` plus
+  each row's own k gathered rows.  The reference packs K/V per row for ``flash_attn_varlen_func`` (``:1597-1670``);
+  here the gathered rows land in a dense ``[bs,H,max_k,128]`` buffer and the attention kernel takes the per-row
+  key count, so the sink/local rows are attended in place and never copied.
+
+Offload mode only, like the reference (``:222-226``).
+"""
+from __future__ import annotations
+
+import math
+import os
+
+import torch
+
+from .. import ops
+from .polar_cache import polar_cache as _polar_cache_base
+
+
+class polar_cache(_polar_cache_base):
+    def __init__(self, valid_start, layer_num, batch_size, max_length, num_key_value_heads, num_heads, head_dim, dtype,
+                 layer_mapping, max_new_length, sink_size, local_size, core=0, nprobe=0, cache_unit_size=0,
+                 cache_cluster_num=0, num_gpus=1, model_size=0, codebook_path=None, collision_ratio: float = 0.3,
+                 candidate_ratio: float = 0.05, final_topk: int = 100, dynamic_update_interval: int = 512,
+                 full_attention_threshold: int = 2000, enable_offload: bool = True, enable_recall: bool = False,
+                 adaptive_topk_threshold: float = 0.85, adaptive_topk_min_k: int = 50,
+                 adaptive_topk_max_k_ratio: float = 0.1) -> None:
+        assert enable_offload, "the adaptive-k variant only supports enable_offload=True"  # reference :222-226
+        # the two ratios are stored like the reference does (:218-219) but, as there, the per-step ratios come from
+        # the retrieval length (_get_adaptive_ratios)
+        super().__init__(valid_start, layer_num, batch_size, max_length, num_key_value_heads, num_heads, head_dim, dtype,
+                         layer_mapping, max_new_length, sink_size, local_size, core, nprobe, cache_unit_size,
+                         cache_cluster_num, num_gpus, model_size, codebook_path=codebook_path, final_topk=final_topk,
+                         dynamic_update_interval=dynamic_update_interval, full_attention_threshold=full_attention_threshold,
+                         enable_offload=True)
+        self.collision_ratio = collision_ratio
+        self.candidate_ratio = candidate_ratio
+        self.enable_recall = enable_recall
+        self.adaptive_topk_threshold = adaptive_topk_threshold
+        self.adaptive_topk_min_k = max(0, int(adaptive_topk_min_k)) if adaptive_topk_min_k is not None else 0
+        r = float(adaptive_topk_max_k_ratio) if adaptive_topk_max_k_ratio is not None else 0.0
+        self.adaptive_topk_max_k_ratio = min(1.0, max(0.0, r))
+        # the caps the reference actually applies (:255-257): environment overrides with the same names
+        self._HARDCODED_MAX_K = int(os.environ.get("ADAPTIVE_TOPK_MAX_K", "800"))
+        self._HARDCODED_MIN_K = int(os.environ.get("ADAPTIVE_TOPK_MIN_K", "100"))
+        self._adaptive_topk_buffer_cap = self._HARDCODED_MAX_K
+        self._attn_scale = 1.0 / math.sqrt(self.head_dim)
+
+        dev, bs, H = self.device, self.batch_size, self.kv_head
+        self._sl_vnorm_cache = [torch.zeros((bs, H, self.gpu_kv_capacity), dtype=torch.float32, device=dev)
+                                for _ in range(layer_num)]
+        self.value_norm_gpu = [torch.zeros((bs, H, self.unified_kv_capacity), dtype=torch.float32, device=dev)
+                               for _ in range(layer_num)]
+        cap = max(1, self._adaptive_topk_buffer_cap)
+        self._topk_k = torch.zeros((bs, H, cap, self.head_dim), dtype=self.dtype, device=dev)
+        self._topk_v = torch.zeros((bs, H, cap, self.head_dim), dtype=self.dtype, device=dev)
+        V = bs * H
+        self._cu_seqlens_dense = (torch.arange(V + 1, dtype=torch.int64) * cap).to(torch.int32).to(dev)
+        self._cu_seqlens_topk_cpu = torch.zeros(V + 1, dtype=torch.int32, pin_memory=True)
+        self.last_adaptive_k = None  # [bs, H] int64 of the most recent retrieval step
+
+    # ------------------------------------------------------------ ratios
+    def _get_adaptive_ratios(self, retrieval_len):
+        """(candidate_ratio, collision_ratio) by retrieval-zone length (reference :2107-2128)."""
+        if retrieval_len < 5000:
+            return 0.5, 0.5
+        if retrieval_len < 10000:
+            return 0.25, 0.3
+        if retrieval_len < 30000:
+            return 0.2, 0.25
+        return 0.05, 0.2
+
+    # ------------------------------------------------ value-norm bookkeeping
+    def _vnorm(self, values):
+        """||v||_2 per token as the reference computes it: in the tensor's dtype, then widened (:680, :756, :1179)."""
+        return torch.linalg.vector_norm(values.to(self.dtype), dim=-1).to(torch.float32)
+
+    def _on_prefill(self, layer_idx, b0, b1, values_bhsd, retrieval, local_len):
+        S0 = self.sink_size
+        sl = self._sl_vnorm_cache[layer_idx]
+        if retrieval == 0:  # short prompt: all tokens are dense GPU rows (:680)
+            sl[b0:b1, :, :local_len] = self._vnorm(values_bhsd[:, :, :local_len])
+            return
+        r_end = S0 + retrieval
+        sl[b0:b1, :, :S0] = self._vnorm(values_bhsd[:, :, :S0])                              # :704
+        sl[b0:b1, :, S0:S0 + local_len] = self._vnorm(values_bhsd[:, :, r_end:r_end + local_len])  # :706
+        self.value_norm_gpu[layer_idx][b0:b1, :, S0:r_end] = self._vnorm(values_bhsd[:, :, S0:r_end])  # :753-756
+
+    def _on_decode_write(self, layer_idx, slot, value_states):
+        self._sl_vnorm_cache[layer_idx][:, :, slot] = self._vnorm(value_states[:, 0])             # :1179
+
+    def _on_refresh(self, layer_idx, r):
+        S0, n, L = self.sink_size, r.n_new, self.local_size
+        sl = self._sl_vnorm_cache[layer_idx]
+        self.value_norm_gpu[layer_idx][:, :, r.encode_abs0:r.encode_abs0 + n] = sl[:, :, S0:S0 + n]  # :1075-1078
+        sl[:, :, S0:S0 + L] = sl[:, :, S0 + n:S0 + n + L].clone()                                 # :1130-1133
+
+    # ---------------------------------------------------------------- compute
+    def _pack_indices(self, dense_indices, adaptive_k, topk_cap):
+        """Dense [bs,H,cap] indices -> packed [sum(k)] in (b, h) row-major order (reference :1817-1832)."""
+        V = adaptive_k.numel()
+        mask = torch.arange(topk_cap, device=dense_indices.device).unsqueeze(0) < adaptive_k.view(V, 1)
+        return dense_indices.contiguous().view(V, topk_cap)[mask]
+
+    def _compute_adaptive_topk(self, query_avg, sink_local_keys, sl_vnorm, all_cand_scores, all_cand_indices, layer_idx,
+                               threshold):
+        """Per-row k and the packed indices (reference :1684-1815).  Returns (adaptive_k [bs,H] int64,
+        indices_packed [sum(k)] int64, global_k int)."""
+        cand_len = all_cand_scores.shape[-1]
+        effective_max_k = min(self._HARDCODED_MAX_K, cand_len)
+        effective_min_k = min(self._HARDCODED_MIN_K, effective_max_k)
+        topk_cap = effective_max_k
+        # logits of the dense tokens: a plain library contraction, as in the reference (:1731)
+        logits_sl = torch.einsum("bhd,bhkd->bhk", query_avg, sink_local_keys).to(torch.float32) * self._attn_scale
+        adaptive_k, topk_ids = ops.adaptive_topk(logits_sl, sl_vnorm, all_cand_scores, self._attn_scale, all_cand_indices,
+                                                 float(threshold), topk_cap, value_norm=self.value_norm_gpu[layer_idx],
+                                                 vn_offset=self.sink_size)
+        adaptive_k.clamp_(min=max(1, effective_min_k), max=max(1, effective_max_k))               # :1759
+        global_k = int(adaptive_k.max().item())                                                   # the step's one host sync
+        return adaptive_k, self._pack_indices(topk_ids, adaptive_k, topk_cap), global_k
+
+    def compute(self, queries, layer_idx):
+        """Decode attention for one token: [bs,1,Hq,D] -> [bs,1,Hq,D] (reference :1391-1677)."""
+        z = self._zones[layer_idx]
+        total = z.seq_len
+        n_keys = self.cpu_valid_end[layer_idx]
+        min_total = max(self.FULL_ATTENTION_THRESHOLD, self.sink_size + self.local_size + self.final_topk * 2)
+        if total < min_total or n_keys <= 0:
+            return super().compute(queries, layer_idx)  # dense branch
+        q = queries.contiguous()
+        bs, H, G, D = self.batch_size, self.kv_head, self.group_size, self.head_dim
+        n_keys, n_cand, _, tiers = self.retrieval_shape(layer_idx)
+        self._wait_offload(layer_idx)
+        cand, scores = self._plan.run_candidates(q, self._srht_signs, self._mag_centers, self.cluster_key_counts_gpu[layer_idx],
+                                                 self._codes_km[layer_idx], self._nib_km[layer_idx], self._w_km[layer_idx],
+                                                 self.sink_size, n_keys, tiers, n_cand)
+        kg, vg = self.unified_keys_gpu[layer_idx], self.unified_values_gpu[layer_idx]
+        sl_end = z.gpu_prefix_rows                                   # sink + local + update buffer rows
+        query_avg = q[:, 0].view(bs, H, G, D).mean(dim=2)            # :1418-1419
+        adaptive_k, indices_packed, global_k = self._compute_adaptive_topk(
+            query_avg, kg[:, :, :sl_end], self._sl_vnorm_cache[layer_idx][:, :, :sl_end], scores, cand, layer_idx,
+            self.adaptive_topk_threshold)
+        self.last_adaptive_k = adaptive_k
+        # ragged UVA gather: row vh receives its own k rows at [vh*cap, vh*cap + k) of the dense buffer (:1634-1644)
+        cu = self._cu_seqlens_topk_cpu
+        torch.cumsum(adaptive_k.reshape(-1).to("cpu", dtype=torch.int32), dim=0, out=cu[1:])
+        cu_topk = cu.to(self.device, non_blocking=True)
+        cap = self._topk_k.shape[2]
+        ops.gather_uva_packed(self.unified_keys_cpu[layer_idx], self.unified_values_cpu[layer_idx],
+                              self._topk_k.view(bs * H * cap, D), self._topk_v.view(bs * H * cap, D), indices_packed,
+                              cu_topk, self._cu_seqlens_dense, 0, global_k)
+        row_keys = (adaptive_k + sl_end).to(torch.int32).contiguous()
+        return self._attention.run(q, [(kg, vg, 0, sl_end), (self._topk_k, self._topk_v, 0, global_k)], row_keys=row_keys)

@@ -86,14 +86,19 @@ constexpr int kPartStride = 130;
 template <bool BF16, int G>
 __global__ __launch_bounds__(kAttThreads) void pkv_attn_partial_kernel(const void *__restrict__ q, int n_kv_heads,
                                                                        int group, int g0, int g_count, AttSegs segs,
-                                                                       int64_t total, int64_t per_split,
-                                                                       float scale_log2e, float *__restrict__ ws) {
+                                                                       int64_t total, const int32_t *__restrict__ row_keys,
+                                                                       int64_t per_split, float scale_log2e,
+                                                                       float *__restrict__ ws) {
   const int split = blockIdx.x, row = blockIdx.y;
   const int b = row / n_kv_heads, h = row % n_kv_heads;
   const int tid = threadIdx.x;
   const int lane16 = tid & 15;        // owns dims 8*lane16 .. +7
   const int grp = tid >> 4;           // 16 key slots per workgroup step
 
+  if (row_keys) {  // ragged rows: this (b, h) attends to its first row_keys[row] keys only
+    const int64_t rk = row_keys[row];
+    total = rk < total ? (rk > 0 ? rk : 1) : total;
+  }
   const int64_t j0 = (int64_t)split * per_split;
   const int64_t j1 = (j0 + per_split < total) ? j0 + per_split : total;
   // per segment: byte address of this lane's 16 bytes of "concatenated key 0" (may lie before the tensor)
@@ -270,8 +275,8 @@ extern "C" size_t pkv_decode_attention_ws_bytes(int bs, int n_kv_heads, int grou
 }
 
 extern "C" int pkv_decode_attention(const void *q, int dtype, int bs, int n_kv_heads, int group,
-                                    const pkv_attn_segment *segments, int n_segments, float scale, void *out, void *ws,
-                                    size_t ws_bytes, void *stream) {
+                                    const pkv_attn_segment *segments, int n_segments, const int32_t *row_keys,
+                                    float scale, void *out, void *ws, size_t ws_bytes, void *stream) {
   PKV_REQUIRE(q && segments && out && ws, "pkv_decode_attention: null pointer");
   PKV_REQUIRE(dtype == PKV_DTYPE_F32 || dtype == PKV_DTYPE_BF16, "unknown dtype %d", dtype);
   PKV_REQUIRE(bs > 0 && n_kv_heads > 0 && (int64_t)bs * n_kv_heads <= 65535, "bad shape bs=%d kv_heads=%d", bs,
@@ -314,7 +319,7 @@ extern "C" int pkv_decode_attention(const void *q, int dtype, int bs, int n_kv_h
   dim3 grid((unsigned)n_splits, (unsigned)rows);
 #define PKV_ATT(BF, GG, G0, GC)                                                                                  \
   hipLaunchKernelGGL((pkv_attn_partial_kernel<BF, GG>), grid, dim3(kAttThreads), 0, s, q, n_kv_heads, group, G0, GC, \
-                     sg, total, per_split, scale_log2e, (float *)ws)
+                     sg, total, row_keys, per_split, scale_log2e, (float *)ws)
   const bool bf = dtype == PKV_DTYPE_BF16;
   for (int g0 = 0; g0 < group; g0 += 4) {  // four query heads per launch: more would not fit the registers
     const int gc = group - g0 < 4 ? group - g0 : 4;

@@ -83,7 +83,7 @@ extern "C" int pkv_retrieve_ws_view(void *ws, int rows, int64_t n_keys, int64_t 
 
 extern "C" int pkv_retrieve(const pkv_retrieve_args *a, void *ws, size_t ws_bytes, void *stream) {
   PKV_REQUIRE(a != nullptr, "pkv_retrieve: null args");
-  PKV_REQUIRE(a->q && a->signs && a->centers && a->cluster_counts && a->codes && a->nib && a->weight && a->out_ids,
+  PKV_REQUIRE(a->q && a->signs && a->centers && a->cluster_counts && a->codes && a->nib && a->weight,
               "pkv_retrieve: null pointer");
   PKV_REQUIRE(a->dtype == PKV_DTYPE_F32 || a->dtype == PKV_DTYPE_BF16, "unknown dtype %d", a->dtype);
   PKV_REQUIRE(a->bs > 0 && a->n_kv_heads > 0 && a->group > 0, "bad shape bs=%d kv_heads=%d group=%d", a->bs,
@@ -141,6 +141,7 @@ extern "C" int pkv_retrieve(const pkv_retrieve_args *a, void *ws, size_t ws_byte
                                   qhat, qnorm, a->centers, cand, scores, s);
   }
   if (rc) return rc;
+  if (!a->out_ids) return PKV_OK;  // candidates only: the caller reads them out of the workspace
   rc = pkv_launch_topk_f32(scores, a->n_cand, cand, a->n_cand, rows, a->n_cand, a->k, a->out_ids, a->out_scores,
                            nullptr, 0, s);
   if (rc) return rc;

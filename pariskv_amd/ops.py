@@ -396,9 +396,11 @@ class DecodeAttention:
         nbytes = max(nbytes, bs * n_kv_heads * 64 * group * 130 * 4)
         self.ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
 
-    def run(self, queries: torch.Tensor, segments, scale: float = None, out: torch.Tensor = None) -> torch.Tensor:
+    def run(self, queries: torch.Tensor, segments, scale: float = None, out: torch.Tensor = None,
+            row_keys: torch.Tensor = None) -> torch.Tensor:
         """queries [bs,1,Hq,128] (or [bs,Hq,128]); segments: list of (k, v, row0, n_rows) with k, v
-        [bs,Hkv,rows,128] tensors whose rows are contiguous.  Returns a tensor shaped like `queries`."""
+        [bs,Hkv,rows,128] tensors whose rows are contiguous; row_keys: optional int32 [bs,Hkv] number of keys
+        (in concatenated order) each row attends to.  Returns a tensor shaped like `queries`."""
         q = queries if queries.is_contiguous() else queries.contiguous()
         _cuda(q)
         _need(q.shape[-1] == HEAD_DIM and q.numel() == self.bs * self.H * self.G * HEAD_DIM, "queries: [bs,1,Hq,128]")
@@ -418,8 +420,13 @@ class DecodeAttention:
             out = torch.empty_like(q)
         if scale is None:
             scale = 1.0 / math.sqrt(HEAD_DIM)
+        if row_keys is not None:
+            _cuda(row_keys)
+            _need(row_keys.dtype == torch.int32 and row_keys.is_contiguous() and row_keys.numel() == self.bs * self.H,
+                  "row_keys: contiguous int32 [bs,Hkv]")
         _lib.check(_lib.lib().pkv_decode_attention(_p(q), _dt(q.dtype), self.bs, self.H, self.G, segs, len(segments),
-                                                   float(scale), _p(out), _p(self.ws), self.ws.numel(), _stream(q)))
+                                                   _p(row_keys), float(scale), _p(out), _p(self.ws), self.ws.numel(),
+                                                   _stream(q)))
         return out
 
 
@@ -452,8 +459,18 @@ class RetrievePlan:
         self.ws = torch.empty(int(nbytes) + (1 << 16), dtype=torch.uint8, device=device)
         self.max = (max_keys, max_cand, max_k)
 
+    def run_candidates(self, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts,
+                       n_cand):
+        """Collision vote + candidate select + 4-bit rerank only.  Returns (cand int64 [bs,H,n_cand] in the select's
+        fixed order, scores float32 [bs,H,n_cand]) as views of the workspace, valid until the next run."""
+        self.run(queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, 1,
+                 candidates_only=True)
+        cand = self.view("cand", n_keys, n_cand, 1, torch.int64).view(self.bs, self.H, n_cand)
+        scores = self.view("scores", n_keys, n_cand, 1, torch.float32).view(self.bs, self.H, n_cand)
+        return cand, scores
+
     def run(self, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, k,
-            out_ids=None, out_scores=None, gather=None):
+            out_ids=None, out_scores=None, gather=None, candidates_only=False):
         """Returns out_ids int64 [bs,H,k].  ``gather`` = dict(src_k, src_v, from_host, idx_offset, dst_k, dst_v, dst_row0)."""
         lib = _lib.lib()
         need = lib.pkv_retrieve_ws_bytes(self.rows, n_keys, n_cand, k)
@@ -462,7 +479,7 @@ class RetrievePlan:
             self.ws = torch.empty(int(need), dtype=torch.uint8, device=self.device)
         q = queries.reshape(self.bs, -1, HEAD_DIM)
         _need(q.is_contiguous() and q.shape[1] == self.H * self.group, "queries must be contiguous [bs,1,Hq,128]")
-        if out_ids is None:
+        if out_ids is None and not candidates_only:
             out_ids = torch.empty(self.bs, self.H, k, dtype=torch.int64, device=self.device)
         a = _lib.RetrieveArgs()
         a.q, a.dtype, a.bs, a.n_kv_heads, a.group = q.data_ptr(), _dt(q.dtype), self.bs, self.H, self.group
@@ -475,7 +492,7 @@ class RetrievePlan:
         for i, t in enumerate(tier_counts):
             a.tier_counts[i] = int(t)
         a.n_tiers, a.n_cand, a.k = len(tier_counts), n_cand, k
-        a.out_ids = out_ids.data_ptr()
+        a.out_ids = None if candidates_only else out_ids.data_ptr()
         a.out_scores = out_scores.data_ptr() if out_scores is not None else None
         if gather is not None:
             sk, sv, dk, dv = gather["src_k"], gather["src_v"], gather["dst_k"], gather["dst_v"]

@@ -164,3 +164,90 @@ def test_single_sample_prefill_and_constructor_errors():
         _make_cache(True, 1, 2, 4, 1, 100, 8, 4, 32, 16, 40, codebook_path="/nonexistent.json")
     with pytest.raises(ValueError):
         polar_cache([0], 1, 1, 100, 2, 4, 64, torch.bfloat16, {0: DEV}, 8, 4, 32)
+
+
+def test_adaptive_k_cache_decode_loop():
+    """Adaptive-k variant (reference polar_cache_adaptivek_varlen.py): value-norm caches follow the K/V slots
+    through prefill, decode writes and index refreshes; per-row k and the selected set equal the CPU oracle's on
+    the cache's own index; attention equals an fp32 softmax over sink ++ each row's own selection ++ dense tail."""
+    from pariskv_amd.cache_hub.polar_cache_adaptivek_varlen import polar_cache as adaptive_cache
+
+    bs, Hkv, Hq, layers, S, steps = 2, 2, 8, 2, 3000, 40
+    sink, local, I = 4, 64, 16
+    G = Hq // Hkv
+    thr = 0.6
+    cache = adaptive_cache(valid_start=[0] * bs, layer_num=layers, batch_size=bs, max_length=S + steps + 10,
+                           num_key_value_heads=Hkv, num_heads=Hq, head_dim=128, dtype=torch.bfloat16,
+                           layer_mapping={i: DEV for i in range(layers)}, max_new_length=steps + 10, sink_size=sink,
+                           local_size=local, core=1, nprobe=1, cache_unit_size=1, cache_cluster_num=1, num_gpus=1,
+                           model_size=7, final_topk=100, dynamic_update_interval=I, full_attention_threshold=100,
+                           enable_offload=True, adaptive_topk_threshold=thr)
+    cache._HARDCODED_MAX_K, cache._HARDCODED_MIN_K = 300, 20   # what ADAPTIVE_TOPK_MAX_K / _MIN_K would set
+    with pytest.raises(AssertionError):
+        adaptive_cache([0], 1, 1, 100, 2, 4, 128, torch.bfloat16, {0: DEV}, 8, 4, 32, enable_offload=False)
+    gen = torch.Generator().manual_seed(3)
+    hist_k, hist_v = [None] * layers, [None] * layers
+    for l in range(layers):
+        k, v = _synth_kv(gen, bs, S, Hkv)
+        v = v * (0.25 + 2.0 * torch.rand(bs, S, Hkv, 1, generator=gen)).to(torch.bfloat16)  # uneven value norms
+        hist_k[l], hist_v[l] = k, v
+        cache.prefill_update_kv_cache(None, k.to(DEV), v.to(DEV), l, 0)
+    signs = O.srht_signs(42)
+    scale = 1.0 / math.sqrt(128)
+    seen_k = set()
+    for step in range(steps):
+        for l in range(layers):
+            k1, v1 = _synth_kv(gen, bs, 1, Hkv)
+            # queries near a handful of recent keys make the attention mass concentrate, so k varies by row
+            q = (hist_k[l][:, -3:].float().mean(dim=1).repeat_interleave(G, dim=1) * 0.3
+                 + 0.5 * torch.randn(bs, Hq, 128, generator=gen)).to(torch.bfloat16).view(bs, 1, Hq, 128)
+            hist_k[l] = torch.cat([hist_k[l], k1], dim=1)
+            hist_v[l] = torch.cat([hist_v[l], v1], dim=1)
+            cache.decode_update_kv_cache(k1.to(DEV), v1.to(DEV), l)
+            out = cache.compute(q.to(DEV), l)
+            if step % 7 != 0 and step not in (I - 1, I, 2 * I - 1):
+                continue
+            torch.cuda.synchronize()
+            total = S + step + 1
+            z = cache._zones[l]
+            n_keys, n_cand, _, tiers = cache.retrieval_shape(l)
+            assert n_keys == z.encoded and z.seq_len == total
+            sl_end = z.gpu_prefix_rows
+            # value norms: retrieval zone by absolute position, dense rows by GPU slot
+            vn_ref = torch.linalg.vector_norm(hist_v[l], dim=-1).float().permute(0, 2, 1)      # [bs, H, total]
+            assert torch.equal(cache.value_norm_gpu[l][:, :, sink:sink + n_keys].cpu(), vn_ref[:, :, sink:sink + n_keys])
+            dense_pos = torch.cat([torch.arange(sink), torch.arange(sink + n_keys, total)])
+            assert sl_end == len(dense_pos)
+            assert torch.equal(cache._sl_vnorm_cache[l][:, :, :sl_end].cpu(), vn_ref[:, :, dense_pos])
+            codes = cache._codes_km[l].cpu().numpy()
+            nib = cache._nib_km[l].cpu().numpy()
+            w = cache._w_km[l].float().cpu().numpy()
+            cc = cache.cluster_key_counts_gpu[l].cpu().numpy()
+            ak = cache.last_adaptive_k.cpu().numpy()
+            qd = q.to(DEV)
+            q_avg = qd[:, 0].view(bs, Hkv, G, 128).mean(dim=2)
+            sl_logits = (torch.einsum("bhd,bhkd->bhk", q_avg, cache.unified_keys_gpu[l][:, :, :sl_end]).float() * scale).cpu().numpy()
+            sl_vnorm = cache._sl_vnorm_cache[l][:, :, :sl_end].cpu().numpy()
+            for b in range(bs):
+                K = hist_k[l][b].permute(1, 0, 2)
+                V = hist_v[l][b].permute(1, 0, 2)
+                ref = torch.empty(Hq, 128)
+                for h in range(Hkv):
+                    zone = slice(sink, sink + n_keys)
+                    qh, qn = O.query_prep(q[b, 0, h * G:(h + 1) * G].float().numpy(), signs, O.BF16)
+                    lut = O.tier_lut(O.rank_centroids(qh, O.BF16), cc[b, h], tiers)
+                    cand_ref, _ = O.select_candidates(O.collision_count(codes[b, h][zone], lut), n_cand)
+                    sc = O.rerank(cand_ref, nib[b, h][zone].reshape(-1, 16, 4), w[b, h][zone], qh, qn)
+                    vn = cache.value_norm_gpu[l][b, h].cpu().numpy()[cand_ref + sink]
+                    cap_k = min(cache._HARDCODED_MAX_K, n_cand)
+                    k_ref, ids_ref = O.adaptive_topk(sl_logits[b, h], sl_vnorm[b, h], sc * np.float32(scale), vn, cand_ref,
+                                                     thr, cap_k)
+                    k_ref = min(max(k_ref, min(cache._HARDCODED_MIN_K, cap_k)), cap_k)
+                    assert int(ak[b, h]) == k_ref, f"step {step} layer {l} row {(b, h)}: k {ak[b, h]} vs {k_ref}"
+                    seen_k.add(k_ref)
+                    sel = torch.cat([torch.arange(sink), torch.from_numpy(ids_ref[:k_ref]) + sink,
+                                     torch.arange(sink + n_keys, total)])
+                    ref[h * G:(h + 1) * G] = _ref_attention(q[b, 0, h * G:(h + 1) * G], K[h:h + 1, sel], V[h:h + 1, sel], G=G * 10)
+                err = (out[b, 0].float().cpu() - ref).abs().max().item()
+                assert err < 2e-2, f"attention differs by {err} at step {step} layer {l}"
+    assert len(seen_k) >= 3, f"k should vary across rows and steps, saw {sorted(seen_k)}"
