@@ -802,3 +802,31 @@ def test_decode_attention_argument_errors(ops):
     bad = ops.DecodeAttention(1, 2, 9, 64, DEV)
     with pytest.raises(RuntimeError, match="group must be"):
         bad.run(torch.zeros(1, 1, 18, 128, dtype=torch.bfloat16, device=DEV), [(k, k, 0, 8)])
+
+
+# --------------------------------------------------- randomised small shapes
+
+
+def test_retrieve_random_shapes_vs_oracle(ops):
+    """Whole retrieval on 14 seeded random shapes (ragged key counts, group sizes 1-7, candidate counts from 1 to
+    every key, k from 1 to the candidate count, both dtype chains): final indices bit-exact against the oracle."""
+    rng = np.random.default_rng(2024)
+    shapes = [(1, 1, 1, 50, 1, 1), (1, 2, 7, 333, 333, 17), (2, 1, 3, 4097, 4096, 4096), (1, 1, 4, 8193, 5000, 1)]
+    while len(shapes) < 14:
+        N = int(rng.integers(60, 20000))
+        C = int(rng.integers(1, N + 1))
+        shapes.append((int(rng.integers(1, 3)), int(rng.integers(1, 3)), int(rng.integers(1, 8)), N, C,
+                       int(rng.integers(1, C + 1))))
+    for i, (bs, H, G, N, C, K) in enumerate(shapes):
+        dtype = O.BF16 if i % 3 else O.F32
+        _say(f"random shape {i}: bs={bs} H={H} G={G} N={N} C={C} K={K} dtype={dtype}")
+        w = W.make_workload(f"rand{i}", bs, H, G, N, C, K, dtype, float(rng.choice([0.2, 0.3, 0.5])), seed0=100 + i,
+                            with_values=False)
+        plan, out, scores = _run_fused(ops, w)
+        for r in range(w.R):
+            b, h = divmod(r, w.H)
+            ref = O.retrieve_row(w.queries[b, h * G:(h + 1) * G], w.signs, w.dtype, w.codes[r], w.nib[r], w.weight[r],
+                                 w.cluster_counts[r], w.tiers, C, K)
+            assert np.array_equal(out[b, h].cpu().numpy(), ref), f"shape {i} row {r}"
+            s = scores[b, h].cpu().numpy()
+            assert np.all(s[:-1] >= s[1:])
