@@ -7,14 +7,16 @@
 // flash_attn_func on [bs, S, H, D]); here the segments are read where they lie.
 //
 // HBM-bound: 512 B (one K row + one V row, bf16) per key and KV head, read once for
-// all G query heads.  Split over the key axis (flash-decoding): grid (n_splits, R),
-// every 16 lanes own one key at a time (16 B of K and of V per lane, so a wave
-// instruction moves four whole rows), keep a running (max, sum, output) per query
-// head, and the partial results are merged first inside the workgroup, then across
-// splits by a second small launch.
+// all G query heads.  Split over the key axis (flash-decoding): grid (n_splits, R);
+// every split keeps a running (max, sum, output) per query head and the partial
+// results are merged by a second small launch.
+//   bf16: one wave per split on the matrix cores (v_mfma_f32_16x16x32_bf16), see below.
+//   fp32: 256 threads per split, every 16 lanes own one key at a time (a wave
+//         instruction moves four whole rows), fp32 FMA and lane-exchange reductions.
 //
-// Arithmetic: products and sums in fp32, exp2 with the scale folded in; the output is
-// rounded to the input dtype.  Not bit-reproducible against another summation order -
+// Arithmetic: products and sums in fp32 (bf16 path: bf16 x bf16 products accumulated in
+// fp32, probabilities rounded to bf16 before P.V as flash-attn does), exp2 with the scale
+// folded in; the output is rounded to the input dtype.  Not bit-reproducible against another summation order -
 // the tolerance of this row is 2e-2 absolute in bf16.
 #include "pkv_common.h"
 
@@ -222,6 +224,154 @@ __global__ __launch_bounds__(kAttThreads) void pkv_attn_partial_kernel(const voi
   }
 }
 
+// ---- bf16 inputs: the same partial step on the matrix cores ----
+//
+// One wave per workgroup, 32 keys per step, v_mfma_f32_16x16x32_bf16 throughout.
+//   scores:  S^T[key][head] = K[key][dim] . Q^T[dim][head]: A = 16 keys x 32 dims (lane (r, j) holds dims
+//            32c + 8j .. +7 of key r: one 128-bit load), B = the query heads (zero columns past `group`),
+//            4 instructions per 16 keys.  Lane (n, j) receives the scores of head n for keys 4j .. 4j+3 of the
+//            tile - which is exactly where the next product wants the probabilities, so nothing is moved.
+//   output:  O[head][dim] += P[head][key] . V[key][dim] over the 32 keys of two tiles: lane (n, j) supplies its
+//            8 probabilities as A; for B it loads dims 8n .. 8n+7 of its 8 keys (rows read whole, 16 lanes per
+//            row) and regroups them with byte permutes so that instruction m covers the dims 8n + m.
+// The running maximum of head n lives in the lanes n, n+16, n+32, n+48; the output rows of head h live in lanes
+// with j == h / 4.  group <= 16, all heads of the KV head in one pass.
+typedef __bf16 pkv_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float pkv_f32x4 __attribute__((ext_vector_type(4)));
+constexpr int kMfmaStepKeys = 32;
+
+__device__ __forceinline__ pkv_f32x4 mfma_bf16(pkv_u32x4 a, pkv_u32x4 b, pkv_f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pkv_bf16x8, a), __builtin_bit_cast(pkv_bf16x8, b), c,
+                                                 0, 0, 0);
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return (uint32_t)pkv_f32_to_bf16_bits(lo) | ((uint32_t)pkv_f32_to_bf16_bits(hi) << 16);
+}
+
+__global__ __launch_bounds__(PKV_WAVE) void pkv_attn_partial_mfma_kernel(const void *__restrict__ q, int n_kv_heads,
+                                                                         int group, AttSegs segs, int64_t total,
+                                                                         const int32_t *__restrict__ row_keys,
+                                                                         int64_t per_split, float scale_log2e,
+                                                                         float *__restrict__ ws) {
+  const int split = blockIdx.x, row = blockIdx.y;
+  const int b = row / n_kv_heads, h = row % n_kv_heads;
+  const int lane = threadIdx.x;
+  const int n = lane & 15, j = lane >> 4;
+  if (row_keys) {
+    const int64_t rk = row_keys[row];
+    total = rk < total ? (rk > 0 ? rk : 1) : total;
+  }
+  const int64_t j0 = (int64_t)split * per_split;
+  const int64_t j1 = (j0 + per_split < total) ? j0 + per_split : total;
+
+  // per segment: byte address of "concatenated key 0" for this (b, h)
+  const char *kb[PKV_ATTN_MAX_SEGMENTS], *vb[PKV_ATTN_MAX_SEGMENTS];
+#pragma unroll
+  for (int s = 0; s < PKV_ATTN_MAX_SEGMENTS; ++s) {
+    const int64_t first = s == 0 ? 0 : segs.end[s - 1];
+    const int64_t off = ((int64_t)b * segs.stride_b[s] + (int64_t)h * segs.stride_h[s] + (segs.row0[s] - first) * 128) * 2;
+    kb[s] = (const char *)segs.k[s] + off;
+    vb[s] = (const char *)segs.v[s] + off;
+  }
+  auto row_ptr = [&](const char *const (&base)[PKV_ATTN_MAX_SEGMENTS], int64_t key) {
+    const uint32_t jj = (uint32_t)(key < j1 ? key : j1 - 1);
+    const char *p = base[0];
+#pragma unroll
+    for (int s = 1; s < PKV_ATTN_MAX_SEGMENTS; ++s)
+      if (s < segs.n && jj >= (uint32_t)segs.end[s - 1]) p = base[s];
+    return p + jj * 256u;
+  };
+
+  const pkv_u32x4 zero4 = {0u, 0u, 0u, 0u};
+  pkv_u32x4 qb[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+    qb[c] = n < group ? *(const pkv_u32x4 *)((const uint16_t *)q + ((int64_t)row * group + n) * 128 + 32 * c + 8 * j) : zero4;
+
+  float m_run = kNegBig, l_part = 0.f;
+  pkv_f32x4 o[8];
+#pragma unroll
+  for (int m = 0; m < 8; ++m) o[m] = pkv_f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int64_t jb = j0; jb < j1; jb += kMfmaStepKeys) {
+    // K: two tiles of 16 keys, lane (n, j) reads dims 32c + 8j .. +7 of key jb + 16t + n
+    pkv_u32x4 ka[2][4], vr[8];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const char *kp = row_ptr(kb, jb + 16 * t + n) + 16 * j;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) ka[t][c] = __builtin_nontemporal_load((const pkv_u32x4 *)(kp + 64 * c));
+    }
+    // V: dims 8n .. 8n+7 of the 8 keys whose probabilities this lane will hold
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      vr[e] = __builtin_nontemporal_load((const pkv_u32x4 *)(row_ptr(vb, jb + 16 * (e >> 2) + 4 * j + (e & 3)) + 16 * n));
+
+    pkv_f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      s0 = mfma_bf16(ka[0][c], qb[c], s0);
+      s1 = mfma_bf16(ka[1][c], qb[c], s1);
+    }
+    float sc[8];
+    bool valid[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      valid[e] = jb + 16 * (e >> 2) + 4 * j + (e & 3) < j1;
+      const float raw = (e < 4) ? s0[e & 3] : s1[e & 3];
+      sc[e] = valid[e] ? raw * scale_log2e : kNegBig;
+    }
+    float mx = sc[0];
+#pragma unroll
+    for (int e = 1; e < 8; ++e) mx = fmaxf(mx, sc[e]);
+    mx = fmaxf(mx, __shfl_xor(mx, 16, PKV_WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, PKV_WAVE));
+    const float m_new = fmaxf(m_run, mx);
+    const float corr = exp2f(m_run - m_new);
+    m_run = m_new;
+    float p[8], psum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      p[e] = valid[e] ? exp2f(sc[e] - m_new) : 0.f;
+      psum += p[e];
+    }
+    l_part = l_part * corr + psum;
+    const pkv_u32x4 pa = {pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]),
+                          pack_bf16x2(p[6], p[7])};
+    // the output rows of this lane belong to heads 4j .. 4j+3: fetch their correction factors
+    float cr[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) cr[i] = __shfl(corr, 4 * j + i, PKV_WAVE);
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {
+      // element m of each of the eight V vectors: dword m/2, half m%2
+      const uint32_t sel = (m & 1) ? 0x07060302u : 0x05040100u;
+      pkv_u32x4 bm;
+      bm.x = __builtin_amdgcn_perm(vr[1][m >> 1], vr[0][m >> 1], sel);
+      bm.y = __builtin_amdgcn_perm(vr[3][m >> 1], vr[2][m >> 1], sel);
+      bm.z = __builtin_amdgcn_perm(vr[5][m >> 1], vr[4][m >> 1], sel);
+      bm.w = __builtin_amdgcn_perm(vr[7][m >> 1], vr[6][m >> 1], sel);
+      pkv_f32x4 acc = o[m];
+      acc.x *= cr[0], acc.y *= cr[1], acc.z *= cr[2], acc.w *= cr[3];
+      o[m] = mfma_bf16(pa, bm, acc);
+    }
+  }
+
+  l_part += __shfl_xor(l_part, 16, PKV_WAVE);
+  l_part += __shfl_xor(l_part, 32, PKV_WAVE);
+  float *part = ws + ((int64_t)row * gridDim.x + split) * group * kPartStride;
+  if (j == 0 && n < group) part[n * kPartStride] = m_run, part[n * kPartStride + 1] = l_part;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int head = 4 * j + i;
+    if (head < group) {
+#pragma unroll
+      for (int m = 0; m < 8; ++m) part[head * kPartStride + 2 + 8 * n + m] = o[m][i];
+    }
+  }
+}
+
 // grid R, G*128 threads: merge the splits (at most 64) and normalise.
 template <bool BF16>
 __global__ void pkv_attn_merge_kernel(const float *__restrict__ ws, int n_splits, int G, void *__restrict__ out) {
@@ -266,12 +416,23 @@ int pick_splits(int rows, int64_t total) {
   return (int)s;
 }
 
+// One wave per workgroup on the matrix-core path: enough waves to cover the chip several times over, at
+// least two 32-key steps each (one step each measured no faster, and the merge pays for the extra splits).
+int pick_splits_mfma(int rows, int64_t total) {
+  int64_t s = (4096 + rows - 1) / rows;
+  const int64_t max_by_len = (total + 63) / 64;
+  if (s > max_by_len) s = max_by_len;
+  if (s > 64) s = 64;
+  if (s < 1) s = 1;
+  return (int)s;
+}
+
 }  // namespace
 
 extern "C" size_t pkv_decode_attention_ws_bytes(int bs, int n_kv_heads, int group, int64_t total_keys) {
   if (bs <= 0 || n_kv_heads <= 0 || group <= 0 || total_keys <= 0) return 256;
-  const int rows = bs * n_kv_heads;
-  return pkv_align_up((size_t)rows * pick_splits(rows, total_keys) * group * kPartStride * sizeof(float), 256);
+  // room for the largest split count either path uses (64), whatever the key count and dtype
+  return pkv_align_up((size_t)bs * n_kv_heads * 64 * group * kPartStride * sizeof(float), 256);
 }
 
 extern "C" int pkv_decode_attention(const void *q, int dtype, int bs, int n_kv_heads, int group,
@@ -305,29 +466,34 @@ extern "C" int pkv_decode_attention(const void *q, int dtype, int bs, int n_kv_h
   PKV_REQUIRE(total > 0, "pkv_decode_attention: no keys");
   PKV_REQUIRE(total < ((int64_t)1 << 23), "pkv_decode_attention: at most 2^23 - 1 keys (got %lld)", (long long)total);
   const int rows = bs * n_kv_heads;
-  const int n_splits = pick_splits(rows, total);
+  const bool bf = dtype == PKV_DTYPE_BF16;
+  const int n_splits = bf ? pick_splits_mfma(rows, total) : pick_splits(rows, total);
   const size_t need = (size_t)rows * n_splits * group * kPartStride * sizeof(float);
   if (ws_bytes < need || !pkv_aligned(ws, 16)) {
     pkv_set_error("pkv_decode_attention: workspace of %zu bytes required, got %zu", need, ws_bytes);
     return PKV_ENOMEM;
   }
-  const int step = kAttKeysPerIter * kAttUnroll;
+  const int step = bf ? kMfmaStepKeys : kAttKeysPerIter * kAttUnroll;
   int64_t per_split = (total + n_splits - 1) / n_splits;
   per_split = (per_split + step - 1) / step * step;
   const float scale_log2e = scale * 1.4426950408889634f;
   hipStream_t s = (hipStream_t)stream;
   dim3 grid((unsigned)n_splits, (unsigned)rows);
-#define PKV_ATT(BF, GG, G0, GC)                                                                                  \
-  hipLaunchKernelGGL((pkv_attn_partial_kernel<BF, GG>), grid, dim3(kAttThreads), 0, s, q, n_kv_heads, group, G0, GC, \
+  if (bf) {
+    hipLaunchKernelGGL(pkv_attn_partial_mfma_kernel, grid, dim3(PKV_WAVE), 0, s, q, n_kv_heads, group, sg, total, row_keys,
+                       per_split, scale_log2e, (float *)ws);
+  } else {
+#define PKV_ATT(GG, G0, GC)                                                                                          \
+  hipLaunchKernelGGL((pkv_attn_partial_kernel<false, GG>), grid, dim3(kAttThreads), 0, s, q, n_kv_heads, group, G0, GC, \
                      sg, total, row_keys, per_split, scale_log2e, (float *)ws)
-  const bool bf = dtype == PKV_DTYPE_BF16;
-  for (int g0 = 0; g0 < group; g0 += 4) {  // four query heads per launch: more would not fit the registers
-    const int gc = group - g0 < 4 ? group - g0 : 4;
-    if (gc == 1) { if (bf) PKV_ATT(true, 1, g0, gc); else PKV_ATT(false, 1, g0, gc); }
-    else if (gc == 2) { if (bf) PKV_ATT(true, 2, g0, gc); else PKV_ATT(false, 2, g0, gc); }
-    else { if (bf) PKV_ATT(true, 4, g0, gc); else PKV_ATT(false, 4, g0, gc); }
-  }
+    for (int g0 = 0; g0 < group; g0 += 4) {  // four query heads per launch: more would not fit the registers
+      const int gc = group - g0 < 4 ? group - g0 : 4;
+      if (gc == 1) PKV_ATT(1, g0, gc);
+      else if (gc == 2) PKV_ATT(2, g0, gc);
+      else PKV_ATT(4, g0, gc);
+    }
 #undef PKV_ATT
+  }
   PKV_LAUNCH_CHECK("pkv_attn_partial_kernel");
   if (bf)
     hipLaunchKernelGGL(pkv_attn_merge_kernel<true>, dim3((unsigned)rows), dim3(group * 128), 0, s, (const float *)ws,

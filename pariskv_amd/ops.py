@@ -392,8 +392,6 @@ class DecodeAttention:
         self.bs, self.H, self.G = bs, n_kv_heads, group
         self.max_keys = max_keys
         nbytes = _lib.lib().pkv_decode_attention_ws_bytes(bs, n_kv_heads, group, max(1, max_keys))
-        # the split count never exceeds 64, whatever the key count: size for that
-        nbytes = max(nbytes, bs * n_kv_heads * 64 * group * 130 * 4)
         self.ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
 
     def run(self, queries: torch.Tensor, segments, scale: float = None, out: torch.Tensor = None,
