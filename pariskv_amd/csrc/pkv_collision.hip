@@ -30,9 +30,9 @@ __device__ __forceinline__ int lut_sum16(const uint8_t *__restrict__ l8, pkv_u32
 }
 
 __device__ __forceinline__ void load_lut(uint32_t *s_lut, const uint8_t *__restrict__ lut, int row) {
-  const uint32_t *g = (const uint32_t *)(lut + (int64_t)row * 4096);
-#pragma unroll
-  for (int i = 0; i < 1024 / kScanThreads; ++i) s_lut[threadIdx.x + i * kScanThreads] = g[threadIdx.x + i * kScanThreads];
+  // 4 KB = one 128-bit load per thread
+  const pkv_u32x4 *g = (const pkv_u32x4 *)(lut + (int64_t)row * 4096);
+  ((pkv_u32x4 *)s_lut)[threadIdx.x] = g[threadIdx.x];
 }
 
 // Key-major codes ([key][16] bytes, 16-byte aligned).  grid (n_chunks, R).
@@ -45,7 +45,7 @@ __global__ __launch_bounds__(kScanThreads) void pkv_scan_keymajor_kernel(
   const int b = row / n_kv_heads, h = row % n_kv_heads;
   const int tid = threadIdx.x;
 
-  __shared__ uint32_t s_lut[1024];
+  __shared__ __attribute__((aligned(16))) uint32_t s_lut[1024];
   __shared__ uint32_t s_hist[128 * kHistCopies];  // also reused for the compacted histogram
   load_lut(s_lut, lut, row);
   for (int i = tid; i < 128 * kHistCopies; i += kScanThreads) s_hist[i] = 0;
@@ -102,7 +102,7 @@ __global__ __launch_bounds__(kScanThreads) void pkv_scan_strided_kernel(
   const int b = row / n_kv_heads, h = row % n_kv_heads;
   const int tid = threadIdx.x;
 
-  __shared__ uint32_t s_lut[1024];
+  __shared__ __attribute__((aligned(16))) uint32_t s_lut[1024];
   __shared__ uint32_t s_hist[128 * kHistCopies];  // also reused for the compacted histogram
   load_lut(s_lut, lut, row);
   for (int i = tid; i < 128 * kHistCopies; i += kScanThreads) s_hist[i] = 0;
@@ -145,7 +145,7 @@ __global__ __launch_bounds__(kScanThreads) void pkv_scan_i32_codes_kernel(const 
                                                                           const uint8_t *__restrict__ lut,
                                                                           int32_t *__restrict__ cnt) {
   const int row = blockIdx.y;
-  __shared__ uint32_t s_lut[1024];
+  __shared__ __attribute__((aligned(16))) uint32_t s_lut[1024];
   load_lut(s_lut, lut, row);
   __syncthreads();
   const uint8_t *l8 = (const uint8_t *)s_lut;

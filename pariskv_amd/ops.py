@@ -393,6 +393,7 @@ class DecodeAttention:
         self.max_keys = max_keys
         nbytes = _lib.lib().pkv_decode_attention_ws_bytes(bs, n_kv_heads, group, max(1, max_keys))
         self.ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        self._segs = (_lib.AttnSegment * 4)()  # reused between calls: filling it is most of the host time
 
     def run(self, queries: torch.Tensor, segments, scale: float = None, out: torch.Tensor = None,
             row_keys: torch.Tensor = None) -> torch.Tensor:
@@ -403,7 +404,7 @@ class DecodeAttention:
         _cuda(q)
         _need(q.shape[-1] == HEAD_DIM and q.numel() == self.bs * self.H * self.G * HEAD_DIM, "queries: [bs,1,Hq,128]")
         _need(1 <= len(segments) <= 4, "1..4 key segments")
-        segs = (_lib.AttnSegment * len(segments))()
+        segs = self._segs
         for i, (k, v, row0, n_rows) in enumerate(segments):
             _cuda(k, v)
             _need(k.dtype == q.dtype and v.dtype == q.dtype, "q, k, v must share a dtype")
