@@ -101,19 +101,15 @@ PKV_INTERNAL int pkv_launch_gather(const void *src_k, const void *src_v, int64_t
 typedef unsigned int pkv_u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int pkv_u32x2 __attribute__((ext_vector_type(2)));
 
-__device__ __forceinline__ float pkv_bf16_round(float x) {
-  uint32_t u = __float_as_uint(x);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return __uint_as_float((u | 0x00400000u) & 0xffff0000u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return __uint_as_float(u & 0xffff0000u);
-}
+// Round to nearest even bf16 and widen again: the hardware conversion (v_cvt_pk_bf16_f32) plus a shift.
+__device__ __forceinline__ float pkv_bf16_round(float x) { return (float)(__bf16)x; }
 
 __device__ __forceinline__ float pkv_rdt(float x, int dtype) {
   return dtype == PKV_DTYPE_BF16 ? pkv_bf16_round(x) : x;
 }
 
 __device__ __forceinline__ uint16_t pkv_f32_to_bf16_bits(float x) {
-  return (uint16_t)(__float_as_uint(pkv_bf16_round(x)) >> 16);
+  return __builtin_bit_cast(uint16_t, (__bf16)x);
 }
 
 __device__ __forceinline__ float pkv_bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }

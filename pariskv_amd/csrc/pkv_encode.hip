@@ -27,12 +27,15 @@ __constant__ float c_thresholds[7] = {0.08447265625f, 0.169921875f, 0.2578125f, 
 __constant__ float c_centers[8] = {0.0419921875f, 0.126953125f, 0.212890625f, 0.302734375f,
                                    0.396484375f,  0.5f,         0.6171875f,   0.76171875f};
 
+// BF16 = the rounding chain of the reference's bf16 tensors (compile-time, so that no rounding point branches).
+template <bool BF16>
 __global__ __launch_bounds__(kEncThreads) void pkv_encode_kernel(
-    const void *__restrict__ keys, int dtype, int n_kv_heads, int64_t n_keys, int64_t k_stride_b, int64_t k_stride_h,
+    const void *__restrict__ keys, int n_kv_heads, int64_t n_keys, int64_t k_stride_b, int64_t k_stride_h,
     int64_t k_stride_key, const float *__restrict__ signs, uint8_t *__restrict__ codes, int64_t cs_b, int64_t cs_h,
     int64_t cs_key, int64_t cs_sub, uint8_t *__restrict__ nib, int64_t ns_b, int64_t ns_h, int64_t ns_key,
     int64_t ns_sub, uint16_t *__restrict__ weight, int64_t ws_b, int64_t ws_h, int64_t ws_key, int64_t ws_sub,
     int32_t *__restrict__ cluster_counts, int64_t cc_b, int64_t cc_h) {
+  constexpr int dtype = BF16 ? PKV_DTYPE_BF16 : PKV_DTYPE_F32;
   const int row = blockIdx.y;
   const int b = row / n_kv_heads, h = row % n_kv_heads;
   const int tid = threadIdx.x;
@@ -40,6 +43,9 @@ __global__ __launch_bounds__(kEncThreads) void pkv_encode_kernel(
   const int kq = tid >> 4;  // key slot inside the iteration
 
   __shared__ uint32_t s_hist[16 * 256];
+  __shared__ float s_centers[8];  // magnitude centres, looked up by code (an LDS read instead of a load from constant memory)
+  if (tid < 8) s_centers[tid] = c_centers[tid];
+  if (!cluster_counts) __syncthreads();
   if (cluster_counts) {
     for (int i = tid; i < 16 * 256; i += kEncThreads) s_hist[i] = 0;
     __syncthreads();
@@ -56,7 +62,7 @@ __global__ __launch_bounds__(kEncThreads) void pkv_encode_kernel(
     const int64_t kload = active ? key : n_keys - 1;  // keep all lanes in the shuffles
     const int64_t off = (int64_t)b * k_stride_b + (int64_t)h * k_stride_h + kload * k_stride_key + 8 * s;
     float x[8];
-    if (dtype == PKV_DTYPE_BF16) {
+    if (BF16) {
       const pkv_u32x4 v = *(const pkv_u32x4 *)((const uint16_t *)keys + off);
       const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
@@ -92,11 +98,13 @@ __global__ __launch_bounds__(kEncThreads) void pkv_encode_kernel(
       for (int j = 0; j < 8; ++j) {
         const float u = pkv_rdt(y[j] / rden, dtype);
         const float au = fabsf(u);
-        int t = 0;
-#pragma unroll
-        for (int i = 0; i < 7; ++i) t += (c_thresholds[i] < au) ? 1 : 0;
+        // t = number of thresholds below au (the thresholds ascend): three compares instead of seven
+        const bool b2 = c_thresholds[3] < au;
+        const bool b1 = (b2 ? c_thresholds[5] : c_thresholds[1]) < au;
+        const float tl = b2 ? (b1 ? c_thresholds[6] : c_thresholds[4]) : (b1 ? c_thresholds[2] : c_thresholds[0]);
+        const int t = (b2 ? 4 : 0) + (b1 ? 2 : 0) + ((tl < au) ? 1 : 0);
         packed |= (uint32_t)(((y[j] >= 0.0f) ? 8 : 0) | t) << (4 * j);
-        const float p = pkv_rdt(c_centers[t] * au, dtype);
+        const float p = pkv_rdt(s_centers[t] * au, dtype);
         alpha = (j == 0) ? p : alpha + p;
       }
       if (alpha < 1e-6f) alpha = 1e-6f;
@@ -167,9 +175,12 @@ extern "C" int pkv_encode_append(const void *keys, int dtype, int bs, int n_kv_h
   PKV_REQUIRE(!nib || (pkv_aligned(nib, 4) && ns_b % 4 == 0 && ns_h % 4 == 0 && ns_key % 4 == 0 && ns_sub % 4 == 0),
               "packed 4-bit blocks must be 4-byte aligned");
   dim3 grid((unsigned)((n_keys + kEncKeysPerBlock - 1) / kEncKeysPerBlock), (unsigned)(bs * n_kv_heads));
-  hipLaunchKernelGGL(pkv_encode_kernel, grid, dim3(kEncThreads), 0, (hipStream_t)stream, keys, dtype, n_kv_heads,
-                     n_keys, k_stride_b, k_stride_h, k_stride_key, signs, codes, cs_b, cs_h, cs_key, cs_sub, nib, ns_b,
-                     ns_h, ns_key, ns_sub, weight, ws_b, ws_h, ws_key, ws_sub, cluster_counts, cc_b, cc_h);
+#define PKV_ENC(BF)                                                                                                  \
+  hipLaunchKernelGGL(pkv_encode_kernel<BF>, grid, dim3(kEncThreads), 0, (hipStream_t)stream, keys, n_kv_heads, n_keys, \
+                     k_stride_b, k_stride_h, k_stride_key, signs, codes, cs_b, cs_h, cs_key, cs_sub, nib, ns_b, ns_h,  \
+                     ns_key, ns_sub, weight, ws_b, ws_h, ws_key, ws_sub, cluster_counts, cc_b, cc_h)
+  if (dtype == PKV_DTYPE_BF16) PKV_ENC(true); else PKV_ENC(false);
+#undef PKV_ENC
   PKV_LAUNCH_CHECK("pkv_encode_kernel");
   return PKV_OK;
 }
