@@ -12,7 +12,8 @@ Steps rotate over LAYERS distinct layer indexes (448 MiB each) so that no
 layer's codes are still in the 256 MB last-level cache when it is scanned again,
 as in a real decode step, which walks all layers of the model.
 
-Prints ONE JSON line (see README / DESIGN.md for the field meanings).
+Prints ONE JSON line: metric/value/unit, the per-stage times (`stages_us`), the roofline of the dominant
+kernel (collision scan, timed by its own dispatch timestamps) and the single-thread CPU baseline.
 """
 import argparse
 import ctypes as C
@@ -50,8 +51,8 @@ def main():
                     help="profiling aid: launch only the collision scan (or the calibration copy) --steps times")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (rows would shard across GPUs by (batch, kv-head), "
-              "see DESIGN.md)", file=sys.stderr)
+        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (rows would shard across GPUs by (batch, kv-head))",
+              file=sys.stderr)
         sys.exit(2)
 
     import torch
