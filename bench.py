@@ -171,6 +171,14 @@ def main():
     att_segs = [(dense_k, dense_v, 0, 64), (dst_k, dst_v, 0, K), (dense_k, dense_v, 64, 512)]
     us_attn = timed(lambda i: att.run(layers[i % L]["q"], att_segs, out=att_out), args.steps)
 
+    def step_with_attention(i):  # retrieval + gather + attention from one host call
+        ly = layers[i % L]
+        plan.run(ly["q"], signs, centers, ly["cc"], ly["codes"], ly["nib"], ly["w"], 0, N, tiers, Cn, K, out_ids=out_ids,
+                 gather=gather, attention=(att, att_segs, att_out))
+
+    step_with_attention(0)
+    us_step_attn = timed(step_with_attention, args.steps)
+
     # dominant kernel: the collision scan, timed by its own begin/end timestamps
     kus = C.c_float()
     scan_us = []
@@ -207,7 +215,8 @@ def main():
                    "rows": R, "keys_per_row": N, "candidates": Cn, "topk": K, "collision_ratio": 0.2},
         "stages_us": {"full_retrieval_with_uva_gather": round(us_step, 2), "on_gpu_stages": round(us_gpu, 2),
                       "uva_gather_alone": round(us_gather, 2),
-                      "decode_attention_over_gathered_set": round(us_attn, 2)},
+                      "decode_attention_over_gathered_set": round(us_attn, 2),
+                      "full_step_plus_attention_one_host_call": round(us_step_attn, 2)},
         "hbm_fraction_on_gpu_stages": round(a_hbm / (us_gpu * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
         "algorithmic_bytes": {"hbm_per_step": a_hbm, "pcie_per_step": a_pcie},
         "pcie_GBps_gather": round(a_pcie / (us_gather * 1e-6) / 1e9, 2),

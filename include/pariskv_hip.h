@@ -342,6 +342,24 @@ typedef struct pkv_retrieve_args {
 size_t pkv_retrieve_ws_bytes(int rows, int64_t n_keys, int64_t n_cand, int64_t k);
 int pkv_retrieve(const pkv_retrieve_args *args, void *ws, size_t ws_bytes, void *stream);
 
+/* The whole decode step of one layer from one host call: pkv_retrieve (with its
+ * gather) followed by pkv_decode_attention over the attended set, on the same
+ * stream - polar_cache.compute (cache_hub/polar_cache.py:1002-1107) after the
+ * dense-fallback test.  Queries, dtype and head counts are taken from
+ * `retrieve`; the segments normally include the rows the gather just wrote. */
+typedef struct pkv_attn_args {
+  pkv_attn_segment segments[PKV_ATTN_MAX_SEGMENTS];
+  int n_segments;
+  const int32_t *row_keys;  /* or NULL */
+  float scale;
+  void *out;                /* [bs][n_kv_heads*group][128] in the query dtype */
+  void *ws;
+  size_t ws_bytes;          /* pkv_decode_attention_ws_bytes(...) */
+} pkv_attn_args;
+
+int pkv_decode_step(const pkv_retrieve_args *retrieve, void *ws, size_t ws_bytes,
+                    const pkv_attn_args *attention, void *stream);
+
 /* Names and device pointers of the intermediates inside a pkv_retrieve
  * workspace (for tests and profiling): qhat, qnorm, lut, cnt_u8,
  * chunk_suffix_hist, row_suffix_hist, cand, scores.  Returns PKV_EINVAL for an unknown name. */

@@ -26,6 +26,13 @@ class AttnSegment(C.Structure):
     _fields_ = [("k", _vp), ("v", _vp), ("stride_b", _i64), ("stride_h", _i64), ("row0", _i64), ("n_rows", _i64)]
 
 
+class AttnArgs(C.Structure):
+    """Mirror of ``pkv_attn_args``."""
+
+    _fields_ = [("segments", AttnSegment * 4), ("n_segments", _i), ("row_keys", _vp), ("scale", C.c_float),
+                ("out", _vp), ("ws", _vp), ("ws_bytes", _sz)]
+
+
 class RetrieveArgs(C.Structure):
     """Mirror of ``pkv_retrieve_args``."""
 
@@ -82,6 +89,7 @@ PROTOTYPES = {
     "pkv_decode_attention": (_i, [_vp, _i, _i, _i, _i, C.POINTER(AttnSegment), _i, _vp, C.c_float, _vp, _vp, _sz, _vp]),
     "pkv_retrieve_ws_bytes": (_sz, [_i, _i64, _i64, _i64]),
     "pkv_retrieve": (_i, [C.POINTER(RetrieveArgs), _vp, _sz, _vp]),
+    "pkv_decode_step": (_i, [C.POINTER(RetrieveArgs), _vp, _sz, C.POINTER(AttnArgs), _vp]),
     "pkv_retrieve_ws_view": (_i, [_vp, _i, _i64, _i64, _i64, C.c_char_p, C.POINTER(_vp), C.POINTER(_sz)]),
 }
 

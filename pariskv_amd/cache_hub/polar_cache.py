@@ -382,11 +382,13 @@ class polar_cache(KV_Cache):
         out_ids = self._out_ids[:, :, :topk]
         if not out_ids.is_contiguous():
             out_ids = torch.empty((self.batch_size, self.kv_head, topk), dtype=torch.int64, device=self.device)
+        # retrieval, gather and attention from one host call
         self._plan.run(q, self._srht_signs, self._mag_centers, self.cluster_key_counts_gpu[layer_idx], self._codes_km[layer_idx],
                        self._nib_km[layer_idx], self._w_km[layer_idx], self.sink_size, n_keys, tiers, n_cand, topk,
-                       out_ids=out_ids, gather=gather)
+                       out_ids=out_ids, gather=gather,
+                       attention=(self._attention, [s for s in segments if s[3] > 0], None))
         self.last_topk_indices = out_ids
-        return self._attend(q, segments)
+        return self._plan.attn_out
 
     def sync(self, layer_idx, batch_idx):
         """No-op, as in the reference (:1310-1312)."""

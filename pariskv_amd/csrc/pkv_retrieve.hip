@@ -161,3 +161,13 @@ extern "C" int pkv_retrieve(const pkv_retrieve_args *a, void *ws, size_t ws_byte
   }
   return rc;
 }
+
+extern "C" int pkv_decode_step(const pkv_retrieve_args *retrieve, void *ws, size_t ws_bytes,
+                               const pkv_attn_args *attention, void *stream) {
+  PKV_REQUIRE(retrieve && attention, "pkv_decode_step: null args");
+  int rc = pkv_retrieve(retrieve, ws, ws_bytes, stream);
+  if (rc) return rc;
+  return pkv_decode_attention(retrieve->q, retrieve->dtype, retrieve->bs, retrieve->n_kv_heads, retrieve->group,
+                              attention->segments, attention->n_segments, attention->row_keys, attention->scale,
+                              attention->out, attention->ws, attention->ws_bytes, stream);
+}

@@ -401,10 +401,17 @@ class DecodeAttention:
         [bs,Hkv,rows,128] tensors whose rows are contiguous; row_keys: optional int32 [bs,Hkv] number of keys
         (in concatenated order) each row attends to.  Returns a tensor shaped like `queries`."""
         q = queries if queries.is_contiguous() else queries.contiguous()
+        segs, out, scale = self._prepare(q, segments, scale, out, row_keys, self._segs)
+        _lib.check(_lib.lib().pkv_decode_attention(_p(q), _dt(q.dtype), self.bs, self.H, self.G, segs, len(segments),
+                                                   _p(row_keys), float(scale), _p(out), _p(self.ws), self.ws.numel(),
+                                                   _stream(q)))
+        return out
+
+    def _prepare(self, q, segments, scale, out, row_keys, segs):
+        """Validate and fill the C segment array `segs`; returns (segs, out, scale)."""
         _cuda(q)
         _need(q.shape[-1] == HEAD_DIM and q.numel() == self.bs * self.H * self.G * HEAD_DIM, "queries: [bs,1,Hq,128]")
         _need(1 <= len(segments) <= 4, "1..4 key segments")
-        segs = self._segs
         for i, (k, v, row0, n_rows) in enumerate(segments):
             _cuda(k, v)
             _need(k.dtype == q.dtype and v.dtype == q.dtype, "q, k, v must share a dtype")
@@ -423,10 +430,15 @@ class DecodeAttention:
             _cuda(row_keys)
             _need(row_keys.dtype == torch.int32 and row_keys.is_contiguous() and row_keys.numel() == self.bs * self.H,
                   "row_keys: contiguous int32 [bs,Hkv]")
-        _lib.check(_lib.lib().pkv_decode_attention(_p(q), _dt(q.dtype), self.bs, self.H, self.G, segs, len(segments),
-                                                   _p(row_keys), float(scale), _p(out), _p(self.ws), self.ws.numel(),
-                                                   _stream(q)))
-        return out
+        return segs, out, scale
+
+    def c_args(self, q, segments, scale=None, out=None, row_keys=None):
+        """(pkv_attn_args, out) for pkv_decode_step: the same call as :meth:`run`, deferred."""
+        a = _lib.AttnArgs()
+        _, out, scale = self._prepare(q, segments, scale, out, row_keys, a.segments)
+        a.n_segments, a.row_keys, a.scale = len(segments), _p(row_keys), float(scale)
+        a.out, a.ws, a.ws_bytes = _p(out), _p(self.ws), self.ws.numel()
+        return a, out
 
 
 def gather_cpu(src: torch.Tensor, index: torch.Tensor, out: torch.Tensor, n_threads: int = 1) -> None:
@@ -469,8 +481,10 @@ class RetrievePlan:
         return cand, scores
 
     def run(self, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, k,
-            out_ids=None, out_scores=None, gather=None, candidates_only=False):
-        """Returns out_ids int64 [bs,H,k].  ``gather`` = dict(src_k, src_v, from_host, idx_offset, dst_k, dst_v, dst_row0)."""
+            out_ids=None, out_scores=None, gather=None, candidates_only=False, attention=None):
+        """Returns out_ids int64 [bs,H,k].  ``gather`` = dict(src_k, src_v, from_host, idx_offset, dst_k, dst_v, dst_row0).
+        ``attention`` = (DecodeAttention, segments, out or None): the attention over those segments is launched by the
+        same C call, after the gather (pkv_decode_step); the output tensor is then in ``self.attn_out``."""
         lib = _lib.lib()
         need = lib.pkv_retrieve_ws_bytes(self.rows, n_keys, n_cand, k)
         _need(need > 0, "need 0 < k <= n_cand <= n_keys")
@@ -499,7 +513,14 @@ class RetrievePlan:
             a.src_len, a.idx_offset = sk.shape[2], int(gather.get("idx_offset", 0))
             a.dst_k, a.dst_v, a.dst_len, a.dst_row0 = dk.data_ptr(), dv.data_ptr(), dk.shape[2], int(gather.get("dst_row0", 0))
             a.row_bytes = sk.shape[3] * sk.element_size()
-        _lib.check(lib.pkv_retrieve(C.byref(a), _p(self.ws), self.ws.numel(), _stream(self.ws)))
+        if attention is None:
+            _lib.check(lib.pkv_retrieve(C.byref(a), _p(self.ws), self.ws.numel(), _stream(self.ws)))
+        else:
+            att, segments, att_out = attention
+            _need(not candidates_only, "attention needs the final top-k")
+            qq = queries if queries.is_contiguous() else queries.contiguous()
+            aa, self.attn_out = att.c_args(qq, segments, out=att_out)
+            _lib.check(lib.pkv_decode_step(C.byref(a), _p(self.ws), self.ws.numel(), C.byref(aa), _stream(self.ws)))
         return out_ids
 
     def view(self, name: str, n_keys: int, n_cand: int, k: int, dtype: torch.dtype) -> torch.Tensor:

@@ -830,3 +830,42 @@ def test_retrieve_random_shapes_vs_oracle(ops):
             assert np.array_equal(out[b, h].cpu().numpy(), ref), f"shape {i} row {r}"
             s = scores[b, h].cpu().numpy()
             assert np.all(s[:-1] >= s[1:])
+
+
+def test_decode_step_single_call_equals_separate_calls(ops, wl_small_bf16):
+    """pkv_decode_step (retrieve + gather + attention from one host call) against the three separate entry points."""
+    w = wl_small_bf16
+    d = W.to_device(w, DEV, torch)
+    g = torch.Generator(device=DEV).manual_seed(3)
+    src_k = torch.randn(w.bs, w.H, w.N, 128, generator=g, device=DEV).to(torch.bfloat16)
+    src_v = torch.randn(w.bs, w.H, w.N, 128, generator=g, device=DEV).to(torch.bfloat16)
+    dense_k = torch.randn(w.bs, w.H, 40, 128, generator=g, device=DEV).to(torch.bfloat16)
+    dense_v = torch.randn(w.bs, w.H, 40, 128, generator=g, device=DEV).to(torch.bfloat16)
+    plan = ops.RetrievePlan(w.bs, w.H, w.G, w.N, DEV, w.N, w.C, w.K)
+    att = ops.DecodeAttention(w.bs, w.H, w.G, 40 + w.K, DEV)
+    outs = []
+    for fused in (False, True):
+        dst_k = torch.zeros(w.bs, w.H, w.K, 128, dtype=torch.bfloat16, device=DEV)
+        dst_v = torch.zeros_like(dst_k)
+        gather = dict(src_k=src_k, src_v=src_v, from_host=False, dst_k=dst_k, dst_v=dst_v)
+        segs = [(dense_k, dense_v, 0, 8), (dst_k, dst_v, 0, w.K), (dense_k, dense_v, 8, 32)]
+        args = (d["queries"], d["signs"], d["centers"], d["cluster_counts"], d["codes_km"], d["nib_km"], d["w_km"], 0, w.N,
+                w.tiers, w.C, w.K)
+        if fused:
+            ids = plan.run(*args, gather=gather, attention=(att, segs, None))
+            out = plan.attn_out
+        else:
+            ids = plan.run(*args, gather=gather)
+            out = att.run(d["queries"], segs)
+        torch.cuda.synchronize()
+        outs.append((ids.clone(), out.clone(), dst_k.clone()))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][2], outs[1][2])
+    assert torch.equal(outs[0][1], outs[1][1]) and outs[1][1].shape == d["queries"].shape
+    # and the attention agrees with the oracle on the gathered rows of one (b, h)
+    b, h = 1, 0
+    sel = outs[1][0][b, h].cpu()
+    kk = torch.cat([dense_k[b, h, :8].cpu(), src_k[b, h].cpu()[sel], dense_k[b, h, 8:40].cpu()]).float().numpy()
+    vv = torch.cat([dense_v[b, h, :8].cpu(), src_v[b, h].cpu()[sel], dense_v[b, h, 8:40].cpu()]).float().numpy()
+    qq = d["queries"][b, 0, h * w.G:(h + 1) * w.G].float().cpu().numpy()
+    got = outs[1][1][b, 0, h * w.G:(h + 1) * w.G].float().cpu().numpy()
+    assert np.abs(got - O.attention(qq, kk, vv)).max() <= 2e-2
