@@ -869,3 +869,46 @@ def test_decode_step_single_call_equals_separate_calls(ops, wl_small_bf16):
     qq = d["queries"][b, 0, h * w.G:(h + 1) * w.G].float().cpu().numpy()
     got = outs[1][1][b, 0, h * w.G:(h + 1) * w.G].float().cpu().numpy()
     assert np.abs(got - O.attention(qq, kk, vv)).max() <= 2e-2
+
+
+def test_decode_step_replays_from_a_captured_graph(ops, wl_small_bf16):
+    """The launch sequence allocates nothing, synchronises nothing and records no memset: it can be captured into
+    a graph once and replayed.  Three replays with different queries and eager work in between, each checked
+    against the eager result of the same inputs."""
+    w = wl_small_bf16
+    d = W.to_device(w, DEV, torch)
+    g = torch.Generator(device=DEV).manual_seed(4)
+    src_k = torch.randn(w.bs, w.H, w.N, 128, generator=g, device=DEV).to(torch.bfloat16)
+    src_v = torch.randn(w.bs, w.H, w.N, 128, generator=g, device=DEV).to(torch.bfloat16)
+    plan = ops.RetrievePlan(w.bs, w.H, w.G, w.N, DEV, w.N, w.C, w.K)
+    att = ops.DecodeAttention(w.bs, w.H, w.G, w.K, DEV)
+    dst_k = torch.zeros(w.bs, w.H, w.K, 128, dtype=torch.bfloat16, device=DEV)
+    dst_v = torch.zeros_like(dst_k)
+    gather = dict(src_k=src_k, src_v=src_v, from_host=False, dst_k=dst_k, dst_v=dst_v)
+    q_static = d["queries"].clone()
+    ids_static = torch.zeros(w.bs, w.H, w.K, dtype=torch.int64, device=DEV)
+    out_static = torch.zeros_like(q_static)
+
+    def step():
+        plan.run(q_static, d["signs"], d["centers"], d["cluster_counts"], d["codes_km"], d["nib_km"], d["w_km"], 0, w.N,
+                 w.tiers, w.C, w.K, out_ids=ids_static, gather=gather, attention=(att, [(dst_k, dst_v, 0, w.K)], out_static))
+
+    step()  # warm-up outside the capture (module load, workspace sizing)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for rep in range(3):
+        q_new = (d["queries"].float() + 0.3 * torch.randn(d["queries"].shape, generator=g, device=DEV)).to(torch.bfloat16)
+        q_static.copy_(q_new)
+        ids_static.zero_(), out_static.zero_(), dst_k.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        got_ids, got_out = ids_static.clone(), out_static.clone()
+        scratch = torch.randn(1 << 20, device=DEV).sum().item()  # unrelated eager work between replays
+        ids_static.zero_(), out_static.zero_()
+        step()
+        torch.cuda.synchronize()
+        assert torch.equal(got_ids, ids_static), f"replay {rep}: indices differ from the eager run"
+        assert torch.equal(got_out, out_static), f"replay {rep}: attention differs from the eager run"
+        assert scratch == scratch
