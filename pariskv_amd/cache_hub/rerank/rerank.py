@@ -38,3 +38,30 @@ def partial_rerank_cuda(coarse_indices, key_4bit, key_block_weight, q_blocks, q_
     centers = mag_centers.to(torch.float32).contiguous()
     scores, v4b = ops.rerank4(coarse_indices, key_4bit, key_block_weight, qhat, qn, centers, want_v4b=return_v4b)
     return scores, v4b
+
+
+def _coarse_filter_truncate(cache_cnt: torch.Tensor, candidate_ratio: float) -> tuple:
+    """Top ``ceil(kv_len * candidate_ratio)`` keys by vote count (reference ``:119-124``).  Returns
+    ``(coarse_indices int64 [bs,H,C], C)``; fixed order: counts above the threshold by ascending key, then the
+    ties at the threshold by ascending key."""
+    import math
+
+    bs, H, kv_len = cache_cnt.shape
+    n_cand = max(1, int(math.ceil(kv_len * candidate_ratio)))
+    idx = ops.bucket_topk(cache_cnt.reshape(bs * H, kv_len), n_cand)
+    return idx.view(bs, H, n_cand), n_cand
+
+
+def rerank_rabitq_fused(cache_cnt, key_4bit, key_block_weight, q_blocks, q_norm, mag_centers, candidate_ratio: float,
+                        final_topk: int, B: int, m: int) -> tuple:
+    """Coarse filter by vote count, 4-bit rerank, final top-k (reference ``:266-293``).  Returns
+    ``(final_indices [bs,H,final_topk], approx_scores, v4b)``; the last two are ``None`` when the candidate set is
+    not larger than ``final_topk``."""
+    coarse_indices, max_candidates = _coarse_filter_truncate(cache_cnt, candidate_ratio)
+    if max_candidates <= final_topk:
+        return coarse_indices[:, :, :final_topk], None, None
+    approx_scores, v4b = partial_rerank_cuda(coarse_indices, key_4bit, key_block_weight, q_blocks, q_norm, mag_centers, B, m)
+    bs, H, C = approx_scores.shape
+    final = ops.topk_f32(approx_scores.view(bs * H, C), final_topk, ids=coarse_indices.view(bs * H, C))
+    final_indices = final[0] if isinstance(final, tuple) else final
+    return final_indices.view(bs, H, final_topk), approx_scores, v4b

@@ -912,3 +912,34 @@ def test_decode_step_replays_from_a_captured_graph(ops, wl_small_bf16):
         assert torch.equal(got_ids, ids_static), f"replay {rep}: indices differ from the eager run"
         assert torch.equal(got_out, out_static), f"replay {rep}: attention differs from the eager run"
         assert scratch == scratch
+
+
+def test_rerank_rabitq_fused_helper(ops, wl_small_bf16):
+    """rerank_rabitq_fused (reference rerank.py:266-293): coarse filter + rerank + final top-k from the vote counts."""
+    from pariskv_amd.cache_hub.rerank.rerank import rerank_rabitq_fused
+
+    w = wl_small_bf16
+    d = W.to_device(w, DEV, torch)
+    codes_km, nib_km, w_km = d["codes_km"], d["nib_km"], d["w_km"]
+    k4 = nib_km.view(w.bs, w.H, w.N, 16, 4).permute(0, 1, 3, 2, 4)   # reference-shaped views of key-major memory
+    kw = w_km.permute(0, 1, 3, 2)
+    cb = codes_km.permute(0, 1, 3, 2)
+    qhat, qnorm, lut, _ = ops.query_prep_lut(d["queries"], w.H, d["signs"], d["cluster_counts"], w.tiers)
+    cnt, _, _ = ops.collision_scan(cb, lut, out_dtype=torch.int32)
+    ratio, final_k = 0.05, 40
+    ids, scores, v4b = rerank_rabitq_fused(cnt, k4, kw, qhat.view(w.bs, w.H, 16, 8), qnorm.view(w.bs, w.H, 1),
+                                           ops.mag_centers(DEV), ratio, final_k, 16, 8)
+    torch.cuda.synchronize()
+    n_cand = int(math.ceil(w.N * ratio))
+    assert ids.shape == (w.bs, w.H, final_k) and scores.shape == (w.bs, w.H, n_cand)
+    for r in range(w.R):
+        b, h = divmod(r, w.H)
+        st = W.oracle_stages(w, r)
+        cand, _ = O.select_candidates(st["cnt"], n_cand)
+        sc = O.rerank(cand, w.nib[r], w.weight[r], st["qhat"], st["qnorm"])
+        final, _ = O.topk_f32(sc, cand, final_k)
+        assert np.array_equal(ids[b, h].cpu().numpy(), final)
+    # candidate set not larger than final_topk: the coarse indices come back, nothing is scored
+    ids2, s2, v2 = rerank_rabitq_fused(cnt, k4, kw, qhat.view(w.bs, w.H, 16, 8), qnorm.view(w.bs, w.H, 1),
+                                       ops.mag_centers(DEV), 0.001, 40, 16, 8)
+    assert s2 is None and v2 is None and ids2.shape[2] == int(math.ceil(w.N * 0.001))
