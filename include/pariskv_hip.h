@@ -201,6 +201,17 @@ int pkv_gather_hbm(const void *src_k, const void *src_v, int64_t src_len,
                    void *dst_k, void *dst_v, int64_t dst_len, int64_t dst_row0,
                    int bs, int n_kv_heads, int row_bytes, void *stream);
 
+/* One decode token per sequence written into the K/V stores: replaces the two
+ * indexed assignments unified_keys_gpu[layer][:, :, pos, :] = key_states[:, 0]
+ * (and values) of decode_update_kv_cache (cache_hub/polar_cache.py:848-856)
+ * with one launch.  k_new/v_new: device rows of row_bytes bytes addressed
+ * k_new + b*new_stride_b + h*new_stride_h; dst_k/dst_v: device
+ * [bs][h][dst_len] rows addressed dst + b*dst_stride_b + h*dst_stride_h +
+ * slot*row_bytes.  All strides in BYTES, multiples of 16. */
+int pkv_append_kv(const void *k_new, const void *v_new, int64_t new_stride_b, int64_t new_stride_h,
+                  void *dst_k, void *dst_v, int64_t dst_stride_b, int64_t dst_stride_h, int64_t dst_len,
+                  int64_t slot, int bs, int n_kv_heads, int row_bytes, void *stream);
+
 /* Ragged form used by the adaptive-k cache variant (kernel source absent from
  * the reference; contract from the call site
  * cache_hub/polar_cache_adaptivek_varlen.py:1634-1644, layout :1573-1586).

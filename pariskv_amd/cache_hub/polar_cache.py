@@ -140,6 +140,7 @@ class polar_cache(KV_Cache):
         max_keys = max(1, cap - sink_size)
         max_cand = max(1, math.ceil(max_keys * 0.5))
         self._plan = ops.RetrievePlan(bs, H, self.group_size, cap, dev, max_keys, max_cand, max(1, min(final_topk, max_cand)))
+        self._bound = [None] * layer_num  # per layer: (n_keys, ops.BoundStep, topk, out_ids, index of the local segment)
         self._out_ids = torch.empty((bs, H, max(1, final_topk)), dtype=torch.int64, device=dev)
         self._attention = ops.DecodeAttention(bs, H, self.group_size, self.unified_kv_capacity, dev)
         self.last_topk_indices = None  # [bs, H, K] of the most recent retrieval (zone-relative), for inspection
@@ -262,8 +263,9 @@ class polar_cache(KV_Cache):
         """Append one token ([bs,1,Hkv,D]); refresh the index when this layer's update buffer fills (:827-881)."""
         z = self._zones[layer_idx]
         slot = z.append_slot()
-        self.unified_keys_gpu[layer_idx][:, :, slot, :] = key_states[:, 0]
-        self.unified_values_gpu[layer_idx][:, :, slot, :] = value_states[:, 0]
+        if key_states.dtype != self.dtype or value_states.dtype != self.dtype:
+            key_states, value_states = key_states.to(self.dtype), value_states.to(self.dtype)
+        ops.append_kv(key_states, value_states, self.unified_keys_gpu[layer_idx], self.unified_values_gpu[layer_idx], slot)
         self._on_decode_write(layer_idx, slot, value_states)
         refresh = z.appended()
         self.current_seq_len[layer_idx] = z.seq_len
@@ -366,11 +368,31 @@ class polar_cache(KV_Cache):
             if not (k.stride(3) == 1 and k.stride(2) == self.head_dim and v.stride() == k.stride()):
                 k, v = k.contiguous(), v.contiguous()
             return self._attend(queries.contiguous(), [(k, v, 0, k.shape[2])])
+        q = queries if queries.is_contiguous() else queries.contiguous()
+        step = self._bound[layer_idx]
+        if step is None or step[0] != n_keys:
+            step = self._bind_step(layer_idx, q, n_keys)
+        _, bound, topk, out_ids, local_seg = step
+        # what moves with every token: where the gathered rows go / how long the dense tail is
+        if self.enable_offload:
+            prefix = z.gpu_prefix_rows
+            bound.a.dst_row0 = prefix
+            bound.segs[0].n_rows = prefix + topk
+        else:
+            bound.segs[local_seg].row0 = z.local_start
+            bound.segs[local_seg].n_rows = z.dense_tail_len
+        self._wait_offload(layer_idx)
+        self.last_topk_indices = out_ids
+        return bound.launch(q)  # retrieval, gather and attention from one host call
+
+    def _bind_step(self, layer_idx, q, n_keys):
+        """Build and validate the argument blocks of this layer's decode step; they stay valid until the next index
+        refresh changes ``n_keys`` (every pointer in them belongs to a tensor this object keeps)."""
+        z = self._zones[layer_idx]
         n_keys, n_cand, topk, tiers = self.retrieval_shape(layer_idx)
         kg, vg = self.unified_keys_gpu[layer_idx], self.unified_values_gpu[layer_idx]
-        q = queries.contiguous()
+        local_seg = 0
         if self.enable_offload:
-            self._wait_offload(layer_idx)
             prefix = z.gpu_prefix_rows
             gather = dict(src_k=self.unified_keys_cpu[layer_idx], src_v=self.unified_values_cpu[layer_idx], from_host=True,
                           idx_offset=0, dst_k=kg, dst_v=vg, dst_row0=prefix)
@@ -379,16 +401,17 @@ class polar_cache(KV_Cache):
             ak, av = self._attn_k, self._attn_v
             gather = dict(src_k=kg, src_v=vg, from_host=False, idx_offset=self.sink_size, dst_k=ak, dst_v=av, dst_row0=0)
             segments = [(kg, vg, 0, self.sink_size), (ak, av, 0, topk), (kg, vg, z.local_start, z.dense_tail_len)]
+            segments = [s for s in segments if s[3] > 0]
+            local_seg = len(segments) - 1
         out_ids = self._out_ids[:, :, :topk]
         if not out_ids.is_contiguous():
             out_ids = torch.empty((self.batch_size, self.kv_head, topk), dtype=torch.int64, device=self.device)
-        # retrieval, gather and attention from one host call
-        self._plan.run(q, self._srht_signs, self._mag_centers, self.cluster_key_counts_gpu[layer_idx], self._codes_km[layer_idx],
-                       self._nib_km[layer_idx], self._w_km[layer_idx], self.sink_size, n_keys, tiers, n_cand, topk,
-                       out_ids=out_ids, gather=gather,
-                       attention=(self._attention, [s for s in segments if s[3] > 0], None))
-        self.last_topk_indices = out_ids
-        return self._plan.attn_out
+        bound = self._plan.bind(q, self._srht_signs, self._mag_centers, self.cluster_key_counts_gpu[layer_idx],
+                                self._codes_km[layer_idx], self._nib_km[layer_idx], self._w_km[layer_idx], self.sink_size,
+                                n_keys, tiers, n_cand, topk, out_ids, gather, self._attention, segments)
+        step = (n_keys, bound, topk, out_ids, local_seg)
+        self._bound[layer_idx] = step
+        return step
 
     def sync(self, layer_idx, batch_idx):
         """No-op, as in the reference (:1310-1312)."""

@@ -368,6 +368,26 @@ def gather_hbm(src_k, src_v, idx, dst_k, dst_v, idx_offset: int = 0, dst_row0: i
     _gather(_lib.lib().pkv_gather_hbm, src_k, src_v, idx, dst_k, dst_v, idx_offset, dst_row0)
 
 
+def append_kv(key_states, value_states, dst_k, dst_v, slot: int) -> None:
+    """dst_k[:, :, slot, :] = key_states[:, 0] and the same for values, in one launch
+    (decode_update_kv_cache, cache_hub/polar_cache.py:848-856).  key_states/value_states [bs,1,Hkv,D];
+    dst_k/dst_v [bs,Hkv,rows,D] with contiguous rows."""
+    bs, one, H, D = key_states.shape
+    es = key_states.element_size()
+    _need(one == 1 and value_states.shape == key_states.shape and key_states.stride(3) == 1 and
+          value_states.stride() == key_states.stride(), "key_states, value_states: [bs,1,Hkv,D], same strides")
+    _need(dst_k.dtype == key_states.dtype and dst_v.dtype == key_states.dtype and value_states.dtype == key_states.dtype,
+          "append: dtypes differ")
+    _need(dst_k.shape == dst_v.shape and dst_k.stride() == dst_v.stride() and dst_k.stride(3) == 1 and
+          dst_k.stride(2) == D and tuple(dst_k.shape[:2]) == (bs, H) and dst_k.shape[3] == D,
+          "dst_k, dst_v: [bs,Hkv,rows,D] with contiguous rows")
+    _need(key_states.is_cuda and dst_k.is_cuda, "append: tensors must be on the GPU")
+    _lib.check(_lib.lib().pkv_append_kv(
+        key_states.data_ptr(), value_states.data_ptr(), key_states.stride(0) * es, key_states.stride(2) * es,
+        dst_k.data_ptr(), dst_v.data_ptr(), dst_k.stride(0) * es, dst_k.stride(1) * es, dst_k.shape[2], slot, bs, H,
+        D * es, _stream(dst_k)))
+
+
 def gather_uva_packed(src_k, src_v, k_packed, v_packed, indices_packed, cu_seqlens_topk, cu_seqlens_k,
                       sink_local_end: int, global_k: int) -> None:
     bs, H, src_len, D = src_k.shape
@@ -458,6 +478,33 @@ def gather_cpu(src: torch.Tensor, index: torch.Tensor, out: torch.Tensor, n_thre
 # ------------------------------------------------------- fused decode step
 
 
+class BoundStep:
+    """The argument blocks of one layer's pkv_decode_step, validated once.  A launch patches only what moves with
+    every token: the query and output pointers and, through ``a`` / ``segs``, the caller's row counts.  Filling and
+    checking the blocks costs more host time than the seven launches themselves, which matters when the K/V live in
+    HBM and the GPU side of a step is a few tens of microseconds."""
+
+    __slots__ = ("a", "aa", "segs", "keep", "_ra", "_raa", "_ws", "_ws_bytes", "_fn", "_numel", "_dtype")
+
+    def __init__(self, plan, a, aa, keep, q):
+        self.a, self.aa, self.segs, self.keep = a, aa, aa.segments, keep
+        self._ra, self._raa = C.byref(a), C.byref(aa)
+        self._ws, self._ws_bytes = _p(plan.ws), plan.ws.numel()
+        self._fn = _lib.lib().pkv_decode_step
+        self._numel, self._dtype = q.numel(), q.dtype
+
+    def launch(self, q: torch.Tensor) -> torch.Tensor:
+        """q: contiguous [bs,1,Hq,128] of the bound dtype.  Returns the attention output, shaped like q."""
+        _need(q.is_cuda and q.is_contiguous() and q.numel() == self._numel and q.dtype == self._dtype,
+              "queries must be contiguous [bs,1,Hq,128] of the cache dtype")
+        out = torch.empty_like(q)
+        self.a.q, self.aa.out = q.data_ptr(), out.data_ptr()
+        rc = self._fn(self._ra, self._ws, self._ws_bytes, self._raa, torch.cuda.current_stream(q.device).cuda_stream)
+        if rc != 0:
+            _lib.check(rc)
+        return out
+
+
 class RetrievePlan:
     """Persistent workspace + argument block for :func:`pkv_retrieve` on key-major storage."""
 
@@ -480,11 +527,9 @@ class RetrievePlan:
         scores = self.view("scores", n_keys, n_cand, 1, torch.float32).view(self.bs, self.H, n_cand)
         return cand, scores
 
-    def run(self, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, k,
-            out_ids=None, out_scores=None, gather=None, candidates_only=False, attention=None):
-        """Returns out_ids int64 [bs,H,k].  ``gather`` = dict(src_k, src_v, from_host, idx_offset, dst_k, dst_v, dst_row0).
-        ``attention`` = (DecodeAttention, segments, out or None): the attention over those segments is launched by the
-        same C call, after the gather (pkv_decode_step); the output tensor is then in ``self.attn_out``."""
+    def _fill(self, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, k,
+              out_ids, out_scores, gather, candidates_only):
+        """Validate one retrieval's operands and return its C argument block."""
         lib = _lib.lib()
         need = lib.pkv_retrieve_ws_bytes(self.rows, n_keys, n_cand, k)
         _need(need > 0, "need 0 < k <= n_cand <= n_keys")
@@ -492,8 +537,6 @@ class RetrievePlan:
             self.ws = torch.empty(int(need), dtype=torch.uint8, device=self.device)
         q = queries.reshape(self.bs, -1, HEAD_DIM)
         _need(q.is_contiguous() and q.shape[1] == self.H * self.group, "queries must be contiguous [bs,1,Hq,128]")
-        if out_ids is None and not candidates_only:
-            out_ids = torch.empty(self.bs, self.H, k, dtype=torch.int64, device=self.device)
         a = _lib.RetrieveArgs()
         a.q, a.dtype, a.bs, a.n_kv_heads, a.group = q.data_ptr(), _dt(q.dtype), self.bs, self.H, self.group
         a.signs, a.centers, a.cluster_counts = signs.data_ptr(), centers.data_ptr(), cluster_counts.data_ptr()
@@ -513,6 +556,18 @@ class RetrievePlan:
             a.src_len, a.idx_offset = sk.shape[2], int(gather.get("idx_offset", 0))
             a.dst_k, a.dst_v, a.dst_len, a.dst_row0 = dk.data_ptr(), dv.data_ptr(), dk.shape[2], int(gather.get("dst_row0", 0))
             a.row_bytes = sk.shape[3] * sk.element_size()
+        return a
+
+    def run(self, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, k,
+            out_ids=None, out_scores=None, gather=None, candidates_only=False, attention=None):
+        """Returns out_ids int64 [bs,H,k].  ``gather`` = dict(src_k, src_v, from_host, idx_offset, dst_k, dst_v, dst_row0).
+        ``attention`` = (DecodeAttention, segments, out or None): the attention over those segments is launched by the
+        same C call, after the gather (pkv_decode_step); the output tensor is then in ``self.attn_out``."""
+        lib = _lib.lib()
+        if out_ids is None and not candidates_only:
+            out_ids = torch.empty(self.bs, self.H, k, dtype=torch.int64, device=self.device)
+        a = self._fill(queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, k,
+                       out_ids, out_scores, gather, candidates_only)
         if attention is None:
             _lib.check(lib.pkv_retrieve(C.byref(a), _p(self.ws), self.ws.numel(), _stream(self.ws)))
         else:
@@ -522,6 +577,16 @@ class RetrievePlan:
             aa, self.attn_out = att.c_args(qq, segments, out=att_out)
             _lib.check(lib.pkv_decode_step(C.byref(a), _p(self.ws), self.ws.numel(), C.byref(aa), _stream(self.ws)))
         return out_ids
+
+    def bind(self, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, k,
+             out_ids, gather, att, segments):
+        """Validate everything :meth:`run` would and keep the two argument blocks of pkv_decode_step for repeated
+        launches with the same operands (one layer between two index refreshes): see :class:`BoundStep`."""
+        a = self._fill(queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, k,
+                       out_ids, None, gather, False)
+        aa, _ = att.c_args(queries, segments, out=queries)  # out is patched at every launch
+        keep = (signs, centers, cluster_counts, codes_km, nib_km, w_km, out_ids, gather, att, segments, self.ws)
+        return BoundStep(self, a, aa, keep, queries)
 
     def view(self, name: str, n_keys: int, n_cand: int, k: int, dtype: torch.dtype) -> torch.Tensor:
         """An intermediate of the last :meth:`run` (qhat, qnorm, lut, cnt_u8, chunk_hist, cand, scores)."""

@@ -943,3 +943,28 @@ def test_rerank_rabitq_fused_helper(ops, wl_small_bf16):
     ids2, s2, v2 = rerank_rabitq_fused(cnt, k4, kw, qhat.view(w.bs, w.H, 16, 8), qnorm.view(w.bs, w.H, 1),
                                        ops.mag_centers(DEV), 0.001, 40, 16, 8)
     assert s2 is None and v2 is None and ids2.shape[2] == int(math.ceil(w.N * 0.001))
+
+
+def test_append_kv_equals_indexed_assignment(ops):
+    """pkv_append_kv against the two indexed assignments it replaces (reference polar_cache.py:848-856), with
+    contiguous and strided new rows and a strided (sliced-batch) store."""
+    g = torch.Generator().manual_seed(5)
+    bs, H, cap, D = 3, 4, 37, 128
+    for dtype in (torch.bfloat16, torch.float32):
+        kg = torch.randn(bs + 1, H, cap, D, generator=g).to(dtype).to(DEV)
+        vg = torch.randn(bs + 1, H, cap, D, generator=g).to(dtype).to(DEV)
+        dk, dv = kg[1:], vg[1:]
+        fused = torch.randn(bs, 1, 3 * H, D, generator=g).to(dtype).to(DEV)   # rows of a fused projection: strided heads
+        for k1, v1 in ((fused[:, :, :H], fused[:, :, 2 * H:]),
+                       (fused[:, :, H:2 * H].contiguous(), fused[:, :, :H].contiguous())):
+            for slot in (0, 17, cap - 1):
+                wk, wv = dk.clone(), dv.clone()
+                wk[:, :, slot, :] = k1[:, 0]
+                wv[:, :, slot, :] = v1[:, 0]
+                ops.append_kv(k1, v1, dk, dv, slot)
+                torch.cuda.synchronize()
+                assert torch.equal(dk, wk) and torch.equal(dv, wv)
+        with pytest.raises(RuntimeError, match="slot"):
+            ops.append_kv(fused[:, :, :H], fused[:, :, H:2 * H], dk, dv, cap)
+    with pytest.raises(RuntimeError):
+        ops.append_kv(fused[:, :, :H], fused[:, :, H:2 * H + 1], dk, dv, 0)
