@@ -352,11 +352,14 @@ float pkv_o_expf(float x) {
   return y * u2f((uint32_t)(e + 127) << 23);
 }
 
-/* Sum in a fixed parallel-friendly order: 1024 strided partial sums (element i
- * goes to lane i mod 1024, accumulated in increasing i), then a pairwise tree
- * over the 1024 lanes (stride 1, 2, 4, ...). */
+/* Sum in a fixed parallel-friendly order.  The input is cut into slices of 8192
+ * consecutive elements.  Inside a slice element j goes to lane j mod 1024,
+ * accumulated in increasing j, then a pairwise tree runs over the 1024 lanes
+ * (stride 1, 2, 4, ...).  The slice sums are added in slice order, the first
+ * one taken as it is.  (Up to 8192 elements this is one slice.) */
 #define PKV_O_SUM_LANES 1024
-static float sum_lanes(const float *x, int64_t n) {
+#define PKV_O_SUM_SLICE 8192
+static float sum_slice(const float *x, int64_t n) {
   float lane[PKV_O_SUM_LANES];
   for (int t = 0; t < PKV_O_SUM_LANES; ++t) {
     float acc = 0.0f;
@@ -368,6 +371,13 @@ static float sum_lanes(const float *x, int64_t n) {
   return lane[0];
 }
 
+static float sum_lanes(const float *x, int64_t n) {
+  float total = sum_slice(x, n < PKV_O_SUM_SLICE ? n : PKV_O_SUM_SLICE);
+  for (int64_t s0 = PKV_O_SUM_SLICE; s0 < n; s0 += PKV_O_SUM_SLICE)
+    total = total + sum_slice(x + s0, n - s0 < PKV_O_SUM_SLICE ? n - s0 : PKV_O_SUM_SLICE);
+  return total;
+}
+
 int64_t pkv_o_adaptive_topk(const float *sl_logits, const float *sl_vnorm, int64_t sl,
                             const float *cand_logits, const float *cand_vnorm,
                             const int64_t *cand_ids, int64_t n_cand, float threshold,
@@ -376,7 +386,7 @@ int64_t pkv_o_adaptive_topk(const float *sl_logits, const float *sl_vnorm, int64
   float g = -INFINITY;
   for (int64_t i = 0; i < sl; ++i) g = sl_logits[i] > g ? sl_logits[i] : g;
   for (int64_t i = 0; i < n_cand; ++i) g = cand_logits[i] > g ? cand_logits[i] : g;
-  float *ben_sl = (float *)malloc((size_t)(sl > 0 ? sl : 1) * sizeof(float));
+  float *ben_sl = (float *)calloc((size_t)(sl > 0 ? sl : 1), sizeof(float));
   float *ben = (float *)malloc((size_t)(n_cand > 0 ? n_cand : 1) * sizeof(float));
   for (int64_t i = 0; i < sl; ++i) ben_sl[i] = pkv_o_expf(sl_logits[i] - g) * sl_vnorm[i];
   for (int64_t i = 0; i < n_cand; ++i) ben[i] = pkv_o_expf(cand_logits[i] - g) * cand_vnorm[i];
@@ -389,10 +399,17 @@ int64_t pkv_o_adaptive_topk(const float *sl_logits, const float *sl_vnorm, int64
   if (total <= 0.0f) {
     k = 1; /* :304-306 */
   } else {
-    float cs = 0.0f, tgt = threshold * total;
+    /* :300-303 cumulative sum of the sorted benefits, in a fixed two-level order:
+     * blocks of 64 consecutive elements are summed left to right (run), the block
+     * totals are summed left to right (before), prefix = before + run. */
+    float tgt = threshold * total, before = 0.0f, run = 0.0f;
     for (int64_t i = 0; i < k_out; ++i) {
-      cs = cs + ben[pos[i]];
-      if (sl_benefit + cs >= tgt) {
+      if (i % 64 == 0) {
+        before = before + run; /* total of the previous block (0 at the start) */
+        run = 0.0f;
+      }
+      run = run + ben[pos[i]];
+      if (sl_benefit + (before + run) >= tgt) {
         k = i + 1;
         break;
       }

@@ -121,6 +121,11 @@ void pkv_o_gather_rows(const void *src, const int64_t *idx, int64_t k,
 float pkv_o_expf(float x);
 
 /* adaptive_k_fused/adaptive_topk.py:255-313 (adaptive_topk_ref), fp32.
+ * Summation orders are fixed (the reference leaves them to torch): the two
+ * benefit sums run over slices of 8192 elements (lane j mod 1024 in increasing
+ * j, pairwise tree over the 1024 lanes, slice sums left to right); the
+ * cumulative sum over the sorted benefits runs left to right inside blocks of
+ * 64 and left to right over the block totals.
  * Returns adaptive k (before any min/max clamp by the caller);
  * out_ids[k_out] = candidate ids in descending benefit order
  * (ties: smaller candidate position first). */

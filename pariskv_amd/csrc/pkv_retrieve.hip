@@ -12,13 +12,13 @@ PKV_INTERNAL int pkv_launch_identity_fill(int64_t *out, int64_t len, int64_t k, 
 namespace {
 
 struct WsLayout {
-  size_t qhat, qnorm, lut, cnt, hist, rowsuf, cand, scores, total;
+  size_t qhat, qnorm, lut, cnt, hist, rowsuf, cand, scores, topk, topk_bytes, total;
   int64_t cnt_stride;
   int chunk_keys;
   int64_t n_chunks;
 };
 
-WsLayout layout(int rows, int64_t n_keys, int64_t n_cand, int64_t /*k*/) {
+WsLayout layout(int rows, int64_t n_keys, int64_t n_cand, int64_t k) {
   WsLayout w;
   size_t off = 0;
   auto take = [&](size_t bytes) {
@@ -37,6 +37,8 @@ WsLayout layout(int rows, int64_t n_keys, int64_t n_cand, int64_t /*k*/) {
   w.rowsuf = take((size_t)rows * 128 * sizeof(uint32_t));
   w.cand = take((size_t)rows * (size_t)n_cand * sizeof(int64_t));
   w.scores = take((size_t)rows * (size_t)n_cand * sizeof(float));
+  w.topk_bytes = pkv_topk_ws_bytes_impl(rows, n_cand, k);  // lists of the multi-workgroup top-k (wide rows only)
+  w.topk = take(w.topk_bytes);
   w.total = off;
   return w;
 }
@@ -143,7 +145,7 @@ extern "C" int pkv_retrieve(const pkv_retrieve_args *a, void *ws, size_t ws_byte
   if (rc) return rc;
   if (!a->out_ids) return PKV_OK;  // candidates only: the caller reads them out of the workspace
   rc = pkv_launch_topk_f32(scores, a->n_cand, cand, a->n_cand, rows, a->n_cand, a->k, a->out_ids, a->out_scores,
-                           nullptr, 0, s);
+                           (char *)ws + w.topk, w.topk_bytes, s);
   if (rc) return rc;
   if (a->src_k) {
     PKV_REQUIRE(a->src_v && a->dst_k && a->dst_v, "pkv_retrieve: gather needs src_v, dst_k, dst_v");

@@ -617,30 +617,181 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
 #undef PKV_SORT_K
 }
 
-// len > 8192, k <= 8192: 8-bit MSB-first radix passes over the row find the k winners
-// exactly; they are collected into LDS and sorted.
-__global__ __launch_bounds__(kTopkThreads) void pkv_topk_radix_kernel(const float *__restrict__ x, int64_t x_stride,
-                                                                      const int64_t *__restrict__ ids,
-                                                                      int64_t ids_stride, int64_t len, int P,
-                                                                      int64_t k, int64_t *__restrict__ out_ids,
-                                                                      float *__restrict__ out_vals) {
+// ------------------------------------------------- rows wider than one workgroup
+//
+// More than 8192 keys in a row: the row is cut into slices of 8192 keys, one workgroup (8 keys per
+// thread) each, and the k winners are found in three steps.
+//   histogram  every slice adds bits [BINSHIFT, BINSHIFT+11) of its 64-bit keys to a 2048-bin
+//              histogram of the row: in LDS first, then one global atomic per non-empty bin;
+//   compact    every slice derives the threshold bin b* from the row histogram (the bin in which the
+//              k-th largest key lies) and appends its keys above b* to list A (fewer than k in the
+//              whole row) and its keys inside b* to list B, slots handed out by two row counters;
+//   finish     one workgroup per row picks the k - |A| largest keys of list B exactly (radix select in
+//              registers; streamed if B has more than 8192 keys) and sorts the k winners.
+// Keys are distinct, so the order in which the lists are filled does not reach the result.
+constexpr int kWideSlice = 8192;
+constexpr int kWideBins = 2048;
+constexpr int kWideRowWords = kWideBins + 8;  // per-row control block: histogram, |A|, |B|, padding
+
+struct ScoreKeys {  // key i of a row of scores with optional ids
+  const float *x;
+  const int64_t *ids;
+  __device__ __forceinline__ uint64_t operator()(int64_t i) const { return make_key(x, ids, i); }
+};
+
+constexpr int kWideE = kWideSlice / kTopkThreads;  // keys per thread
+
+// The slice's keys, element e of thread t = slice*8192 + e*1024 + t; 0 beyond the row's end.  The loads are
+// unconditional (clamped index) so that all of them are in flight together.
+template <typename KeyFn>
+__device__ __forceinline__ void wide_load_keys(KeyFn key_of, int64_t len, int slice, uint64_t (&keys)[kWideE]) {
+#pragma unroll
+  for (int e = 0; e < kWideE; ++e) {
+    const int64_t i = (int64_t)slice * kWideSlice + e * kTopkThreads + threadIdx.x;
+    const uint64_t key = key_of(i < len ? i : len - 1);
+    keys[e] = i < len ? key : 0ull;
+  }
+}
+
+template <int BINSHIFT>
+__device__ __forceinline__ void wide_hist_slice(const uint64_t (&keys)[kWideE], int64_t len, int slice, uint32_t *s_bins,
+                                                uint32_t *__restrict__ g_hist) {
+  const int tid = threadIdx.x;
+  for (int b = tid; b < kWideBins; b += kTopkThreads) s_bins[b] = 0;
+  __syncthreads();
+#pragma unroll
+  for (int e = 0; e < kWideE; ++e) {
+    const int64_t i = (int64_t)slice * kWideSlice + e * kTopkThreads + tid;
+    wave_hist_add(s_bins, (uint32_t)(keys[e] >> BINSHIFT) & (kWideBins - 1), i < len, 1);
+  }
+  __syncthreads();
+  for (int b = tid; b < kWideBins; b += kTopkThreads) {
+    const uint32_t c = s_bins[b];
+    if (c) atomicAdd(&g_hist[b], c);
+  }
+}
+
+// s_tmp: 24 words.  ctl: the row's control block (histogram complete at launch).  Every workgroup
+// reserves its share of both lists with one atomic each.
+template <int BINSHIFT>
+__device__ __forceinline__ void wide_compact_slice(const uint64_t (&keys)[kWideE], int64_t len, int slice, uint32_t k,
+                                                   uint32_t *__restrict__ ctl, uint64_t *__restrict__ list_a,
+                                                   uint64_t *__restrict__ list_b, uint32_t *s_tmp) {
+  const int tid = threadIdx.x;
+  // thread t owns bins 2047 - 2t and 2046 - 2t: an exclusive scan over threads counts the keys in higher bins
+  const uint32_t h0 = ctl[kWideBins - 1 - 2 * tid], h1 = ctl[kWideBins - 2 - 2 * tid];
+  if (tid == 0) s_tmp[16] = 0;
+  int total;
+  uint32_t above = (uint32_t)pkv_block_excl_scan<kTopkThreads>((int)(h0 + h1), (int *)s_tmp, total);
+  if (above < k && above + h0 >= k) s_tmp[16] = (uint32_t)(kWideBins - 1 - 2 * tid);
+  above += h0;
+  if (above < k && above + h1 >= k) s_tmp[16] = (uint32_t)(kWideBins - 2 - 2 * tid);
+  __syncthreads();
+  const uint32_t bstar = s_tmp[16];
+  uint32_t in_a = 0, in_b = 0, n_a = 0, n_b = 0;  // bit e: key e goes to list A / B
+#pragma unroll
+  for (int e = 0; e < kWideE; ++e) {
+    const int64_t i = (int64_t)slice * kWideSlice + e * kTopkThreads + tid;
+    const uint32_t bin = (uint32_t)(keys[e] >> BINSHIFT) & (kWideBins - 1);
+    const bool a = i < len && bin > bstar, b = i < len && bin == bstar;
+    in_a |= (uint32_t)a << e, in_b |= (uint32_t)b << e;
+    n_a += a, n_b += b;
+  }
+  // both counts in one scan: a slice holds at most 8192 keys, so 16 bits each are enough
+  const uint32_t excl = (uint32_t)pkv_block_excl_scan<kTopkThreads>((int)(n_a | (n_b << 16)), (int *)s_tmp, total);
+  if (tid == 0) s_tmp[17] = atomicAdd(&ctl[kWideBins], (uint32_t)total & 0xffffu);
+  if (tid == PKV_WAVE) s_tmp[18] = atomicAdd(&ctl[kWideBins + 1], (uint32_t)total >> 16);
+  __syncthreads();
+  uint32_t slot_a = s_tmp[17] + (excl & 0xffffu), slot_b = s_tmp[18] + (excl >> 16);
+#pragma unroll
+  for (int e = 0; e < kWideE; ++e) {
+    if ((in_a >> e) & 1u) {
+      if (slot_a < k) list_a[slot_a] = keys[e];
+      ++slot_a;
+    }
+    if ((in_b >> e) & 1u) {
+      if ((int64_t)slot_b < len) list_b[slot_b] = keys[e];
+      ++slot_b;
+    }
+  }
+}
+
+// The k winners into s_keys[0 .. k) in any order (zero padded up to max(P, 1024)).  All 1024 threads.
+__device__ __forceinline__ void wide_finish_select(uint32_t k, int P, const uint32_t *__restrict__ ctl,
+                                                   const uint64_t *__restrict__ list_a,
+                                                   const uint64_t *__restrict__ list_b, int64_t len, uint64_t *s_keys,
+                                                   uint32_t *s_hist, uint32_t *s_bcast, uint32_t *s_counter) {
+  const int tid = threadIdx.x;
+  uint32_t n_a = ctl[kWideBins], n_b = ctl[kWideBins + 1];
+  if (n_a > k) n_a = k;  // cannot happen with a consistent histogram; keeps every index in range
+  if ((int64_t)n_b > len) n_b = (uint32_t)len;
+  const uint32_t need = k - n_a;
+  for (int i = tid; i < (P < 1024 ? 1024 : P); i += kTopkThreads) s_keys[i] = (uint32_t)i < n_a ? list_a[i] : 0ull;
+  if (tid == 0) *s_counter = n_a;
+  __syncthreads();
+  if (need == 0) return;
+  if (n_b <= (uint32_t)kWideSlice) {
+    uint64_t v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t i = (uint32_t)(tid + e * kTopkThreads);
+      v[e] = i < n_b ? list_b[i] : 0ull;
+    }
+    uint64_t prefix = 0;
+    int shift = 0;
+    if (need < n_b) radix_select_regs<8>(v, need, s_hist, s_bcast, prefix, shift);  // else: all of B
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const bool win = v[e] != 0ull && (v[e] >> shift) >= (prefix >> shift);
+      const uint32_t slot = wave_take_slots(s_counter, win);
+      if (win && slot < k) s_keys[slot] = v[e];
+    }
+  } else {
+    auto key_of = [&](int64_t i) { return list_b[i]; };
+    uint64_t prefix;
+    int shift;
+    radix_select_streamed(key_of, (int64_t)n_b, need, s_hist, s_bcast, prefix, shift);
+    collect_winners_streamed(key_of, (int64_t)n_b, k, prefix, shift, s_counter, s_keys);
+  }
+  __syncthreads();
+}
+
+// grid (slices, rows).  ctl: u32 [rows][kWideRowWords], zero at launch.
+__global__ __launch_bounds__(kTopkThreads) void pkv_topk_wide_hist_kernel(const float *__restrict__ x, int64_t x_stride,
+                                                                          const int64_t *__restrict__ ids,
+                                                                          int64_t ids_stride, int64_t len,
+                                                                          uint32_t *__restrict__ ctl) {
+  __shared__ uint32_t s_bins[kWideBins];
+  const int row = blockIdx.y;
+  uint64_t keys[kWideE];
+  wide_load_keys(ScoreKeys{x + (int64_t)row * x_stride, ids ? ids + (int64_t)row * ids_stride : nullptr}, len, blockIdx.x,
+                 keys);
+  wide_hist_slice<53>(keys, len, blockIdx.x, s_bins, ctl + (int64_t)row * kWideRowWords);
+}
+
+__global__ __launch_bounds__(kTopkThreads) void pkv_topk_wide_compact_kernel(
+    const float *__restrict__ x, int64_t x_stride, const int64_t *__restrict__ ids, int64_t ids_stride, int64_t len,
+    int64_t k, uint32_t *__restrict__ ctl, uint64_t *__restrict__ list_a, uint64_t *__restrict__ list_b) {
+  __shared__ uint32_t s_tmp[24];
+  const int row = blockIdx.y;
+  uint64_t keys[kWideE];
+  wide_load_keys(ScoreKeys{x + (int64_t)row * x_stride, ids ? ids + (int64_t)row * ids_stride : nullptr}, len, blockIdx.x,
+                 keys);
+  wide_compact_slice<53>(keys, len, blockIdx.x, (uint32_t)k, ctl + (int64_t)row * kWideRowWords, list_a + (int64_t)row * k,
+                         list_b + (int64_t)row * len, s_tmp);
+}
+
+// grid rows; dynamic LDS max(P,1024)*8 bytes.
+__global__ __launch_bounds__(kTopkThreads) void pkv_topk_wide_finish_kernel(
+    int64_t len, int P, int64_t k, const uint32_t *__restrict__ ctl, const uint64_t *__restrict__ list_a,
+    const uint64_t *__restrict__ list_b, int64_t *__restrict__ out_ids, float *__restrict__ out_vals) {
   extern __shared__ uint64_t s_keys[];
   __shared__ uint32_t s_hist[512];
   __shared__ uint32_t s_bcast[8];
   __shared__ uint32_t s_counter;
   const int row = blockIdx.x;
-  const int tid = threadIdx.x;
-  const float *xr = x + (int64_t)row * x_stride;
-  const int64_t *ir = ids ? ids + (int64_t)row * ids_stride : nullptr;
-  auto key_of = [&](int64_t i) { return make_key(xr, ir, i); };
-
-  if (tid == 0) s_counter = 0;
-  for (int i = tid; i < (P < 1024 ? 1024 : P); i += kTopkThreads) s_keys[i] = 0ull;
-  uint64_t prefix;
-  int shift;
-  radix_select_streamed(key_of, len, (uint32_t)k, s_hist, s_bcast, prefix, shift);
-  collect_winners_streamed(key_of, len, (uint32_t)k, prefix, shift, &s_counter, s_keys);
-  __syncthreads();
+  wide_finish_select((uint32_t)k, P, ctl + (int64_t)row * kWideRowWords, list_a + (int64_t)row * k,
+                     list_b + (int64_t)row * len, len, s_keys, s_hist, s_bcast, &s_counter);
   int64_t *oi = out_ids + (int64_t)row * k;
   float *ov = out_vals ? out_vals + (int64_t)row * k : nullptr;
 #define PKV_SORT_K(NT, E) sort_lds_keys_and_emit<NT, E>(s_keys, k, oi, ov, nullptr)
@@ -711,13 +862,165 @@ __device__ __forceinline__ float cand_logit(const void *__restrict__ scores, int
   return x * scale;
 }
 
-// One workgroup of 1024 threads per row; dynamic LDS P*8 bytes (P = pow2 >= k_out).
+// Sum of x over the workgroup's 1024 lanes for one slice of at most 8192 elements whose per-lane partial
+// sums are `acc`; slices are then added in slice order (the first slice is taken as is).
+__device__ __forceinline__ float add_slice_sum(float total, bool first, float acc, float *s_part) {
+  const float sl = block_tree_sum_1024(acc, s_part);
+  return first ? sl : total + sl;
+}
+
+// sum_i expf(logit_i - g) * vnorm_i over the dense (sink/local) tokens, in slices of 8192.
+__device__ __forceinline__ float dense_benefit_sum(const float *__restrict__ sll, const float *__restrict__ slv,
+                                                   int64_t sl, float g, float *s_part) {
+  float total = 0.f;
+  bool first = true;
+  for (int64_t s0 = 0; s0 < sl || first; s0 += kWideSlice) {
+    float acc = 0.f;
+#pragma unroll
+    for (int e = 0; e < kWideSlice / kTopkThreads; ++e) {
+      const int64_t i = s0 + e * kTopkThreads + threadIdx.x;
+      if (i < sl) acc = acc + pkv_expf(sll[i] - g) * slv[i];
+    }
+    total = add_slice_sum(total, first, acc, s_part);
+    first = false;
+  }
+  return total;
+}
+
+// Running sums of 64 values strictly left to right in fp32: lane l returns carry + v_0 + ... + v_l, added
+// in that order.  The chain of dependent adds runs through the lanes: every step adds a lane's value to
+// its lower neighbour's running sum (DPP wave_shr:1; lane 0 takes the carry), so after step s lanes
+// 0..s hold their final sums.  All 64 lanes must be active.
+__device__ __forceinline__ float wave_running_sum(float val, float carry) {
+  float acc = val;
+#pragma unroll
+  for (int s = 0; s < PKV_WAVE; ++s) {
+    const float below =
+        __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(carry), __float_as_int(acc), 0x138, 0xf, 0xf, false));
+    acc = below + val;
+  }
+  return acc;
+}
+
+// Smallest k <= k_out with sl_benefit + prefix_{k-1} >= tgt over the sorted keys in s_keys (k_out if the
+// target is never reached).  prefix is the cumulative sum of the reference (adaptive_topk.py:300-303) in
+// a fixed two-level order: blocks of 64 consecutive benefits are summed left to right, the block totals
+// are summed left to right, prefix_i = (total of the earlier blocks) + (running sum inside the block).
+// All 1024 threads call it; k_out <= 8192.  s_f: 256 floats, s_k: one word.
+__device__ __forceinline__ int64_t first_k_reaching(const uint64_t *s_keys, int64_t k_out, float sl_benefit, float tgt,
+                                                    float *s_f, uint32_t *s_k) {
+  const int lane = pkv_lane(), wave = threadIdx.x / PKV_WAVE;
+  const int n_blocks = (int)((k_out + PKV_WAVE - 1) / PKV_WAVE);  // <= 128; wave w owns blocks w, w+16, ...
+  float *s_tot = s_f, *s_before = s_f + 128;
+  float run[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int c = wave + 16 * j;
+    run[j] = 0.f;
+    if (c < n_blocks) {
+      const int64_t i = (int64_t)c * PKV_WAVE + lane;
+      run[j] = wave_running_sum(i < k_out ? pkv_from_ordered_u32((uint32_t)(s_keys[i] >> 32)) : 0.f, 0.f);
+      if (lane == PKV_WAVE - 1) s_tot[c] = run[j];
+    }
+  }
+  if (threadIdx.x == 0) *s_k = (uint32_t)k_out;
+  __syncthreads();
+  if (wave == 0) {
+    float carry = 0.f;
+    for (int base = 0; base < n_blocks; base += PKV_WAVE) {
+      const int c = base + lane;
+      const float incl = wave_running_sum(c < n_blocks ? s_tot[c] : 0.f, carry);
+      const float before =
+          __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(carry), __float_as_int(incl), 0x138, 0xf, 0xf, false));
+      if (c < n_blocks) s_before[c] = before;
+      carry = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(incl), PKV_WAVE - 1));
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int c = wave + 16 * j;
+    if (c < n_blocks) {
+      const int64_t i = (int64_t)c * PKV_WAVE + lane;
+      const uint64_t hit = __ballot(i < k_out && sl_benefit + (s_before[c] + run[j]) >= tgt);
+      if (hit && lane == 0) atomicMin(s_k, (uint32_t)(c * PKV_WAVE + __ffsll((long long)hit)));
+    }
+  }
+  __syncthreads();
+  return (int64_t)*s_k;
+}
+
+// Joint maximum of the partial maxima and sum of the per-slice sums of a row, the sums in slice order
+// starting from the first.  All 1024 threads call it (one barrier); s_out: 2 floats.
+__device__ __forceinline__ void combine_slices(const float *__restrict__ pmax, int n_parts,
+                                               const float *__restrict__ ssum, int n_slices, float *s_out, float &g,
+                                               float &csum) {
+  if (threadIdx.x < PKV_WAVE) {
+    const int lane = pkv_lane();
+    float m = -__uint_as_float(0x7f800000u), carry = 0.f;
+    for (int i = lane; i < n_parts; i += PKV_WAVE) m = fmaxf(m, pmax[i]);
+    for (int base = 0; base < n_slices; base += PKV_WAVE) {
+      const int i = base + lane;
+      const float acc = wave_running_sum(i < n_slices ? ssum[i] : 0.f, carry);
+      carry = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(acc), PKV_WAVE - 1));
+    }
+#pragma unroll
+    for (int x = 1; x < PKV_WAVE; x <<= 1) m = fmaxf(m, __shfl_xor(m, x, PKV_WAVE));
+    if (lane == 0) s_out[0] = m, s_out[1] = carry;
+  }
+  __syncthreads();
+  g = s_out[0];
+  csum = s_out[1];
+}
+
+// Shared tail: s_keys[0 .. P) holds the k_out winners (zero padded, any order).  Sorts them, finds k,
+// writes adaptive_k[row] and the candidate ids in benefit order.
+__device__ __forceinline__ void adaptive_tail(uint64_t *s_keys, int P, int64_t k_out, float sl_benefit, float total,
+                                              float threshold, const int64_t *__restrict__ ci, int64_t n_cand,
+                                              int64_t *__restrict__ adaptive_k_row, int64_t *__restrict__ ids_row,
+                                              float *s_f, uint32_t *s_k) {
+#define PKV_SORT_K(NT, E) sort_lds_keys_and_emit<NT, E>(s_keys, 0, nullptr, nullptr, s_keys)
+  PKV_DISPATCH_E(P, PKV_SORT_K);
+#undef PKV_SORT_K
+  int64_t k = 1;  // total <= 0: adaptive_topk.py:304-306
+  if (total > 0.f) k = first_k_reaching(s_keys, k_out, sl_benefit, threshold * total, s_f, s_k);
+  if (threadIdx.x == 0) *adaptive_k_row = k;
+  for (int64_t i = threadIdx.x; i < k_out; i += kTopkThreads) {
+    const uint32_t pos = ~(uint32_t)s_keys[i];
+    ids_row[i] = (pos < (uint64_t)n_cand) ? ci[pos] : 0;
+  }
+}
+
+struct AdkRow {  // one row's operands
+  const float *sll, *slv;
+  const char *cs;
+  const int64_t *ci;
+  const float *cv, *vn;
+};
+
+__device__ __forceinline__ AdkRow adk_row(int row, const float *sl_logits, int64_t sl_stride, const float *sl_vnorm,
+                                          int64_t slv_stride, const void *cand_scores, int cand_dtype,
+                                          const float *cand_vnorm, const float *value_norm, int64_t vn_stride,
+                                          const int64_t *cand_ids, int64_t n_cand) {
+  AdkRow r;
+  r.sll = sl_logits + (int64_t)row * sl_stride;
+  r.slv = sl_vnorm + (int64_t)row * slv_stride;
+  r.cs = (const char *)cand_scores + (int64_t)row * n_cand * (cand_dtype == PKV_DTYPE_BF16 ? 2 : 4);
+  r.ci = cand_ids + (int64_t)row * n_cand;
+  r.cv = cand_vnorm ? cand_vnorm + (int64_t)row * n_cand : nullptr;
+  r.vn = value_norm ? value_norm + (int64_t)row * vn_stride : nullptr;
+  return r;
+}
+
+// n_cand <= 1024*EIN <= 8192: one workgroup per row, everything in registers.  Dynamic LDS P*8 bytes
+// (P = pow2 >= k_out, at least 1024 keys).
+template <int EIN>
 __global__ __launch_bounds__(kTopkThreads) void pkv_adaptive_topk_kernel(
     const float *__restrict__ sl_logits, int64_t sl_stride, const float *__restrict__ sl_vnorm, int64_t slv_stride,
     int64_t sl, const void *__restrict__ cand_scores, int cand_dtype, float cand_scale,
     const float *__restrict__ cand_vnorm, const float *__restrict__ value_norm, int64_t vn_stride, int64_t vn_offset,
-    const int64_t *__restrict__ cand_ids, int64_t n_cand, float threshold, int64_t k_out, int P,
-    int64_t *__restrict__ adaptive_k, int64_t *__restrict__ topk_ids, float *__restrict__ ws_ben) {
+    const int64_t *__restrict__ cand_ids, int n_cand, float threshold, int64_t k_out, int P,
+    int64_t *__restrict__ adaptive_k, int64_t *__restrict__ topk_ids) {
   extern __shared__ uint64_t s_keys[];
   __shared__ float s_part[16];
   __shared__ uint32_t s_hist[512];
@@ -725,68 +1028,195 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adaptive_topk_kernel(
   __shared__ uint32_t s_counter;
   const int row = blockIdx.x;
   const int tid = threadIdx.x;
-  const float *sll = sl_logits + (int64_t)row * sl_stride;
-  const float *slv = sl_vnorm + (int64_t)row * slv_stride;
-  const char *cs = (const char *)cand_scores + (int64_t)row * n_cand * (cand_dtype == PKV_DTYPE_BF16 ? 2 : 4);
-  const int64_t *ci = cand_ids + (int64_t)row * n_cand;
-  const float *cv = cand_vnorm ? cand_vnorm + (int64_t)row * n_cand : nullptr;
-  const float *vn = value_norm ? value_norm + (int64_t)row * vn_stride : nullptr;
-  float *ben = ws_ben + (int64_t)row * n_cand;
-
-  // joint max of the dense (sink/local) logits and the candidate logits
+  const AdkRow r = adk_row(row, sl_logits, sl_stride, sl_vnorm, slv_stride, cand_scores, cand_dtype, cand_vnorm,
+                           value_norm, vn_stride, cand_ids, n_cand);
+  // candidate logits and value norms: element i = tid + e*1024, so a lane adds its elements in increasing i
+  float logit[EIN], vnorm[EIN];
+#pragma unroll
+  for (int e = 0; e < EIN; ++e) {
+    const int i = tid + e * kTopkThreads, ii = i < n_cand ? i : n_cand - 1;  // clamped: the loads carry no branch
+    const float lg = cand_logit(r.cs, cand_dtype, cand_scale, ii);
+    const float vv = r.cv ? r.cv[ii] : r.vn[r.ci[ii] + vn_offset];
+    logit[e] = i < n_cand ? lg : -__uint_as_float(0x7f800000u);
+    vnorm[e] = i < n_cand ? vv : 0.f;
+  }
   float m = -__uint_as_float(0x7f800000u);
-  for (int64_t i = tid; i < sl; i += kTopkThreads) m = fmaxf(m, sll[i]);
-  for (int64_t i = tid; i < n_cand; i += kTopkThreads) m = fmaxf(m, cand_logit(cs, cand_dtype, cand_scale, i));
-  const float g = block_max_1024(m, s_part);
-
+  for (int64_t i = tid; i < sl; i += kTopkThreads) m = fmaxf(m, r.sll[i]);
+#pragma unroll
+  for (int e = 0; e < EIN; ++e) m = fmaxf(m, logit[e]);
+  const float g = block_max_1024(m, s_part);  // joint max (adaptive_topk.py:282-286)
+  const float sl_benefit = dense_benefit_sum(r.sll, r.slv, sl, g, s_part);
+  uint64_t v[EIN];
   float acc = 0.f;
-  for (int64_t i = tid; i < sl; i += kTopkThreads) acc = acc + pkv_expf(sll[i] - g) * slv[i];
-  const float sl_benefit = block_tree_sum_1024(acc, s_part);
-  acc = 0.f;
-  for (int64_t i = tid; i < n_cand; i += kTopkThreads) {
-    const float vnorm = cv ? cv[i] : vn[ci[i] + vn_offset];
-    const float b = pkv_expf(cand_logit(cs, cand_dtype, cand_scale, i) - g) * vnorm;
-    ben[i] = b;
+#pragma unroll
+  for (int e = 0; e < EIN; ++e) {
+    const int i = tid + e * kTopkThreads;
+    const float b = i < n_cand ? pkv_expf(logit[e] - g) * vnorm[e] : 0.f;
     acc = acc + b;
+    v[e] = i < n_cand ? (((uint64_t)pkv_ordered_u32(b) << 32) | (uint64_t)(~(uint32_t)i)) : 0ull;
   }
   const float total = sl_benefit + block_tree_sum_1024(acc, s_part);
-  __syncthreads();  // ben[] of this row is complete (written and read by this workgroup only)
 
   // the k_out largest (benefit, ~position) keys
-  auto key_of = [&](int64_t i) { return make_key(ben, nullptr, i); };
   if (tid == 0) s_counter = 0;
   for (int i = tid; i < (P < 1024 ? 1024 : P); i += kTopkThreads) s_keys[i] = 0ull;
-  uint64_t prefix;
-  int shift;
-  radix_select_streamed(key_of, n_cand, (uint32_t)k_out, s_hist, s_bcast, prefix, shift);
-  collect_winners_streamed(key_of, n_cand, (uint32_t)k_out, prefix, shift, &s_counter, s_keys);
+  uint64_t prefix = 0;
+  int shift = 0;
+  if (k_out < n_cand) radix_select_regs<EIN>(v, (uint32_t)k_out, s_hist, s_bcast, prefix, shift);
+  else __syncthreads();
+#pragma unroll
+  for (int e = 0; e < EIN; ++e) {
+    const bool win = v[e] != 0ull && (v[e] >> shift) >= (prefix >> shift);
+    const uint32_t slot = wave_take_slots(&s_counter, win);
+    if (win && slot < (uint32_t)k_out) s_keys[slot] = v[e];
+  }
   __syncthreads();
-#define PKV_SORT_K(NT, E) sort_lds_keys_and_emit<NT, E>(s_keys, 0, nullptr, nullptr, s_keys)
-  PKV_DISPATCH_E(P, PKV_SORT_K);
-#undef PKV_SORT_K
+  adaptive_tail(s_keys, P, k_out, sl_benefit, total, threshold, r.ci, n_cand, adaptive_k + row,
+                topk_ids + (int64_t)row * k_out, (float *)s_hist, &s_counter);
+}
 
-  // smallest k with sl_benefit + cumsum_k >= threshold * total (sequential fp32 cumsum)
-  if (tid == 0) {
-    int64_t k = k_out;
-    if (total <= 0.f) {
-      k = 1;
-    } else {
-      float csum = 0.f;
-      const float tgt = threshold * total;
-      for (int64_t i = 0; i < k_out; ++i) {
-        csum = csum + pkv_from_ordered_u32((uint32_t)(s_keys[i] >> 32));
-        if (sl_benefit + csum >= tgt) {
-          k = i + 1;
-          break;
-        }
-      }
+// ---- n_cand > 8192: slices of 8192 candidates, one workgroup each ----
+// Workspace per row: ben f32 [n_cand]; gathered norms f32 [n_cand]; partial maxima f32 [n_cand/2048];
+// slice sums f32 [n_slices];
+// control block u32 [kWideRowWords]; list A u64 [k_out]; list B u64 [n_cand].
+
+struct BenefitKeys {  // key i = (benefit, ~position)
+  const float *ben;
+  __device__ __forceinline__ uint64_t operator()(int64_t i) const { return make_key(ben, nullptr, i); }
+};
+
+// grid (parts, rows) x 256 threads, 2048 candidates per workgroup: partial maxima of the logits (part 0 also
+// covers the dense logits and clears the row's control block for the later launches) and, when the value
+// norms come from the per-position table, the candidates' norms gathered into ws_vn.  The gather is a
+// random 4-byte read per candidate and is bound by how many misses one CU keeps in flight, hence the
+// small workgroups: they spread it over the whole chip.
+constexpr int kAdkPart = 2048;
+constexpr int kAdkPartThreads = 256;
+
+__global__ __launch_bounds__(kAdkPartThreads) void pkv_adk_max_gather_kernel(
+    const float *__restrict__ sl_logits, int64_t sl_stride, int64_t sl, const void *__restrict__ cand_scores,
+    int cand_dtype, float cand_scale, const float *__restrict__ value_norm, int64_t vn_stride, int64_t vn_offset,
+    const int64_t *__restrict__ cand_ids, int64_t n_cand, float *__restrict__ ws_max, float *__restrict__ ws_vn,
+    uint32_t *__restrict__ ctl) {
+  __shared__ float s_part[kAdkPartThreads / PKV_WAVE];
+  const int row = blockIdx.y, part = blockIdx.x, tid = threadIdx.x;
+  const char *cs = (const char *)cand_scores + (int64_t)row * n_cand * (cand_dtype == PKV_DTYPE_BF16 ? 2 : 4);
+  constexpr int E = kAdkPart / kAdkPartThreads;
+  if (value_norm) {
+    const int64_t *ci = cand_ids + (int64_t)row * n_cand;
+    const float *vn = value_norm + (int64_t)row * vn_stride;
+    float vv[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int64_t i = (int64_t)part * kAdkPart + e * kAdkPartThreads + tid;
+      vv[e] = vn[ci[i < n_cand ? i : n_cand - 1] + vn_offset];
     }
-    adaptive_k[row] = k;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int64_t i = (int64_t)part * kAdkPart + e * kAdkPartThreads + tid;
+      if (i < n_cand) ws_vn[(int64_t)row * n_cand + i] = vv[e];
+    }
   }
-  for (int64_t i = tid; i < k_out; i += kTopkThreads) {
-    const uint32_t pos = ~(uint32_t)s_keys[i];
-    topk_ids[(int64_t)row * k_out + i] = (pos < (uint64_t)n_cand) ? ci[pos] : 0;
+  float m = -__uint_as_float(0x7f800000u);
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const int64_t i = (int64_t)part * kAdkPart + e * kAdkPartThreads + tid;
+    const float lg = cand_logit(cs, cand_dtype, cand_scale, i < n_cand ? i : n_cand - 1);
+    m = fmaxf(m, lg);  // a clamped index repeats the row's last candidate: harmless for a maximum
   }
+  if (part == 0) {
+    const float *sll = sl_logits + (int64_t)row * sl_stride;
+    for (int64_t i = tid; i < sl; i += kAdkPartThreads) m = fmaxf(m, sll[i]);
+    for (int i = tid; i < kWideRowWords; i += kAdkPartThreads) ctl[(int64_t)row * kWideRowWords + i] = 0;
+  }
+#pragma unroll
+  for (int x = 1; x < PKV_WAVE; x <<= 1) m = fmaxf(m, __shfl_xor(m, x, PKV_WAVE));
+  if (pkv_lane() == 0) s_part[tid / PKV_WAVE] = m;
+  __syncthreads();
+  if (tid == 0) {
+#pragma unroll
+    for (int w = 1; w < kAdkPartThreads / PKV_WAVE; ++w) m = fmaxf(m, s_part[w]);
+    ws_max[(int64_t)row * gridDim.x + part] = m;
+  }
+}
+
+// grid (slices, rows) x 1024: benefits of the slice into ws_ben, their sum (lane order, then the 1024-lane tree)
+// into ws_sum, and their top key bits into the row histogram.
+__global__ __launch_bounds__(kTopkThreads) void pkv_adk_benefit_kernel(
+    const void *__restrict__ cand_scores, int cand_dtype, float cand_scale, const float *__restrict__ cand_vnorm,
+    int64_t n_cand, const float *__restrict__ ws_max, int n_parts, float *__restrict__ ws_ben,
+    float *__restrict__ ws_sum, uint32_t *__restrict__ ctl) {
+  __shared__ float s_part[16];
+  __shared__ uint32_t s_bins[kWideBins];
+  const int row = blockIdx.y, slice = blockIdx.x, tid = threadIdx.x, n_slices = gridDim.x;
+  const char *cs = (const char *)cand_scores + (int64_t)row * n_cand * (cand_dtype == PKV_DTYPE_BF16 ? 2 : 4);
+  const float *cv = cand_vnorm + (int64_t)row * n_cand;  // the caller's, or the ones gathered by the first launch
+  float *ben = ws_ben + (int64_t)row * n_cand;
+  float g = -__uint_as_float(0x7f800000u);
+  for (int w = tid & (PKV_WAVE - 1); w < n_parts; w += PKV_WAVE) g = fmaxf(g, ws_max[(int64_t)row * n_parts + w]);
+#pragma unroll
+  for (int x = 1; x < PKV_WAVE; x <<= 1) g = fmaxf(g, __shfl_xor(g, x, PKV_WAVE));
+  float lg[kWideE], vv[kWideE];
+#pragma unroll
+  for (int e = 0; e < kWideE; ++e) {
+    const int64_t i = (int64_t)slice * kWideSlice + e * kTopkThreads + tid, ii = i < n_cand ? i : n_cand - 1;
+    lg[e] = cand_logit(cs, cand_dtype, cand_scale, ii);
+    vv[e] = cv[ii];
+  }
+  float acc = 0.f;
+  uint64_t keys[kWideE];
+#pragma unroll
+  for (int e = 0; e < kWideE; ++e) {
+    const int64_t i = (int64_t)slice * kWideSlice + e * kTopkThreads + tid;
+    const float b = pkv_expf(lg[e] - g) * vv[e];
+    keys[e] = 0ull;
+    if (i < n_cand) {
+      ben[i] = b;
+      acc = acc + b;
+      keys[e] = ((uint64_t)pkv_ordered_u32(b) << 32) | (uint64_t)(~(uint32_t)i);
+    }
+  }
+  const float ssum = block_tree_sum_1024(acc, s_part);
+  if (tid == 0) ws_sum[(int64_t)row * n_slices + slice] = ssum;
+  wide_hist_slice<52>(keys, n_cand, slice, s_bins, ctl + (int64_t)row * kWideRowWords);
+}
+
+__global__ __launch_bounds__(kTopkThreads) void pkv_adk_compact_kernel(const float *__restrict__ ws_ben, int64_t n_cand,
+                                                                       int64_t k_out, uint32_t *__restrict__ ctl,
+                                                                       uint64_t *__restrict__ list_a,
+                                                                       uint64_t *__restrict__ list_b) {
+  __shared__ uint32_t s_tmp[24];
+  const int row = blockIdx.y;
+  uint64_t keys[kWideE];
+  wide_load_keys(BenefitKeys{ws_ben + (int64_t)row * n_cand}, n_cand, blockIdx.x, keys);
+  wide_compact_slice<52>(keys, n_cand, blockIdx.x, (uint32_t)k_out,
+                         ctl + (int64_t)row * kWideRowWords, list_a + (int64_t)row * k_out,
+                         list_b + (int64_t)row * n_cand, s_tmp);
+}
+
+// grid rows; dynamic LDS max(P,1024)*8 bytes.
+__global__ __launch_bounds__(kTopkThreads) void pkv_adk_finish_kernel(
+    const float *__restrict__ sl_logits, int64_t sl_stride, const float *__restrict__ sl_vnorm, int64_t slv_stride,
+    int64_t sl, const int64_t *__restrict__ cand_ids, int64_t n_cand, int n_slices, int n_parts, float threshold,
+    int64_t k_out, int P,
+    const float *__restrict__ ws_max, const float *__restrict__ ws_sum, const uint32_t *__restrict__ ctl,
+    const uint64_t *__restrict__ list_a, const uint64_t *__restrict__ list_b, int64_t *__restrict__ adaptive_k,
+    int64_t *__restrict__ topk_ids) {
+  extern __shared__ uint64_t s_keys[];
+  __shared__ float s_part[16];
+  __shared__ uint32_t s_hist[512];
+  __shared__ uint32_t s_bcast[8];
+  __shared__ uint32_t s_counter;
+  const int row = blockIdx.x;
+  float g, csum;
+  combine_slices(ws_max + (int64_t)row * n_parts, n_parts, ws_sum + (int64_t)row * n_slices, n_slices, s_part, g, csum);
+  const float sl_benefit = dense_benefit_sum(sl_logits + (int64_t)row * sl_stride, sl_vnorm + (int64_t)row * slv_stride,
+                                             sl, g, s_part);
+  const float total = sl_benefit + csum;
+  wide_finish_select((uint32_t)k_out, P, ctl + (int64_t)row * kWideRowWords, list_a + (int64_t)row * k_out,
+                     list_b + (int64_t)row * n_cand, n_cand, s_keys, s_hist, s_bcast, &s_counter);
+  adaptive_tail(s_keys, P, k_out, sl_benefit, total, threshold, cand_ids + (int64_t)row * n_cand, n_cand,
+                adaptive_k + row, topk_ids + (int64_t)row * k_out, (float *)s_hist, &s_counter);
 }
 
 static size_t lds_bytes(int P) { return (size_t)(P < 1024 ? 1024 : P) * 8; }
@@ -892,18 +1322,38 @@ extern "C" int pkv_bucket_topk(const int32_t *x, int64_t x_stride, int rows, int
   return pkv_launch_select(cnt, cs, row_suf, hist, ck, rows, len, k, out, s);
 }
 
-size_t pkv_topk_ws_bytes_impl(int, int64_t, int64_t) { return 256; }
+// Wide rows (len > 8192): control blocks, list A [rows][k], list B [rows][len].
+struct WideWs {
+  size_t ctl, list_a, list_b, total;
+};
+static WideWs wide_ws_layout(int rows, int64_t len, int64_t k, size_t off) {
+  WideWs w;
+  w.ctl = off = pkv_align_up(off, 256);
+  off += (size_t)rows * kWideRowWords * sizeof(uint32_t);
+  w.list_a = off = pkv_align_up(off, 256);
+  off += (size_t)rows * (size_t)k * sizeof(uint64_t);
+  w.list_b = off = pkv_align_up(off, 256);
+  off += (size_t)rows * (size_t)len * sizeof(uint64_t);
+  w.total = pkv_align_up(off, 256);
+  return w;
+}
+
+size_t pkv_topk_ws_bytes_impl(int rows, int64_t len, int64_t k) {
+  if (rows <= 0 || len <= kTopkMaxSort || k <= 0) return 256;
+  return wide_ws_layout(rows, len, k, 0).total;
+}
 
 extern "C" size_t pkv_topk_f32_ws_bytes(int rows, int64_t len, int64_t k) {
   return pkv_topk_ws_bytes_impl(rows, len, k);
 }
 
 int pkv_launch_topk_f32(const float *x, int64_t x_stride, const int64_t *ids, int64_t ids_stride, int rows,
-                        int64_t len, int64_t k, int64_t *out_ids, float *out_vals, void *, size_t, hipStream_t s) {
+                        int64_t len, int64_t k, int64_t *out_ids, float *out_vals, void *ws, size_t ws_bytes,
+                        hipStream_t s) {
   PKV_REQUIRE(x && out_ids, "pkv_topk_f32: null pointer");
   PKV_REQUIRE(k > 0, "k must be positive");
   PKV_REQUIRE(k <= len, "k cannot exceed sequence length");
-  PKV_REQUIRE(rows > 0 && len < ((int64_t)1 << 31), "bad shape rows=%d len=%lld", rows, (long long)len);
+  PKV_REQUIRE(rows > 0 && rows <= 65535 && len < ((int64_t)1 << 31), "bad shape rows=%d len=%lld", rows, (long long)len);
   if (len <= kTopkMaxSort && pow2_ceil(k) * 2 <= pow2_ceil(len) && pow2_ceil(len) >= 2048) {
     const int P = pow2_ceil(k);
     const int ein = pow2_ceil(len) / kTopkThreads;
@@ -921,10 +1371,28 @@ int pkv_launch_topk_f32(const float *x, int64_t x_stride, const int64_t *ids, in
   } else {
     PKV_REQUIRE(k <= kTopkMaxSort, "k up to %d supported when len > %d (got %lld)", kTopkMaxSort, kTopkMaxSort,
                 (long long)k);
+    const size_t need = pkv_topk_ws_bytes_impl(rows, len, k);
+    if (!ws || ws_bytes < need || !pkv_aligned(ws, 256)) {
+      pkv_set_error("pkv_topk_f32: rows of more than %d keys need a workspace of %zu bytes (256-aligned), got %zu",
+                    kTopkMaxSort, need, ws_bytes);
+      return PKV_ENOMEM;
+    }
+    const WideWs w = wide_ws_layout(rows, len, k, 0);
+    uint32_t *ctl = (uint32_t *)((char *)ws + w.ctl);
+    uint64_t *list_a = (uint64_t *)((char *)ws + w.list_a), *list_b = (uint64_t *)((char *)ws + w.list_b);
     const int P = pow2_ceil(k);
-    hipLaunchKernelGGL(pkv_topk_radix_kernel, dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes(P), s, x,
-                       x_stride, ids, ids_stride, len, P, k, out_ids, out_vals);
-    PKV_LAUNCH_CHECK("pkv_topk_radix_kernel");
+    const dim3 grid((unsigned)((len + kWideSlice - 1) / kWideSlice), (unsigned)rows);
+    hipLaunchKernelGGL(pkv_zero_u32_kernel, dim3((unsigned)((rows * kWideRowWords + 255) / 256)), dim3(256), 0, s, ctl,
+                       (int64_t)rows * kWideRowWords);
+    PKV_LAUNCH_CHECK("pkv_zero_u32_kernel");
+    hipLaunchKernelGGL(pkv_topk_wide_hist_kernel, grid, dim3(kTopkThreads), 0, s, x, x_stride, ids, ids_stride, len, ctl);
+    PKV_LAUNCH_CHECK("pkv_topk_wide_hist_kernel");
+    hipLaunchKernelGGL(pkv_topk_wide_compact_kernel, grid, dim3(kTopkThreads), 0, s, x, x_stride, ids, ids_stride, len, k,
+                       ctl, list_a, list_b);
+    PKV_LAUNCH_CHECK("pkv_topk_wide_compact_kernel");
+    hipLaunchKernelGGL(pkv_topk_wide_finish_kernel, dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes(P), s, len, P, k,
+                       ctl, list_a, list_b, out_ids, out_vals);
+    PKV_LAUNCH_CHECK("pkv_topk_wide_finish_kernel");
   }
   return PKV_OK;
 }
@@ -936,9 +1404,31 @@ extern "C" int pkv_topk_f32(const float *x, int64_t x_stride, const int64_t *ids
                              (hipStream_t)stream);
 }
 
-extern "C" size_t pkv_adaptive_topk_ws_bytes(int rows, int64_t n_cand, int64_t) {
-  if (rows <= 0 || n_cand <= 0) return 256;
-  return pkv_align_up((size_t)rows * (size_t)n_cand * sizeof(float), 256);
+struct AdkWs {
+  size_t ben, vn, smax, ssum;
+  WideWs wide;
+  size_t total;
+};
+static AdkWs adk_ws_layout(int rows, int64_t n_cand, int64_t k_out) {
+  AdkWs w;
+  const size_t n_slices = (size_t)((n_cand + kWideSlice - 1) / kWideSlice);
+  size_t off = 0;
+  w.ben = off;
+  off = pkv_align_up(off + (size_t)rows * (size_t)n_cand * sizeof(float), 256);
+  w.vn = off;
+  off = pkv_align_up(off + (size_t)rows * (size_t)n_cand * sizeof(float), 256);
+  w.smax = off;
+  off = pkv_align_up(off + (size_t)rows * (size_t)((n_cand + kAdkPart - 1) / kAdkPart) * sizeof(float), 256);
+  w.ssum = off;
+  off = pkv_align_up(off + (size_t)rows * n_slices * sizeof(float), 256);
+  w.wide = wide_ws_layout(rows, n_cand, k_out, off);
+  w.total = w.wide.total;
+  return w;
+}
+
+extern "C" size_t pkv_adaptive_topk_ws_bytes(int rows, int64_t n_cand, int64_t k_out) {
+  if (rows <= 0 || n_cand <= kTopkMaxSort || k_out <= 0) return 256;
+  return adk_ws_layout(rows, n_cand, k_out).total;
 }
 
 extern "C" int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, const float *sl_vnorm, int64_t slv_stride,
@@ -950,19 +1440,48 @@ extern "C" int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, cons
               "pkv_adaptive_topk: null pointer");
   PKV_REQUIRE(sl >= 0 && (sl == 0 || (sl_logits && sl_vnorm)), "pkv_adaptive_topk: dense logits missing");
   PKV_REQUIRE(cand_dtype == PKV_DTYPE_F32 || cand_dtype == PKV_DTYPE_BF16, "unknown candidate score dtype %d", cand_dtype);
-  PKV_REQUIRE(rows > 0 && n_cand > 0 && n_cand < ((int64_t)1 << 31) && k_out > 0 && k_out <= n_cand,
+  PKV_REQUIRE(rows > 0 && rows <= 65535 && n_cand > 0 && n_cand < ((int64_t)1 << 31) && k_out > 0 && k_out <= n_cand,
               "need 0 < k_out <= n_cand (k_out=%lld n_cand=%lld rows=%d)", (long long)k_out, (long long)n_cand, rows);
   PKV_REQUIRE(k_out <= kTopkMaxSort, "k_out up to %d supported (got %lld)", kTopkMaxSort, (long long)k_out);
-  const size_t need = pkv_adaptive_topk_ws_bytes(rows, n_cand, k_out);
-  if (!ws || ws_bytes < need || !pkv_aligned(ws, 16)) {
-    pkv_set_error("pkv_adaptive_topk: workspace of %zu bytes required, got %zu", need, ws_bytes);
+  hipStream_t s = (hipStream_t)stream;
+  const int P = pow2_ceil(k_out);
+  if (n_cand <= kTopkMaxSort) {  // one workgroup per row, no workspace
+    const int ein = pow2_ceil(n_cand) / kTopkThreads;
+#define PKV_ADK(EIN)                                                                                                  \
+  hipLaunchKernelGGL((pkv_adaptive_topk_kernel<EIN>), dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes(P), s,      \
+                     sl_logits, sl_stride, sl_vnorm, slv_stride, sl, cand_scores, cand_dtype, cand_scale, cand_vnorm, \
+                     value_norm, vn_stride, vn_offset, cand_ids, (int)n_cand, threshold, k_out, P, adaptive_k, topk_ids)
+    if (ein <= 1) PKV_ADK(1); else if (ein == 2) PKV_ADK(2); else if (ein == 4) PKV_ADK(4); else PKV_ADK(8);
+#undef PKV_ADK
+    PKV_LAUNCH_CHECK("pkv_adaptive_topk_kernel");
+    return PKV_OK;
+  }
+  const AdkWs w = adk_ws_layout(rows, n_cand, k_out);
+  if (!ws || ws_bytes < w.total || !pkv_aligned(ws, 256)) {
+    pkv_set_error("pkv_adaptive_topk: workspace of %zu bytes (256-aligned) required, got %zu", w.total, ws_bytes);
     return PKV_ENOMEM;
   }
-  const int P = pow2_ceil(k_out);
-  hipLaunchKernelGGL(pkv_adaptive_topk_kernel, dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes(P),
-                     (hipStream_t)stream, sl_logits, sl_stride, sl_vnorm, slv_stride, sl, cand_scores, cand_dtype,
-                     cand_scale, cand_vnorm, value_norm, vn_stride, vn_offset, cand_ids, n_cand, threshold, k_out, P,
-                     adaptive_k, topk_ids, (float *)ws);
-  PKV_LAUNCH_CHECK("pkv_adaptive_topk_kernel");
+  char *base = (char *)ws;
+  float *ben = (float *)(base + w.ben), *smax = (float *)(base + w.smax), *ssum = (float *)(base + w.ssum);
+  uint32_t *ctl = (uint32_t *)(base + w.wide.ctl);
+  uint64_t *list_a = (uint64_t *)(base + w.wide.list_a), *list_b = (uint64_t *)(base + w.wide.list_b);
+  float *gathered = (float *)(base + w.vn);
+  const int n_slices = (int)((n_cand + kWideSlice - 1) / kWideSlice);
+  const int n_parts = (int)((n_cand + kAdkPart - 1) / kAdkPart);
+  const dim3 grid((unsigned)n_slices, (unsigned)rows);
+  hipLaunchKernelGGL(pkv_adk_max_gather_kernel, dim3((unsigned)n_parts, (unsigned)rows), dim3(kAdkPartThreads), 0, s,
+                     sl_logits, sl_stride, sl, cand_scores, cand_dtype, cand_scale, cand_vnorm ? nullptr : value_norm,
+                     vn_stride, vn_offset, cand_ids, n_cand, smax, gathered, ctl);
+  PKV_LAUNCH_CHECK("pkv_adk_max_gather_kernel");
+  hipLaunchKernelGGL(pkv_adk_benefit_kernel, grid, dim3(kTopkThreads), 0, s, cand_scores, cand_dtype, cand_scale,
+                     cand_vnorm ? cand_vnorm : gathered, n_cand, smax, n_parts, ben, ssum, ctl);
+  PKV_LAUNCH_CHECK("pkv_adk_benefit_kernel");
+  hipLaunchKernelGGL(pkv_adk_compact_kernel, grid, dim3(kTopkThreads), 0, s, ben, n_cand, k_out, ctl, list_a, list_b);
+  PKV_LAUNCH_CHECK("pkv_adk_compact_kernel");
+  hipLaunchKernelGGL(pkv_adk_finish_kernel, dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes(P), s, sl_logits,
+                     sl_stride, sl_vnorm, slv_stride, sl, cand_ids, n_cand, n_slices, n_parts, threshold, k_out, P, smax, ssum,
+                     ctl,
+                     list_a, list_b, adaptive_k, topk_ids);
+  PKV_LAUNCH_CHECK("pkv_adk_finish_kernel");
   return PKV_OK;
 }

@@ -266,8 +266,10 @@ def topk_f32(x: torch.Tensor, k: int, ids: Optional[torch.Tensor] = None, want_v
         _need(ids.dtype == torch.int64 and tuple(ids.shape) == (rows, L) and ids.stride(1) == 1, "ids: int64 [rows,L]")
     out = torch.empty(rows, k, dtype=torch.int64, device=x.device)
     vals = torch.empty(rows, k, dtype=torch.float32, device=x.device) if want_values else None
+    nbytes = _lib.lib().pkv_topk_f32_ws_bytes(rows, L, k)   # 256 unless rows are wider than one workgroup sorts
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device) if nbytes > 256 else None
     _lib.check(_lib.lib().pkv_topk_f32(_p(x), x.stride(0), _p(ids), ids.stride(0) if ids is not None else 0, rows, L, k,
-                                       _p(out), _p(vals), None, 0, _stream(x)))
+                                       _p(out), _p(vals), _p(ws), nbytes if ws is not None else 0, _stream(x)))
     return (out, vals) if want_values else out
 
 

@@ -294,6 +294,37 @@ def test_topk_f32_exact(ops, rows, L, k):
     assert torch.equal(vals, tv)
 
 
+def test_topk_f32_wide_rows_edge_cases(ops):
+    """Rows wider than one workgroup sorts (more than 8192 keys): the multi-workgroup histogram / compaction
+    path with a threshold bin that holds the whole row (constant scores: every key ties, ids decide), one that
+    holds more than 8192 keys, k = 8192, len = 8193, and mixed signs with infinities."""
+    rng = np.random.default_rng(99)
+    cases = []
+    L = 30000
+    cases.append(("constant", np.full((2, L), 1.25, np.float32), 700))
+    x = rng.standard_normal((3, L)).astype(np.float32)
+    x[:, : L // 2] = np.float32(0.75) + rng.integers(0, 4, (3, L // 2)).astype(np.float32) * np.float32(2.0 ** -20)
+    cases.append(("crowded threshold bin", x, 9000 // 2))
+    cases.append(("k=8192", rng.standard_normal((2, 70000)).astype(np.float32), 8192))
+    cases.append(("len=8193", rng.standard_normal((5, 8193)).astype(np.float32), 100))
+    y = (rng.standard_normal((2, 20001)) * 1e3).astype(np.float32)
+    y[0, 5], y[0, 77], y[1, 20000] = np.inf, -np.inf, np.inf
+    y[:, 100:4000] = -np.abs(y[:, 100:4000])
+    cases.append(("signs and infinities", y, 3000))
+    for name, x, k in cases:
+        _say(f"topk_f32 wide: {name} {x.shape} k={k}")
+        rows, L = x.shape
+        ids = np.stack([rng.permutation(3 * L)[:L] for _ in range(rows)]).astype(np.int64)
+        out, vals = ops.topk_f32(torch.from_numpy(x).to(DEV), k, torch.from_numpy(ids).to(DEV), want_values=True)
+        torch.cuda.synchronize()
+        for r in range(rows):
+            ref_ids, ref_pos = O.topk_f32(x[r], ids[r], k)
+            assert np.array_equal(out[r].cpu().numpy(), ref_ids), name
+            assert np.array_equal(vals[r].cpu().numpy(), x[r][ref_pos]), name
+    with pytest.raises(RuntimeError, match="k up to"):
+        ops.topk_f32(torch.zeros(1, 20000, device=DEV), 8193)
+
+
 def test_radix_topk_float_api(ops):
     from pariskv_amd.cache_hub.topk import radix_topk, fast_topk, fast_topk_with_ratio
 
@@ -652,6 +683,55 @@ def test_adaptive_topk_value_norm_gather_and_edges(ops):
     ak, ids = ops.adaptive_topk(z[..., :1], one[..., :1], z, 1.0, torch.arange(50, device=DEV).flip(0).view(1, 1, 50).contiguous(),
                                 0.95, 10, cand_vnorm=one)
     assert int(ak) == 10 and ids[0, 0].cpu().tolist() == list(range(49, 39, -1))
+
+
+@pytest.mark.parametrize("sl,Cn,k_out,thr,mode", [(9000, 3000, 3000, 0.97, "cv"),       # dense sum over two slices, k_out == n_cand
+                                                  (0, 20000, 4096, 0.5, "cv"),          # no dense tokens, wide path, early k
+                                                  (300, 40000, 8192, 0.999, "gather"),  # wide path, largest k_out, norm gather
+                                                  (300, 8192, 1000, 0.6, "gather"),     # widest one-workgroup row
+                                                  (300, 8193, 1000, 0.6, "gather"),     # narrowest multi-workgroup row
+                                                  (50, 30000, 500, 0.9, "ties")])       # quantised benefits: crowded bins
+def test_adaptive_topk_shapes_and_orders(ops, sl, Cn, k_out, thr, mode):
+    """Adaptive-k against the CPU checker on shapes that exercise each summation / selection branch: k exact,
+    ids identical (both follow the same fixed orders)."""
+    _say(f"adaptive_topk sl={sl} C={Cn} k_out={k_out} thr={thr} {mode}")
+    g = torch.Generator().manual_seed(sl * 31 + Cn)
+    H, cap, off = 3, 50000, 17
+    sc = torch.randn(1, H, Cn, generator=g) * 6 + 4
+    if mode == "ties":
+        sc = torch.round(sc)
+    sll = torch.randn(1, H, sl, generator=g) * 2 + 6
+    slv = torch.rand(1, H, sl, generator=g) + 0.5
+    ci = torch.stack([torch.randperm(cap - off, generator=g)[:Cn] for _ in range(H)]).view(1, H, Cn)
+    scale = 0.25
+    if mode == "gather":
+        vn = torch.rand(1, H, cap, generator=g) + 0.5
+        ak, ids = ops.adaptive_topk(sll.to(DEV), slv.to(DEV), sc.to(DEV), scale, ci.to(DEV), thr, k_out,
+                                    value_norm=vn.to(DEV), vn_offset=off)
+        cv = torch.stack([vn[0, h][ci[0, h] + off] for h in range(H)]).view(1, H, Cn)
+    else:
+        cv = torch.rand(1, H, Cn, generator=g) + 0.5 if mode == "cv" else torch.ones(1, H, Cn)
+        ak, ids = ops.adaptive_topk(sll.to(DEV), slv.to(DEV), sc.to(DEV), scale, ci.to(DEV), thr, k_out, cand_vnorm=cv.to(DEV))
+    torch.cuda.synchronize()
+    ks = []
+    for h in range(H):
+        k_ref, ids_ref = O.adaptive_topk(sll[0, h].numpy(), slv[0, h].numpy(), (sc[0, h] * np.float32(scale)).numpy(),
+                                         cv[0, h].numpy(), ci[0, h].numpy(), thr, k_out)
+        assert int(ak[0, h]) == k_ref
+        assert np.array_equal(ids[0, h].cpu().numpy(), ids_ref)
+        ks.append(k_ref)
+    if thr <= 0.6:
+        assert max(ks) < k_out  # the threshold is reached inside the list in these cases
+
+
+def test_adaptive_topk_wide_zero_mass(ops):
+    """total <= 0 on the multi-workgroup path: k = 1 (adaptive_topk.py:304-306); ids still ordered by position."""
+    Cn = 10000
+    z = torch.zeros(1, 2, Cn, device=DEV)
+    ci = torch.arange(Cn, device=DEV).flip(0).expand(1, 2, Cn).contiguous()
+    ak, ids = ops.adaptive_topk(z[..., :7], z[..., :7], z, 1.0, ci, 0.95, 300, cand_vnorm=z)
+    assert ak.flatten().tolist() == [1, 1]
+    assert ids[0, 1].cpu().tolist() == list(range(Cn - 1, Cn - 301, -1))
 
 
 # ---------------------------------- BASELINE config 4: 1M keys, adaptive-k, packed gather
