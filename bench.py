@@ -47,8 +47,10 @@ def main():
     ap.add_argument("--candidates", type=int, default=4096)
     ap.add_argument("--topk", type=int, default=1024)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["scan", "copy"], default=None,
-                    help="profiling aid: launch only the collision scan (or the calibration copy) --steps times")
+    ap.add_argument("--only", choices=["scan", "copy", "adaptive"], default=None,
+                    help="profiling aid: launch only the collision scan, the calibration copy, or the adaptive-k stage "
+                         "(--candidates scores per row, dense prefix 1600, value norms gathered from a --context table, "
+                         "list length --topk) --steps times")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (rows would shard across GPUs by (batch, kv-head))",
@@ -65,6 +67,20 @@ def main():
     N, Cn, K, L = args.context, args.candidates, args.topk, args.layers
     R = bs * H
     lib = _lib.lib()
+
+    if args.only == "adaptive":
+        g = torch.Generator(device=dev).manual_seed(0)
+        scores = torch.randn(bs, H, Cn, generator=g, device=dev) * 20 + 30
+        cand = torch.stack([torch.randperm(N, generator=g, device=dev)[:Cn].sort().values for _ in range(R)]).view(bs, H, Cn)
+        vnorm = torch.rand(bs, H, N, generator=g, device=dev) + 0.5
+        sl_logits = torch.randn(bs, H, 1600, generator=g, device=dev) * 2
+        sl_vnorm = torch.rand(bs, H, 1600, generator=g, device=dev) + 0.5
+        for _ in range(args.warmup + args.steps):
+            ak, _ = ops.adaptive_topk(sl_logits, sl_vnorm, scores, 1.0 / math.sqrt(D), cand, 0.95, K, value_norm=vnorm)
+        torch.cuda.synchronize()
+        print(json.dumps({"only": "adaptive", "launches": args.warmup + args.steps, "rows": R, "candidates": Cn,
+                          "list": K, "adaptive_k_row0": int(ak.flatten()[0])}))
+        return
 
     # ---------------------------------------------------------------- inputs
     signs = ops.srht_signs(dev)
@@ -169,7 +185,16 @@ def main():
     att = ops.DecodeAttention(bs, H, G, 576 + K, dev)
     att_out = torch.empty(bs, 1, H * G, D, dtype=torch.bfloat16, device=dev)
     att_segs = [(dense_k, dense_v, 0, 64), (dst_k, dst_v, 0, K), (dense_k, dense_v, 64, 512)]
-    us_attn = timed(lambda i: att.run(layers[i % L]["q"], att_segs, out=att_out), args.steps)
+    att_args = [att.c_args(ly["q"], att_segs, out=att_out)[0] for ly in layers]   # validated once: the loop below
+    att_q = [C.c_void_p(ly["q"].data_ptr()) for ly in layers]                      # must not be bound by host time
+
+    def attention_only(i):
+        a = att_args[i % L]
+        lib.pkv_decode_attention(att_q[i % L], _lib.DTYPE_BF16, bs, H, G, a.segments, a.n_segments, None, a.scale, a.out,
+                                 a.ws, a.ws_bytes, stream)
+
+    att.run(layers[0]["q"], att_segs, out=att_out)  # checked call first
+    us_attn = timed(attention_only, args.steps)
 
     def step_with_attention(i):  # retrieval + gather + attention from one host call
         ly = layers[i % L]
