@@ -47,10 +47,13 @@ def main():
     ap.add_argument("--candidates", type=int, default=4096)
     ap.add_argument("--topk", type=int, default=1024)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["scan", "copy", "adaptive"], default=None,
+    ap.add_argument("--only", choices=["scan", "copy", "adaptive", "decode-loop"], default=None,
                     help="profiling aid: launch only the collision scan, the calibration copy, or the adaptive-k stage "
                          "(--candidates scores per row, dense prefix 1600, value norms gathered from a --context table, "
-                         "list length --topk) --steps times")
+                         "list length --topk) --steps times; decode-loop: the polar_cache class itself, --layers layers, "
+                         "--context prompt tokens, --steps generated tokens (append + retrieval + gather + attention per "
+                         "layer, index refresh and host offload every 1024 tokens)")
+    ap.add_argument("--no-offload", action="store_true", help="decode-loop: keep K/V in HBM (config 2's mode)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (rows would shard across GPUs by (batch, kv-head))",
@@ -67,6 +70,50 @@ def main():
     N, Cn, K, L = args.context, args.candidates, args.topk, args.layers
     R = bs * H
     lib = _lib.lib()
+
+    if args.only == "decode-loop":
+        from pariskv_amd.attn_hub import polar_decode_attn
+        from pariskv_amd.cache_hub.polar_cache import polar_cache
+
+        S, T = N, args.steps
+        cache = polar_cache(valid_start=[0] * bs, layer_num=L, batch_size=bs, max_length=S + T + 8, num_key_value_heads=H,
+                            num_heads=H * G, head_dim=D, dtype=torch.bfloat16, layer_mapping={i: dev for i in range(L)},
+                            max_new_length=T + 8, sink_size=64, local_size=512, core=1, nprobe=1, cache_unit_size=1,
+                            cache_cluster_num=1, num_gpus=1, model_size=8, final_topk=K, dynamic_update_interval=1024,
+                            full_attention_threshold=2000, enable_offload=not args.no_offload)
+        g = torch.Generator(device=dev).manual_seed(0)
+        t0 = time.perf_counter()
+        for l in range(L):
+            k = torch.randn(bs, S, H, D, generator=g, device=dev, dtype=torch.bfloat16)
+            k[..., [7, 31, 64, 101]] *= 10.0
+            v = torch.randn(bs, S, H, D, generator=g, device=dev, dtype=torch.bfloat16)
+            cache.prefill_update_kv_cache(None, k, v, l, 0)
+            del k, v
+        torch.cuda.synchronize()
+        t_prefill = time.perf_counter() - t0
+        k1 = torch.randn(T, bs, 1, H, D, generator=g, device=dev, dtype=torch.bfloat16)
+        v1 = torch.randn(T, bs, 1, H, D, generator=g, device=dev, dtype=torch.bfloat16)
+        q = torch.randn(bs, 1, H * G, D, generator=g, device=dev, dtype=torch.bfloat16)
+        torch.cuda.synchronize()
+        tok_us, issue = [], 0.0
+        for t in range(T):
+            a = time.perf_counter()
+            for l in range(L):
+                cache.decode_update_kv_cache(k1[t], v1[t], l)
+                polar_decode_attn(q, None, None, l, cache)
+            b = time.perf_counter()
+            torch.cuda.synchronize()
+            tok_us.append((time.perf_counter() - a) * 1e6)
+            issue += b - a
+        body = sorted(tok_us[8:])
+        print(json.dumps({"only": "decode-loop", "offload": not args.no_offload, "layers": L, "batch": bs, "prompt": S,
+                          "generated": T, "final_topk": K, "prefill_s": round(t_prefill, 2),
+                          "us_per_layer_step_median": round(body[len(body) // 2] / L, 1),
+                          "us_per_layer_step_mean": round(sum(tok_us[8:]) / len(tok_us[8:]) / L, 1),
+                          "us_per_layer_step_worst_token": round(body[-1] / L, 1),
+                          "host_issue_us_per_layer_step": round(issue * 1e6 / T / L, 1),
+                          "index_refreshes": T // 1024}))
+        return
 
     if args.only == "adaptive":
         g = torch.Generator(device=dev).manual_seed(0)

@@ -212,6 +212,21 @@ int pkv_append_kv(const void *k_new, const void *v_new, int64_t new_stride_b, in
                   void *dst_k, void *dst_v, int64_t dst_stride_b, int64_t dst_stride_h, int64_t dst_len,
                   int64_t slot, int bs, int n_kv_heads, int row_bytes, void *stream);
 
+/* The oldest tokens of a layer leave the GPU: replaces the copy_() of staged
+ * [bs][h][n][d] tensors into slices of the pinned host tensors on the side
+ * stream (cache_hub/polar_cache.py:457-471 at prefill, :778-799 at an index
+ * refresh), which torch executes as a strided device-to-host copy.  One
+ * kernel writes the rows through the host store's device mapping:
+ *   dst[(b,h)][dst_row0 + r] = src + b*src_stride_b + h*src_stride_h + r*src_stride_row
+ * for r < n_rows, K and V.  src: device memory, strides in BYTES (multiples
+ * of 16), so the model's [bs][seq][h][d] layout can be read in place;
+ * dst_k_host/dst_v_host: pinned, device-mapped host memory
+ * [bs][h][dst_len][row_bytes].  Asynchronous on `stream`; the host store is
+ * complete when the stream reaches the caller's next event. */
+int pkv_offload_rows(const void *src_k, const void *src_v, int64_t src_stride_b, int64_t src_stride_h,
+                     int64_t src_stride_row, void *dst_k_host, void *dst_v_host, int64_t dst_len,
+                     int64_t dst_row0, int64_t n_rows, int bs, int n_kv_heads, int row_bytes, void *stream);
+
 /* Ragged form used by the adaptive-k cache variant (kernel source absent from
  * the reference; contract from the call site
  * cache_hub/polar_cache_adaptivek_varlen.py:1634-1644, layout :1573-1586).

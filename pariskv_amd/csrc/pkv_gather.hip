@@ -86,6 +86,26 @@ __global__ __launch_bounds__(kGatherThreads) void pkv_append_rows_kernel(
   (kv ? dst_v : dst_k)[b * dst_stride_b + h * dst_stride_h + slot * vpr + lane] = val;
 }
 
+// Blocks of consecutive rows, one block per (batch, head), from the GPU into the pinned host store:
+// dst[(b,h)][dst_row0 + r] = src[(b,h)][r] for K and V.  16-byte vectors, a wave writes 1 KB of
+// consecutive host memory per instruction (posted PCIe writes).  grid-stride over all vectors.
+__global__ __launch_bounds__(kGatherThreads) void pkv_offload_rows_kernel(
+    const pkv_u32x4 *__restrict__ src_k, const pkv_u32x4 *__restrict__ src_v, int64_t src_stride_b,
+    int64_t src_stride_h, int64_t src_stride_row, pkv_u32x4 *__restrict__ dst_k, pkv_u32x4 *__restrict__ dst_v,
+    int64_t dst_len, int64_t dst_row0, int64_t n_rows, int n_heads, int64_t n_vec, int vpr) {
+  const int64_t per_head = n_rows * vpr;  // vectors of one (b, h) block
+  for (int64_t g = (int64_t)blockIdx.x * kGatherThreads + threadIdx.x; g < n_vec;
+       g += (int64_t)gridDim.x * kGatherThreads) {
+    const int64_t kvbh = g / per_head, in_block = g % per_head;
+    const int kv = (int)(kvbh & 1);
+    const int64_t bh = kvbh >> 1, b = bh / n_heads, h = bh % n_heads;
+    const int64_t row = in_block / vpr;
+    const int lane = (int)(in_block % vpr);
+    const pkv_u32x4 val = (kv ? src_v : src_k)[b * src_stride_b + h * src_stride_h + row * src_stride_row + lane];
+    (kv ? dst_v : dst_k)[(bh * dst_len + dst_row0 + row) * vpr + lane] = val;
+  }
+}
+
 // Plain streaming copy of n 16-byte vectors (calibration of HBM counters, tests).
 __global__ __launch_bounds__(256) void pkv_copy_kernel(const pkv_u32x4 *__restrict__ src, pkv_u32x4 *__restrict__ dst,
                                                        int64_t n) {
@@ -177,6 +197,33 @@ extern "C" int pkv_append_kv(const void *k_new, const void *v_new, int64_t new_s
                      new_stride_b / 16, new_stride_h / 16, (pkv_u32x4 *)dst_k, (pkv_u32x4 *)dst_v, dst_stride_b / 16,
                      dst_stride_h / 16, slot, n_kv_heads, n_tasks, vpr);
   PKV_LAUNCH_CHECK("pkv_append_rows_kernel");
+  return PKV_OK;
+}
+
+extern "C" int pkv_offload_rows(const void *src_k, const void *src_v, int64_t src_stride_b, int64_t src_stride_h,
+                                int64_t src_stride_row, void *dst_k_host, void *dst_v_host, int64_t dst_len,
+                                int64_t dst_row0, int64_t n_rows, int bs, int n_kv_heads, int row_bytes, void *stream) {
+  int rc = check_common(src_k, src_v, dst_k_host, dst_v_host, bs * n_kv_heads, row_bytes);
+  if (rc) return rc;
+  PKV_REQUIRE(bs > 0 && n_kv_heads > 0 && n_rows > 0 && dst_row0 >= 0 && dst_row0 + n_rows <= dst_len,
+              "offload: rows [%lld, %lld) outside the host store of %lld rows", (long long)dst_row0,
+              (long long)(dst_row0 + n_rows), (long long)dst_len);
+  PKV_REQUIRE(src_stride_b % 16 == 0 && src_stride_h % 16 == 0 && src_stride_row % 16 == 0 && src_stride_row >= row_bytes,
+              "offload: strides are bytes, multiples of 16");
+  const void *dk, *dv;
+  rc = device_view_of_host(dst_k_host, &dk);
+  if (rc) return rc;
+  rc = device_view_of_host(dst_v_host, &dv);
+  if (rc) return rc;
+  const int vpr = row_bytes / 16;
+  const int64_t n_vec = (int64_t)2 * bs * n_kv_heads * n_rows * vpr;
+  int64_t blocks = (n_vec + kGatherThreads - 1) / kGatherThreads;
+  if (blocks > 8192) blocks = 8192;
+  hipLaunchKernelGGL(pkv_offload_rows_kernel, dim3((unsigned)blocks), dim3(kGatherThreads), 0, (hipStream_t)stream,
+                     (const pkv_u32x4 *)src_k, (const pkv_u32x4 *)src_v, src_stride_b / 16, src_stride_h / 16,
+                     src_stride_row / 16, (pkv_u32x4 *)const_cast<void *>(dk), (pkv_u32x4 *)const_cast<void *>(dv), dst_len,
+                     dst_row0, n_rows, n_kv_heads, n_vec, vpr);
+  PKV_LAUNCH_CHECK("pkv_offload_rows_kernel");
   return PKV_OK;
 }
 

@@ -390,6 +390,26 @@ def append_kv(key_states, value_states, dst_k, dst_v, slot: int) -> None:
         D * es, _stream(dst_k)))
 
 
+def offload_rows(src_k, src_v, dst_k_cpu, dst_v_cpu, dst_row0: int, stream=None) -> None:
+    """dst_cpu[:, :, dst_row0:dst_row0+n] = src for K and V in one launch on ``stream`` (default: the current one).
+    src_k/src_v: GPU [bs,H,n,D] views with any batch / head / row strides (last dim contiguous); dst_*_cpu: pinned
+    CPU [bs,H,rows,D] (a batch slice of a contiguous tensor is fine).  Asynchronous
+    (cache_hub/polar_cache.py:457-471, :778-799)."""
+    bs, H, n, D = src_k.shape
+    es = src_k.element_size()
+    _need(src_k.is_cuda and src_v.is_cuda and src_v.shape == src_k.shape and src_v.stride() == src_k.stride() and
+          src_k.stride(3) == 1 and src_v.dtype == src_k.dtype, "src_k, src_v: GPU [bs,H,n,D], same strides, contiguous rows")
+    for t in (dst_k_cpu, dst_v_cpu):
+        _need(t.is_cpu and t.is_pinned() and t.dtype == src_k.dtype and t.dim() == 4 and tuple(t.shape[:2]) == (bs, H) and
+              t.shape[3] == D and t.stride(3) == 1 and t.stride(2) == D and t.stride(1) == t.shape[2] * D and
+              (bs == 1 or t.stride(0) == H * t.stride(1)), "dst: pinned CPU [bs,H,rows,D], contiguous")
+    s = stream if stream is not None else torch.cuda.current_stream(src_k.device)
+    _lib.check(_lib.lib().pkv_offload_rows(
+        src_k.data_ptr(), src_v.data_ptr(), src_k.stride(0) * es, src_k.stride(1) * es, src_k.stride(2) * es,
+        dst_k_cpu.data_ptr(), dst_v_cpu.data_ptr(), dst_k_cpu.shape[2], dst_row0, n, bs, H, D * es,
+        C.c_void_p(s.cuda_stream)))
+
+
 def gather_uva_packed(src_k, src_v, k_packed, v_packed, indices_packed, cu_seqlens_topk, cu_seqlens_k,
                       sink_local_end: int, global_k: int) -> None:
     bs, H, src_len, D = src_k.shape

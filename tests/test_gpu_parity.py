@@ -1048,3 +1048,33 @@ def test_append_kv_equals_indexed_assignment(ops):
             ops.append_kv(fused[:, :, :H], fused[:, :, H:2 * H], dk, dv, cap)
     with pytest.raises(RuntimeError):
         ops.append_kv(fused[:, :, :H], fused[:, :, H:2 * H + 1], dk, dv, 0)
+
+
+def test_offload_rows_equals_sliced_copy(ops):
+    """pkv_offload_rows against the sliced copy_ it replaces (reference polar_cache.py:457-471, :778-799): rows read in
+    place from the model's [bs,seq,h,d] layout and from a partly filled staging buffer, into a batch slice of the pinned
+    store; rows outside the written window stay untouched."""
+    g = torch.Generator().manual_seed(3)
+    bs, H, cap, D = 3, 4, 50, 128
+    kc = torch.randn(bs + 1, H, cap, D, generator=g).to(torch.bfloat16).pin_memory()
+    vc = torch.randn(bs + 1, H, cap, D, generator=g).to(torch.bfloat16).pin_memory()
+    want_k, want_v = kc.clone(), vc.clone()
+    model_k = torch.randn(bs, 40, H, D, generator=g).to(torch.bfloat16).to(DEV)    # [bs, seq, h, d]
+    model_v = torch.randn(bs, 40, H, D, generator=g).to(torch.bfloat16).to(DEV)
+    src_k, src_v = model_k[:, 5:33].permute(0, 2, 1, 3), model_v[:, 5:33].permute(0, 2, 1, 3)
+    ops.offload_rows(src_k, src_v, kc[1:], vc[1:], 7)
+    want_k[1:, :, 7:35] = src_k.cpu()
+    want_v[1:, :, 7:35] = src_v.cpu()
+    stage_k = torch.randn(bs, H, 16, D, generator=g).to(torch.bfloat16).to(DEV)   # staging buffer, first 9 rows valid
+    stage_v = torch.randn(bs, H, 16, D, generator=g).to(torch.bfloat16).to(DEV)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    ops.offload_rows(stage_k[:, :, :9], stage_v[:, :, :9], kc[:bs], vc[:bs], cap - 9, stream=side)
+    want_k[:bs, :, cap - 9:] = stage_k[:, :, :9].cpu()
+    want_v[:bs, :, cap - 9:] = stage_v[:, :, :9].cpu()
+    torch.cuda.synchronize()
+    assert torch.equal(kc, want_k) and torch.equal(vc, want_v)
+    with pytest.raises(RuntimeError, match="outside the host store"):
+        ops.offload_rows(stage_k, stage_v, kc[:bs], vc[:bs], cap - 9)
+    with pytest.raises(RuntimeError):
+        ops.offload_rows(stage_k, stage_v, kc[:bs].clone(), vc[:bs], 0)   # not pinned
