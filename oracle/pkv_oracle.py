@@ -238,14 +238,26 @@ def retrieve_row(q, signs, dtype, codes, nib, weight, cluster_counts, tiers, n_c
 # ------------------------------------------------------------------ fixtures
 
 
-def srht_signs(seed: int = 42):
-    """SRHT diagonal D in {+-1}^128.  The reference draws it from the CUDA
-    generator (polar_cache.py:59-63), which a CPU cannot reproduce; the build
-    fixes it as this CPU-generator draw."""
-    import torch
+def philox4x32_10(ctr, key):
+    """Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3", SC'11), one block:
+    ctr 4 x uint32, key 2 x uint32 -> 4 x uint32.  Pinned by the Random123 known-answer vectors."""
+    c = [np.uint64(x) for x in ctr]
+    k = [np.uint64(x) for x in key]
+    m0, m1 = np.uint64(0xD2511F53), np.uint64(0xCD9E8D57)
+    w0, w1, mask, s32 = np.uint64(0x9E3779B9), np.uint64(0xBB67AE85), np.uint64(0xFFFFFFFF), np.uint64(32)
+    for _ in range(10):
+        p0, p1 = m0 * c[0], m1 * c[2]
+        c = [(p1 >> s32) ^ c[1] ^ k[0], p1 & mask, (p0 >> s32) ^ c[3] ^ k[1], p0 & mask]
+        k = [(k[0] + w0) & mask, (k[1] + w1) & mask]
+    return [int(x) for x in c]
 
-    g = torch.Generator().manual_seed(seed)
-    return (torch.randint(0, 2, (D,), generator=g).to(torch.float32) * 2 - 1).numpy()
+
+def srht_signs(seed: int = 42):
+    """SRHT diagonal D in {+-1}^128 (polar_cache.py:57-63: manual_seed(seed), then randint(0, 2, (128,)) * 2 - 1 on
+    the GPU).  torch's device generator is Philox4x32-10 keyed by the seed; element i of the first draw after seeding
+    is word 0 of the block with counter (0, 0, i, 0), reduced modulo the range."""
+    bits = [philox4x32_10((0, 0, i, 0), (seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF))[0] % 2 for i in range(D)]
+    return np.asarray([2.0 * b - 1.0 for b in bits], dtype=np.float32)
 
 
 def synth_keys(n, seed, outliers=(7, 31, 64, 101), bf16=False, drift_deg_per_1k=0.0):

@@ -52,12 +52,27 @@ def _cuda(*ts):
             _need(t.is_cuda, "tensor must be on the GPU")
 
 
+def _philox4x32_10(ctr, key):
+    """One block of the Philox4x32-10 counter-based generator (Salmon et al., SC'11): 4 x uint32 out."""
+    m0, m1, w0, w1, mask = 0xD2511F53, 0xCD9E8D57, 0x9E3779B9, 0xBB67AE85, 0xFFFFFFFF
+    c, k = list(ctr), list(key)
+    for _ in range(10):
+        p0, p1 = m0 * c[0], m1 * c[2]
+        c = [(p1 >> 32) ^ c[1] ^ k[0], p1 & mask, (p0 >> 32) ^ c[3] ^ k[1], p0 & mask]
+        k = [(k[0] + w0) & mask, (k[1] + w1) & mask]
+    return c
+
+
 def srht_signs(device, seed: int = 42) -> torch.Tensor:
-    """SRHT diagonal in {+-1}^128 as float32.  The reference draws it from the
-    device generator (``polar_cache.py:59-63``); here it is a CPU-generator draw
-    so that every machine gets the same vector."""
-    g = torch.Generator().manual_seed(seed)
-    return (torch.randint(0, 2, (HEAD_DIM,), generator=g).to(torch.float32) * 2 - 1).to(device)
+    """SRHT diagonal in {+-1}^128 as float32: the vector the reference draws with
+    ``torch.manual_seed(seed); torch.randint(0, 2, (128,), device=gpu) * 2 - 1`` (``polar_cache.py:57-63``).
+
+    torch's device generator is Philox4x32-10 with key = seed, subsequence = element index and offset 0 for the first
+    draw after seeding, and ``randint`` keeps the first word modulo the range; this evaluates the same function on the
+    host, so the vector needs no GPU, does not touch any generator state and is the same on every machine."""
+    mask = 0xFFFFFFFF
+    bits = [_philox4x32_10((0, 0, i, 0), (seed & mask, (seed >> 32) & mask))[0] % 2 for i in range(HEAD_DIM)]
+    return torch.tensor([2.0 * b - 1.0 for b in bits], dtype=torch.float32, device=device)
 
 
 def mag_centers(device) -> torch.Tensor:

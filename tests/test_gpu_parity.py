@@ -1025,6 +1025,22 @@ def test_rerank_rabitq_fused_helper(ops, wl_small_bf16):
     assert s2 is None and v2 is None and ids2.shape[2] == int(math.ceil(w.N * 0.001))
 
 
+def test_srht_signs_equal_the_device_generator_draw(ops):
+    """The reference draws the SRHT diagonal from torch's device generator (polar_cache.py:57-63); the host
+    restatement used here must give the same vector, for the shipped seed and others, and leave the generators alone."""
+    cpu_state, dev_state = torch.get_rng_state(), torch.cuda.get_rng_state(0)
+    for seed in (42, 0, 7, 123456789012):
+        before = torch.get_rng_state(), torch.cuda.get_rng_state(0)
+        mine = ops.srht_signs(DEV, seed)
+        assert torch.equal(torch.get_rng_state(), before[0]) and torch.equal(torch.cuda.get_rng_state(0), before[1])
+        torch.manual_seed(seed)
+        ref = torch.randint(0, 2, (128,), device=DEV, dtype=torch.bfloat16) * 2 - 1   # the reference's expression
+        assert torch.equal(mine, ref.float())
+        assert np.array_equal(O.srht_signs(seed), mine.cpu().numpy())
+    torch.set_rng_state(cpu_state)
+    torch.cuda.set_rng_state(dev_state, 0)
+
+
 def test_append_kv_equals_indexed_assignment(ops):
     """pkv_append_kv against the two indexed assignments it replaces (reference polar_cache.py:848-856), with
     contiguous and strided new rows and a strided (sliced-batch) store."""

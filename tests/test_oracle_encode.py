@@ -46,6 +46,29 @@ def test_sign_codebook_is_bit_enumeration():
             assert (s[c, j] > 0) == bool((c >> j) & 1)
 
 
+def test_philox_known_answers_and_srht_signs(oracle):
+    """The SRHT sign vector is a Philox4x32-10 draw (the generator behind torch's device RNG).  The block function is
+    pinned by the three known-answer vectors of the Random123 distribution (zeros, ones, digits of pi); the sign
+    vector by its definition from the block function, by the product's independent host restatement, and by
+    balance (a gross indexing error would not give 128 fair coin flips from 128 counters)."""
+    kat = [((0, 0, 0, 0), (0, 0), (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)),
+           ((0xffffffff,) * 4, (0xffffffff,) * 2, (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)),
+           ((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0),
+            (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1))]
+    for ctr, key, want in kat:
+        assert tuple(oracle.philox4x32_10(ctr, key)) == want
+    from pariskv_amd import ops
+
+    for seed in (42, 0, 123456789012):
+        s = oracle.srht_signs(seed)
+        assert s.dtype == np.float32 and s.shape == (128,) and set(np.unique(s)) == {-1.0, 1.0}
+        assert [oracle.philox4x32_10((0, 0, i, 0), (seed & 0xffffffff, seed >> 32))[0] % 2 for i in range(128)] == \
+            [int(x > 0) for x in s]
+        assert np.array_equal(ops.srht_signs("cpu", seed).numpy(), s)
+        assert 40 <= int((s > 0).sum()) <= 88
+    assert oracle.srht_signs(42)[:12].tolist() == [1, 1, -1, -1, 1, 1, -1, -1, -1, 1, 1, 1]
+
+
 def test_fwht_matches_hadamard_matrix(oracle):
     H = scipy.linalg.hadamard(128).astype(np.float64)
     g = np.random.default_rng(0)

