@@ -54,6 +54,7 @@ def main():
                          "--context prompt tokens, --steps generated tokens (append + retrieval + gather + attention per "
                          "layer, index refresh and host offload every 1024 tokens)")
     ap.add_argument("--no-offload", action="store_true", help="decode-loop: keep K/V in HBM (config 2's mode)")
+    ap.add_argument("--adaptive", action="store_true", help="decode-loop: the adaptive-k cache class (config 4's mode)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (rows would shard across GPUs by (batch, kv-head))",
@@ -73,7 +74,10 @@ def main():
 
     if args.only == "decode-loop":
         from pariskv_amd.attn_hub import polar_decode_attn
-        from pariskv_amd.cache_hub.polar_cache import polar_cache
+        if args.adaptive:
+            from pariskv_amd.cache_hub.polar_cache_adaptivek_varlen import polar_cache
+        else:
+            from pariskv_amd.cache_hub.polar_cache import polar_cache
 
         S, T = N, args.steps
         cache = polar_cache(valid_start=[0] * bs, layer_num=L, batch_size=bs, max_length=S + T + 8, num_key_value_heads=H,
@@ -95,7 +99,7 @@ def main():
         v1 = torch.randn(T, bs, 1, H, D, generator=g, device=dev, dtype=torch.bfloat16)
         q = torch.randn(bs, 1, H * G, D, generator=g, device=dev, dtype=torch.bfloat16)
         torch.cuda.synchronize()
-        tok_us, issue = [], 0.0
+        tok_us, issue = [], []
         for t in range(T):
             a = time.perf_counter()
             for l in range(L):
@@ -104,14 +108,15 @@ def main():
             b = time.perf_counter()
             torch.cuda.synchronize()
             tok_us.append((time.perf_counter() - a) * 1e6)
-            issue += b - a
+            issue.append((b - a) * 1e6)
         body = sorted(tok_us[8:])
-        print(json.dumps({"only": "decode-loop", "offload": not args.no_offload, "layers": L, "batch": bs, "prompt": S,
+        print(json.dumps({"only": "decode-loop", "cache": "adaptive-k" if args.adaptive else "fixed-k",
+                          "offload": not args.no_offload, "layers": L, "batch": bs, "prompt": S,
                           "generated": T, "final_topk": K, "prefill_s": round(t_prefill, 2),
                           "us_per_layer_step_median": round(body[len(body) // 2] / L, 1),
                           "us_per_layer_step_mean": round(sum(tok_us[8:]) / len(tok_us[8:]) / L, 1),
                           "us_per_layer_step_worst_token": round(body[-1] / L, 1),
-                          "host_issue_us_per_layer_step": round(issue * 1e6 / T / L, 1),
+                          "host_issue_us_per_layer_step": round(sorted(issue[8:])[len(issue[8:]) // 2] / L, 1),
                           "index_refreshes": T // 1024}))
         return
 

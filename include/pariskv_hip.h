@@ -227,6 +227,17 @@ int pkv_offload_rows(const void *src_k, const void *src_v, int64_t src_stride_b,
                      int64_t src_stride_row, void *dst_k_host, void *dst_v_host, int64_t dst_len,
                      int64_t dst_row0, int64_t n_rows, int bs, int n_kv_heads, int row_bytes, void *stream);
 
+/* pkv_gather_uva with a per-row count: row (b, h) moves only its first
+ * row_counts[b*h_count + h] selected rows (int64 on the device, values in
+ * [0, k]); the other slots of dst are left untouched.  For the adaptive-k
+ * cache (cache_hub/polar_cache_adaptivek_varlen.py:1597-1670), whose attention
+ * takes the per-row key count: the ragged selection then needs neither the
+ * packing of the indices nor a host read of the counts. */
+int pkv_gather_uva_ragged(const void *src_k, const void *src_v, int64_t src_len,
+                          const int64_t *idx, int64_t k, const int64_t *row_counts, int64_t idx_offset,
+                          void *dst_k, void *dst_v, int64_t dst_len, int64_t dst_row0,
+                          int bs, int n_kv_heads, int row_bytes, void *stream);
+
 /* Ragged form used by the adaptive-k cache variant (kernel source absent from
  * the reference; contract from the call site
  * cache_hub/polar_cache_adaptivek_varlen.py:1634-1644, layout :1573-1586).

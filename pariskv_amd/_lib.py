@@ -79,6 +79,7 @@ PROTOTYPES = {
     "pkv_gather_hbm": (_i, [_vp, _vp, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i, _i, _i, _vp]),
     "pkv_append_kv": (_i, [_vp, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i, _i, _i, _vp]),
     "pkv_offload_rows": (_i, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i, _i, _i, _vp]),
+    "pkv_gather_uva_ragged": (_i, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i64, _i64, _i, _i, _i, _vp]),
     "pkv_gather_uva_packed": (_i, [_vp, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _i64, _i, _i, _i, _vp]),
     "pkv_gather_cpu": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i, _i]),
     "pkv_host_alloc_mapped": (_i, [_sz, C.POINTER(_vp)]),

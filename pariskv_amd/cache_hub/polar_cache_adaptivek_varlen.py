@@ -10,10 +10,11 @@ What differs from :class:`polar_cache`:
   ``:1130-1133``, ``:1179``): ``_sl_vnorm_cache [bs,H,gpu_rows]`` for the dense GPU rows and ``value_norm_gpu
   [bs,H,capacity]`` by absolute position for the retrieval zone;
 * ``compute`` stops the retrieval after the rerank (all candidates with their scores), runs the adaptive-k
-  kernel, gathers the ragged selection with the packed UVA gather and attends over ``[sink | local | buffer]`` plus
-  each row's own k gathered rows.  The reference packs K/V per row for ``flash_attn_varlen_func`` (``:1597-1670``);
-  here the gathered rows land in a dense ``[bs,H,max_k,128]`` buffer and the attention kernel takes the per-row
-  key count, so the sink/local rows are attended in place and never copied.
+  kernel, gathers each row's own k rows over UVA and attends over ``[sink | local | buffer]`` plus those rows.  The
+  reference packs indices and K/V per row for ``flash_attn_varlen_func`` and reads the largest k back to the host
+  (``:1597-1670``); here the gathered rows land in a dense ``[bs,H,max_k,128]`` buffer, the gather and the attention
+  kernel take the per-row count from device memory, the sink/local rows are attended in place, and the step has no
+  host synchronisation.
 
 Offload mode only, like the reference (``:222-226``).
 """
@@ -65,9 +66,6 @@ class polar_cache(_polar_cache_base):
         cap = max(1, self._adaptive_topk_buffer_cap)
         self._topk_k = torch.zeros((bs, H, cap, self.head_dim), dtype=self.dtype, device=dev)
         self._topk_v = torch.zeros((bs, H, cap, self.head_dim), dtype=self.dtype, device=dev)
-        V = bs * H
-        self._cu_seqlens_dense = (torch.arange(V + 1, dtype=torch.int64) * cap).to(torch.int32).to(dev)
-        self._cu_seqlens_topk_cpu = torch.zeros(V + 1, dtype=torch.int32, pin_memory=True)
         self.last_adaptive_k = None  # [bs, H] int64 of the most recent retrieval step
 
     # ------------------------------------------------------------ ratios
@@ -113,10 +111,10 @@ class polar_cache(_polar_cache_base):
         mask = torch.arange(topk_cap, device=dense_indices.device).unsqueeze(0) < adaptive_k.view(V, 1)
         return dense_indices.contiguous().view(V, topk_cap)[mask]
 
-    def _compute_adaptive_topk(self, query_avg, sink_local_keys, sl_vnorm, all_cand_scores, all_cand_indices, layer_idx,
-                               threshold):
-        """Per-row k and the packed indices (reference :1684-1815).  Returns (adaptive_k [bs,H] int64,
-        indices_packed [sum(k)] int64, global_k int)."""
+    def _adaptive_topk_device(self, query_avg, sink_local_keys, sl_vnorm, all_cand_scores, all_cand_indices, layer_idx,
+                              threshold):
+        """Per-row k and the candidate ids in benefit order, all on the GPU (reference :1684-1759).
+        Returns (adaptive_k [bs,H] int64 after the clamp, topk_ids [bs,H,topk_cap] int64, topk_cap)."""
         cand_len = all_cand_scores.shape[-1]
         effective_max_k = min(self._HARDCODED_MAX_K, cand_len)
         effective_min_k = min(self._HARDCODED_MIN_K, effective_max_k)
@@ -127,7 +125,15 @@ class polar_cache(_polar_cache_base):
                                                  float(threshold), topk_cap, value_norm=self.value_norm_gpu[layer_idx],
                                                  vn_offset=self.sink_size)
         adaptive_k.clamp_(min=max(1, effective_min_k), max=max(1, effective_max_k))               # :1759
-        global_k = int(adaptive_k.max().item())                                                   # the step's one host sync
+        return adaptive_k, topk_ids, topk_cap
+
+    def _compute_adaptive_topk(self, query_avg, sink_local_keys, sl_vnorm, all_cand_scores, all_cand_indices, layer_idx,
+                               threshold):
+        """The reference's return form (:1684-1832): (adaptive_k [bs,H] int64, indices_packed [sum(k)] int64,
+        global_k int).  Reads k back to the host; :meth:`compute` does not go through here."""
+        adaptive_k, topk_ids, topk_cap = self._adaptive_topk_device(query_avg, sink_local_keys, sl_vnorm, all_cand_scores,
+                                                                    all_cand_indices, layer_idx, threshold)
+        global_k = int(adaptive_k.max().item())
         return adaptive_k, self._pack_indices(topk_ids, adaptive_k, topk_cap), global_k
 
     def compute(self, queries, layer_idx):
@@ -148,17 +154,15 @@ class polar_cache(_polar_cache_base):
         kg, vg = self.unified_keys_gpu[layer_idx], self.unified_values_gpu[layer_idx]
         sl_end = z.gpu_prefix_rows                                   # sink + local + update buffer rows
         query_avg = q[:, 0].view(bs, H, G, D).mean(dim=2)            # :1418-1419
-        adaptive_k, indices_packed, global_k = self._compute_adaptive_topk(
+        adaptive_k, topk_ids, topk_cap = self._adaptive_topk_device(
             query_avg, kg[:, :, :sl_end], self._sl_vnorm_cache[layer_idx][:, :, :sl_end], scores, cand, layer_idx,
             self.adaptive_topk_threshold)
         self.last_adaptive_k = adaptive_k
-        # ragged UVA gather: row vh receives its own k rows at [vh*cap, vh*cap + k) of the dense buffer (:1634-1644)
-        cu = self._cu_seqlens_topk_cpu
-        torch.cumsum(adaptive_k.reshape(-1).to("cpu", dtype=torch.int32), dim=0, out=cu[1:])
-        cu_topk = cu.to(self.device, non_blocking=True)
-        cap = self._topk_k.shape[2]
-        ops.gather_uva_packed(self.unified_keys_cpu[layer_idx], self.unified_values_cpu[layer_idx],
-                              self._topk_k.view(bs * H * cap, D), self._topk_v.view(bs * H * cap, D), indices_packed,
-                              cu_topk, self._cu_seqlens_dense, 0, global_k)
-        row_keys = (adaptive_k + sl_end).to(torch.int32).contiguous()
-        return self._attention.run(q, [(kg, vg, 0, sl_end), (self._topk_k, self._topk_v, 0, global_k)], row_keys=row_keys)
+        # ragged UVA gather: row (b, h) receives its own k rows at the head of its slice of the dense buffer.  The
+        # reference packs the indices and reads the largest k back to the host to size its launch (:1597-1644); the
+        # attention below takes the per-row key count instead, so neither the packing nor the host read is needed and
+        # the step never waits for the GPU.
+        ops.gather_uva_ragged(self.unified_keys_cpu[layer_idx], self.unified_values_cpu[layer_idx], topk_ids, adaptive_k,
+                              self._topk_k, self._topk_v)
+        row_keys = (adaptive_k + sl_end).to(torch.int32)
+        return self._attention.run(q, [(kg, vg, 0, sl_end), (self._topk_k, self._topk_v, 0, topk_cap)], row_keys=row_keys)

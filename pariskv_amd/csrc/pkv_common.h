@@ -92,7 +92,7 @@ PKV_INTERNAL int pkv_launch_topk_f32(const float *x, int64_t x_stride, const int
                                      void *ws, size_t ws_bytes, hipStream_t s);
 PKV_INTERNAL int pkv_launch_gather(const void *src_k, const void *src_v, int64_t src_len, const int64_t *idx,
                                    int64_t k, int64_t idx_offset, void *dst_k, void *dst_v, int64_t dst_len,
-                                   int64_t dst_row0, int rows, int row_bytes, hipStream_t s);
+                                   int64_t dst_row0, int rows, int row_bytes, hipStream_t s, const int64_t *row_counts = nullptr);
 
 // -------------------------------------------------------------- device side
 

@@ -13,12 +13,14 @@ namespace {
 constexpr int kGatherThreads = 256;
 constexpr int kGatherUnroll = 4;  // independent row reads per lane
 
-// task t in [0, rows*k*2): kv = t & 1, (row, slot) = divmod(t >> 1, k).
+// task t in [0, rows*k*2): kv = t & 1, (row, slot) = divmod(t >> 1, k).  With row_counts, row r only
+// moves its first row_counts[r] slots (the others leave dst untouched).
 // `vpr` = 16-byte vectors per row; consecutive lanes cover one row.
 __global__ __launch_bounds__(kGatherThreads) void pkv_gather_rows_kernel(
     const pkv_u32x4 *__restrict__ src_k, const pkv_u32x4 *__restrict__ src_v, int64_t src_len,
     const int64_t *__restrict__ idx, int64_t k, int64_t idx_offset, pkv_u32x4 *__restrict__ dst_k,
-    pkv_u32x4 *__restrict__ dst_v, int64_t dst_len, int64_t dst_row0, int64_t n_tasks, int vpr) {
+    pkv_u32x4 *__restrict__ dst_v, int64_t dst_len, int64_t dst_row0, int64_t n_tasks, int vpr,
+    const int64_t *__restrict__ row_counts) {
   const int64_t lanes_per_block = kGatherThreads;
   const int64_t g0 = (int64_t)blockIdx.x * lanes_per_block * kGatherUnroll + threadIdx.x;
   pkv_u32x4 val[kGatherUnroll];
@@ -34,6 +36,7 @@ __global__ __launch_bounds__(kGatherThreads) void pkv_gather_rows_kernel(
       const int kv = (int)(task & 1);
       const int64_t rs = task >> 1;
       const int64_t row = rs / k, slot = rs % k;
+      if (row_counts && slot >= row_counts[row]) continue;  // ragged selection: this row takes fewer than k
       const int64_t i = idx[rs] + idx_offset;
       const pkv_u32x4 *src = kv ? src_v : src_k;
       pkv_u32x4 *d = kv ? dst_v : dst_k;
@@ -139,7 +142,7 @@ int device_view_of_host(const void *host, const void **dev) {
 
 int pkv_launch_gather(const void *src_k, const void *src_v, int64_t src_len, const int64_t *idx, int64_t k,
                       int64_t idx_offset, void *dst_k, void *dst_v, int64_t dst_len, int64_t dst_row0, int rows,
-                      int row_bytes, hipStream_t s) {
+                      int row_bytes, hipStream_t s, const int64_t *row_counts) {
   int rc = check_common(src_k, src_v, dst_k, dst_v, rows, row_bytes);
   if (rc) return rc;
   PKV_REQUIRE(idx && k > 0 && src_len > 0 && dst_row0 >= 0 && dst_row0 + k <= dst_len,
@@ -153,7 +156,7 @@ int pkv_launch_gather(const void *src_k, const void *src_v, int64_t src_len, con
   PKV_REQUIRE(blocks < ((int64_t)1 << 31), "gather too large");
   hipLaunchKernelGGL(pkv_gather_rows_kernel, dim3((unsigned)blocks), dim3(kGatherThreads), 0, s,
                      (const pkv_u32x4 *)src_k, (const pkv_u32x4 *)src_v, src_len, idx, k, idx_offset,
-                     (pkv_u32x4 *)dst_k, (pkv_u32x4 *)dst_v, dst_len, dst_row0, n_tasks, vpr);
+                     (pkv_u32x4 *)dst_k, (pkv_u32x4 *)dst_v, dst_len, dst_row0, n_tasks, vpr, row_counts);
   PKV_LAUNCH_CHECK("pkv_gather_rows_kernel");
   return PKV_OK;
 }
@@ -225,6 +228,20 @@ extern "C" int pkv_offload_rows(const void *src_k, const void *src_v, int64_t sr
                      dst_row0, n_rows, n_kv_heads, n_vec, vpr);
   PKV_LAUNCH_CHECK("pkv_offload_rows_kernel");
   return PKV_OK;
+}
+
+extern "C" int pkv_gather_uva_ragged(const void *src_k, const void *src_v, int64_t src_len, const int64_t *idx, int64_t k,
+                                     const int64_t *row_counts, int64_t idx_offset, void *dst_k, void *dst_v,
+                                     int64_t dst_len, int64_t dst_row0, int bs, int n_kv_heads, int row_bytes,
+                                     void *stream) {
+  PKV_REQUIRE(src_k && src_v && row_counts, "ragged gather: null pointer");
+  const void *dk, *dv;
+  int rc = device_view_of_host(src_k, &dk);
+  if (rc) return rc;
+  rc = device_view_of_host(src_v, &dv);
+  if (rc) return rc;
+  return pkv_launch_gather(dk, dv, src_len, idx, k, idx_offset, dst_k, dst_v, dst_len, dst_row0, bs * n_kv_heads,
+                           row_bytes, (hipStream_t)stream, row_counts);
 }
 
 extern "C" int pkv_gather_uva_packed(const void *src_k, const void *src_v, int64_t src_len, const int64_t *idx_packed,

@@ -380,6 +380,17 @@ def gather_uva(src_k, src_v, idx, dst_k, dst_v, idx_offset: int = 0, dst_row0: i
     _gather(_lib.lib().pkv_gather_uva, src_k, src_v, idx, dst_k, dst_v, idx_offset, dst_row0)
 
 
+def gather_uva_ragged(src_k, src_v, idx, row_counts, dst_k, dst_v, idx_offset: int = 0, dst_row0: int = 0) -> None:
+    """:func:`gather_uva` where row (b, h) moves only its first ``row_counts[b, h]`` indices (int64 [bs,H] on the GPU,
+    values in [0, K]); the remaining dst rows are left as they are."""
+    _need(src_k.is_cpu and src_v.is_cpu and src_k.is_pinned() and src_v.is_pinned(), "src must be pinned CPU tensors")
+    _need(row_counts.is_cuda and row_counts.dtype == torch.int64 and row_counts.is_contiguous() and
+          row_counts.numel() == idx.shape[0] * idx.shape[1], "row_counts: contiguous int64 [bs,H] on the GPU")
+    fn = _lib.lib().pkv_gather_uva_ragged
+    _gather(lambda sk, sv, sl, ix, k, *rest: fn(sk, sv, sl, ix, k, _p(row_counts), *rest), src_k, src_v, idx, dst_k, dst_v,
+            idx_offset, dst_row0)
+
+
 def gather_hbm(src_k, src_v, idx, dst_k, dst_v, idx_offset: int = 0, dst_row0: int = 0) -> None:
     _need(src_k.is_cuda and src_v.is_cuda, "src must be GPU tensors")
     _gather(_lib.lib().pkv_gather_hbm, src_k, src_v, idx, dst_k, dst_v, idx_offset, dst_row0)

@@ -1041,6 +1041,28 @@ def test_srht_signs_equal_the_device_generator_draw(ops):
     torch.cuda.set_rng_state(dev_state, 0)
 
 
+def test_gather_uva_ragged_moves_only_each_rows_prefix(ops):
+    """pkv_gather_uva_ragged: row (b, h) fetches its first row_counts[b, h] selected rows; the rest of dst is untouched;
+    counts 0 and K included."""
+    g = torch.Generator().manual_seed(8)
+    bs, H, N, K, D = 2, 3, 500, 40, 128
+    sk = torch.randn(bs, H, N, D, generator=g).to(torch.bfloat16).pin_memory()
+    sv = torch.randn(bs, H, N, D, generator=g).to(torch.bfloat16).pin_memory()
+    idx = torch.stack([torch.randperm(N, generator=g)[:K] for _ in range(bs * H)]).view(bs, H, K)
+    counts = torch.tensor([[0, K, 7], [1, 39, 20]], dtype=torch.int64)
+    dk = torch.full((bs, H, K + 5, D), 3.0, dtype=torch.bfloat16, device=DEV)
+    dv = torch.full((bs, H, K + 5, D), 5.0, dtype=torch.bfloat16, device=DEV)
+    want_k, want_v = dk.cpu().clone(), dv.cpu().clone()
+    ops.gather_uva_ragged(sk, sv, idx.to(DEV), counts.to(DEV), dk, dv, dst_row0=2)
+    torch.cuda.synchronize()
+    for b in range(bs):
+        for h in range(H):
+            c = int(counts[b, h])
+            want_k[b, h, 2:2 + c] = sk[b, h][idx[b, h, :c]]
+            want_v[b, h, 2:2 + c] = sv[b, h][idx[b, h, :c]]
+    assert torch.equal(dk.cpu(), want_k) and torch.equal(dv.cpu(), want_v)
+
+
 def test_append_kv_equals_indexed_assignment(ops):
     """pkv_append_kv against the two indexed assignments it replaces (reference polar_cache.py:848-856), with
     contiguous and strided new rows and a strided (sliced-batch) store."""
