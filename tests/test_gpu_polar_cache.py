@@ -251,3 +251,55 @@ def test_adaptive_k_cache_decode_loop():
                 err = (out[b, 0].float().cpu() - ref).abs().max().item()
                 assert err < 2e-2, f"attention differs by {err} at step {step} layer {l}"
     assert len(seen_k) >= 3, f"k should vary across rows and steps, saw {sorted(seen_k)}"
+
+
+def test_reference_multibatch_smoke_shape():
+    """The reference's own integration smoke (tests/test_multibatch_smoke.py:23-117): batch 8 in lockstep, 28 layers,
+    4 KV heads x GQA 8, prefill 20480, 50 decode steps, sink 128 / local 256, refresh every 128 tokens, offload on,
+    integer device ids in layer_mapping, the shipped codebook file -- same constructor call minus the two keywords
+    that the reference class itself no longer accepts.  Beyond "does not crash": outputs are finite and, at the last
+    step, one layer's retrieved indices equal the CPU oracle's on the cache's own index."""
+    import os
+
+    from pariskv_amd.cache_hub.polar_cache import polar_cache
+
+    print("reference multibatch smoke shape", flush=True)
+    bs, layers, Hkv, Hq, D, S, steps = 8, 28, 4, 32, 128, 20480, 50
+    max_new = steps + 100
+    codebook = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "codebook_d128_m8_Kr1_Kw256_rabitq_sign.json")
+    cache = polar_cache(valid_start=[0] * bs, layer_num=layers, batch_size=bs, max_length=S + max_new,
+                        num_key_value_heads=Hkv, num_heads=Hq, head_dim=D, dtype=torch.bfloat16,
+                        layer_mapping={i: 0 for i in range(layers)}, max_new_length=max_new, sink_size=128, local_size=256,
+                        core=1, nprobe=1, cache_unit_size=1, cache_cluster_num=1, num_gpus=1, model_size=7,
+                        codebook_path=codebook, final_topk=100, dynamic_update_interval=128, enable_offload=True)
+    g = torch.Generator(device=DEV).manual_seed(0)
+    rnd = lambda *shape: torch.randn(*shape, generator=g, device=DEV, dtype=torch.bfloat16)
+    for l in range(layers):
+        k_out, v_out = cache.prefill_update_kv_cache(rnd(bs, 8, Hkv * 8, D), rnd(bs, S, Hkv, D), rnd(bs, S, Hkv, D), l, batch_idx=0)
+        assert k_out.shape == (bs, S, Hkv, D) and v_out.shape == (bs, S, Hkv, D)
+    assert cache.current_seq_len[0] == S
+    probe = layers - 3
+    for step in range(steps):
+        for l in range(layers):
+            q = rnd(bs, 1, Hq, D)
+            cache.decode_update_kv_cache(rnd(bs, 1, Hkv, D), rnd(bs, 1, Hkv, D), l)
+            out = cache.compute(q, l)
+            if step == steps - 1 and l == probe:
+                q_probe, ids_probe = q.clone(), cache.last_topk_indices.clone()
+        if step % 10 == 0 or step == steps - 1:
+            assert out.shape == (bs, 1, Hq, D) and bool(torch.isfinite(out.float()).all())
+    torch.cuda.synchronize()
+    assert cache.current_seq_len == [S + steps] * layers and cache.context == S + steps
+    n_keys, n_cand, kk, tiers = cache.retrieval_shape(probe)
+    assert kk == 100 and n_keys == S - 128 - 256          # 50 tokens: no refresh yet (interval 128)
+    signs = O.srht_signs(42)
+    G = Hq // Hkv
+    for b, h in ((0, 0), (5, 3)):
+        zone = slice(128, 128 + n_keys)
+        codes = cache._codes_km[probe][b, h, zone].cpu().numpy()
+        nib = cache._nib_km[probe][b, h, zone].cpu().numpy().reshape(-1, 16, 4)
+        w = cache._w_km[probe][b, h, zone].float().cpu().numpy()
+        cc = cache.cluster_key_counts_gpu[probe][b, h].cpu().numpy()
+        ref = O.retrieve_row(q_probe[b, 0, h * G:(h + 1) * G].float().cpu().numpy(), signs, O.BF16, codes, nib, w, cc, tiers,
+                             n_cand, kk)
+        assert np.array_equal(ids_probe[b, h].cpu().numpy(), ref)
