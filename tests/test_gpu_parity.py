@@ -888,11 +888,12 @@ def test_decode_attention_argument_errors(ops):
 
 
 def test_retrieve_random_shapes_vs_oracle(ops):
-    """Whole retrieval on 14 seeded random shapes (ragged key counts, group sizes 1-7, candidate counts from 1 to
+    """Whole retrieval on 16 seeded shapes (ragged key counts, group sizes 1-7, candidate counts from 1 to
     every key, k from 1 to the candidate count, both dtype chains): final indices bit-exact against the oracle."""
     rng = np.random.default_rng(2024)
-    shapes = [(1, 1, 1, 50, 1, 1), (1, 2, 7, 333, 333, 17), (2, 1, 3, 4097, 4096, 4096), (1, 1, 4, 8193, 5000, 1)]
-    while len(shapes) < 14:
+    shapes = [(1, 1, 1, 50, 1, 1), (1, 2, 7, 333, 333, 17), (2, 1, 3, 4097, 4096, 4096), (1, 1, 4, 8193, 5000, 1),
+              (1, 2, 4, 30000, 12000, 3000), (1, 1, 2, 20000, 20000, 8192)]   # candidate rows wider than one workgroup sorts
+    while len(shapes) < 16:
         N = int(rng.integers(60, 20000))
         C = int(rng.integers(1, N + 1))
         shapes.append((int(rng.integers(1, 3)), int(rng.integers(1, 3)), int(rng.integers(1, 8)), N, C,
