@@ -303,13 +303,20 @@ int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, const float *sl
 
 #define PKV_ATTN_MAX_SEGMENTS 4
 
-/* One run of consecutive K/V rows (head_dim 128, rows contiguous: 128 elements
- * apart) inside tensors laid out [bs][n_kv_heads][rows][128]; strides in
- * elements.  Rows row0 .. row0+n_rows-1 of every (b, h) take part. */
+/* One run of K/V rows (head_dim 128, rows contiguous: 128 elements apart)
+ * inside tensors laid out [bs][n_kv_heads][rows][128]; strides in elements.
+ * idx == NULL: rows row0 .. row0+n_rows-1 of every (b, h) take part.
+ * idx != NULL (device int64, [bs*n_kv_heads][idx_stride]): row (b, h) attends
+ * to rows row0 + idx[(b*n_kv_heads+h)*idx_stride + j], j < n_rows - the
+ * selected rows are read where they lie, which replaces the torch.gather of
+ * the no-offload branch (cache_hub/polar_cache.py:1089-1095) altogether.
+ * Index values are clamped to [0, idx_limit). */
 typedef struct pkv_attn_segment {
   const void *k, *v;
   int64_t stride_b, stride_h;
   int64_t row0, n_rows;
+  const int64_t *idx;
+  int64_t idx_stride, idx_limit;
 } pkv_attn_segment;
 
 /* Replaces the torch.cat of sink / top-k / local K and V followed by

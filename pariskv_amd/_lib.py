@@ -23,7 +23,8 @@ _vp, _i, _i64, _sz = C.c_void_p, C.c_int, C.c_int64, C.c_size_t
 class AttnSegment(C.Structure):
     """Mirror of ``pkv_attn_segment``."""
 
-    _fields_ = [("k", _vp), ("v", _vp), ("stride_b", _i64), ("stride_h", _i64), ("row0", _i64), ("n_rows", _i64)]
+    _fields_ = [("k", _vp), ("v", _vp), ("stride_b", _i64), ("stride_h", _i64), ("row0", _i64), ("n_rows", _i64),
+                ("idx", _vp), ("idx_stride", _i64), ("idx_limit", _i64)]
 
 
 class AttnArgs(C.Structure):

@@ -112,15 +112,12 @@ class polar_cache(KV_Cache):
             self._offload_keys_buffer = [torch.empty((bs, H, I, D), dtype=dtype, device=dev) for _ in range(layer_num)]
             self._offload_values_buffer = [torch.empty((bs, H, I, D), dtype=dtype, device=dev) for _ in range(layer_num)]
         else:
-            # GPU rows: every token at its absolute position; a separate buffer holds the attended set
+            # GPU rows: every token at its absolute position
             self.gpu_kv_capacity = self.unified_kv_capacity
             rows = self.unified_kv_capacity
             self.unified_keys_cpu = None
             self.unified_values_cpu = None
             self.cpu_valid_end = None
-            att_rows = max(1, final_topk)  # the gathered top-k rows; sink and local window are attended in place
-            self._attn_k = torch.zeros((bs, H, att_rows, D), dtype=dtype, device=dev)
-            self._attn_v = torch.zeros((bs, H, att_rows, D), dtype=dtype, device=dev)
         self.unified_keys_gpu = [torch.zeros((bs, H, rows, D), dtype=dtype, device=dev) for _ in range(layer_num)]
         self.unified_values_gpu = [torch.zeros((bs, H, rows, D), dtype=dtype, device=dev) for _ in range(layer_num)]
 
@@ -140,6 +137,7 @@ class polar_cache(KV_Cache):
         max_keys = max(1, cap - sink_size)
         max_cand = max(1, math.ceil(max_keys * 0.5))
         self._plan = ops.RetrievePlan(bs, H, self.group_size, cap, dev, max_keys, max_cand, max(1, min(final_topk, max_cand)))
+        self._attn_k = self._attn_v = None  # no-offload mode with few rows: staging buffer of the selected rows
         self._bound = [None] * layer_num  # per layer: (n_keys, ops.BoundStep, topk, out_ids, index of the local segment)
         self._out_ids = torch.empty((bs, H, max(1, final_topk)), dtype=torch.int64, device=dev)
         self._attention = ops.DecodeAttention(bs, H, self.group_size, self.unified_kv_capacity, dev)
@@ -399,15 +397,30 @@ class polar_cache(KV_Cache):
             gather = dict(src_k=self.unified_keys_cpu[layer_idx], src_v=self.unified_values_cpu[layer_idx], from_host=True,
                           idx_offset=0, dst_k=kg, dst_v=vg, dst_row0=prefix)
             segments = [(kg, vg, 0, prefix + topk)]  # [sink | local + buffer | gathered top-k], one run
-        else:
-            ak, av = self._attn_k, self._attn_v
-            gather = dict(src_k=kg, src_v=vg, from_host=False, idx_offset=self.sink_size, dst_k=ak, dst_v=av, dst_row0=0)
-            segments = [(kg, vg, 0, self.sink_size), (ak, av, 0, topk), (kg, vg, z.local_start, z.dense_tail_len)]
-            segments = [s for s in segments if s[3] > 0]
-            local_seg = len(segments) - 1
         out_ids = self._out_ids[:, :, :topk]
         if not out_ids.is_contiguous():
             out_ids = torch.empty((self.batch_size, self.kv_head, topk), dtype=torch.int64, device=self.device)
+        if not self.enable_offload:
+            # The reference gathers sink ++ top-k ++ local rows into a new tensor (:1089-1095).  Sink and local window
+            # are always attended in place here.  The selected rows are either a segment addressed through the index
+            # list the retrieval just wrote (nothing is copied, one launch fewer) or gathered into a small buffer
+            # first: with few (batch, kv-head) rows the extra dependent index load inside the attention kernel costs
+            # more than the gather launch (65.2 vs 62.8 us per layer-step at 8 rows x 32K keys; 111.9 vs 113.2 us at
+            # 32 rows x 128K keys).
+            if self.batch_groups >= 16:
+                gather = None
+                selected = (kg, vg, self.sink_size, topk, out_ids)
+            else:
+                if self._attn_k is None or self._attn_k.shape[2] < topk:
+                    shape = (self.batch_size, self.kv_head, max(topk, self.final_topk), self.head_dim)
+                    self._attn_k = torch.zeros(shape, dtype=self.dtype, device=self.device)
+                    self._attn_v = torch.zeros(shape, dtype=self.dtype, device=self.device)
+                gather = dict(src_k=kg, src_v=vg, from_host=False, idx_offset=self.sink_size, dst_k=self._attn_k,
+                              dst_v=self._attn_v, dst_row0=0)
+                selected = (self._attn_k, self._attn_v, 0, topk)
+            segments = [(kg, vg, 0, self.sink_size), selected, (kg, vg, z.local_start, z.dense_tail_len)]
+            segments = [s for s in segments if s[3] > 0]
+            local_seg = len(segments) - 1
         bound = self._plan.bind(q, self._srht_signs, self._mag_centers, self.cluster_key_counts_gpu[layer_idx],
                                 self._codes_km[layer_idx], self._nib_km[layer_idx], self._w_km[layer_idx], self.sink_size,
                                 n_keys, tiers, n_cand, topk, out_ids, gather, self._attention, segments)

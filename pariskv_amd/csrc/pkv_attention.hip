@@ -37,8 +37,31 @@ struct AttSegs {
   int64_t stride_b[PKV_ATTN_MAX_SEGMENTS], stride_h[PKV_ATTN_MAX_SEGMENTS];
   int64_t row0[PKV_ATTN_MAX_SEGMENTS];
   int64_t end[PKV_ATTN_MAX_SEGMENTS];  // exclusive end of the segment in the concatenated key order
+  const int64_t *idx[PKV_ATTN_MAX_SEGMENTS];  // per segment: selected rows (relative to row0) or nullptr
+  int64_t idx_stride[PKV_ATTN_MAX_SEGMENTS], idx_limit[PKV_ATTN_MAX_SEGMENTS];
   int n;
 };
+
+// Row (inside the (b, h) slab of its segment, row0 included) and segment of concatenated key jj, packed as
+// row | segment << 29.  Indexed segments cost one dependent 8-byte load.
+__device__ __forceinline__ uint32_t att_resolve_row(const AttSegs &segs, int row, uint32_t jj) {
+  int s = 0;
+  uint32_t first = 0;
+#pragma unroll
+  for (int t = 1; t < PKV_ATTN_MAX_SEGMENTS; ++t)
+    if (t < segs.n && jj >= (uint32_t)segs.end[t - 1]) s = t, first = (uint32_t)segs.end[t - 1];
+  const int64_t *ip = segs.idx[0];
+  int64_t stride = segs.idx_stride[0], limit = segs.idx_limit[0], row0 = segs.row0[0];
+#pragma unroll
+  for (int t = 1; t < PKV_ATTN_MAX_SEGMENTS; ++t)
+    if (s == t) ip = segs.idx[t], stride = segs.idx_stride[t], limit = segs.idx_limit[t], row0 = segs.row0[t];
+  int64_t r = jj - first;
+  if (ip) {
+    r = ip[(int64_t)row * stride + r];
+    r = r < 0 ? 0 : (r >= limit ? limit - 1 : r);
+  }
+  return (uint32_t)(r + row0) | ((uint32_t)s << 29);
+}
 
 // Eight consecutive elements as loaded (16 B of bf16, or 32 B of fp32) and their fp32 values.  Kept
 // apart so that a load can be issued a whole step before its data is touched.
@@ -85,7 +108,7 @@ __device__ __forceinline__ void load8(const void *base, int64_t elem_off, float 
 // Partial results layout: ws[((row * n_splits + split) * G + g) * 130 + {0: max, 1: sum, 2..129: output}].
 constexpr int kPartStride = 130;
 
-template <bool BF16, int G>
+template <bool BF16, int G, bool INDEXED>
 __global__ __launch_bounds__(kAttThreads) void pkv_attn_partial_kernel(const void *__restrict__ q, int n_kv_heads,
                                                                        int group, int g0, int g_count, AttSegs segs,
                                                                        int64_t total, const int32_t *__restrict__ row_keys,
@@ -103,14 +126,15 @@ __global__ __launch_bounds__(kAttThreads) void pkv_attn_partial_kernel(const voi
   }
   const int64_t j0 = (int64_t)split * per_split;
   const int64_t j1 = (j0 + per_split < total) ? j0 + per_split : total;
-  // per segment: byte address of this lane's 16 bytes of "concatenated key 0" (may lie before the tensor)
+  // per segment: byte address of this lane's 16 bytes of "concatenated key 0" (may lie before the tensor);
+  // with indexed segments: of row 0 of the (b, h) slab
   const int esz = BF16 ? 2 : 4;
   const char *kb[PKV_ATTN_MAX_SEGMENTS], *vb[PKV_ATTN_MAX_SEGMENTS];
 #pragma unroll
   for (int s = 0; s < PKV_ATTN_MAX_SEGMENTS; ++s) {
     const int64_t first = s == 0 ? 0 : segs.end[s - 1];
     const int64_t off = ((int64_t)b * segs.stride_b[s] + (int64_t)h * segs.stride_h[s] +
-                         (segs.row0[s] - first) * 128 + 8 * lane16) * esz;
+                         (INDEXED ? 0 : (segs.row0[s] - first) * 128) + 8 * lane16) * esz;
     kb[s] = (const char *)segs.k[s] + off;
     vb[s] = (const char *)segs.v[s] + off;
   }
@@ -123,10 +147,19 @@ __global__ __launch_bounds__(kAttThreads) void pkv_attn_partial_kernel(const voi
       const int64_t j = jb + u * kAttKeysPerIter + grp;
       const uint32_t jj = (uint32_t)(j < j1 ? j : j1 - 1);  // fewer than 2^24 keys
       const char *kp = kb[0], *vp = vb[0];
+      uint32_t rownum = jj;
+      if (INDEXED) {
+        const uint32_t packed = att_resolve_row(segs, row, jj);
+        rownum = packed & 0x1fffffffu;
 #pragma unroll
-      for (int s = 1; s < PKV_ATTN_MAX_SEGMENTS; ++s)
-        if (s < segs.n && jj >= (uint32_t)segs.end[s - 1]) kp = kb[s], vp = vb[s];
-      const uint32_t boff = jj * (uint32_t)(128 * esz);
+        for (int s = 1; s < PKV_ATTN_MAX_SEGMENTS; ++s)
+          if ((packed >> 29) == (uint32_t)s) kp = kb[s], vp = vb[s];
+      } else {
+#pragma unroll
+        for (int s = 1; s < PKV_ATTN_MAX_SEGMENTS; ++s)
+          if (s < segs.n && jj >= (uint32_t)segs.end[s - 1]) kp = kb[s], vp = vb[s];
+      }
+      const uint64_t boff = (uint64_t)rownum * (uint32_t)(128 * esz);
       load_raw8<BF16>(kp + boff, 0, kd[u]);
       load_raw8<BF16>(vp + boff, 0, vd[u]);
     }
@@ -148,7 +181,6 @@ __global__ __launch_bounds__(kAttThreads) void pkv_attn_partial_kernel(const voi
     for (int d = 0; d < 8; ++d) o[g][d] = 0.f;
   }
 
-  if (j0 < j1) fetch(j0, kn, vn);
   for (int64_t jb = j0; jb < j1; jb += kAttKeysPerIter * kAttUnroll) {
     bool valid[kAttUnroll];
 #pragma unroll
@@ -249,6 +281,7 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return (uint32_t)pkv_f32_to_bf16_bits(lo) | ((uint32_t)pkv_f32_to_bf16_bits(hi) << 16);
 }
 
+template <bool INDEXED>
 __global__ __launch_bounds__(PKV_WAVE) void pkv_attn_partial_mfma_kernel(const void *__restrict__ q, int n_kv_heads,
                                                                          int group, AttSegs segs, int64_t total,
                                                                          const int32_t *__restrict__ row_keys,
@@ -265,18 +298,30 @@ __global__ __launch_bounds__(PKV_WAVE) void pkv_attn_partial_mfma_kernel(const v
   const int64_t j0 = (int64_t)split * per_split;
   const int64_t j1 = (j0 + per_split < total) ? j0 + per_split : total;
 
-  // per segment: byte address of "concatenated key 0" for this (b, h)
+  // per segment: byte address of "concatenated key 0" for this (b, h); with indexed segments: of row 0 of the slab
   const char *kb[PKV_ATTN_MAX_SEGMENTS], *vb[PKV_ATTN_MAX_SEGMENTS];
 #pragma unroll
   for (int s = 0; s < PKV_ATTN_MAX_SEGMENTS; ++s) {
     const int64_t first = s == 0 ? 0 : segs.end[s - 1];
-    const int64_t off = ((int64_t)b * segs.stride_b[s] + (int64_t)h * segs.stride_h[s] + (segs.row0[s] - first) * 128) * 2;
+    const int64_t off = ((int64_t)b * segs.stride_b[s] + (int64_t)h * segs.stride_h[s] +
+                         (INDEXED ? 0 : (segs.row0[s] - first) * 128)) * 2;
     kb[s] = (const char *)segs.k[s] + off;
     vb[s] = (const char *)segs.v[s] + off;
   }
+  // INDEXED: lane l holds the resolved row of key blk0 + l for the current block of 64 keys (two steps);
+  // the rows a lane needs are then fetched from the owning lanes, so the index loads are one per key.
+  uint32_t my_row = 0;
+  int64_t blk0 = j0;
   auto row_ptr = [&](const char *const (&base)[PKV_ATTN_MAX_SEGMENTS], int64_t key) {
     const uint32_t jj = (uint32_t)(key < j1 ? key : j1 - 1);
     const char *p = base[0];
+    if (INDEXED) {
+      const uint32_t packed = (uint32_t)__shfl((int)my_row, (int)(jj - (uint32_t)blk0), PKV_WAVE);
+#pragma unroll
+      for (int s = 1; s < PKV_ATTN_MAX_SEGMENTS; ++s)
+        if ((packed >> 29) == (uint32_t)s) p = base[s];
+      return p + (uint64_t)(packed & 0x1fffffffu) * 256u;
+    }
 #pragma unroll
     for (int s = 1; s < PKV_ATTN_MAX_SEGMENTS; ++s)
       if (s < segs.n && jj >= (uint32_t)segs.end[s - 1]) p = base[s];
@@ -295,6 +340,11 @@ __global__ __launch_bounds__(PKV_WAVE) void pkv_attn_partial_mfma_kernel(const v
   for (int m = 0; m < 8; ++m) o[m] = pkv_f32x4{0.f, 0.f, 0.f, 0.f};
 
   for (int64_t jb = j0; jb < j1; jb += kMfmaStepKeys) {
+    if (INDEXED && ((jb - j0) & (PKV_WAVE - 1)) == 0) {
+      blk0 = jb;
+      const int64_t key = jb + lane;
+      my_row = att_resolve_row(segs, row, (uint32_t)(key < j1 ? key : j1 - 1));
+    }
     // K: two tiles of 16 keys, lane (n, j) reads dims 32c + 8j .. +7 of key jb + 16t + n
     pkv_u32x4 ka[2][4], vr[8];
 #pragma unroll
@@ -449,6 +499,7 @@ extern "C" int pkv_decode_attention(const void *q, int dtype, int bs, int n_kv_h
   AttSegs sg;
   memset(&sg, 0, sizeof sg);
   int64_t total = 0;
+  bool indexed = false;
   for (int i = 0; i < n_segments; ++i) {
     const pkv_attn_segment &s = segments[i];
     PKV_REQUIRE(s.n_rows >= 0 && s.row0 >= 0, "segment %d: negative extent", i);
@@ -459,6 +510,13 @@ extern "C" int pkv_decode_attention(const void *q, int dtype, int bs, int n_kv_h
     sg.k[sg.n] = s.k, sg.v[sg.n] = s.v;
     sg.stride_b[sg.n] = s.stride_b, sg.stride_h[sg.n] = s.stride_h;
     sg.row0[sg.n] = s.row0;
+    if (s.idx) {
+      PKV_REQUIRE(pkv_aligned(s.idx, 8) && s.idx_stride >= s.n_rows && s.idx_limit > 0 &&
+                      s.row0 + s.idx_limit < ((int64_t)1 << 29),
+                  "segment %d: indexed rows need idx_stride >= n_rows and 0 < idx_limit (row0 + idx_limit < 2^29)", i);
+      sg.idx[sg.n] = s.idx, sg.idx_stride[sg.n] = s.idx_stride, sg.idx_limit[sg.n] = s.idx_limit;
+      indexed = true;
+    }
     total += s.n_rows;
     sg.end[sg.n] = total;
     ++sg.n;
@@ -480,18 +538,27 @@ extern "C" int pkv_decode_attention(const void *q, int dtype, int bs, int n_kv_h
   hipStream_t s = (hipStream_t)stream;
   dim3 grid((unsigned)n_splits, (unsigned)rows);
   if (bf) {
-    hipLaunchKernelGGL(pkv_attn_partial_mfma_kernel, grid, dim3(PKV_WAVE), 0, s, q, n_kv_heads, group, sg, total, row_keys,
-                       per_split, scale_log2e, (float *)ws);
+    if (indexed)
+      hipLaunchKernelGGL(pkv_attn_partial_mfma_kernel<true>, grid, dim3(PKV_WAVE), 0, s, q, n_kv_heads, group, sg, total,
+                         row_keys, per_split, scale_log2e, (float *)ws);
+    else
+      hipLaunchKernelGGL(pkv_attn_partial_mfma_kernel<false>, grid, dim3(PKV_WAVE), 0, s, q, n_kv_heads, group, sg, total,
+                         row_keys, per_split, scale_log2e, (float *)ws);
   } else {
-#define PKV_ATT(GG, G0, GC)                                                                                          \
-  hipLaunchKernelGGL((pkv_attn_partial_kernel<false, GG>), grid, dim3(kAttThreads), 0, s, q, n_kv_heads, group, G0, GC, \
-                     sg, total, row_keys, per_split, scale_log2e, (float *)ws)
+#define PKV_ATT(GG, G0, GC, IDX)                                                                                  \
+  hipLaunchKernelGGL((pkv_attn_partial_kernel<false, GG, IDX>), grid, dim3(kAttThreads), 0, s, q, n_kv_heads, group, G0, \
+                     GC, sg, total, row_keys, per_split, scale_log2e, (float *)ws)
+#define PKV_ATT_G(G0, GC, IDX)            \
+  do {                                    \
+    if (GC == 1) PKV_ATT(1, G0, GC, IDX); \
+    else if (GC == 2) PKV_ATT(2, G0, GC, IDX); \
+    else PKV_ATT(4, G0, GC, IDX);         \
+  } while (0)
     for (int g0 = 0; g0 < group; g0 += 4) {  // four query heads per launch: more would not fit the registers
       const int gc = group - g0 < 4 ? group - g0 : 4;
-      if (gc == 1) PKV_ATT(1, g0, gc);
-      else if (gc == 2) PKV_ATT(2, g0, gc);
-      else PKV_ATT(4, g0, gc);
+      if (indexed) PKV_ATT_G(g0, gc, true); else PKV_ATT_G(g0, gc, false);
     }
+#undef PKV_ATT_G
 #undef PKV_ATT
   }
   PKV_LAUNCH_CHECK("pkv_attn_partial_kernel");

@@ -465,9 +465,11 @@ class DecodeAttention:
 
     def run(self, queries: torch.Tensor, segments, scale: float = None, out: torch.Tensor = None,
             row_keys: torch.Tensor = None) -> torch.Tensor:
-        """queries [bs,1,Hq,128] (or [bs,Hq,128]); segments: list of (k, v, row0, n_rows) with k, v
-        [bs,Hkv,rows,128] tensors whose rows are contiguous; row_keys: optional int32 [bs,Hkv] number of keys
-        (in concatenated order) each row attends to.  Returns a tensor shaped like `queries`."""
+        """queries [bs,1,Hq,128] (or [bs,Hq,128]); segments: list of (k, v, row0, n_rows) or (k, v, row0, n_rows, idx)
+        with k, v [bs,Hkv,rows,128] tensors whose rows are contiguous.  Without ``idx`` a segment is rows
+        row0 .. row0+n_rows-1; with ``idx`` (int64 [bs,Hkv,>=n_rows] on the GPU) it is rows row0 + idx[b,h,j], read in
+        place (values outside the tensor are clamped).  row_keys: optional int32 [bs,Hkv] number of keys (in
+        concatenated order) each row attends to.  Returns a tensor shaped like `queries`."""
         q = queries if queries.is_contiguous() else queries.contiguous()
         segs, out, scale = self._prepare(q, segments, scale, out, row_keys, self._segs)
         _lib.check(_lib.lib().pkv_decode_attention(_p(q), _dt(q.dtype), self.bs, self.H, self.G, segs, len(segments),
@@ -480,16 +482,26 @@ class DecodeAttention:
         _cuda(q)
         _need(q.shape[-1] == HEAD_DIM and q.numel() == self.bs * self.H * self.G * HEAD_DIM, "queries: [bs,1,Hq,128]")
         _need(1 <= len(segments) <= 4, "1..4 key segments")
-        for i, (k, v, row0, n_rows) in enumerate(segments):
+        for i, seg in enumerate(segments):
+            k, v, row0, n_rows = seg[:4]
+            idx = seg[4] if len(seg) > 4 else None
             _cuda(k, v)
             _need(k.dtype == q.dtype and v.dtype == q.dtype, "q, k, v must share a dtype")
             _need(k.dim() == 4 and k.shape == v.shape and k.stride() == v.stride() and k.shape[3] == HEAD_DIM and
                   k.stride(3) == 1 and k.stride(2) == HEAD_DIM and tuple(k.shape[:2]) == (self.bs, self.H),
                   "k, v: [bs,Hkv,rows,128] with contiguous rows")
-            _need(0 <= row0 and row0 + n_rows <= k.shape[2], "segment rows out of range")
             segs[i].k, segs[i].v = _p(k), _p(v)
             segs[i].stride_b, segs[i].stride_h = k.stride(0), k.stride(1)
             segs[i].row0, segs[i].n_rows = row0, n_rows
+            if idx is None:
+                _need(0 <= row0 and row0 + n_rows <= k.shape[2], "segment rows out of range")
+                segs[i].idx, segs[i].idx_stride, segs[i].idx_limit = None, 0, 0
+            else:  # the segment's rows are row0 + idx[b, h, :n_rows], read where they lie
+                _cuda(idx)
+                _need(idx.dtype == torch.int64 and idx.is_contiguous() and idx.dim() == 3 and
+                      tuple(idx.shape[:2]) == (self.bs, self.H) and idx.shape[2] >= n_rows and 0 <= row0 < k.shape[2],
+                      "segment indices: contiguous int64 [bs,Hkv,>=n_rows]")
+                segs[i].idx, segs[i].idx_stride, segs[i].idx_limit = _p(idx), idx.shape[2], k.shape[2] - row0
         if out is None:
             out = torch.empty_like(q)
         if scale is None:

@@ -869,6 +869,49 @@ def test_decode_attention_segments_vs_oracle(ops, dtype, group, lens):
             assert np.abs(got[b, h] - ref).max() <= tol, (b, h, np.abs(got[b, h] - ref).max())
 
 
+@pytest.mark.parametrize("dtype,group,K", [(torch.bfloat16, 4, 300), (torch.bfloat16, 8, 77), (torch.bfloat16, 1, 1500),
+                                           (torch.float32, 4, 130), (torch.float32, 7, 64)])
+def test_decode_attention_indexed_segment_equals_gathered(ops, dtype, group, K):
+    """A segment given as an index list (rows row0 + idx[b,h,j], read in place) against the same rows gathered into a
+    buffer first (reference polar_cache.py:1089-1095 + 1097-1105): the two outputs are identical, and both match the
+    CPU oracle.  Sink and local segments surround the indexed one, as in the no-offload decode step; a ragged
+    row_keys case and out-of-range indices (clamped, no fault) are included."""
+    bs, H, cap, sink, tail0, tail = 2, 3, 2500, 5, 2300, 140
+    _say(f"indexed attention dtype={dtype} G={group} K={K}")
+    g = torch.Generator(device=DEV).manual_seed(21)
+    q = (torch.randn(bs, 1, H * group, 128, generator=g, device=DEV) * 1.5).to(dtype)
+    kk = torch.randn(bs, H, cap, 128, generator=g, device=DEV).to(dtype)
+    vv = torch.randn(bs, H, cap, 128, generator=g, device=DEV).to(dtype)
+    idx = torch.stack([torch.randperm(tail0 - sink, generator=g, device=DEV)[:K + 9] for _ in range(bs * H)]).view(bs, H, K + 9)
+    gk = torch.empty(bs, H, K, 128, dtype=dtype, device=DEV)
+    gv = torch.empty_like(gk)
+    ops.gather_hbm(kk, vv, idx[:, :, :K].contiguous(), gk, gv, idx_offset=sink)
+    att = ops.DecodeAttention(bs, H, group, sink + K + tail, DEV)
+    for row_keys in (None, torch.tensor([[sink + K + tail, sink + 3, sink + K], [40 if K > 40 else K, sink + K + 1, 1]],
+                                        dtype=torch.int32, device=DEV)):
+        a = att.run(q, [(kk, vv, 0, sink), (kk, vv, sink, K, idx), (kk, vv, tail0, tail)], row_keys=row_keys).clone()
+        b_ = att.run(q, [(kk, vv, 0, sink), (gk, gv, 0, K), (kk, vv, tail0, tail)], row_keys=row_keys).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(a, b_)
+    kc = torch.cat([kk[:, :, :sink], gk, kk[:, :, tail0:tail0 + tail]], dim=2).float().cpu().numpy()
+    vc = torch.cat([vv[:, :, :sink], gv, vv[:, :, tail0:tail0 + tail]], dim=2).float().cpu().numpy()
+    full = att.run(q, [(kk, vv, 0, sink), (kk, vv, sink, K, idx), (kk, vv, tail0, tail)])
+    got = full.float().cpu().numpy().reshape(bs, H, group, 128)
+    qc = q.float().cpu().numpy().reshape(bs, H, group, 128)
+    tol = 2e-2 if dtype == torch.bfloat16 else 1e-4
+    for b in range(bs):
+        for h in range(H):
+            assert np.abs(got[b, h] - O.attention(qc[b, h], kc[b, h], vc[b, h])).max() <= tol
+    wild = idx.clone()
+    wild[:, :, ::7] = 10 ** 9          # far outside the tensor: clamped to its last row, must not fault
+    wild[:, :, 3::11] = -5
+    out = att.run(q, [(kk, vv, sink, K, wild)])
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out.float()).all())
+    with pytest.raises(RuntimeError, match="segment indices"):
+        att.run(q, [(kk, vv, sink, K, idx.to(torch.int32))])
+
+
 def test_decode_attention_argument_errors(ops):
     att = ops.DecodeAttention(1, 2, 4, 64, DEV)
     q = torch.zeros(1, 1, 8, 128, dtype=torch.bfloat16, device=DEV)

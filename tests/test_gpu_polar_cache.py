@@ -46,12 +46,12 @@ def _synth_kv(gen, bs, S, Hkv):
     return k.to(torch.bfloat16), v.to(torch.bfloat16)
 
 
-@pytest.mark.parametrize("offload", [True, False])
-def test_decode_loop_matches_oracle_and_dense_reference(offload):
+@pytest.mark.parametrize("offload,bs,Hkv", [(True, 2, 2), (False, 2, 2), (False, 4, 4)])  # 16 rows: selected rows attended in place
+def test_decode_loop_matches_oracle_and_dense_reference(offload, bs, Hkv):
     from pariskv_amd.attn_hub import polar_decode_attn
 
-    print(f"polar_cache decode loop offload={offload}", flush=True)
-    bs, Hkv, Hq, layers, S, steps = 2, 2, 8, 2, 3000, 70
+    print(f"polar_cache decode loop offload={offload} bs={bs} Hkv={Hkv}", flush=True)
+    Hq, layers, S, steps = 4 * Hkv, 2, 3000, 70
     sink, local, I, topk = 4, 64, 32, 200
     G = Hq // Hkv
     cache = _make_cache(offload, bs, Hkv, Hq, layers, S, steps + 10, sink, local, I, topk)
