@@ -266,6 +266,12 @@ int pkv_gather_cpu(const void *src, const int64_t *src_strides4, const int64_t *
  * reference. */
 int pkv_copy_bytes(const void *src, void *dst, size_t bytes, void *stream);
 
+/* Streaming read of `bytes` bytes with the collision scan's access pattern and
+ * no other work (the words are xor-ed into a 256-byte device sink): what a
+ * read-only kernel pulls out of HBM on the device at hand, the yardstick
+ * beside the published peak.  No counterpart in the reference. */
+int pkv_read_bytes(const void *src, size_t bytes, void *sink256, void *stream);
+
 /* Pinned host memory that kernels can read in place (hipHostMalloc, mapped).
  * The reference relies on torch's pin_memory=True for the same purpose
  * (cache_hub/polar_cache.py:226-237). */

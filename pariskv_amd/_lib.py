@@ -70,6 +70,7 @@ PROTOTYPES = {
     "pkv_collision_scan_timed": (_i, [_vp, _i64, _i64, _i64, _i64, _i, _i, _i64, _vp, _vp, _i64, _vp, _vp, _i,
                                       C.POINTER(C.c_float), _vp]),
     "pkv_copy_bytes": (_i, [_vp, _vp, _sz, _vp]),
+    "pkv_read_bytes": (_i, [_vp, _sz, _vp, _vp]),
     "pkv_bucket_topk_ws_bytes": (_sz, [_i, _i64]),
     "pkv_bucket_topk": (_i, [_vp, _i64, _i, _i64, _i64, _vp, _vp, _sz, _vp]),
     "pkv_topk_f32_ws_bytes": (_sz, [_i, _i64, _i64]),

@@ -116,6 +116,30 @@ __global__ __launch_bounds__(256) void pkv_copy_kernel(const pkv_u32x4 *__restri
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = src[i];
 }
 
+// Plain streaming read of n 16-byte vectors (what a read-only kernel can pull out of HBM; one word per
+// wave is written so that the loads cannot be dropped).  Same access pattern as the collision scan:
+// 256-thread workgroups, four 128-bit non-temporal loads per thread in flight.
+__global__ __launch_bounds__(256) void pkv_read_kernel(const pkv_u32x4 *__restrict__ src, uint32_t *__restrict__ sink,
+                                                       int64_t n) {
+  constexpr int kChunk = 4096;  // vectors per workgroup: one contiguous 64 KB slab, like a scan chunk
+  const int64_t k0 = (int64_t)blockIdx.x * kChunk, k1 = k0 + kChunk < n ? k0 + kChunk : n;
+  uint32_t acc = 0;
+  for (int64_t i = k0 + threadIdx.x; i < k1; i += 4 * 256) {
+    pkv_u32x4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int64_t j = i + u * 256;
+      v[u] = j < k1 ? __builtin_nontemporal_load(src + j) : pkv_u32x4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+  }
+#pragma unroll
+  for (int m = 1; m < PKV_WAVE; m <<= 1) acc ^= (uint32_t)__shfl_xor((int)acc, m, PKV_WAVE);
+  // a plain store: the sink only keeps the loads alive, and atomics on a few shared words would dominate the kernel
+  if ((threadIdx.x & (PKV_WAVE - 1)) == 0) sink[(blockIdx.x * 4 + threadIdx.x / PKV_WAVE) & 63] = acc;
+}
+
 int check_common(const void *src_k, const void *src_v, const void *dst_k, const void *dst_v, int rows, int row_bytes) {
   PKV_REQUIRE(src_k && src_v && dst_k && dst_v, "gather: null pointer");
   PKV_REQUIRE(rows > 0, "gather: bad row count %d", rows);
@@ -269,6 +293,19 @@ extern "C" int pkv_gather_uva_packed(const void *src_k, const void *src_v, int64
                      (const pkv_u32x4 *)dk, (const pkv_u32x4 *)dv, src_len, idx_packed, cu_topk, cu_k, sink_local_end,
                      (pkv_u32x4 *)dst_k, (pkv_u32x4 *)dst_v, total_k, vpr);
   PKV_LAUNCH_CHECK("pkv_gather_packed_kernel");
+  return PKV_OK;
+}
+
+extern "C" int pkv_read_bytes(const void *src, size_t bytes, void *sink256, void *stream) {
+  PKV_REQUIRE(src && sink256 && bytes % 16 == 0 && pkv_aligned(src, 16) && pkv_aligned(sink256, 4),
+              "pkv_read_bytes: 16-byte aligned buffer and size, 256-byte sink required");
+  if (bytes == 0) return PKV_OK;
+  const int64_t n = (int64_t)(bytes / 16);
+  const int64_t blocks = (n + 4095) / 4096;
+  PKV_REQUIRE(blocks < ((int64_t)1 << 31), "pkv_read_bytes: too large");
+  hipLaunchKernelGGL(pkv_read_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                     (const pkv_u32x4 *)src, (uint32_t *)sink256, n);
+  PKV_LAUNCH_CHECK("pkv_read_kernel");
   return PKV_OK;
 }
 
