@@ -224,6 +224,14 @@ def main():
     t_wall = time.perf_counter() - t_wall0
     us_gpu = timed(lambda i: step(i, False), args.steps)    # on-GPU stages only
 
+    def step_any_order(i):  # what polar_cache.compute asks for: the same k ids as a set, final sort left out
+        ly = layers[i % L]
+        plan.run(ly["q"], signs, centers, ly["cc"], ly["codes"], ly["nib"], ly["w"], 0, N, tiers, Cn, K, out_ids=out_ids,
+                 any_order=True)
+
+    step_any_order(0)
+    us_gpu_any = timed(step_any_order, args.steps)
+
     def gather_only(i):
         ops.gather_uva(kcpu, vcpu, out_ids, dst_k, dst_v)
 
@@ -301,6 +309,7 @@ def main():
                                f"(UVA gather), {L} rotating layers",
                    "rows": R, "keys_per_row": N, "candidates": Cn, "topk": K, "collision_ratio": 0.2},
         "stages_us": {"full_retrieval_with_uva_gather": round(us_step, 2), "on_gpu_stages": round(us_gpu, 2),
+                      "on_gpu_stages_ids_in_any_order": round(us_gpu_any, 2),
                       "uva_gather_alone": round(us_gather, 2),
                       "decode_attention_over_gathered_set": round(us_attn, 2),
                       "full_step_plus_attention_one_host_call": round(us_step_attn, 2)},

@@ -387,6 +387,10 @@ typedef struct pkv_retrieve_args {
   void *dst_k, *dst_v;
   int64_t dst_len, dst_row0;
   int row_bytes;
+  /* 0: out_ids in descending score order (torch.topk's order, cache_hub/polar_cache.py:1300-1302).
+   * 1: the same k ids in an unspecified but fixed order (a function of the inputs only), for callers that
+   *    use them as a set, as polar_cache.compute does (gather + attention): the final sort is left out. */
+  int any_order;
 } pkv_retrieve_args;
 
 size_t pkv_retrieve_ws_bytes(int rows, int64_t n_keys, int64_t n_cand, int64_t k);

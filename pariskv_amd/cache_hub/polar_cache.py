@@ -382,7 +382,7 @@ class polar_cache(KV_Cache):
             bound.segs[local_seg].row0 = z.local_start
             bound.segs[local_seg].n_rows = z.dense_tail_len
         self._wait_offload(layer_idx)
-        self.last_topk_indices = out_ids
+        self.last_topk_indices = out_ids  # the selected set; its order is fixed but not by score (the sort is left out)
         return bound.launch(q)  # retrieval, gather and attention from one host call
 
     def _bind_step(self, layer_idx, q, n_keys):
@@ -423,7 +423,7 @@ class polar_cache(KV_Cache):
             local_seg = len(segments) - 1
         bound = self._plan.bind(q, self._srht_signs, self._mag_centers, self.cluster_key_counts_gpu[layer_idx],
                                 self._codes_km[layer_idx], self._nib_km[layer_idx], self._w_km[layer_idx], self.sink_size,
-                                n_keys, tiers, n_cand, topk, out_ids, gather, self._attention, segments)
+                                n_keys, tiers, n_cand, topk, out_ids, gather, self._attention, segments, any_order=True)
         step = (n_keys, bound, topk, out_ids, local_seg)
         self._bound[layer_idx] = step
         return step

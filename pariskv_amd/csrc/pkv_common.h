@@ -89,7 +89,7 @@ PKV_INTERNAL int pkv_launch_rerank(const int64_t *cand, int bs, int n_kv_heads, 
 PKV_INTERNAL size_t pkv_topk_ws_bytes_impl(int rows, int64_t len, int64_t k);
 PKV_INTERNAL int pkv_launch_topk_f32(const float *x, int64_t x_stride, const int64_t *ids, int64_t ids_stride,
                                      int rows, int64_t len, int64_t k, int64_t *out_ids, float *out_vals,
-                                     void *ws, size_t ws_bytes, hipStream_t s);
+                                     void *ws, size_t ws_bytes, hipStream_t s, bool any_order = false);
 PKV_INTERNAL int pkv_launch_gather(const void *src_k, const void *src_v, int64_t src_len, const int64_t *idx,
                                    int64_t k, int64_t idx_offset, void *dst_k, void *dst_v, int64_t dst_len,
                                    int64_t dst_row0, int rows, int row_bytes, hipStream_t s, const int64_t *row_counts = nullptr);

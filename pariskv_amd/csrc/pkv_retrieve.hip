@@ -145,7 +145,7 @@ extern "C" int pkv_retrieve(const pkv_retrieve_args *a, void *ws, size_t ws_byte
   if (rc) return rc;
   if (!a->out_ids) return PKV_OK;  // candidates only: the caller reads them out of the workspace
   rc = pkv_launch_topk_f32(scores, a->n_cand, cand, a->n_cand, rows, a->n_cand, a->k, a->out_ids, a->out_scores,
-                           (char *)ws + w.topk, w.topk_bytes, s);
+                           (char *)ws + w.topk, w.topk_bytes, s, a->any_order != 0);
   if (rc) return rc;
   if (a->src_k) {
     PKV_REQUIRE(a->src_v && a->dst_k && a->dst_v, "pkv_retrieve: gather needs src_v, dst_k, dst_v");

@@ -580,7 +580,10 @@ __device__ __forceinline__ void collect_winners_streamed(KeyFn key_of, int64_t l
 }
 
 // len <= 8192 and k well below len: select the k winners exactly, then sort only those.
-template <int EIN>
+// SORTED = false leaves the sort out: the winners come out in the order of their positions in the row
+// (a fixed function of the inputs), for callers that use them as a set (gather + attention).  A thread then
+// owns EIN consecutive positions, so that one exclusive scan over the threads gives every winner its slot.
+template <int EIN, bool SORTED>
 __global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
     const float *__restrict__ x, int64_t x_stride, const int64_t *__restrict__ ids, int64_t ids_stride, int len, int P,
     int64_t k, int64_t *__restrict__ out_ids, float *__restrict__ out_vals) {
@@ -595,14 +598,35 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
   uint64_t v[EIN];
 #pragma unroll
   for (int e = 0; e < EIN; ++e) {
-    const int i = tid + e * kTopkThreads;
+    const int i = SORTED ? tid + e * kTopkThreads : tid * EIN + e;
     v[e] = i < len ? make_key(xr, ir, i) : 0ull;
   }
   if (tid == 0) s_counter = 0;
-  for (int i = tid; i < (P < 1024 ? 1024 : P); i += kTopkThreads) s_keys[i] = 0ull;
+  if (SORTED)
+    for (int i = tid; i < (P < 1024 ? 1024 : P); i += kTopkThreads) s_keys[i] = 0ull;
   uint64_t prefix;
   int shift;
   radix_select_regs<EIN>(v, (uint32_t)k, s_hist, s_bcast, prefix, shift);
+  int64_t *oi = out_ids + (int64_t)row * k;
+  float *ov = out_vals ? out_vals + (int64_t)row * k : nullptr;
+  if (!SORTED) {
+    int mine = 0;
+#pragma unroll
+    for (int e = 0; e < EIN; ++e) mine += (v[e] >> shift) >= (prefix >> shift) && v[e] != 0ull;
+    int total;
+    int slot = pkv_block_excl_scan<kTopkThreads>(mine, (int *)s_hist, total);  // s_hist is free again
+#pragma unroll
+    for (int e = 0; e < EIN; ++e) {
+      if ((v[e] >> shift) >= (prefix >> shift) && v[e] != 0ull) {
+        if (slot < k) {
+          oi[slot] = (int64_t)(uint32_t)(~(uint32_t)v[e]);
+          if (ov) ov[slot] = pkv_from_ordered_u32((uint32_t)(v[e] >> 32));
+        }
+        ++slot;
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int e = 0; e < EIN; ++e) {
     const bool win = (v[e] >> shift) >= (prefix >> shift) && v[e] != 0ull;
@@ -610,8 +634,6 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
     if (win && slot < (uint32_t)k) s_keys[slot] = v[e];
   }
   __syncthreads();
-  int64_t *oi = out_ids + (int64_t)row * k;
-  float *ov = out_vals ? out_vals + (int64_t)row * k : nullptr;
 #define PKV_SORT_K(NT, E) sort_lds_keys_and_emit<NT, E>(s_keys, k, oi, ov, nullptr)
   PKV_DISPATCH_E(P, PKV_SORT_K);
 #undef PKV_SORT_K
@@ -1349,7 +1371,7 @@ extern "C" size_t pkv_topk_f32_ws_bytes(int rows, int64_t len, int64_t k) {
 
 int pkv_launch_topk_f32(const float *x, int64_t x_stride, const int64_t *ids, int64_t ids_stride, int rows,
                         int64_t len, int64_t k, int64_t *out_ids, float *out_vals, void *ws, size_t ws_bytes,
-                        hipStream_t s) {
+                        hipStream_t s, bool any_order) {
   PKV_REQUIRE(x && out_ids, "pkv_topk_f32: null pointer");
   PKV_REQUIRE(k > 0, "k must be positive");
   PKV_REQUIRE(k <= len, "k cannot exceed sequence length");
@@ -1357,10 +1379,17 @@ int pkv_launch_topk_f32(const float *x, int64_t x_stride, const int64_t *ids, in
   if (len <= kTopkMaxSort && pow2_ceil(k) * 2 <= pow2_ceil(len) && pow2_ceil(len) >= 2048) {
     const int P = pow2_ceil(k);
     const int ein = pow2_ceil(len) / kTopkThreads;
-#define PKV_SEL(EIN)                                                                                              \
-  hipLaunchKernelGGL((pkv_topk_select_sort_kernel<EIN>), dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes(P), s, \
-                     x, x_stride, ids, ids_stride, (int)len, P, k, out_ids, out_vals)
-    if (ein <= 2) PKV_SEL(2); else if (ein == 4) PKV_SEL(4); else PKV_SEL(8);
+#define PKV_SEL(EIN, SORTED)                                                                                      \
+  hipLaunchKernelGGL((pkv_topk_select_sort_kernel<EIN, SORTED>), dim3((unsigned)rows), dim3(kTopkThreads),        \
+                     lds_bytes(P), s, x, x_stride, ids, ids_stride, (int)len, P, k, out_ids, out_vals)
+#define PKV_SEL_E(SORTED)             \
+  do {                                \
+    if (ein <= 2) PKV_SEL(2, SORTED); \
+    else if (ein == 4) PKV_SEL(4, SORTED); \
+    else PKV_SEL(8, SORTED);          \
+  } while (0)
+    if (any_order) PKV_SEL_E(false); else PKV_SEL_E(true);
+#undef PKV_SEL_E
 #undef PKV_SEL
     PKV_LAUNCH_CHECK("pkv_topk_select_sort_kernel");
   } else if (len <= kTopkMaxSort) {
@@ -1401,7 +1430,7 @@ extern "C" int pkv_topk_f32(const float *x, int64_t x_stride, const int64_t *ids
                             int64_t len, int64_t k, int64_t *out_ids, float *out_vals, void *ws, size_t ws_bytes,
                             void *stream) {
   return pkv_launch_topk_f32(x, x_stride, ids, ids_stride, rows, len, k, out_ids, out_vals, ws, ws_bytes,
-                             (hipStream_t)stream);
+                             (hipStream_t)stream, false);
 }
 
 struct AdkWs {

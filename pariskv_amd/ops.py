@@ -588,7 +588,7 @@ class RetrievePlan:
         return cand, scores
 
     def _fill(self, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, k,
-              out_ids, out_scores, gather, candidates_only):
+              out_ids, out_scores, gather, candidates_only, any_order=False):
         """Validate one retrieval's operands and return its C argument block."""
         lib = _lib.lib()
         need = lib.pkv_retrieve_ws_bytes(self.rows, n_keys, n_cand, k)
@@ -610,6 +610,7 @@ class RetrievePlan:
         a.n_tiers, a.n_cand, a.k = len(tier_counts), n_cand, k
         a.out_ids = None if candidates_only else out_ids.data_ptr()
         a.out_scores = out_scores.data_ptr() if out_scores is not None else None
+        a.any_order = int(bool(any_order))
         if gather is not None:
             sk, sv, dk, dv = gather["src_k"], gather["src_v"], gather["dst_k"], gather["dst_v"]
             a.src_k, a.src_v, a.gather_from_host = sk.data_ptr(), sv.data_ptr(), int(bool(gather["from_host"]))
@@ -619,15 +620,16 @@ class RetrievePlan:
         return a
 
     def run(self, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, k,
-            out_ids=None, out_scores=None, gather=None, candidates_only=False, attention=None):
-        """Returns out_ids int64 [bs,H,k].  ``gather`` = dict(src_k, src_v, from_host, idx_offset, dst_k, dst_v, dst_row0).
+            out_ids=None, out_scores=None, gather=None, candidates_only=False, attention=None, any_order=False):
+        """Returns out_ids int64 [bs,H,k] in descending score order, or, with ``any_order``, the same ids in an
+        unspecified fixed order (the final sort is left out; enough for gather + attention).  ``gather`` = dict(src_k, src_v, from_host, idx_offset, dst_k, dst_v, dst_row0).
         ``attention`` = (DecodeAttention, segments, out or None): the attention over those segments is launched by the
         same C call, after the gather (pkv_decode_step); the output tensor is then in ``self.attn_out``."""
         lib = _lib.lib()
         if out_ids is None and not candidates_only:
             out_ids = torch.empty(self.bs, self.H, k, dtype=torch.int64, device=self.device)
         a = self._fill(queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, k,
-                       out_ids, out_scores, gather, candidates_only)
+                       out_ids, out_scores, gather, candidates_only, any_order)
         if attention is None:
             _lib.check(lib.pkv_retrieve(C.byref(a), _p(self.ws), self.ws.numel(), _stream(self.ws)))
         else:
@@ -639,11 +641,11 @@ class RetrievePlan:
         return out_ids
 
     def bind(self, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, k,
-             out_ids, gather, att, segments):
+             out_ids, gather, att, segments, any_order=False):
         """Validate everything :meth:`run` would and keep the two argument blocks of pkv_decode_step for repeated
         launches with the same operands (one layer between two index refreshes): see :class:`BoundStep`."""
         a = self._fill(queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, k,
-                       out_ids, None, gather, False)
+                       out_ids, None, gather, False, any_order)
         aa, _ = att.c_args(queries, segments, out=queries)  # out is patched at every launch
         keep = (signs, centers, cluster_counts, codes_km, nib_km, w_km, out_ids, gather, att, segments, self.ws)
         return BoundStep(self, a, aa, keep, queries)

@@ -472,6 +472,37 @@ def _run_fused(ops, w, gather_host=False):
 
 
 @pytest.mark.parametrize("wl_name", ["wl_cfg1", "wl_cfg2", "wl_small_bf16"])
+def test_retrieve_any_order_is_the_same_set_in_candidate_order(ops, request, wl_name):
+    """any_order leaves the final sort out: the k ids are the sorted mode's ids exactly (as a set, scores attached
+    to the right ids), they come in the order of the candidate list (a fixed order), and two runs agree bit for bit."""
+    w = request.getfixturevalue(wl_name)
+    _say(f"retrieve any_order {w.name}")
+    d = W.to_device(w, DEV, torch)
+    plan = ops.RetrievePlan(w.bs, w.H, w.G, w.N, DEV, w.N, w.C, w.K)
+    args = (d["queries"], d["signs"], d["centers"], d["cluster_counts"], d["codes_km"], d["nib_km"], d["w_km"], 0, w.N, w.tiers,
+            w.C, w.K)
+    s_sorted = torch.empty(w.bs, w.H, w.K, dtype=torch.float32, device=DEV)
+    s_any = torch.empty_like(s_sorted)
+    ids_sorted = plan.run(*args, out_scores=s_sorted).clone()
+    ids_any = plan.run(*args, out_scores=s_any, any_order=True).clone()
+    cand = plan.view("cand", w.N, w.C, w.K, torch.int64).view(w.R, w.C).cpu().numpy()
+    ids_again = plan.run(*args, any_order=True)
+    torch.cuda.synchronize()
+    assert torch.equal(ids_any, ids_again)
+    a, b_ = ids_sorted.view(w.R, w.K).cpu().numpy(), ids_any.view(w.R, w.K).cpu().numpy()
+    sa, sb = s_sorted.view(w.R, w.K).cpu().numpy(), s_any.view(w.R, w.K).cpu().numpy()
+    for r in range(w.R):
+        assert np.array_equal(np.sort(a[r]), np.sort(b_[r]))
+        assert dict(zip(a[r].tolist(), sa[r].tolist())) == dict(zip(b_[r].tolist(), sb[r].tolist()))
+        if 2048 <= w.C <= 8192 and 4 * w.K <= w.C:   # the select kernel without its sort: candidate-list order
+            pos = {int(key): i for i, key in enumerate(cand[r])}
+            where = [pos[int(key)] for key in b_[r]]
+            assert where == sorted(where)
+        else:                                         # other shapes keep the descending-score order
+            assert np.array_equal(a[r], b_[r])
+
+
+@pytest.mark.parametrize("wl_name", ["wl_cfg1", "wl_cfg2", "wl_small_bf16"])
 def test_retrieve_fused_matches_oracle(ops, request, wl_name):
     w = request.getfixturevalue(wl_name)
     _say(f"retrieve {w.name}: R={w.R} N={w.N} C={w.C} K={w.K}")

@@ -1,8 +1,8 @@
 """End-to-end tests of the polar_cache drop-in on the GPU: prefill, decode appends with index
 refreshes and host offload, retrieval and attention, for several layers.
 
-Checked per step: (1) the retrieved indices equal the CPU oracle's on the cache's own index
-(bit-exact); (2) the attention output equals an fp32 torch softmax attention over
+Checked per step: (1) the retrieved index set equals the CPU oracle's on the cache's own index
+(exact; the cache leaves the final sort out, the order is checked in test_gpu_parity.py); (2) the attention output equals an fp32 torch softmax attention over
 sink ++ selected ++ dense tail taken from the test's own record of every K/V it fed
 (bf16 tolerance 2e-2 abs)."""
 import math
@@ -100,7 +100,8 @@ def test_decode_loop_matches_oracle_and_dense_reference(offload, bs, Hkv):
                         assert np.array_equal(cc[b, h], O.count_cluster_keys(ec))
                     ref_ids = O.retrieve_row(q[b, 0, h * G:(h + 1) * G].float().numpy(), signs, O.BF16, codes[b, h][sl],
                                              nib[b, h][sl].reshape(-1, 16, 4), w[b, h][sl], cc[b, h], tiers, n_cand, kk)
-                    assert np.array_equal(got_ids[b, h], ref_ids), f"step {step} layer {l} row {(b, h)}"
+                    # the cache asks for the selected set in any fixed order (no final sort): compare as sets
+                    assert np.array_equal(np.sort(got_ids[b, h]), np.sort(ref_ids)), f"step {step} layer {l} row {(b, h)}"
                 # fp32 reference attention over sink ++ selected ++ dense tail
                 K = hist_k[l][b].permute(1, 0, 2)  # [Hkv, total, D]
                 V = hist_v[l][b].permute(1, 0, 2)
@@ -302,4 +303,4 @@ def test_reference_multibatch_smoke_shape():
         cc = cache.cluster_key_counts_gpu[probe][b, h].cpu().numpy()
         ref = O.retrieve_row(q_probe[b, 0, h * G:(h + 1) * G].float().cpu().numpy(), signs, O.BF16, codes, nib, w, cc, tiers,
                              n_cand, kk)
-        assert np.array_equal(ids_probe[b, h].cpu().numpy(), ref)
+        assert np.array_equal(np.sort(ids_probe[b, h].cpu().numpy()), np.sort(ref))   # the cache needs the set, not the order
