@@ -304,3 +304,55 @@ def test_reference_multibatch_smoke_shape():
         ref = O.retrieve_row(q_probe[b, 0, h * G:(h + 1) * G].float().cpu().numpy(), signs, O.BF16, codes, nib, w, cc, tiers,
                              n_cand, kk)
         assert np.array_equal(np.sort(ids_probe[b, h].cpu().numpy()), np.sort(ref))   # the cache needs the set, not the order
+
+
+@pytest.mark.parametrize("offload", [True, False])
+def test_prefill_per_sample_and_valid_start_equal_lockstep(offload):
+    """The two prefill entry forms of the reference (polar_cache.py:379-387): one call per sample (bsz == 1, with
+    batch_idx) and one lockstep call for the whole batch, the latter also with a non-zero valid_start that skips
+    left padding.  All three caches must hold the same index, the same K/V rows and give the same first decode step."""
+    bs, Hkv, Hq, S, pad = 3, 2, 8, 2600, 7
+    sink, local, I, topk = 4, 64, 32, 100
+    gen = torch.Generator().manual_seed(12)
+    k, v = _synth_kv(gen, bs, S, Hkv)
+    kd, vd = k.to(DEV), v.to(DEV)
+    lock = _make_cache(offload, bs, Hkv, Hq, 1, S, 20, sink, local, I, topk)
+    lock.prefill_update_kv_cache(None, kd, vd, 0, 0)
+    single = _make_cache(offload, bs, Hkv, Hq, 1, S, 20, sink, local, I, topk)
+    for b in range(bs):
+        ko, vo = single.prefill_update_kv_cache(None, kd[b:b + 1], vd[b:b + 1], 0, b)
+        assert ko.shape == (1, S, Hkv, 128) and torch.equal(vo, vd[b:b + 1])
+    from pariskv_amd.cache_hub.polar_cache import polar_cache
+    padded = polar_cache(valid_start=[pad] * bs, layer_num=1, batch_size=bs, max_length=S + pad + 20, num_key_value_heads=Hkv,
+                         num_heads=Hq, head_dim=128, dtype=torch.bfloat16, layer_mapping={0: DEV}, max_new_length=20,
+                         sink_size=sink, local_size=local, core=1, nprobe=1, cache_unit_size=1, cache_cluster_num=1, num_gpus=1,
+                         model_size=7, final_topk=topk, dynamic_update_interval=I, full_attention_threshold=100,
+                         enable_offload=offload)
+    junk_k, junk_v = _synth_kv(gen, bs, pad, Hkv)
+    ko, vo = padded.prefill_update_kv_cache(None, torch.cat([junk_k.to(DEV), kd], dim=1), torch.cat([junk_v.to(DEV), vd], dim=1), 0, 0)
+    assert torch.equal(ko, kd) and torch.equal(vo, vd)                       # the states from valid_start on
+    assert padded.prefill_update_kv_cache(None, torch.cat([junk_k.to(DEV), kd], dim=1), torch.cat([junk_v.to(DEV), vd], dim=1),
+                                          0, 1)[0].shape == (bs, S, Hkv, 128)  # batch_idx != 0: slices only
+    torch.cuda.synchronize()
+    k1, v1 = _synth_kv(gen, bs, 1, Hkv)
+    q = (k.float().mean(dim=1).repeat_interleave(Hq // Hkv, dim=1) + 0.5 * torch.randn(bs, Hq, 128, generator=gen))
+    q = q.to(torch.bfloat16).view(bs, 1, Hq, 128).to(DEV)
+    outs = []
+    for c in (lock, single, padded):
+        assert c.current_seq_len == [S] and c.context == S
+        c.decode_update_kv_cache(k1.to(DEV), v1.to(DEV), 0)
+        outs.append((c.compute(q, 0).clone(), c.last_topk_indices.clone()))
+    torch.cuda.synchronize()
+    for c in (single, padded):
+        assert torch.equal(c.cluster_key_counts_gpu[0], lock.cluster_key_counts_gpu[0])
+        for name in ("_codes_km", "_nib_km", "_w_km", "unified_keys_gpu", "unified_values_gpu"):
+            a, b_ = getattr(c, name)[0], getattr(lock, name)[0]
+            rows = min(a.shape[2], b_.shape[2])     # the padded cache was sized for a longer prompt
+            assert torch.equal(a[:, :, :rows], b_[:, :, :rows]), name
+        if offload:
+            n = lock.cpu_valid_end[0]
+            assert c.cpu_valid_end[0] == n
+            assert torch.equal(c.unified_keys_cpu[0][:, :, :n], lock.unified_keys_cpu[0][:, :, :n])
+            assert torch.equal(c.unified_values_cpu[0][:, :, :n], lock.unified_values_cpu[0][:, :, :n])
+    for out, ids in outs[1:]:
+        assert torch.equal(ids, outs[0][1]) and torch.equal(out, outs[0][0])
