@@ -1013,6 +1013,11 @@ __device__ __forceinline__ void adaptive_tail(uint64_t *s_keys, int P, int64_t k
   }
 }
 
+// Position in a row of the per-position value-norm table, kept inside the row whatever the candidate id says.
+__device__ __forceinline__ int64_t vn_index(int64_t pos, int64_t row_len) {
+  return pos < 0 ? 0 : (pos >= row_len ? row_len - 1 : pos);
+}
+
 struct AdkRow {  // one row's operands
   const float *sll, *slv;
   const char *cs;
@@ -1058,7 +1063,7 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adaptive_topk_kernel(
   for (int e = 0; e < EIN; ++e) {
     const int i = tid + e * kTopkThreads, ii = i < n_cand ? i : n_cand - 1;  // clamped: the loads carry no branch
     const float lg = cand_logit(r.cs, cand_dtype, cand_scale, ii);
-    const float vv = r.cv ? r.cv[ii] : r.vn[r.ci[ii] + vn_offset];
+    const float vv = r.cv ? r.cv[ii] : r.vn[vn_index(r.ci[ii] + vn_offset, vn_stride)];
     logit[e] = i < n_cand ? lg : -__uint_as_float(0x7f800000u);
     vnorm[e] = i < n_cand ? vv : 0.f;
   }
@@ -1131,7 +1136,7 @@ __global__ __launch_bounds__(kAdkPartThreads) void pkv_adk_max_gather_kernel(
 #pragma unroll
     for (int e = 0; e < E; ++e) {
       const int64_t i = (int64_t)part * kAdkPart + e * kAdkPartThreads + tid;
-      vv[e] = vn[ci[i < n_cand ? i : n_cand - 1] + vn_offset];
+      vv[e] = vn[vn_index(ci[i < n_cand ? i : n_cand - 1] + vn_offset, vn_stride)];
     }
 #pragma unroll
     for (int e = 0; e < E; ++e) {
@@ -1468,6 +1473,7 @@ extern "C" int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, cons
   PKV_REQUIRE(cand_scores && cand_ids && adaptive_k && topk_ids && (cand_vnorm || value_norm),
               "pkv_adaptive_topk: null pointer");
   PKV_REQUIRE(sl >= 0 && (sl == 0 || (sl_logits && sl_vnorm)), "pkv_adaptive_topk: dense logits missing");
+  PKV_REQUIRE(cand_vnorm || vn_stride > 0, "pkv_adaptive_topk: value_norm needs its row length (vn_stride)");
   PKV_REQUIRE(cand_dtype == PKV_DTYPE_F32 || cand_dtype == PKV_DTYPE_BF16, "unknown candidate score dtype %d", cand_dtype);
   PKV_REQUIRE(rows > 0 && rows <= 65535 && n_cand > 0 && n_cand < ((int64_t)1 << 31) && k_out > 0 && k_out <= n_cand,
               "need 0 < k_out <= n_cand (k_out=%lld n_cand=%lld rows=%d)", (long long)k_out, (long long)n_cand, rows);
