@@ -47,12 +47,14 @@ def main():
     ap.add_argument("--candidates", type=int, default=4096)
     ap.add_argument("--topk", type=int, default=1024)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["scan", "copy", "adaptive", "decode-loop"], default=None,
+    ap.add_argument("--only", choices=["scan", "copy", "adaptive", "decode-loop", "model-decode"], default=None,
                     help="profiling aid: launch only the collision scan, the calibration copy, or the adaptive-k stage "
                          "(--candidates scores per row, dense prefix 1600, value norms gathered from a --context table, "
                          "list length --topk) --steps times; decode-loop: the polar_cache class itself, --layers layers, "
                          "--context prompt tokens, --steps generated tokens (append + retrieval + gather + attention per "
-                         "layer, index refresh and host offload every 1024 tokens)")
+                         "layer, index refresh and host offload every 1024 tokens); model-decode: the same loop inside a "
+                         "random-initialised Qwen3-8B-shaped decoder (config 5: --layers 36 --batch 8 --context 65536 "
+                         "--topk 100 --steps 256), end-to-end decode tokens/s")
     ap.add_argument("--no-offload", action="store_true", help="decode-loop: keep K/V in HBM (config 2's mode)")
     ap.add_argument("--adaptive", action="store_true", help="decode-loop: the adaptive-k cache class (config 4's mode)")
     args = ap.parse_args()
@@ -71,6 +73,52 @@ def main():
     N, Cn, K, L = args.context, args.candidates, args.topk, args.layers
     R = bs * H
     lib = _lib.lib()
+
+    if args.only == "model-decode":
+        from pariskv_amd.cache_hub.polar_cache import polar_cache
+        from pariskv_amd.model_hub import QwenConfig, QwenModel
+
+        S, T = N, args.steps
+        cfg = QwenConfig(num_layers=L)
+        cache = polar_cache(valid_start=[0] * bs, layer_num=L, batch_size=bs, max_length=S + T + 8,
+                            num_key_value_heads=cfg.num_key_value_heads, num_heads=cfg.num_heads, head_dim=cfg.head_dim,
+                            dtype=torch.bfloat16, layer_mapping={i: dev for i in range(L)}, max_new_length=T + 8,
+                            sink_size=64, local_size=512, core=1, nprobe=1, cache_unit_size=1, cache_cluster_num=1,
+                            num_gpus=1, model_size=8, final_topk=K, dynamic_update_interval=1024,
+                            full_attention_threshold=2000, enable_offload=not args.no_offload)
+        g = torch.Generator(device=dev).manual_seed(0)
+        t0 = time.perf_counter()
+        # the prompt's K/V are synthetic (the prompt is not run through the model): keys ~ N(mean_t, 1) with four
+        # outlier channels and a mean that rotates by 0.5 degrees per 1K tokens in the (0, 1) plane; values ~ N(0, 1)
+        ang = torch.arange(S, device=dev, dtype=torch.float32) * (0.5 / 1000.0) * (math.pi / 180.0)
+        for l in range(L):
+            k = torch.randn(bs, S, H, D, generator=g, device=dev, dtype=torch.bfloat16)
+            k[..., 0] += ang.cos().to(torch.bfloat16)[None, :, None]
+            k[..., 1] += ang.sin().to(torch.bfloat16)[None, :, None]
+            k[..., [7, 31, 64, 101]] *= 10.0
+            v = torch.randn(bs, S, H, D, generator=g, device=dev, dtype=torch.bfloat16)
+            cache.prefill_update_kv_cache(None, k, v, l, 0)
+            del k, v
+        torch.cuda.synchronize()
+        t_prefill = time.perf_counter() - t0
+        model = QwenModel(cfg, cache, device=dev, max_positions=S + T + 8)
+        ids = torch.randint(0, cfg.vocab_size, (bs, 1), generator=g, device=dev)
+        for _ in range(args.warmup):
+            ids = model.decode_forward(ids).argmax(dim=-1)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(T - args.warmup):
+            ids = model.decode_forward(ids).argmax(dim=-1)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        n_tok = T - args.warmup
+        print(json.dumps({"only": "model-decode", "model": "Qwen3-8B shape, random init, bf16", "layers": L, "batch": bs,
+                          "prompt": S, "generated": T, "timed_tokens": n_tok, "offload": not args.no_offload,
+                          "final_topk": K, "cache_fill_s": round(t_prefill, 2),
+                          "ms_per_token": round(dt * 1e3 / n_tok, 3),
+                          "decode_tokens_per_s": round(bs * n_tok / dt, 1),
+                          "us_per_layer": round(dt * 1e6 / n_tok / L, 1)}))
+        return
 
     if args.only == "decode-loop":
         from pariskv_amd.attn_hub import polar_decode_attn

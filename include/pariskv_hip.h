@@ -205,10 +205,13 @@ int pkv_gather_hbm(const void *src_k, const void *src_v, int64_t src_len,
  * indexed assignments unified_keys_gpu[layer][:, :, pos, :] = key_states[:, 0]
  * (and values) of decode_update_kv_cache (cache_hub/polar_cache.py:848-856)
  * with one launch.  k_new/v_new: device rows of row_bytes bytes addressed
- * k_new + b*new_stride_b + h*new_stride_h; dst_k/dst_v: device
- * [bs][h][dst_len] rows addressed dst + b*dst_stride_b + h*dst_stride_h +
- * slot*row_bytes.  All strides in BYTES, multiples of 16. */
-int pkv_append_kv(const void *k_new, const void *v_new, int64_t new_stride_b, int64_t new_stride_h,
+ * k_new + b*k_stride_b + h*k_stride_h (and likewise for v_new: the two often
+ * are slices of one fused projection output with different strides);
+ * dst_k/dst_v: device [bs][h][dst_len] rows addressed
+ * dst + b*dst_stride_b + h*dst_stride_h + slot*row_bytes.
+ * All strides in BYTES, multiples of 16. */
+int pkv_append_kv(const void *k_new, int64_t k_stride_b, int64_t k_stride_h,
+                  const void *v_new, int64_t v_stride_b, int64_t v_stride_h,
                   void *dst_k, void *dst_v, int64_t dst_stride_b, int64_t dst_stride_h, int64_t dst_len,
                   int64_t slot, int bs, int n_kv_heads, int row_bytes, void *stream);
 
@@ -342,6 +345,21 @@ int pkv_decode_attention(const void *q, int dtype, int bs, int n_kv_heads, int g
                          const pkv_attn_segment *segments, int n_segments,
                          const int32_t *row_keys, float scale,
                          void *out, void *ws, size_t ws_bytes, void *stream);
+
+/* ------------------------------------------------- decode glue (model side) */
+
+/* One decode token per sequence between the fused QKV projection and the cache:
+ * RMSNorm of every query and key head (weights bf16 [128], or both NULL for
+ * models without q_norm / k_norm) followed by the rotary embedding in
+ * rotate-half form with the position's cos / sin rows (bf16 [64] each).
+ * Replaces the split + head_rmsnorm + apply_rotary_pos_emb sequence of the
+ * reference's decode step (model_hub/qwen.py:327-340, 410-431, 434-498).
+ * qkv: bf16 [bs][stride_b] with the q heads, then the k heads, then v;
+ * q_out bf16 [bs][n_q_heads][128], k_out bf16 [bs][n_kv_heads][128].
+ * head_dim 128, bf16 only; fp32 arithmetic, one rounding at the end. */
+int pkv_qk_norm_rope(const void *qkv, int64_t stride_b, int bs, int n_q_heads, int n_kv_heads,
+                     const void *q_weight, const void *k_weight, float eps,
+                     const void *cos_row, const void *sin_row, void *q_out, void *k_out, void *stream);
 
 /* ------------------------------------------------------- fused decode step */
 

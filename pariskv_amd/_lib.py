@@ -79,7 +79,7 @@ PROTOTYPES = {
                          _vp, _vp, _vp, _vp, _vp, _vp]),
     "pkv_gather_uva": (_i, [_vp, _vp, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i, _i, _i, _vp]),
     "pkv_gather_hbm": (_i, [_vp, _vp, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i, _i, _i, _vp]),
-    "pkv_append_kv": (_i, [_vp, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i, _i, _i, _vp]),
+    "pkv_append_kv": (_i, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i, _i, _i, _vp]),
     "pkv_offload_rows": (_i, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i, _i, _i, _vp]),
     "pkv_gather_uva_ragged": (_i, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i64, _i64, _i, _i, _i, _vp]),
     "pkv_gather_uva_packed": (_i, [_vp, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _i64, _i, _i, _i, _vp]),
@@ -92,6 +92,7 @@ PROTOTYPES = {
                                C.c_float, _i64, _i, _vp, _vp, _vp, _sz, _vp]),
     "pkv_decode_attention_ws_bytes": (_sz, [_i, _i, _i, _i64]),
     "pkv_decode_attention": (_i, [_vp, _i, _i, _i, _i, C.POINTER(AttnSegment), _i, _vp, C.c_float, _vp, _vp, _sz, _vp]),
+    "pkv_qk_norm_rope": (_i, [_vp, _i64, _i, _i, _i, _vp, _vp, C.c_float, _vp, _vp, _vp, _vp, _vp]),
     "pkv_retrieve_ws_bytes": (_sz, [_i, _i64, _i64, _i64]),
     "pkv_retrieve": (_i, [C.POINTER(RetrieveArgs), _vp, _sz, _vp]),
     "pkv_decode_step": (_i, [C.POINTER(RetrieveArgs), _vp, _sz, C.POINTER(AttnArgs), _vp]),

@@ -104,9 +104,9 @@ class polar_cache(KV_Cache):
             self._copy_stream = torch.cuda.Stream(device=dev)
             self._copy_events = [torch.cuda.Event() for _ in range(layer_num)]
             self._offload_inflight = [False] * layer_num
-            self.unified_keys_cpu = [torch.zeros((bs, H, self.cpu_kv_capacity, D), dtype=dtype, pin_memory=True)
+            self.unified_keys_cpu = [ops.alloc_pinned((bs, H, self.cpu_kv_capacity, D), dtype)
                                      for _ in range(layer_num)]
-            self.unified_values_cpu = [torch.zeros((bs, H, self.cpu_kv_capacity, D), dtype=dtype, pin_memory=True)
+            self.unified_values_cpu = [ops.alloc_pinned((bs, H, self.cpu_kv_capacity, D), dtype)
                                        for _ in range(layer_num)]
             self.cpu_valid_end = [0] * layer_num
             self._offload_keys_buffer = [torch.empty((bs, H, I, D), dtype=dtype, device=dev) for _ in range(layer_num)]

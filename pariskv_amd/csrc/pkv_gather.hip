@@ -77,15 +77,15 @@ __global__ __launch_bounds__(kGatherThreads) void pkv_gather_packed_kernel(
 // the [bs][h][dst_len] K and V stores.  Lane g: (task, lane) = divmod(g, vpr),
 // kv = task & 1, (b, h) = divmod(task >> 1, n_heads).  Strides in 16-byte vectors.
 __global__ __launch_bounds__(kGatherThreads) void pkv_append_rows_kernel(
-    const pkv_u32x4 *__restrict__ k_new, const pkv_u32x4 *__restrict__ v_new, int64_t new_stride_b,
-    int64_t new_stride_h, pkv_u32x4 *__restrict__ dst_k, pkv_u32x4 *__restrict__ dst_v, int64_t dst_stride_b,
-    int64_t dst_stride_h, int64_t slot, int n_heads, int n_tasks, int vpr) {
+    const pkv_u32x4 *__restrict__ k_new, const pkv_u32x4 *__restrict__ v_new, int64_t k_stride_b, int64_t k_stride_h,
+    int64_t v_stride_b, int64_t v_stride_h, pkv_u32x4 *__restrict__ dst_k, pkv_u32x4 *__restrict__ dst_v,
+    int64_t dst_stride_b, int64_t dst_stride_h, int64_t slot, int n_heads, int n_tasks, int vpr) {
   const int g = blockIdx.x * kGatherThreads + threadIdx.x;
   const int task = g / vpr, lane = g % vpr;
   if (task >= n_tasks) return;
   const int kv = task & 1;
   const int b = (task >> 1) / n_heads, h = (task >> 1) % n_heads;
-  const pkv_u32x4 val = (kv ? v_new : k_new)[b * new_stride_b + h * new_stride_h + lane];
+  const pkv_u32x4 val = kv ? v_new[b * v_stride_b + h * v_stride_h + lane] : k_new[b * k_stride_b + h * k_stride_h + lane];
   (kv ? dst_v : dst_k)[b * dst_stride_b + h * dst_stride_h + slot * vpr + lane] = val;
 }
 
@@ -205,24 +205,25 @@ extern "C" int pkv_gather_uva(const void *src_k, const void *src_v, int64_t src_
                            row_bytes, (hipStream_t)stream);
 }
 
-extern "C" int pkv_append_kv(const void *k_new, const void *v_new, int64_t new_stride_b, int64_t new_stride_h,
-                             void *dst_k, void *dst_v, int64_t dst_stride_b, int64_t dst_stride_h, int64_t dst_len,
-                             int64_t slot, int bs, int n_kv_heads, int row_bytes, void *stream) {
+extern "C" int pkv_append_kv(const void *k_new, int64_t k_stride_b, int64_t k_stride_h, const void *v_new,
+                             int64_t v_stride_b, int64_t v_stride_h, void *dst_k, void *dst_v, int64_t dst_stride_b,
+                             int64_t dst_stride_h, int64_t dst_len, int64_t slot, int bs, int n_kv_heads, int row_bytes,
+                             void *stream) {
   int rc = check_common(k_new, v_new, dst_k, dst_v, bs * n_kv_heads, row_bytes);
   if (rc) return rc;
   PKV_REQUIRE(bs > 0 && n_kv_heads > 0 && (int64_t)bs * n_kv_heads <= (1 << 20), "append: bad batch/head count");
   PKV_REQUIRE(slot >= 0 && slot < dst_len, "append: slot %lld outside [0, %lld)", (long long)slot, (long long)dst_len);
-  PKV_REQUIRE(new_stride_b % 16 == 0 && new_stride_h % 16 == 0 && dst_stride_b % 16 == 0 && dst_stride_h % 16 == 0 &&
-                  new_stride_h >= row_bytes && new_stride_b >= 0 && dst_stride_h >= dst_len * row_bytes &&
-                  dst_stride_b >= 0,
+  PKV_REQUIRE(k_stride_b % 16 == 0 && k_stride_h % 16 == 0 && v_stride_b % 16 == 0 && v_stride_h % 16 == 0 &&
+                  dst_stride_b % 16 == 0 && dst_stride_h % 16 == 0 && k_stride_h >= row_bytes && v_stride_h >= row_bytes &&
+                  k_stride_b >= 0 && v_stride_b >= 0 && dst_stride_h >= dst_len * row_bytes && dst_stride_b >= 0,
               "append: strides are bytes, multiples of 16, rows must not overlap");
   const int vpr = row_bytes / 16;
   const int n_tasks = bs * n_kv_heads * 2;
   const int lanes = n_tasks * vpr;
   hipLaunchKernelGGL(pkv_append_rows_kernel, dim3((unsigned)((lanes + kGatherThreads - 1) / kGatherThreads)),
                      dim3(kGatherThreads), 0, (hipStream_t)stream, (const pkv_u32x4 *)k_new, (const pkv_u32x4 *)v_new,
-                     new_stride_b / 16, new_stride_h / 16, (pkv_u32x4 *)dst_k, (pkv_u32x4 *)dst_v, dst_stride_b / 16,
-                     dst_stride_h / 16, slot, n_kv_heads, n_tasks, vpr);
+                     k_stride_b / 16, k_stride_h / 16, v_stride_b / 16, v_stride_h / 16, (pkv_u32x4 *)dst_k,
+                     (pkv_u32x4 *)dst_v, dst_stride_b / 16, dst_stride_h / 16, slot, n_kv_heads, n_tasks, vpr);
   PKV_LAUNCH_CHECK("pkv_append_rows_kernel");
   return PKV_OK;
 }

@@ -403,7 +403,7 @@ def append_kv(key_states, value_states, dst_k, dst_v, slot: int) -> None:
     bs, one, H, D = key_states.shape
     es = key_states.element_size()
     _need(one == 1 and value_states.shape == key_states.shape and key_states.stride(3) == 1 and
-          value_states.stride() == key_states.stride(), "key_states, value_states: [bs,1,Hkv,D], same strides")
+          value_states.stride(3) == 1, "key_states, value_states: [bs,1,Hkv,D] with contiguous rows")
     _need(dst_k.dtype == key_states.dtype and dst_v.dtype == key_states.dtype and value_states.dtype == key_states.dtype,
           "append: dtypes differ")
     _need(dst_k.shape == dst_v.shape and dst_k.stride() == dst_v.stride() and dst_k.stride(3) == 1 and
@@ -411,8 +411,8 @@ def append_kv(key_states, value_states, dst_k, dst_v, slot: int) -> None:
           "dst_k, dst_v: [bs,Hkv,rows,D] with contiguous rows")
     _need(key_states.is_cuda and dst_k.is_cuda, "append: tensors must be on the GPU")
     _lib.check(_lib.lib().pkv_append_kv(
-        key_states.data_ptr(), value_states.data_ptr(), key_states.stride(0) * es, key_states.stride(2) * es,
-        dst_k.data_ptr(), dst_v.data_ptr(), dst_k.stride(0) * es, dst_k.stride(1) * es, dst_k.shape[2], slot, bs, H,
+        key_states.data_ptr(), key_states.stride(0) * es, key_states.stride(2) * es,
+        value_states.data_ptr(), value_states.stride(0) * es, value_states.stride(2) * es, dst_k.data_ptr(), dst_v.data_ptr(), dst_k.stride(0) * es, dst_k.stride(1) * es, dst_k.shape[2], slot, bs, H,
         D * es, _stream(dst_k)))
 
 
@@ -519,6 +519,51 @@ class DecodeAttention:
         a.n_segments, a.row_keys, a.scale = len(segments), _p(row_keys), float(scale)
         a.out, a.ws, a.ws_bytes = _p(out), _p(self.ws), self.ws.numel()
         return a, out
+
+
+def qk_norm_rope(qkv: torch.Tensor, n_q_heads: int, n_kv_heads: int, q_weight, k_weight, eps: float,
+                 cos_row: torch.Tensor, sin_row: torch.Tensor):
+    """Per-head RMSNorm of q and k plus rotary embedding for one decode token per sequence, one launch
+    (model_hub/qwen.py:327-340, 410-431, 434-498).  qkv bf16 [bs,1,(Hq+2Hkv)*128] (last dim contiguous); cos_row /
+    sin_row bf16 [64] of the token's position.  Returns (q [bs,1,Hq,128], k [bs,1,Hkv,128])."""
+    bs = qkv.shape[0]
+    _need(qkv.is_cuda and qkv.dtype == torch.bfloat16 and qkv.stride(-1) == 1 and qkv.numel() == bs * qkv.shape[-1] and
+          qkv.shape[-1] >= (n_q_heads + 2 * n_kv_heads) * HEAD_DIM, "qkv: bf16 [bs,1,(Hq+2Hkv)*128]")
+    for t in (cos_row, sin_row):
+        _need(t.is_cuda and t.dtype == torch.bfloat16 and t.numel() == HEAD_DIM // 2 and t.is_contiguous(), "cos/sin: bf16 [64]")
+    for t in (q_weight, k_weight):
+        _need(t is None or (t.is_cuda and t.dtype == torch.bfloat16 and t.numel() == HEAD_DIM and t.is_contiguous()),
+              "norm weights: bf16 [128]")
+    q = torch.empty(bs, 1, n_q_heads, HEAD_DIM, dtype=torch.bfloat16, device=qkv.device)
+    k = torch.empty(bs, 1, n_kv_heads, HEAD_DIM, dtype=torch.bfloat16, device=qkv.device)
+    _lib.check(_lib.lib().pkv_qk_norm_rope(_p(qkv), qkv.stride(0), bs, n_q_heads, n_kv_heads, _p(q_weight), _p(k_weight),
+                                           float(eps), _p(cos_row), _p(sin_row), _p(q), _p(k), _stream(qkv)))
+    return q, k
+
+
+def alloc_pinned(shape, dtype: torch.dtype, zero: bool = False) -> torch.Tensor:
+    """Pinned, device-mapped host tensor of exactly the requested size, optionally zero-filled (``pkv_host_alloc_mapped`` =
+    hipHostMalloc).  torch's own pinned allocator rounds every block up to a power of two, which nearly doubles the
+    host footprint of an offloaded K/V store whose per-layer tensors are just over 1 GiB (72 x 1.07 GiB become
+    144 GiB); these blocks are freed when the tensor and its views are gone."""
+    import weakref
+
+    import numpy as np
+
+    n_elems = 1
+    for d in shape:
+        n_elems *= int(d)
+    esz = torch.empty((), dtype=dtype).element_size()
+    nbytes = max(1, n_elems * esz)
+    ptr = C.c_void_p()
+    _lib.check(_lib.lib().pkv_host_alloc_mapped(nbytes, C.byref(ptr)))
+    buf = (C.c_uint8 * nbytes).from_address(ptr.value)
+    arr = np.frombuffer(buf, dtype=np.uint8, count=nbytes)
+    weakref.finalize(buf, _lib.lib().pkv_host_free, C.c_void_p(ptr.value))   # arr and every tensor view keep buf alive
+    t = torch.from_numpy(arr)
+    if zero:
+        t.zero_()
+    return t[:n_elems * esz].view(dtype).view(*shape)
 
 
 def gather_cpu(src: torch.Tensor, index: torch.Tensor, out: torch.Tensor, n_threads: int = 1) -> None:

@@ -356,3 +356,110 @@ def test_prefill_per_sample_and_valid_start_equal_lockstep(offload):
             assert torch.equal(c.unified_values_cpu[0][:, :, :n], lock.unified_values_cpu[0][:, :, :n])
     for out, ids in outs[1:]:
         assert torch.equal(ids, outs[0][1]) and torch.equal(out, outs[0][0])
+
+
+def test_model_decode_glue_matches_dense_model():
+    """The decode glue (reference model_hub/LLM.py:157-198 + qwen.py ops) on a small random Qwen3-shaped model: with a
+    prompt short enough that the cache attends to every token, each decode step must equal a plain fp32 restatement of
+    the same decoder that keeps its own K/V history (RMSNorm, per-head q/k norm, rotary embedding, GQA attention,
+    SiLU-gated MLP), to bf16 tolerance; then a long prompt runs the retrieval path for a few steps."""
+    import torch.nn.functional as F
+
+    from pariskv_amd.model_hub import QwenConfig, QwenModel
+
+    cfg = QwenConfig(hidden_size=256, num_layers=2, num_heads=8, num_key_value_heads=2, head_dim=128, intermediate_size=512,
+                     vocab_size=1000)
+    bs, S, steps = 2, 40, 6
+    cache = _make_cache(True, bs, cfg.num_key_value_heads, cfg.num_heads, cfg.num_layers, S, steps + 4, 4, 64, 32, 100, thr=2000)
+    gen = torch.Generator().manual_seed(4)
+    hk, hv = [], []
+    for l in range(cfg.num_layers):
+        k, v = _synth_kv(gen, bs, S, cfg.num_key_value_heads)
+        k = (k.float() * 0.1).to(torch.bfloat16)
+        hk.append(k.float()), hv.append(v.float())
+        cache.prefill_update_kv_cache(None, k.to(DEV), v.to(DEV), l, 0)
+    model = QwenModel(cfg, cache, device=DEV, max_positions=S + steps + 8, seed=1)
+    f = lambda t: t.float().cpu()
+
+    def rms(x, w, eps):
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w
+
+    def ref_step(ids, pos):
+        x = f(model.embed_tokens)[ids]                                   # [bs, 1, h]
+        for l, ly in enumerate(model.layers):
+            y = rms(x, f(ly.input_layernorm_weight), cfg.rms_norm_eps)
+            qkv = y @ f(ly.wqkv).T
+            q, k, v = qkv.split([cfg.num_heads * 128, cfg.num_key_value_heads * 128, cfg.num_key_value_heads * 128], dim=-1)
+            q = rms(q.view(bs, 1, cfg.num_heads, 128), f(ly.q_norm_weight), cfg.rms_norm_eps)
+            k = rms(k.view(bs, 1, cfg.num_key_value_heads, 128), f(ly.k_norm_weight), cfg.rms_norm_eps)
+            c, s = f(model.cos_cache)[pos][None, None, None, :], f(model.sin_cache)[pos][None, None, None, :]
+            rot = lambda t: torch.cat((t[..., :64] * c - t[..., 64:] * s, t[..., 64:] * c + t[..., :64] * s), dim=-1)
+            q, k = rot(q), rot(k)
+            hk[l] = torch.cat([hk[l], k], dim=1)
+            hv[l] = torch.cat([hv[l], v.view(bs, 1, cfg.num_key_value_heads, 128)], dim=1)
+            G = cfg.num_heads // cfg.num_key_value_heads
+            kk, vv = hk[l].repeat_interleave(G, dim=2), hv[l].repeat_interleave(G, dim=2)     # [bs, T, Hq, D]
+            att = F.scaled_dot_product_attention(q.transpose(1, 2), kk.transpose(1, 2), vv.transpose(1, 2))   # [bs,Hq,1,D]
+            x = x + att.transpose(1, 2).reshape(bs, 1, -1) @ f(ly.wo).T
+            y = rms(x, f(ly.post_attention_layernorm_weight), cfg.rms_norm_eps)
+            gu = y @ f(ly.gate_up_proj).T
+            x = x + (F.silu(gu[..., :cfg.intermediate_size]) * gu[..., cfg.intermediate_size:]) @ f(ly.down_proj).T
+        return rms(x, f(model.norm_weight), cfg.rms_norm_eps) @ f(model.lm_head).T
+
+    ids = torch.randint(0, cfg.vocab_size, (bs, 1), generator=gen)
+    for step in range(steps):
+        logits = model.decode_forward(ids.to(DEV))
+        ref = ref_step(ids, S + step)
+        assert logits.shape == (bs, 1, cfg.vocab_size) and logits.dtype == torch.float32
+        err = (logits.cpu() - ref).abs().max().item()
+        assert err < 0.15 * ref.abs().max().item() + 0.05, f"step {step}: logits differ by {err}"
+        ids = ref.argmax(dim=-1)
+    assert cache.context == S + steps
+    # long prompt: the same glue over the retrieval path (offload, index refresh inside the run)
+    S2 = 3000
+    cache2 = _make_cache(True, bs, cfg.num_key_value_heads, cfg.num_heads, cfg.num_layers, S2, 50, 4, 64, 32, 100)
+    for l in range(cfg.num_layers):
+        k, v = _synth_kv(gen, bs, S2, cfg.num_key_value_heads)
+        cache2.prefill_update_kv_cache(None, k.to(DEV), v.to(DEV), l, 0)
+    model2 = QwenModel(cfg, cache2, device=DEV, max_positions=S2 + 64, seed=1)
+    ids = torch.randint(0, cfg.vocab_size, (bs, 1), generator=gen).to(DEV)
+    for step in range(40):
+        logits = model2.decode_forward(ids)
+        ids = logits.argmax(dim=-1)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(logits).all()) and cache2.context == S2 + 40 and cache2._zones[0].encoded > S2 - 68
+
+
+def test_qk_norm_rope_matches_torch_ops():
+    """pkv_qk_norm_rope against the reference's op sequence (qwen.py:327-340 head_rmsnorm of q and k, :434-498 rotary
+    embedding) evaluated in fp32 on the same bf16 inputs: within one bf16 rounding of the result; with and without
+    norm weights; q/k read from a fused projection output with a padded row stride."""
+    from pariskv_amd import ops
+
+    g = torch.Generator(device=DEV).manual_seed(2)
+    bs, Hq, Hkv, D = 3, 32, 8, 128
+    width = (Hq + 2 * Hkv) * D
+    buf = torch.randn(bs, 1, width + 64, generator=g, device=DEV).to(torch.bfloat16)
+    qkv = buf[..., :width]                                   # row stride larger than the row
+    qw = (1 + 0.1 * torch.randn(D, generator=g, device=DEV)).to(torch.bfloat16)
+    kw = (1 + 0.1 * torch.randn(D, generator=g, device=DEV)).to(torch.bfloat16)
+    ang = torch.rand(D // 2, generator=g, device=DEV) * 6.28
+    cos, sin = ang.cos().to(torch.bfloat16), ang.sin().to(torch.bfloat16)
+    eps = 1e-6
+
+    def ref(x, heads, w):
+        x = x.float().reshape(bs, 1, heads, D)
+        if w is not None:
+            x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+        c, s = cos.float(), sin.float()
+        return torch.cat((x[..., :64] * c - x[..., 64:] * s, x[..., 64:] * c + x[..., :64] * s), dim=-1)
+
+    for weights in ((qw, kw), (None, None)):
+        q, k = ops.qk_norm_rope(qkv, Hq, Hkv, weights[0], weights[1], eps, cos, sin)
+        torch.cuda.synchronize()
+        assert q.shape == (bs, 1, Hq, D) and k.shape == (bs, 1, Hkv, D)
+        for got, want in ((q, ref(qkv[..., :Hq * D], Hq, weights[0])), (k, ref(qkv[..., Hq * D:(Hq + Hkv) * D], Hkv, weights[1]))):
+            err = (got.float() - want).abs()
+            assert bool((err <= want.abs() * 2 ** -7 + 1e-6).all()), float(err.max())
+    with pytest.raises(RuntimeError, match="go together"):
+        ops.qk_norm_rope(qkv, Hq, Hkv, qw, None, eps, cos, sin)
