@@ -361,6 +361,19 @@ int pkv_qk_norm_rope(const void *qkv, int64_t stride_b, int bs, int n_q_heads, i
                      const void *q_weight, const void *k_weight, float eps,
                      const void *cos_row, const void *sin_row, void *q_out, void *k_out, void *stream);
 
+/* out_sum = x + residual (bf16; residual may be NULL: out_sum = x) and
+ * out_norm = RMSNorm(out_sum) * weight over the last dimension, one launch:
+ * the residual add and the layer norm that follows it in the decode step
+ * (model_hub/LLM.py:186-193, qwen.py:395-407).  x, residual, out_* bf16
+ * [rows][width]; weight bf16 [width]; width % 8 == 0, at most 16384; out_sum may be NULL. */
+int pkv_add_rmsnorm(const void *x, const void *residual, const void *weight, float eps, int rows, int width,
+                    void *out_sum, void *out_norm, void *stream);
+
+/* out[r][j] = silu(gate_up[r][j]) * gate_up[r][inter + j] (bf16): the gate of the
+ * MLP (model_hub/qwen.py:377-381, flashinfer.activation.silu_and_mul there).
+ * gate_up bf16 [rows][row_stride >= 2*inter]; out bf16 [rows][inter]. */
+int pkv_silu_mul(const void *gate_up, int64_t row_stride, int rows, int inter, void *out, void *stream);
+
 /* ------------------------------------------------------- fused decode step */
 
 /* One layer's retrieval for one decode step, key-major storage:

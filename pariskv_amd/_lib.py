@@ -93,6 +93,8 @@ PROTOTYPES = {
     "pkv_decode_attention_ws_bytes": (_sz, [_i, _i, _i, _i64]),
     "pkv_decode_attention": (_i, [_vp, _i, _i, _i, _i, C.POINTER(AttnSegment), _i, _vp, C.c_float, _vp, _vp, _sz, _vp]),
     "pkv_qk_norm_rope": (_i, [_vp, _i64, _i, _i, _i, _vp, _vp, C.c_float, _vp, _vp, _vp, _vp, _vp]),
+    "pkv_add_rmsnorm": (_i, [_vp, _vp, _vp, C.c_float, _i, _i, _vp, _vp, _vp]),
+    "pkv_silu_mul": (_i, [_vp, _i64, _i, _i, _vp, _vp]),
     "pkv_retrieve_ws_bytes": (_sz, [_i, _i64, _i64, _i64]),
     "pkv_retrieve": (_i, [C.POINTER(RetrieveArgs), _vp, _sz, _vp]),
     "pkv_decode_step": (_i, [C.POINTER(RetrieveArgs), _vp, _sz, C.POINTER(AttnArgs), _vp]),

@@ -42,6 +42,83 @@ __global__ __launch_bounds__(256) void pkv_qk_norm_rope_kernel(const uint16_t *_
   dst[lane + 64] = pkv_f32_to_bf16_bits(y2);
 }
 
+// out_sum = x + residual (residual may be NULL), out_norm = RMSNorm(out_sum) * weight.  One workgroup of 256
+// threads per token row; width a multiple of 8 up to 16384 (8 bf16 per 128-bit access, at most 8 accesses
+// per thread).  fp32 arithmetic; out_sum is rounded to bf16 first and the norm is taken of the rounded sum,
+// as a separate add followed by a norm would.
+__global__ __launch_bounds__(256) void pkv_add_rmsnorm_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ residual,
+                                                              const uint16_t *__restrict__ weight, float eps, int width,
+                                                              uint16_t *__restrict__ out_sum, uint16_t *__restrict__ out_norm) {
+  __shared__ float s_part[4];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const int n_vec = width / 8;
+  float v[8][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    const int vec = tid + r * 256;
+    if (vec < n_vec) {
+      const pkv_u32x4 a = *(const pkv_u32x4 *)(x + (int64_t)row * width + vec * 8);
+      pkv_u32x4 b = {0u, 0u, 0u, 0u};
+      if (residual) b = *(const pkv_u32x4 *)(residual + (int64_t)row * width + vec * 8);
+      const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
+      uint32_t ow[4];
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        const float lo = pkv_bf16_round(__uint_as_float(aw[p] << 16) + __uint_as_float(bw[p] << 16));
+        const float hi = pkv_bf16_round(__uint_as_float(aw[p] & 0xffff0000u) + __uint_as_float(bw[p] & 0xffff0000u));
+        v[r][2 * p] = lo, v[r][2 * p + 1] = hi;
+        ss += lo * lo + hi * hi;
+        ow[p] = (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xffff0000u);
+      }
+      if (out_sum) *(pkv_u32x4 *)(out_sum + (int64_t)row * width + vec * 8) = pkv_u32x4{ow[0], ow[1], ow[2], ow[3]};
+    }
+  }
+#pragma unroll
+  for (int m = 1; m < PKV_WAVE; m <<= 1) ss += __shfl_xor(ss, m, PKV_WAVE);
+  if (pkv_lane() == 0) s_part[tid / PKV_WAVE] = ss;
+  __syncthreads();
+  const float inv = 1.0f / sqrtf((s_part[0] + s_part[1] + s_part[2] + s_part[3]) / (float)width + eps);
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    const int vec = tid + r * 256;
+    if (vec < n_vec) {
+      const pkv_u32x4 w4 = *(const pkv_u32x4 *)(weight + vec * 8);
+      const uint32_t ww[4] = {w4.x, w4.y, w4.z, w4.w};
+      uint32_t ow[4];
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        const float lo = v[r][2 * p] * inv * __uint_as_float(ww[p] << 16);
+        const float hi = v[r][2 * p + 1] * inv * __uint_as_float(ww[p] & 0xffff0000u);
+        ow[p] = (uint32_t)pkv_f32_to_bf16_bits(lo) | ((uint32_t)pkv_f32_to_bf16_bits(hi) << 16);
+      }
+      *(pkv_u32x4 *)(out_norm + (int64_t)row * width + vec * 8) = pkv_u32x4{ow[0], ow[1], ow[2], ow[3]};
+    }
+  }
+}
+
+// out[row][j] = silu(gate_up[row][j]) * gate_up[row][inter + j], bf16, 8 elements per thread.
+__global__ __launch_bounds__(256) void pkv_silu_mul_kernel(const uint16_t *__restrict__ gate_up, int64_t row_stride, int inter,
+                                                           uint16_t *__restrict__ out, int64_t n_vec_total) {
+  const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= n_vec_total) return;
+  const int per_row = inter / 8;
+  const int64_t row = g / per_row;
+  const int vec = (int)(g % per_row);
+  const pkv_u32x4 a = *(const pkv_u32x4 *)(gate_up + row * row_stride + vec * 8);
+  const pkv_u32x4 b = *(const pkv_u32x4 *)(gate_up + row * row_stride + inter + vec * 8);
+  const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
+  uint32_t ow[4];
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const float g0 = __uint_as_float(aw[p] << 16), g1 = __uint_as_float(aw[p] & 0xffff0000u);
+    const float u0 = __uint_as_float(bw[p] << 16), u1 = __uint_as_float(bw[p] & 0xffff0000u);
+    const float s0 = pkv_bf16_round(g0 / (1.0f + __expf(-g0))), s1 = pkv_bf16_round(g1 / (1.0f + __expf(-g1)));
+    ow[p] = (uint32_t)pkv_f32_to_bf16_bits(s0 * u0) | ((uint32_t)pkv_f32_to_bf16_bits(s1 * u1) << 16);
+  }
+  *(pkv_u32x4 *)(out + row * inter + vec * 8) = pkv_u32x4{ow[0], ow[1], ow[2], ow[3]};
+}
+
 }  // namespace
 
 extern "C" int pkv_qk_norm_rope(const void *qkv, int64_t stride_b, int bs, int n_q_heads, int n_kv_heads,
@@ -58,5 +135,30 @@ extern "C" int pkv_qk_norm_rope(const void *qkv, int64_t stride_b, int bs, int n
                      (const uint16_t *)k_weight, eps, (const uint16_t *)cos_row, (const uint16_t *)sin_row,
                      (uint16_t *)q_out, (uint16_t *)k_out, n_tasks);
   PKV_LAUNCH_CHECK("pkv_qk_norm_rope_kernel");
+  return PKV_OK;
+}
+
+extern "C" int pkv_add_rmsnorm(const void *x, const void *residual, const void *weight, float eps, int rows, int width,
+                               void *out_sum, void *out_norm, void *stream) {
+  PKV_REQUIRE(x && weight && out_norm, "pkv_add_rmsnorm: null pointer");
+  PKV_REQUIRE(rows > 0 && width > 0 && width % 8 == 0 && width <= 16384, "pkv_add_rmsnorm: width must be a multiple of 8 up to 16384 (got %d)", width);
+  PKV_REQUIRE(pkv_aligned(x, 16) && pkv_aligned(weight, 16) && pkv_aligned(out_norm, 16) &&
+                  (!residual || pkv_aligned(residual, 16)) && (!out_sum || pkv_aligned(out_sum, 16)),
+              "pkv_add_rmsnorm: 16-byte aligned buffers required");
+  hipLaunchKernelGGL(pkv_add_rmsnorm_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, (const uint16_t *)x,
+                     (const uint16_t *)residual, (const uint16_t *)weight, eps, width, (uint16_t *)out_sum,
+                     (uint16_t *)out_norm);
+  PKV_LAUNCH_CHECK("pkv_add_rmsnorm_kernel");
+  return PKV_OK;
+}
+
+extern "C" int pkv_silu_mul(const void *gate_up, int64_t row_stride, int rows, int inter, void *out, void *stream) {
+  PKV_REQUIRE(gate_up && out && rows > 0 && inter > 0 && inter % 8 == 0 && row_stride >= 2 * (int64_t)inter && row_stride % 8 == 0,
+              "pkv_silu_mul: bad shape rows=%d inter=%d stride=%lld", rows, inter, (long long)row_stride);
+  PKV_REQUIRE(pkv_aligned(gate_up, 16) && pkv_aligned(out, 16), "pkv_silu_mul: 16-byte aligned buffers required");
+  const int64_t n_vec = (int64_t)rows * (inter / 8);
+  hipLaunchKernelGGL(pkv_silu_mul_kernel, dim3((unsigned)((n_vec + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const uint16_t *)gate_up, row_stride, inter, (uint16_t *)out, n_vec);
+  PKV_LAUNCH_CHECK("pkv_silu_mul_kernel");
   return PKV_OK;
 }

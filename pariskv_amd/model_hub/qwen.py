@@ -163,11 +163,39 @@ class QwenModel:
                                        layer.post_attention_layernorm_weight)
         return residual + self.mlp(hidden_states, layer)
 
+    def _attention_block(self, layer_idx, normed):
+        """QKV projection, head norms + rotary embedding, cache update and decode attention, output projection."""
+        layer = self.layers[layer_idx]
+        bsz, seq_len, _ = normed.shape
+        qkv = F.linear(normed, layer.wqkv)
+        pos = self._position
+        q, k = ops.qk_norm_rope(qkv, self.num_heads, self.num_key_value_heads, layer.q_norm_weight, layer.k_norm_weight,
+                                layer.q_norm_variance_epsilon or 0.0, self.cos_cache[pos], self.sin_cache[pos])
+        v = qkv[..., (self.num_heads + self.num_key_value_heads) * self.head_dim:].reshape(bsz, -1, self.num_key_value_heads,
+                                                                                             self.head_dim)
+        k, v = self.kv_cache.decode_update_kv_cache(k, v, layer_idx)
+        attn_out = self.decode_attention(q, k, v, layer_idx)
+        return self.wo(attn_out, layer, bsz, seq_len, attn_out.shape[-2] * attn_out.shape[-1])
+
     def decode_forward(self, inputs_ids):
         """inputs_ids [bs, 1] -> logits [bs, 1, vocab] (fp32)."""
         hidden_states = self.word_embedding(inputs_ids)
         self._position = self.kv_cache.context
-        for ldx in range(self.num_layers):
-            hidden_states = self.layer_decode(ldx, hidden_states)
-        hidden_states = self.layernorm(hidden_states[:, -1:, :], self.norm_variance_epsilon, self.norm_weight)
-        return self.lm(hidden_states)
+        fused = (hidden_states.shape[1] == 1 and self.dtype == torch.bfloat16 and self.head_dim == 128 and
+                 self.hidden_size % 8 == 0 and self.hidden_size <= 16384 and all(ly.bqkv is None for ly in self.layers))
+        if not fused:
+            for ldx in range(self.num_layers):
+                hidden_states = self.layer_decode(ldx, hidden_states)
+            hidden_states = self.layernorm(hidden_states[:, -1:, :], self.norm_variance_epsilon, self.norm_weight)
+            return self.lm(hidden_states)
+        # One token per sequence in bf16: the same arithmetic with each residual add folded into the norm that follows
+        # it (also across the layer boundary) and the MLP gate in one launch.
+        x, pending = hidden_states.contiguous(), None   # residual stream, and what is still to be added to it
+        for ldx, layer in enumerate(self.layers):
+            x, normed = ops.add_rmsnorm(pending if pending is not None else x, x if pending is not None else None,
+                                        layer.input_layernorm_weight, layer.input_layernorm_variance_epsilon)
+            x, normed = ops.add_rmsnorm(self._attention_block(ldx, normed), x, layer.post_attention_layernorm_weight,
+                                        layer.post_attention_layernorm_variance_epsilon)
+            pending = F.linear(ops.silu_mul(F.linear(normed, layer.gate_up_proj)), layer.down_proj)
+        _, normed = ops.add_rmsnorm(pending, x, self.norm_weight, self.norm_variance_epsilon, want_sum=False)
+        return self.lm(normed)

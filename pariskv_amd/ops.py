@@ -541,6 +541,34 @@ def qk_norm_rope(qkv: torch.Tensor, n_q_heads: int, n_kv_heads: int, q_weight, k
     return q, k
 
 
+def add_rmsnorm(x: torch.Tensor, residual, weight: torch.Tensor, eps: float, want_sum: bool = True):
+    """(x + residual, RMSNorm(x + residual) * weight) over the last dimension in one launch; ``residual`` may be None.
+    bf16, contiguous (model_hub/LLM.py:186-193, qwen.py:395-407)."""
+    width = x.shape[-1]
+    rows = x.numel() // width
+    _need(x.is_cuda and x.dtype == torch.bfloat16 and x.is_contiguous() and weight.dtype == torch.bfloat16 and
+          weight.numel() == width and weight.is_contiguous(), "x: contiguous bf16 [..., width]; weight bf16 [width]")
+    _need(residual is None or (residual.shape == x.shape and residual.dtype == x.dtype and residual.is_contiguous()),
+          "residual must match x")
+    out_sum = torch.empty_like(x) if (want_sum and residual is not None) else None
+    out_norm = torch.empty_like(x)
+    _lib.check(_lib.lib().pkv_add_rmsnorm(_p(x), _p(residual), _p(weight), float(eps), rows, width, _p(out_sum), _p(out_norm),
+                                          _stream(x)))
+    return (out_sum if out_sum is not None else x), out_norm
+
+
+def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
+    """silu(gate_up[..., :n]) * gate_up[..., n:] with n = width / 2, bf16, one launch (model_hub/qwen.py:377-381)."""
+    width = gate_up.shape[-1]
+    inter = width // 2
+    rows = gate_up.numel() // width
+    _need(gate_up.is_cuda and gate_up.dtype == torch.bfloat16 and gate_up.is_contiguous() and width % 16 == 0,
+          "gate_up: contiguous bf16 [..., 2n] with n a multiple of 8")
+    out = torch.empty(*gate_up.shape[:-1], inter, dtype=gate_up.dtype, device=gate_up.device)
+    _lib.check(_lib.lib().pkv_silu_mul(_p(gate_up), width, rows, inter, _p(out), _stream(gate_up)))
+    return out
+
+
 def alloc_pinned(shape, dtype: torch.dtype, zero: bool = False) -> torch.Tensor:
     """Pinned, device-mapped host tensor of exactly the requested size, optionally zero-filled (``pkv_host_alloc_mapped`` =
     hipHostMalloc).  torch's own pinned allocator rounds every block up to a power of two, which nearly doubles the

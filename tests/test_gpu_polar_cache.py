@@ -463,3 +463,30 @@ def test_qk_norm_rope_matches_torch_ops():
             assert bool((err <= want.abs() * 2 ** -7 + 1e-6).all()), float(err.max())
     with pytest.raises(RuntimeError, match="go together"):
         ops.qk_norm_rope(qkv, Hq, Hkv, qw, None, eps, cos, sin)
+
+
+def test_add_rmsnorm_and_silu_mul_match_torch_ops():
+    """The two fused element-wise kernels of the decode glue against the torch op sequences they replace (bf16 add then
+    F.rms_norm; F.silu then multiply), element for element up to one bf16 rounding."""
+    import torch.nn.functional as F
+
+    from pariskv_amd import ops
+
+    g = torch.Generator(device=DEV).manual_seed(6)
+    for rows, width in ((8, 4096), (3, 256), (1, 16384), (5, 1000)):
+        x = torch.randn(rows, 1, width, generator=g, device=DEV).to(torch.bfloat16)
+        r = torch.randn(rows, 1, width, generator=g, device=DEV).to(torch.bfloat16)
+        w = (1 + 0.2 * torch.randn(width, generator=g, device=DEV)).to(torch.bfloat16)
+        s, n = ops.add_rmsnorm(x, r, w, 1e-6)
+        want_s = x + r
+        assert torch.equal(s, want_s)
+        want_n = F.rms_norm(want_s.float(), (width,), w.float(), 1e-6)
+        assert bool(((n.float() - want_n).abs() <= want_n.abs() * 2 ** -7 + 1e-6).all())
+        s2, n2 = ops.add_rmsnorm(x, None, w, 1e-6)
+        assert s2 is x and bool(((n2.float() - F.rms_norm(x.float(), (width,), w.float(), 1e-6)).abs()
+                                 <= n2.float().abs() * 2 ** -7 + 1e-6).all())
+    gu = (torch.randn(8, 1, 2 * 12288, generator=g, device=DEV) * 3).to(torch.bfloat16)
+    got = ops.silu_mul(gu)
+    want = F.silu(gu[..., :12288].float()) * gu[..., 12288:].float()
+    assert got.shape == (8, 1, 12288)
+    assert bool(((got.float() - want).abs() <= want.abs() * 2 ** -6 + 1e-6).all())
