@@ -274,7 +274,7 @@ def test_bucket_topk_all_equal_and_clamp(ops):
 
 
 @pytest.mark.parametrize("rows,L,k", [(32, 4096, 1024), (8, 1024, 256), (3, 777, 100), (2, 8192, 8192), (4, 20000, 2048),
-                                      (2, 105000, 2048), (1, 9000, 1)])
+                                      (2, 105000, 2048), (1, 9000, 1), (5, 13107, 1024), (2, 16384, 8192), (3, 16385, 100)])
 def test_topk_f32_exact(ops, rows, L, k):
     _say(f"topk_f32 rows={rows} L={L} k={k}")
     rng = np.random.default_rng(L * 7 + k)
