@@ -490,3 +490,58 @@ def test_add_rmsnorm_and_silu_mul_match_torch_ops():
     want = F.silu(gu[..., :12288].float()) * gu[..., 12288:].float()
     assert got.shape == (8, 1, 12288)
     assert bool(((got.float() - want).abs() <= want.abs() * 2 ** -6 + 1e-6).all())
+
+
+@pytest.mark.parametrize("offload", [True, False])
+def test_fp32_cache_decode_steps(offload):
+    """The cache class with dtype float32 (BASELINE config 1's dtype): fp32 K/V rows (512-byte rows through append,
+    offload and gather), the fp32 encoder / query chains and the fp32 attention kernel.  Index set equal to the
+    oracle's fp32 chain on the cache's own index, attention within 1e-3 of an fp32 softmax over the same rows."""
+    from pariskv_amd.cache_hub.polar_cache import polar_cache
+
+    bs, Hkv, Hq, S, steps = 2, 2, 8, 2500, 40
+    sink, local, I, topk = 4, 64, 32, 150
+    G = Hq // Hkv
+    cache = polar_cache(valid_start=[0] * bs, layer_num=1, batch_size=bs, max_length=S + steps + 8, num_key_value_heads=Hkv,
+                        num_heads=Hq, head_dim=128, dtype=torch.float32, layer_mapping={0: DEV}, max_new_length=steps + 8,
+                        sink_size=sink, local_size=local, core=1, nprobe=1, cache_unit_size=1, cache_cluster_num=1, num_gpus=1,
+                        model_size=7, final_topk=topk, dynamic_update_interval=I, full_attention_threshold=100,
+                        enable_offload=offload)
+    gen = torch.Generator().manual_seed(9)
+    k = torch.randn(bs, S, Hkv, 128, generator=gen)
+    k[..., [7, 31, 64, 101]] *= 10.0
+    v = torch.randn(bs, S, Hkv, 128, generator=gen)
+    cache.prefill_update_kv_cache(None, k.to(DEV), v.to(DEV), 0, 0)
+    signs = O.srht_signs(42)
+    hk, hv = k, v
+    for step in range(steps):
+        k1, v1 = torch.randn(bs, 1, Hkv, 128, generator=gen), torch.randn(bs, 1, Hkv, 128, generator=gen)
+        q = (hk.mean(dim=1).repeat_interleave(G, dim=1) + 0.5 * torch.randn(bs, Hq, 128, generator=gen)).view(bs, 1, Hq, 128)
+        hk, hv = torch.cat([hk, k1], dim=1), torch.cat([hv, v1], dim=1)
+        cache.decode_update_kv_cache(k1.to(DEV), v1.to(DEV), 0)
+        out = cache.compute(q.to(DEV), 0)
+        if step not in (0, I - 1, I, steps - 1):
+            continue
+        torch.cuda.synchronize()
+        assert out.dtype == torch.float32
+        total = S + step + 1
+        n_keys, n_cand, kk, tiers = cache.retrieval_shape(0)
+        ids = cache.last_topk_indices.cpu().numpy()
+        for b in range(bs):
+            ref = torch.empty(Hq, 128)
+            for h in range(Hkv):
+                zone = slice(sink, sink + n_keys)
+                codes = cache._codes_km[0][b, h, zone].cpu().numpy()
+                nib = cache._nib_km[0][b, h, zone].cpu().numpy().reshape(-1, 16, 4)
+                w = cache._w_km[0][b, h, zone].float().cpu().numpy()
+                if step == 0:
+                    ec, en, ew = O.encode(hk[b, sink:sink + n_keys, h].numpy(), signs, O.F32)
+                    assert np.array_equal(codes, ec) and np.array_equal(nib, en) and np.array_equal(w, ew)
+                want = O.retrieve_row(q[b, 0, h * G:(h + 1) * G].numpy(), signs, O.F32, codes, nib, w,
+                                      cache.cluster_key_counts_gpu[0][b, h].cpu().numpy(), tiers, n_cand, kk)
+                assert np.array_equal(np.sort(ids[b, h]), np.sort(want)), (step, b, h)
+                sel = torch.cat([torch.arange(sink), torch.from_numpy(ids[b, h]) + sink, torch.arange(sink + n_keys, total)])
+                ref[h * G:(h + 1) * G] = _ref_attention(q[b, 0, h * G:(h + 1) * G], hk[b].permute(1, 0, 2)[h:h + 1, sel],
+                                                        hv[b].permute(1, 0, 2)[h:h + 1, sel], G=G * 10)
+            err = (out[b, 0].cpu() - ref).abs().max().item()
+            assert err < 1e-3, f"step {step}: attention differs by {err}"
