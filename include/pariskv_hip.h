@@ -48,6 +48,11 @@ extern "C" {
 
 int pkv_version(void);
 const char *pkv_last_error(void);
+/* sizeof of the argument structs as this library was compiled, for a binding to
+ * compare with its own mirror: 0 pkv_attn_segment, 1 pkv_attn_args,
+ * 2 pkv_retrieve_args, 3 pkv_adaptive_args (0 for any other number).
+ * No counterpart in the reference. */
+size_t pkv_struct_bytes(int which);
 
 /* ------------------------------------------------------------------ append */
 
@@ -209,11 +214,17 @@ int pkv_gather_hbm(const void *src_k, const void *src_v, int64_t src_len,
  * are slices of one fused projection output with different strides);
  * dst_k/dst_v: device [bs][h][dst_len] rows addressed
  * dst + b*dst_stride_b + h*dst_stride_h + slot*row_bytes.
- * All strides in BYTES, multiples of 16. */
+ * All strides in BYTES, multiples of 16.
+ * vnorm (optional, device float, rows of 128 elements only: row_bytes 256 = bf16,
+ * 512 = fp32): vnorm[b*vn_stride_b + h*vn_stride_h + slot] = ||v_new[b][h]||_2 in
+ * the rows' dtype, widened - the value-norm bookkeeping of the adaptive-k cache
+ * (cache_hub/polar_cache_adaptivek_varlen.py:1179) in the same launch; strides in
+ * elements. */
 int pkv_append_kv(const void *k_new, int64_t k_stride_b, int64_t k_stride_h,
                   const void *v_new, int64_t v_stride_b, int64_t v_stride_h,
                   void *dst_k, void *dst_v, int64_t dst_stride_b, int64_t dst_stride_h, int64_t dst_len,
-                  int64_t slot, int bs, int n_kv_heads, int row_bytes, void *stream);
+                  int64_t slot, int bs, int n_kv_heads, int row_bytes,
+                  float *vnorm, int64_t vn_stride_b, int64_t vn_stride_h, void *stream);
 
 /* The oldest tokens of a layer leave the GPU: replaces the copy_() of staged
  * [bs][h][n][d] tensors into slices of the pinned host tensors on the side
@@ -300,13 +311,31 @@ int pkv_host_device_pointer(const void *host_ptr, void **dev_ptr);
  * dense_benefit + sum of the k largest candidate benefits >= threshold * total
  * (k_out if never, 1 if total <= 0); topk_ids int64 [rows][k_out] = cand_ids in
  * descending benefit order (ties: candidate position ascending).
+ * k_max > 0: adaptive_k is clamped to [k_min, k_max] before it is written (the
+ * caller's clamp, polar_cache_adaptivek_varlen.py:1759); row_keys (optional,
+ * device int32 [rows]) receives row_keys_base + adaptive_k, the per-row key count
+ * that pkv_decode_attention takes.
  * ws: pkv_adaptive_topk_ws_bytes(rows, n_cand, k_out) bytes. */
 size_t pkv_adaptive_topk_ws_bytes(int rows, int64_t n_cand, int64_t k_out);
 int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, const float *sl_vnorm, int64_t slv_stride,
                       int64_t sl, const void *cand_scores, int cand_dtype, float cand_scale,
                       const float *cand_vnorm, const float *value_norm, int64_t vn_stride, int64_t vn_offset,
                       const int64_t *cand_ids, int64_t n_cand, float threshold, int64_t k_out, int rows,
-                      int64_t *adaptive_k, int64_t *topk_ids, void *ws, size_t ws_bytes, void *stream);
+                      int64_t *adaptive_k, int64_t *topk_ids, int64_t k_min, int64_t k_max,
+                      int32_t *row_keys, int64_t row_keys_base, void *ws, size_t ws_bytes, void *stream);
+
+/* Logits of the dense (sink / local / update buffer) rows against the mean of
+ * each KV head's query group: replaces query.mean over the group plus
+ * torch.einsum("bhd,bhkd->bhk") .to(float32) * scale
+ * (cache_hub/polar_cache_adaptivek_varlen.py:1418-1419, :1731) with one launch.
+ * q [bs][1][n_kv_heads*group][128] contiguous, k rows of 128 elements addressed
+ * k + b*k_stride_b + h*k_stride_h + r*128 (strides in elements), both of dtype;
+ * out float [bs*n_kv_heads][out_stride], first n_rows of each row written.
+ * bf16: the mean and the dot product are each rounded to bf16 (fp32 sums in a
+ * fixed order), as the torch expressions round them. */
+int pkv_dense_logits(const void *q, int dtype, int bs, int n_kv_heads, int group, const void *k,
+                     int64_t k_stride_b, int64_t k_stride_h, int64_t n_rows, float scale, float *out,
+                     int64_t out_stride, void *stream);
 
 /* --------------------------------------------------------- decode attention */
 
@@ -444,6 +473,44 @@ typedef struct pkv_attn_args {
 
 int pkv_decode_step(const pkv_retrieve_args *retrieve, void *ws, size_t ws_bytes,
                     const pkv_attn_args *attention, void *stream);
+
+/* The adaptive-k decode step of one layer from one host call
+ * (cache_hub/polar_cache_adaptivek_varlen.py:1391-1677 after the dense-fallback
+ * test): pkv_retrieve in its candidates-only form (retrieve->out_ids == NULL,
+ * retrieve->src_k == NULL) -> pkv_dense_logits over the first dense_rows rows of
+ * the GPU K store -> pkv_adaptive_topk on the fp32 rerank scores (logit = score
+ * times `scale`) with the value norms looked up by position ->
+ * pkv_gather_uva_ragged of each row's own k rows from the pinned host store ->
+ * pkv_decode_attention with row_keys = row_keys_base + k.  Every field has the
+ * meaning of the same-named argument of those entry points. */
+typedef struct pkv_adaptive_args {
+  const void *dense_k;            /* GPU K store; rows 0 .. dense_rows-1 of each (b, h) are the dense tokens */
+  int64_t dense_stride_b, dense_stride_h;  /* elements */
+  int64_t dense_rows;
+  const float *dense_vnorm;       /* [bs*n_kv_heads][dense_vnorm_stride] */
+  int64_t dense_vnorm_stride;
+  float *dense_logits;            /* scratch [bs*n_kv_heads][dense_logits_stride] */
+  int64_t dense_logits_stride;
+  float scale;                    /* attention scale: logits of dense rows and of candidates */
+  const float *value_norm;        /* [bs*n_kv_heads][vn_stride], candidate id + vn_offset */
+  int64_t vn_stride, vn_offset;
+  float threshold;
+  int64_t k_out, k_min, k_max;
+  int64_t *adaptive_k;            /* [bs*n_kv_heads] */
+  int64_t *topk_ids;              /* [bs*n_kv_heads][k_out] */
+  int32_t *row_keys;              /* [bs*n_kv_heads]; also passed to the attention */
+  int64_t row_keys_base;
+  void *ws;                       /* pkv_adaptive_topk_ws_bytes(rows, n_cand, k_out) */
+  size_t ws_bytes;
+  const void *src_k, *src_v;      /* pinned host K/V stores [bs][h][src_len] rows */
+  int64_t src_len, idx_offset;
+  void *dst_k, *dst_v;            /* GPU [bs][h][dst_len] rows; row (b, h) receives its k rows from dst_row0 on */
+  int64_t dst_len, dst_row0;
+  int row_bytes;
+} pkv_adaptive_args;
+
+int pkv_adaptive_decode_step(const pkv_retrieve_args *retrieve, void *ws, size_t ws_bytes,
+                             const pkv_adaptive_args *adaptive, const pkv_attn_args *attention, void *stream);
 
 /* Names and device pointers of the intermediates inside a pkv_retrieve
  * workspace (for tests and profiling): qhat, qnorm, lut, cnt_u8,

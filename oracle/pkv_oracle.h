@@ -25,8 +25,10 @@
  *   - tie order of pkv_o_rank_centroids, pkv_o_select_candidates and
  *     pkv_o_topk_f32 where the reference's unstable argsort / atomic
  *     compaction leaves it open: the oracle picks (value desc, index asc);
- *   - summation orders of pkv_o_adaptive_topk (the reference leaves them to
- *     torch): k agrees with the reference form within 1.
+ *   - summation orders of pkv_o_adaptive_topk and of the two numpy
+ *     restatements that feed it (dense_logits, value_norm in pkv_oracle.py;
+ *     the reference leaves all of them to torch): k agrees with the reference
+ *     form within 1, logits and norms with torch's within one bf16 step.
  * Everything else, including the SRHT sign vector (a Philox4x32-10 draw,
  * checked against the generator's known-answer vectors and against torch's
  * device generator), is pinned by the tests named in tests/test_oracle_*.py.

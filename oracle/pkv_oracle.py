@@ -219,6 +219,44 @@ def adaptive_topk(sl_logits, sl_vnorm, cand_logits, cand_vnorm, cand_ids, thresh
     return int(k), out
 
 
+def dense_logits(q, keys, scale, dtype):
+    """Logits of the dense (sink / local / buffer) tokens of one KV head against the group-mean query
+    (polar_cache_adaptivek_varlen.py:1418-1419 ``mean(dim=2)``, :1731 ``einsum(...).to(float32) * scale``), numpy.
+    q [G,128], keys [n,128] (bf16-representable values for the bf16 chain).  The mean adds the heads in order and
+    divides by G, like pkv_o_query_prep; the dot product is evaluated in one fixed order: dims in 16 groups of 8,
+    each group left to right, the 16 group sums in a pairwise tree; mean and dot are rounded to the dtype."""
+    q, keys = _f32(q), _f32(keys)
+    rd = bf16_round if dtype == BF16 else (lambda x: x)
+    acc = q[0].copy()
+    for g in range(1, q.shape[0]):
+        acc = acc + q[g]
+    mean = rd(acc / np.float32(q.shape[0]))
+    p = (keys * mean[None, :]).reshape(keys.shape[0], 16, 8)
+    s = p[:, :, 0].copy()
+    for j in range(1, 8):
+        s = s + p[:, :, j]
+    while s.shape[1] > 1:
+        s = s[:, 0::2] + s[:, 1::2]
+    return (rd(s[:, 0]) * np.float32(scale)).astype(np.float32)
+
+
+def value_norm(v, dtype):
+    """||v||_2 of rows [n,128] in the rows' dtype, widened to fp32 (polar_cache_adaptivek_varlen.py:1179
+    ``torch.linalg.vector_norm(value_states, dim=-1).float()``), numpy: squares summed in a fixed order (bf16 rows:
+    16 groups of 8 left to right; fp32 rows: 32 groups of 4; group sums in a pairwise tree), fp32 square root, rounded
+    to the dtype."""
+    v = _f32(v)
+    per = 8 if dtype == BF16 else 4
+    p = (v * v).reshape(v.shape[0], 128 // per, per)
+    s = p[:, :, 0].copy()
+    for j in range(1, per):
+        s = s + p[:, :, j]
+    while s.shape[1] > 1:
+        s = s[:, 0::2] + s[:, 1::2]
+    n = np.sqrt(s[:, 0], dtype=np.float32)
+    return bf16_round(n) if dtype == BF16 else n
+
+
 def retrieve_row(q, signs, dtype, codes, nib, weight, cluster_counts, tiers, n_cand, k):
     """Whole retrieval (query prep .. final top-k) for one (batch, kv-head) row."""
     q = _f32(q).reshape(-1, D)

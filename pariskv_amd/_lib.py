@@ -52,10 +52,26 @@ class RetrieveArgs(C.Structure):
     ]
 
 
+class AdaptiveArgs(C.Structure):
+    """Mirror of ``pkv_adaptive_args``."""
+
+    _fields_ = [
+        ("dense_k", _vp), ("dense_stride_b", _i64), ("dense_stride_h", _i64), ("dense_rows", _i64),
+        ("dense_vnorm", _vp), ("dense_vnorm_stride", _i64), ("dense_logits", _vp), ("dense_logits_stride", _i64),
+        ("scale", C.c_float), ("value_norm", _vp), ("vn_stride", _i64), ("vn_offset", _i64),
+        ("threshold", C.c_float), ("k_out", _i64), ("k_min", _i64), ("k_max", _i64),
+        ("adaptive_k", _vp), ("topk_ids", _vp), ("row_keys", _vp), ("row_keys_base", _i64),
+        ("ws", _vp), ("ws_bytes", _sz),
+        ("src_k", _vp), ("src_v", _vp), ("src_len", _i64), ("idx_offset", _i64),
+        ("dst_k", _vp), ("dst_v", _vp), ("dst_len", _i64), ("dst_row0", _i64), ("row_bytes", _i),
+    ]
+
+
 # name -> (restype, argtypes); one entry per declaration in include/pariskv_hip.h
 PROTOTYPES = {
     "pkv_version": (_i, []),
     "pkv_last_error": (C.c_char_p, []),
+    "pkv_struct_bytes": (_sz, [_i]),
     "pkv_encode_append": (_i, [_vp, _i, _i, _i, _i64, _i64, _i64, _i64, _vp,
                                _vp, _i64, _i64, _i64, _i64,
                                _vp, _i64, _i64, _i64, _i64,
@@ -79,7 +95,8 @@ PROTOTYPES = {
                          _vp, _vp, _vp, _vp, _vp, _vp]),
     "pkv_gather_uva": (_i, [_vp, _vp, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i, _i, _i, _vp]),
     "pkv_gather_hbm": (_i, [_vp, _vp, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i, _i, _i, _vp]),
-    "pkv_append_kv": (_i, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i, _i, _i, _vp]),
+    "pkv_append_kv": (_i, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i, _i, _i,
+                           _vp, _i64, _i64, _vp]),
     "pkv_offload_rows": (_i, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i, _i, _i, _vp]),
     "pkv_gather_uva_ragged": (_i, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i64, _i64, _i, _i, _i, _vp]),
     "pkv_gather_uva_packed": (_i, [_vp, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _i64, _i, _i, _i, _vp]),
@@ -89,7 +106,8 @@ PROTOTYPES = {
     "pkv_host_device_pointer": (_i, [_vp, C.POINTER(_vp)]),
     "pkv_adaptive_topk_ws_bytes": (_sz, [_i, _i64, _i64]),
     "pkv_adaptive_topk": (_i, [_vp, _i64, _vp, _i64, _i64, _vp, _i, C.c_float, _vp, _vp, _i64, _i64, _vp, _i64,
-                               C.c_float, _i64, _i, _vp, _vp, _vp, _sz, _vp]),
+                               C.c_float, _i64, _i, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
+    "pkv_dense_logits": (_i, [_vp, _i, _i, _i, _i, _vp, _i64, _i64, _i64, C.c_float, _vp, _i64, _vp]),
     "pkv_decode_attention_ws_bytes": (_sz, [_i, _i, _i, _i64]),
     "pkv_decode_attention": (_i, [_vp, _i, _i, _i, _i, C.POINTER(AttnSegment), _i, _vp, C.c_float, _vp, _vp, _sz, _vp]),
     "pkv_qk_norm_rope": (_i, [_vp, _i64, _i, _i, _i, _vp, _vp, C.c_float, _vp, _vp, _vp, _vp, _vp]),
@@ -98,6 +116,7 @@ PROTOTYPES = {
     "pkv_retrieve_ws_bytes": (_sz, [_i, _i64, _i64, _i64]),
     "pkv_retrieve": (_i, [C.POINTER(RetrieveArgs), _vp, _sz, _vp]),
     "pkv_decode_step": (_i, [C.POINTER(RetrieveArgs), _vp, _sz, C.POINTER(AttnArgs), _vp]),
+    "pkv_adaptive_decode_step": (_i, [C.POINTER(RetrieveArgs), _vp, _sz, C.POINTER(AdaptiveArgs), C.POINTER(AttnArgs), _vp]),
     "pkv_retrieve_ws_view": (_i, [_vp, _i, _i64, _i64, _i64, C.c_char_p, C.POINTER(_vp), C.POINTER(_sz)]),
 }
 
@@ -129,6 +148,10 @@ def lib():
             fn = getattr(handle, name)
             fn.restype = res
             fn.argtypes = args
+        for which, mirror in enumerate((AttnSegment, AttnArgs, RetrieveArgs, AdaptiveArgs)):
+            if handle.pkv_struct_bytes(which) != C.sizeof(mirror):
+                raise RuntimeError(f"{SO_PATH} was built from another header: {mirror.__name__} is "
+                                   f"{handle.pkv_struct_bytes(which)} bytes there, {C.sizeof(mirror)} here; rebuild it")
         _lib = handle
     return _lib
 

@@ -265,8 +265,7 @@ class polar_cache(KV_Cache):
         slot = z.append_slot()
         if key_states.dtype != self.dtype or value_states.dtype != self.dtype:
             key_states, value_states = key_states.to(self.dtype), value_states.to(self.dtype)
-        ops.append_kv(key_states, value_states, self.unified_keys_gpu[layer_idx], self.unified_values_gpu[layer_idx], slot)
-        self._on_decode_write(layer_idx, slot, value_states)
+        self._append(layer_idx, slot, key_states, value_states)
         refresh = z.appended()
         self.current_seq_len[layer_idx] = z.seq_len
         if layer_idx == 0:
@@ -303,8 +302,8 @@ class polar_cache(KV_Cache):
     def _on_prefill(self, layer_idx, b0, b1, values_bhsd, retrieval, local_len):
         pass
 
-    def _on_decode_write(self, layer_idx, slot, value_states):
-        pass
+    def _append(self, layer_idx, slot, key_states, value_states):
+        ops.append_kv(key_states, value_states, self.unified_keys_gpu[layer_idx], self.unified_values_gpu[layer_idx], slot)
 
     def _on_refresh(self, layer_idx, r):
         pass

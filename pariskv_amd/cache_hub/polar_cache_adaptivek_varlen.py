@@ -66,6 +66,13 @@ class polar_cache(_polar_cache_base):
         cap = max(1, self._adaptive_topk_buffer_cap)
         self._topk_k = torch.zeros((bs, H, cap, self.head_dim), dtype=self.dtype, device=dev)
         self._topk_v = torch.zeros((bs, H, cap, self.head_dim), dtype=self.dtype, device=dev)
+        # operands of the fused step that all layers share
+        self._dense_logits = torch.empty((bs, H, self.gpu_kv_capacity), dtype=torch.float32, device=dev)
+        self._adaptive_k = torch.zeros((bs, H), dtype=torch.int64, device=dev)
+        self._topk_ids = torch.zeros((bs * H * cap,), dtype=torch.int64, device=dev)
+        self._row_keys = torch.zeros((bs, H), dtype=torch.int32, device=dev)
+        self._adk_ws = None
+        self._adaptive_bound = [None] * layer_num  # per layer: (n_keys, ops.BoundAdaptiveStep, topk_cap)
         self.last_adaptive_k = None  # [bs, H] int64 of the most recent retrieval step
 
     # ------------------------------------------------------------ ratios
@@ -95,8 +102,10 @@ class polar_cache(_polar_cache_base):
         sl[b0:b1, :, S0:S0 + local_len] = self._vnorm(values_bhsd[:, :, r_end:r_end + local_len])  # :706
         self.value_norm_gpu[layer_idx][b0:b1, :, S0:r_end] = self._vnorm(values_bhsd[:, :, S0:r_end])  # :753-756
 
-    def _on_decode_write(self, layer_idx, slot, value_states):
-        self._sl_vnorm_cache[layer_idx][:, :, slot] = self._vnorm(value_states[:, 0])             # :1179
+    def _append(self, layer_idx, slot, key_states, value_states):
+        """K/V rows and the value norm of the new token (:1179) in one launch."""
+        ops.append_kv(key_states, value_states, self.unified_keys_gpu[layer_idx], self.unified_values_gpu[layer_idx], slot,
+                      vnorm=self._sl_vnorm_cache[layer_idx])
 
     def _on_refresh(self, layer_idx, r):
         S0, n, L = self.sink_size, r.n_new, self.local_size
@@ -111,20 +120,22 @@ class polar_cache(_polar_cache_base):
         mask = torch.arange(topk_cap, device=dense_indices.device).unsqueeze(0) < adaptive_k.view(V, 1)
         return dense_indices.contiguous().view(V, topk_cap)[mask]
 
+    def _caps(self, cand_len):
+        """(topk_cap, k_min, k_max) for a candidate list of ``cand_len`` (reference :1703-1712, :1759)."""
+        effective_max_k = min(self._HARDCODED_MAX_K, cand_len)
+        effective_min_k = min(self._HARDCODED_MIN_K, effective_max_k)
+        return effective_max_k, max(1, effective_min_k), max(1, effective_max_k)
+
     def _adaptive_topk_device(self, query_avg, sink_local_keys, sl_vnorm, all_cand_scores, all_cand_indices, layer_idx,
                               threshold):
         """Per-row k and the candidate ids in benefit order, all on the GPU (reference :1684-1759).
         Returns (adaptive_k [bs,H] int64 after the clamp, topk_ids [bs,H,topk_cap] int64, topk_cap)."""
-        cand_len = all_cand_scores.shape[-1]
-        effective_max_k = min(self._HARDCODED_MAX_K, cand_len)
-        effective_min_k = min(self._HARDCODED_MIN_K, effective_max_k)
-        topk_cap = effective_max_k
-        # logits of the dense tokens: a plain library contraction, as in the reference (:1731)
-        logits_sl = torch.einsum("bhd,bhkd->bhk", query_avg, sink_local_keys).to(torch.float32) * self._attn_scale
+        topk_cap, k_min, k_max = self._caps(all_cand_scores.shape[-1])
+        # logits of the dense tokens (:1731); a [bs,H,D] mean query is a query group of one head
+        logits_sl = ops.dense_logits(query_avg.contiguous(), sink_local_keys, sink_local_keys.shape[2], self._attn_scale)
         adaptive_k, topk_ids = ops.adaptive_topk(logits_sl, sl_vnorm, all_cand_scores, self._attn_scale, all_cand_indices,
                                                  float(threshold), topk_cap, value_norm=self.value_norm_gpu[layer_idx],
-                                                 vn_offset=self.sink_size)
-        adaptive_k.clamp_(min=max(1, effective_min_k), max=max(1, effective_max_k))               # :1759
+                                                 vn_offset=self.sink_size, k_min=k_min, k_max=k_max)   # clamp: :1759
         return adaptive_k, topk_ids, topk_cap
 
     def _compute_adaptive_topk(self, query_avg, sink_local_keys, sl_vnorm, all_cand_scores, all_cand_indices, layer_idx,
@@ -144,25 +155,44 @@ class polar_cache(_polar_cache_base):
         min_total = max(self.FULL_ATTENTION_THRESHOLD, self.sink_size + self.local_size + self.final_topk * 2)
         if total < min_total or n_keys <= 0:
             return super().compute(queries, layer_idx)  # dense branch
-        q = queries.contiguous()
-        bs, H, G, D = self.batch_size, self.kv_head, self.group_size, self.head_dim
-        n_keys, n_cand, _, tiers = self.retrieval_shape(layer_idx)
+        q = queries if queries.is_contiguous() else queries.contiguous()
+        step = self._adaptive_bound[layer_idx]
+        if step is None or step[0] != n_keys:
+            step = self._bind_adaptive_step(layer_idx, q, n_keys)
+        _, bound, _ = step
+        # what moves with every token: the dense rows (sink + local + update buffer) grow by one
+        sl_end = z.gpu_prefix_rows
+        bound.ad.dense_rows = sl_end
+        bound.ad.row_keys_base = sl_end
+        bound.segs[0].n_rows = sl_end
         self._wait_offload(layer_idx)
-        cand, scores = self._plan.run_candidates(q, self._srht_signs, self._mag_centers, self.cluster_key_counts_gpu[layer_idx],
-                                                 self._codes_km[layer_idx], self._nib_km[layer_idx], self._w_km[layer_idx],
-                                                 self.sink_size, n_keys, tiers, n_cand)
+        self.last_adaptive_k = self._adaptive_k
+        # One host call: candidates + rerank scores -> logits of the dense rows -> adaptive k -> ragged UVA gather (row
+        # (b, h) receives its own k rows at the head of its slice of the dense buffer) -> attention.  The reference
+        # packs the indices and reads the largest k back to the host to size its launch (:1597-1644); the gather and
+        # the attention take the per-row count from device memory instead, so the step never waits for the GPU.
+        return bound.launch(q)
+
+    def _bind_adaptive_step(self, layer_idx, q, n_keys):
+        """Argument blocks of this layer's step, valid until the next index refresh changes ``n_keys``."""
+        z = self._zones[layer_idx]
+        n_keys, n_cand, _, tiers = self.retrieval_shape(layer_idx)
+        topk_cap, k_min, k_max = self._caps(n_cand)
         kg, vg = self.unified_keys_gpu[layer_idx], self.unified_values_gpu[layer_idx]
-        sl_end = z.gpu_prefix_rows                                   # sink + local + update buffer rows
-        query_avg = q[:, 0].view(bs, H, G, D).mean(dim=2)            # :1418-1419
-        adaptive_k, topk_ids, topk_cap = self._adaptive_topk_device(
-            query_avg, kg[:, :, :sl_end], self._sl_vnorm_cache[layer_idx][:, :, :sl_end], scores, cand, layer_idx,
-            self.adaptive_topk_threshold)
-        self.last_adaptive_k = adaptive_k
-        # ragged UVA gather: row (b, h) receives its own k rows at the head of its slice of the dense buffer.  The
-        # reference packs the indices and reads the largest k back to the host to size its launch (:1597-1644); the
-        # attention below takes the per-row key count instead, so neither the packing nor the host read is needed and
-        # the step never waits for the GPU.
-        ops.gather_uva_ragged(self.unified_keys_cpu[layer_idx], self.unified_values_cpu[layer_idx], topk_ids, adaptive_k,
-                              self._topk_k, self._topk_v)
-        row_keys = (adaptive_k + sl_end).to(torch.int32)
-        return self._attention.run(q, [(kg, vg, 0, sl_end), (self._topk_k, self._topk_v, 0, topk_cap)], row_keys=row_keys)
+        sl_end = z.gpu_prefix_rows
+        need = ops.adaptive_topk_ws_bytes(self.batch_groups, n_cand, topk_cap)
+        if self._adk_ws is None or self._adk_ws.numel() < need:
+            self._adk_ws = torch.empty(need, dtype=torch.uint8, device=self.device)
+        adaptive = dict(dense_k=kg, dense_rows=sl_end, dense_vnorm=self._sl_vnorm_cache[layer_idx],
+                        dense_logits=self._dense_logits, scale=self._attn_scale, value_norm=self.value_norm_gpu[layer_idx],
+                        vn_offset=self.sink_size, threshold=self.adaptive_topk_threshold, k_out=topk_cap, k_min=k_min,
+                        k_max=k_max, adaptive_k=self._adaptive_k, topk_ids=self._topk_ids, row_keys=self._row_keys,
+                        row_keys_base=sl_end, ws=self._adk_ws, src_k=self.unified_keys_cpu[layer_idx],
+                        src_v=self.unified_values_cpu[layer_idx], dst_k=self._topk_k, dst_v=self._topk_v)
+        segments = [(kg, vg, 0, sl_end), (self._topk_k, self._topk_v, 0, topk_cap)]
+        bound = self._plan.bind_adaptive(q, self._srht_signs, self._mag_centers, self.cluster_key_counts_gpu[layer_idx],
+                                         self._codes_km[layer_idx], self._nib_km[layer_idx], self._w_km[layer_idx],
+                                         self.sink_size, n_keys, tiers, n_cand, adaptive, self._attention, segments)
+        step = (n_keys, bound, topk_cap)
+        self._adaptive_bound[layer_idx] = step
+        return step

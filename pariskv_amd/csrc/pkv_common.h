@@ -212,20 +212,16 @@ __device__ __forceinline__ float pkv_normalize_rotate_16(const float (&x)[8], co
   return n;
 }
 
-// Group mean of the G query heads of row (b, h), normalised and SRHT-rotated (polar_cache.py:1027-1031,
-// 905-922).  Called by all 64 lanes of ONE wave: 16 lanes per copy of the vector, four identical copies;
-// lane l gets dims 8(l & 15) .. +7 of the rotated unit vector in y[] and the norm of the mean as result.
-// The G heads are added in order; their loads are all issued before the first add (8 at a time, with no
-// branch between them, so that they are in flight together).
+// Mean of the G query heads of row (b, h) (polar_cache.py:1027): lane l of a wave gets dims 8(l & 15) .. +7
+// in x[], rounded to the working dtype.  The G heads are added in order; their loads are all issued before
+// the first add (8 at a time, with no branch between them, so that they are in flight together).
 template <bool BF16>
-__device__ __forceinline__ float pkv_query_mean_rotate_t(const void *__restrict__ q, int b, int h, int n_kv_heads,
-                                                         int group, const float *__restrict__ signs, float (&y)[8]) {
+__device__ __forceinline__ void pkv_query_group_mean_t(const void *__restrict__ q, int b, int h, int n_kv_heads,
+                                                       int group, float (&x)[8]) {
   constexpr int dtype = BF16 ? PKV_DTYPE_BF16 : PKV_DTYPE_F32;
   const int s = pkv_lane() & 15;
   const int64_t base = ((int64_t)b * n_kv_heads * group + (int64_t)h * group) * 128 + 8 * s;
-  float acc[8], sg[8];
-  const float4 s0 = *(const float4 *)(signs + 8 * s), s1 = *(const float4 *)(signs + 8 * s + 4);
-  sg[0] = s0.x, sg[1] = s0.y, sg[2] = s0.z, sg[3] = s0.w, sg[4] = s1.x, sg[5] = s1.y, sg[6] = s1.z, sg[7] = s1.w;
+  float acc[8];
   for (int g0 = 0; g0 < group; g0 += 8) {
     pkv_u32x4 raw[8][BF16 ? 1 : 2];
 #pragma unroll
@@ -259,7 +255,6 @@ __device__ __forceinline__ float pkv_query_mean_rotate_t(const void *__restrict_
       for (int j = 0; j < 8; ++j) acc[j] = first ? v[j] : (live ? acc[j] + v[j] : acc[j]);
     }
   }
-  float x[8];
   if ((group & (group - 1)) == 0) {  // power of two: multiplying by the reciprocal is the same division, exactly
     const float inv = 1.0f / (float)group;
 #pragma unroll
@@ -268,6 +263,20 @@ __device__ __forceinline__ float pkv_query_mean_rotate_t(const void *__restrict_
 #pragma unroll
     for (int j = 0; j < 8; ++j) x[j] = pkv_rdt(acc[j] / (float)group, dtype);
   }
+}
+
+// Group mean of the G query heads of row (b, h), normalised and SRHT-rotated (polar_cache.py:1027-1031,
+// 905-922).  Called by all 64 lanes of ONE wave: 16 lanes per copy of the vector, four identical copies;
+// lane l gets dims 8(l & 15) .. +7 of the rotated unit vector in y[] and the norm of the mean as result.
+template <bool BF16>
+__device__ __forceinline__ float pkv_query_mean_rotate_t(const void *__restrict__ q, int b, int h, int n_kv_heads,
+                                                         int group, const float *__restrict__ signs, float (&y)[8]) {
+  constexpr int dtype = BF16 ? PKV_DTYPE_BF16 : PKV_DTYPE_F32;
+  const int s = pkv_lane() & 15;
+  float x[8], sg[8];
+  const float4 s0 = *(const float4 *)(signs + 8 * s), s1 = *(const float4 *)(signs + 8 * s + 4);
+  sg[0] = s0.x, sg[1] = s0.y, sg[2] = s0.z, sg[3] = s0.w, sg[4] = s1.x, sg[5] = s1.y, sg[6] = s1.z, sg[7] = s1.w;
+  pkv_query_group_mean_t<BF16>(q, b, h, n_kv_heads, group, x);
   return pkv_normalize_rotate_16(x, sg, s, dtype, y);
 }
 

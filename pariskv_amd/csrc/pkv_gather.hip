@@ -76,10 +76,16 @@ __global__ __launch_bounds__(kGatherThreads) void pkv_gather_packed_kernel(
 // One new token per sequence: row (b, h) of k_new / v_new goes to row `slot` of
 // the [bs][h][dst_len] K and V stores.  Lane g: (task, lane) = divmod(g, vpr),
 // kv = task & 1, (b, h) = divmod(task >> 1, n_heads).  Strides in 16-byte vectors.
+// VNORM (0 off, 1 bf16 rows, 2 fp32 rows): the value row's Euclidean norm also goes to
+// vnorm[b*vn_stride_b + h*vn_stride_h + slot] as fp32: a lane adds the squares of its 16 bytes in
+// order, the vpr lanes of the row meet in a pairwise tree (lane ^ 1, 2, 4, ...), then the square
+// root, rounded to bf16 for bf16 rows (the norm of a bf16 tensor is a bf16 tensor).
+template <int VNORM>
 __global__ __launch_bounds__(kGatherThreads) void pkv_append_rows_kernel(
     const pkv_u32x4 *__restrict__ k_new, const pkv_u32x4 *__restrict__ v_new, int64_t k_stride_b, int64_t k_stride_h,
     int64_t v_stride_b, int64_t v_stride_h, pkv_u32x4 *__restrict__ dst_k, pkv_u32x4 *__restrict__ dst_v,
-    int64_t dst_stride_b, int64_t dst_stride_h, int64_t slot, int n_heads, int n_tasks, int vpr) {
+    int64_t dst_stride_b, int64_t dst_stride_h, int64_t slot, int n_heads, int n_tasks, int vpr,
+    float *__restrict__ vnorm, int64_t vn_stride_b, int64_t vn_stride_h) {
   const int g = blockIdx.x * kGatherThreads + threadIdx.x;
   const int task = g / vpr, lane = g % vpr;
   if (task >= n_tasks) return;
@@ -87,6 +93,31 @@ __global__ __launch_bounds__(kGatherThreads) void pkv_append_rows_kernel(
   const int b = (task >> 1) / n_heads, h = (task >> 1) % n_heads;
   const pkv_u32x4 val = kv ? v_new[b * v_stride_b + h * v_stride_h + lane] : k_new[b * k_stride_b + h * k_stride_h + lane];
   (kv ? dst_v : dst_k)[b * dst_stride_b + h * dst_stride_h + slot * vpr + lane] = val;
+  if (VNORM != 0) {  // tasks are whole groups of vpr lanes inside a wave: every lane of a row is here
+    const uint32_t w[4] = {val.x, val.y, val.z, val.w};
+    float acc;
+    if (VNORM == 1) {
+      float e[8];
+#pragma unroll
+      for (int p = 0; p < 4; ++p) e[2 * p] = __uint_as_float(w[p] << 16), e[2 * p + 1] = __uint_as_float(w[p] & 0xffff0000u);
+      acc = e[0] * e[0];
+#pragma unroll
+      for (int j = 1; j < 8; ++j) acc = acc + e[j] * e[j];
+    } else {
+      acc = __uint_as_float(w[0]) * __uint_as_float(w[0]);
+#pragma unroll
+      for (int j = 1; j < 4; ++j) acc = acc + __uint_as_float(w[j]) * __uint_as_float(w[j]);
+    }
+    acc = acc + pkv_lane_xor_f<1>(acc);
+    acc = acc + pkv_lane_xor_f<2>(acc);
+    acc = acc + pkv_lane_xor_f<4>(acc);
+    acc = acc + pkv_lane_xor_f<8>(acc);
+    if (VNORM == 2) acc = acc + pkv_lane_xor_f<16>(acc);
+    if (kv && lane == 0) {
+      const float n = sqrtf(acc);
+      vnorm[b * vn_stride_b + h * vn_stride_h + slot] = VNORM == 1 ? pkv_bf16_round(n) : n;
+    }
+  }
 }
 
 // Blocks of consecutive rows, one block per (batch, head), from the GPU into the pinned host store:
@@ -208,9 +239,11 @@ extern "C" int pkv_gather_uva(const void *src_k, const void *src_v, int64_t src_
 extern "C" int pkv_append_kv(const void *k_new, int64_t k_stride_b, int64_t k_stride_h, const void *v_new,
                              int64_t v_stride_b, int64_t v_stride_h, void *dst_k, void *dst_v, int64_t dst_stride_b,
                              int64_t dst_stride_h, int64_t dst_len, int64_t slot, int bs, int n_kv_heads, int row_bytes,
-                             void *stream) {
+                             float *vnorm, int64_t vn_stride_b, int64_t vn_stride_h, void *stream) {
   int rc = check_common(k_new, v_new, dst_k, dst_v, bs * n_kv_heads, row_bytes);
   if (rc) return rc;
+  PKV_REQUIRE(!vnorm || ((row_bytes == 256 || row_bytes == 512) && vn_stride_b >= 0 && vn_stride_h > slot),
+              "append: value norms need rows of 128 bf16 or fp32 elements and a norm row longer than the slot");
   PKV_REQUIRE(bs > 0 && n_kv_heads > 0 && (int64_t)bs * n_kv_heads <= (1 << 20), "append: bad batch/head count");
   PKV_REQUIRE(slot >= 0 && slot < dst_len, "append: slot %lld outside [0, %lld)", (long long)slot, (long long)dst_len);
   PKV_REQUIRE(k_stride_b % 16 == 0 && k_stride_h % 16 == 0 && v_stride_b % 16 == 0 && v_stride_h % 16 == 0 &&
@@ -220,10 +253,14 @@ extern "C" int pkv_append_kv(const void *k_new, int64_t k_stride_b, int64_t k_st
   const int vpr = row_bytes / 16;
   const int n_tasks = bs * n_kv_heads * 2;
   const int lanes = n_tasks * vpr;
-  hipLaunchKernelGGL(pkv_append_rows_kernel, dim3((unsigned)((lanes + kGatherThreads - 1) / kGatherThreads)),
-                     dim3(kGatherThreads), 0, (hipStream_t)stream, (const pkv_u32x4 *)k_new, (const pkv_u32x4 *)v_new,
-                     k_stride_b / 16, k_stride_h / 16, v_stride_b / 16, v_stride_h / 16, (pkv_u32x4 *)dst_k,
-                     (pkv_u32x4 *)dst_v, dst_stride_b / 16, dst_stride_h / 16, slot, n_kv_heads, n_tasks, vpr);
+  const dim3 grid((unsigned)((lanes + kGatherThreads - 1) / kGatherThreads));
+#define PKV_APPEND(VN)                                                                                              \
+  hipLaunchKernelGGL(pkv_append_rows_kernel<VN>, grid, dim3(kGatherThreads), 0, (hipStream_t)stream,                 \
+                     (const pkv_u32x4 *)k_new, (const pkv_u32x4 *)v_new, k_stride_b / 16, k_stride_h / 16,          \
+                     v_stride_b / 16, v_stride_h / 16, (pkv_u32x4 *)dst_k, (pkv_u32x4 *)dst_v, dst_stride_b / 16,   \
+                     dst_stride_h / 16, slot, n_kv_heads, n_tasks, vpr, vnorm, vn_stride_b, vn_stride_h)
+  if (!vnorm) PKV_APPEND(0); else if (row_bytes == 256) PKV_APPEND(1); else PKV_APPEND(2);
+#undef PKV_APPEND
   PKV_LAUNCH_CHECK("pkv_append_rows_kernel");
   return PKV_OK;
 }

@@ -24,6 +24,16 @@ void pkv_set_error(const char *fmt, ...) {
 
 extern "C" int pkv_version(void) { return 1; }
 
+extern "C" size_t pkv_struct_bytes(int which) {
+  switch (which) {
+    case 0: return sizeof(pkv_attn_segment);
+    case 1: return sizeof(pkv_attn_args);
+    case 2: return sizeof(pkv_retrieve_args);
+    case 3: return sizeof(pkv_adaptive_args);
+    default: return 0;
+  }
+}
+
 extern "C" const char *pkv_last_error(void) { return g_last_error.c_str(); }
 
 extern "C" int pkv_host_alloc_mapped(size_t bytes, void **host_ptr) {

@@ -1,7 +1,8 @@
 // One layer's retrieval for one decode step as a fixed sequence of launches on
 // the caller's stream: query prep + vote table -> collision scan (+ chunk
 // histograms) -> candidate select fused with the 4-bit rerank -> exact top-k ->
-// optional gather of the selected K/V rows (5 launches).
+// optional gather of the selected K/V rows (5 launches).  The adaptive-k step
+// replaces the exact top-k by the dense logits and the adaptive selection.
 //
 // Reference: cache_hub/polar_cache.py:1126-1162 (collision_based_topk_batch),
 // :1207-1231, :1244-1304 and the gather at :1075-1095.
@@ -168,6 +169,40 @@ extern "C" int pkv_decode_step(const pkv_retrieve_args *retrieve, void *ws, size
                                const pkv_attn_args *attention, void *stream) {
   PKV_REQUIRE(retrieve && attention, "pkv_decode_step: null args");
   int rc = pkv_retrieve(retrieve, ws, ws_bytes, stream);
+  if (rc) return rc;
+  return pkv_decode_attention(retrieve->q, retrieve->dtype, retrieve->bs, retrieve->n_kv_heads, retrieve->group,
+                              attention->segments, attention->n_segments, attention->row_keys, attention->scale,
+                              attention->out, attention->ws, attention->ws_bytes, stream);
+}
+
+extern "C" int pkv_adaptive_decode_step(const pkv_retrieve_args *retrieve, void *ws, size_t ws_bytes,
+                                        const pkv_adaptive_args *ad, const pkv_attn_args *attention, void *stream) {
+  PKV_REQUIRE(retrieve && ad && attention, "pkv_adaptive_decode_step: null args");
+  PKV_REQUIRE(!retrieve->out_ids && !retrieve->src_k,
+              "pkv_adaptive_decode_step: the retrieval must be in its candidates-only form (no out_ids, no gather)");
+  PKV_REQUIRE(ad->row_keys && attention->row_keys == ad->row_keys,
+              "pkv_adaptive_decode_step: the attention must read the row_keys the adaptive stage writes");
+  PKV_REQUIRE(ad->dense_rows > 0 && ad->dense_rows <= ad->dense_vnorm_stride && ad->dense_rows <= ad->dense_logits_stride,
+              "pkv_adaptive_decode_step: %lld dense rows exceed the norm / logit rows (%lld, %lld)",
+              (long long)ad->dense_rows, (long long)ad->dense_vnorm_stride, (long long)ad->dense_logits_stride);
+  int rc = pkv_retrieve(retrieve, ws, ws_bytes, stream);
+  if (rc) return rc;
+  const int rows = retrieve->bs * retrieve->n_kv_heads;
+  const WsLayout w = layout(rows, retrieve->n_keys, retrieve->n_cand, retrieve->k);
+  const int64_t *cand = (const int64_t *)((char *)ws + w.cand);
+  const float *scores = (const float *)((char *)ws + w.scores);
+  rc = pkv_dense_logits(retrieve->q, retrieve->dtype, retrieve->bs, retrieve->n_kv_heads, retrieve->group, ad->dense_k,
+                        ad->dense_stride_b, ad->dense_stride_h, ad->dense_rows, ad->scale, ad->dense_logits,
+                        ad->dense_logits_stride, stream);
+  if (rc) return rc;
+  rc = pkv_adaptive_topk(ad->dense_logits, ad->dense_logits_stride, ad->dense_vnorm, ad->dense_vnorm_stride,
+                         ad->dense_rows, scores, PKV_DTYPE_F32, ad->scale, nullptr, ad->value_norm, ad->vn_stride,
+                         ad->vn_offset, cand, retrieve->n_cand, ad->threshold, ad->k_out, rows, ad->adaptive_k,
+                         ad->topk_ids, ad->k_min, ad->k_max, ad->row_keys, ad->row_keys_base, ad->ws, ad->ws_bytes, stream);
+  if (rc) return rc;
+  rc = pkv_gather_uva_ragged(ad->src_k, ad->src_v, ad->src_len, ad->topk_ids, ad->k_out, ad->adaptive_k, ad->idx_offset,
+                             ad->dst_k, ad->dst_v, ad->dst_len, ad->dst_row0, retrieve->bs, retrieve->n_kv_heads,
+                             ad->row_bytes, stream);
   if (rc) return rc;
   return pkv_decode_attention(retrieve->q, retrieve->dtype, retrieve->bs, retrieve->n_kv_heads, retrieve->group,
                               attention->segments, attention->n_segments, attention->row_keys, attention->scale,

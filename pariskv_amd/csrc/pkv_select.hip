@@ -997,16 +997,28 @@ __device__ __forceinline__ void combine_slices(const float *__restrict__ pmax, i
 
 // Shared tail: s_keys[0 .. P) holds the k_out winners (zero padded, any order).  Sorts them, finds k,
 // writes adaptive_k[row] and the candidate ids in benefit order.
+// What the caller does with k right after the kernel, folded into it: the clamp to [k_min, k_max] (off when
+// k_max <= 0) and the per-row key count row_keys[row] = row_keys_base + k that the attention kernel reads.
+struct AdkClamp {
+  int64_t k_min, k_max;
+  int32_t *row_keys;
+  int64_t row_keys_base;
+};
+
 __device__ __forceinline__ void adaptive_tail(uint64_t *s_keys, int P, int64_t k_out, float sl_benefit, float total,
                                               float threshold, const int64_t *__restrict__ ci, int64_t n_cand,
                                               int64_t *__restrict__ adaptive_k_row, int64_t *__restrict__ ids_row,
-                                              float *s_f, uint32_t *s_k) {
+                                              AdkClamp cl, int row, float *s_f, uint32_t *s_k) {
 #define PKV_SORT_K(NT, E) sort_lds_keys_and_emit<NT, E>(s_keys, 0, nullptr, nullptr, s_keys)
   PKV_DISPATCH_E(P, PKV_SORT_K);
 #undef PKV_SORT_K
   int64_t k = 1;  // total <= 0: adaptive_topk.py:304-306
   if (total > 0.f) k = first_k_reaching(s_keys, k_out, sl_benefit, threshold * total, s_f, s_k);
-  if (threadIdx.x == 0) *adaptive_k_row = k;
+  if (threadIdx.x == 0) {
+    if (cl.k_max > 0) k = k < cl.k_min ? cl.k_min : (k > cl.k_max ? cl.k_max : k);
+    *adaptive_k_row = k;
+    if (cl.row_keys) cl.row_keys[row] = (int32_t)(cl.row_keys_base + k);
+  }
   for (int64_t i = threadIdx.x; i < k_out; i += kTopkThreads) {
     const uint32_t pos = ~(uint32_t)s_keys[i];
     ids_row[i] = (pos < (uint64_t)n_cand) ? ci[pos] : 0;
@@ -1047,7 +1059,7 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adaptive_topk_kernel(
     int64_t sl, const void *__restrict__ cand_scores, int cand_dtype, float cand_scale,
     const float *__restrict__ cand_vnorm, const float *__restrict__ value_norm, int64_t vn_stride, int64_t vn_offset,
     const int64_t *__restrict__ cand_ids, int n_cand, float threshold, int64_t k_out, int P,
-    int64_t *__restrict__ adaptive_k, int64_t *__restrict__ topk_ids) {
+    int64_t *__restrict__ adaptive_k, int64_t *__restrict__ topk_ids, AdkClamp cl) {
   extern __shared__ uint64_t s_keys[];
   __shared__ float s_part[16];
   __shared__ uint32_t s_hist[512];
@@ -1099,7 +1111,7 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adaptive_topk_kernel(
   }
   __syncthreads();
   adaptive_tail(s_keys, P, k_out, sl_benefit, total, threshold, r.ci, n_cand, adaptive_k + row,
-                topk_ids + (int64_t)row * k_out, (float *)s_hist, &s_counter);
+                topk_ids + (int64_t)row * k_out, cl, row, (float *)s_hist, &s_counter);
 }
 
 // ---- n_cand > 8192: slices of 8192 candidates, one workgroup each ----
@@ -1228,7 +1240,7 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adk_finish_kernel(
     int64_t k_out, int P,
     const float *__restrict__ ws_max, const float *__restrict__ ws_sum, const uint32_t *__restrict__ ctl,
     const uint64_t *__restrict__ list_a, const uint64_t *__restrict__ list_b, int64_t *__restrict__ adaptive_k,
-    int64_t *__restrict__ topk_ids) {
+    int64_t *__restrict__ topk_ids, AdkClamp cl) {
   extern __shared__ uint64_t s_keys[];
   __shared__ float s_part[16];
   __shared__ uint32_t s_hist[512];
@@ -1243,7 +1255,48 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adk_finish_kernel(
   wide_finish_select((uint32_t)k_out, P, ctl + (int64_t)row * kWideRowWords, list_a + (int64_t)row * k_out,
                      list_b + (int64_t)row * n_cand, n_cand, s_keys, s_hist, s_bcast, &s_counter);
   adaptive_tail(s_keys, P, k_out, sl_benefit, total, threshold, cand_ids + (int64_t)row * n_cand, n_cand,
-                adaptive_k + row, topk_ids + (int64_t)row * k_out, (float *)s_hist, &s_counter);
+                adaptive_k + row, topk_ids + (int64_t)row * k_out, cl, row, (float *)s_hist, &s_counter);
+}
+
+// Logits of the dense (sink / local / buffer) rows against the group-mean query
+// (polar_cache_adaptivek_varlen.py:1418-1419, :1731): out[(b,h)][r] = dtype(mean_g q . K[r]) widened to fp32,
+// times scale.  16 lanes per key row, 8 dims per lane: a lane adds its 8 products in order, the 16 partial
+// sums meet in a pairwise tree (lane ^ 1, 2, 4, 8).  grid (ceil(n_rows / 16), bs * H) x 256 threads.
+constexpr int kDenseLogitThreads = 256;
+
+template <bool BF16>
+__global__ __launch_bounds__(kDenseLogitThreads) void pkv_dense_logits_kernel(
+    const void *__restrict__ q, int n_kv_heads, int group, const void *__restrict__ k, int64_t k_stride_b,
+    int64_t k_stride_h, int64_t n_rows, float scale, float *__restrict__ out, int64_t out_stride) {
+  const int bh = blockIdx.y, b = bh / n_kv_heads, h = bh % n_kv_heads;
+  const int s = threadIdx.x & 15;
+  const int64_t row = (int64_t)blockIdx.x * (kDenseLogitThreads / 16) + (threadIdx.x >> 4);
+  float qa[8];
+  pkv_query_group_mean_t<BF16>(q, b, h, n_kv_heads, group, qa);
+  const int64_t r = row < n_rows ? row : n_rows - 1;
+  const int64_t at = (int64_t)b * k_stride_b + (int64_t)h * k_stride_h + r * 128 + 8 * s;
+  float kv[8];
+  if (BF16) {
+    const pkv_u32x4 w = *(const pkv_u32x4 *)((const uint16_t *)k + at);
+    const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      kv[2 * p] = __uint_as_float(ww[p] << 16);
+      kv[2 * p + 1] = __uint_as_float(ww[p] & 0xffff0000u);
+    }
+  } else {
+    const float4 lo = *(const float4 *)((const float *)k + at), hi = *(const float4 *)((const float *)k + at + 4);
+    kv[0] = lo.x, kv[1] = lo.y, kv[2] = lo.z, kv[3] = lo.w, kv[4] = hi.x, kv[5] = hi.y, kv[6] = hi.z, kv[7] = hi.w;
+  }
+  float acc = qa[0] * kv[0];
+#pragma unroll
+  for (int j = 1; j < 8; ++j) acc = acc + qa[j] * kv[j];
+  acc = acc + pkv_lane_xor_f<1>(acc);
+  acc = acc + pkv_lane_xor_f<2>(acc);
+  acc = acc + pkv_lane_xor_f<4>(acc);
+  acc = acc + pkv_lane_xor_f<8>(acc);
+  if (s == 0 && row < n_rows)
+    out[(int64_t)bh * out_stride + row] = pkv_rdt(acc, BF16 ? PKV_DTYPE_BF16 : PKV_DTYPE_F32) * scale;
 }
 
 static size_t lds_bytes(int P) { return (size_t)(P < 1024 ? 1024 : P) * 8; }
@@ -1469,7 +1522,11 @@ extern "C" int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, cons
                                  int64_t sl, const void *cand_scores, int cand_dtype, float cand_scale,
                                  const float *cand_vnorm, const float *value_norm, int64_t vn_stride, int64_t vn_offset,
                                  const int64_t *cand_ids, int64_t n_cand, float threshold, int64_t k_out, int rows,
-                                 int64_t *adaptive_k, int64_t *topk_ids, void *ws, size_t ws_bytes, void *stream) {
+                                 int64_t *adaptive_k, int64_t *topk_ids, int64_t k_min, int64_t k_max,
+                                 int32_t *row_keys, int64_t row_keys_base, void *ws, size_t ws_bytes, void *stream) {
+  PKV_REQUIRE(k_max <= 0 || (k_min >= 0 && k_min <= k_max), "pkv_adaptive_topk: clamp [%lld, %lld] is empty",
+              (long long)k_min, (long long)k_max);
+  const AdkClamp cl{k_min, k_max, row_keys, row_keys_base};
   PKV_REQUIRE(cand_scores && cand_ids && adaptive_k && topk_ids && (cand_vnorm || value_norm),
               "pkv_adaptive_topk: null pointer");
   PKV_REQUIRE(sl >= 0 && (sl == 0 || (sl_logits && sl_vnorm)), "pkv_adaptive_topk: dense logits missing");
@@ -1485,7 +1542,8 @@ extern "C" int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, cons
 #define PKV_ADK(EIN)                                                                                                  \
   hipLaunchKernelGGL((pkv_adaptive_topk_kernel<EIN>), dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes(P), s,      \
                      sl_logits, sl_stride, sl_vnorm, slv_stride, sl, cand_scores, cand_dtype, cand_scale, cand_vnorm, \
-                     value_norm, vn_stride, vn_offset, cand_ids, (int)n_cand, threshold, k_out, P, adaptive_k, topk_ids)
+                     value_norm, vn_stride, vn_offset, cand_ids, (int)n_cand, threshold, k_out, P, adaptive_k, topk_ids, \
+                     cl)
     if (ein <= 1) PKV_ADK(1); else if (ein == 2) PKV_ADK(2); else if (ein == 4) PKV_ADK(4); else PKV_ADK(8);
 #undef PKV_ADK
     PKV_LAUNCH_CHECK("pkv_adaptive_topk_kernel");
@@ -1516,7 +1574,29 @@ extern "C" int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, cons
   hipLaunchKernelGGL(pkv_adk_finish_kernel, dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes(P), s, sl_logits,
                      sl_stride, sl_vnorm, slv_stride, sl, cand_ids, n_cand, n_slices, n_parts, threshold, k_out, P, smax, ssum,
                      ctl,
-                     list_a, list_b, adaptive_k, topk_ids);
+                     list_a, list_b, adaptive_k, topk_ids, cl);
   PKV_LAUNCH_CHECK("pkv_adk_finish_kernel");
+  return PKV_OK;
+}
+
+extern "C" int pkv_dense_logits(const void *q, int dtype, int bs, int n_kv_heads, int group, const void *k,
+                                int64_t k_stride_b, int64_t k_stride_h, int64_t n_rows, float scale, float *out,
+                                int64_t out_stride, void *stream) {
+  PKV_REQUIRE(q && k && out, "pkv_dense_logits: null pointer");
+  PKV_REQUIRE(dtype == PKV_DTYPE_F32 || dtype == PKV_DTYPE_BF16, "pkv_dense_logits: unknown dtype %d", dtype);
+  PKV_REQUIRE(bs > 0 && n_kv_heads > 0 && group > 0 && (int64_t)bs * n_kv_heads <= 65535 && n_rows > 0 &&
+                  out_stride >= n_rows,
+              "pkv_dense_logits: bad shape bs=%d heads=%d group=%d rows=%lld", bs, n_kv_heads, group, (long long)n_rows);
+  PKV_REQUIRE(k_stride_b % 8 == 0 && k_stride_h % 8 == 0 && pkv_aligned(q, 16) && pkv_aligned(k, 16),
+              "pkv_dense_logits: rows must be 16-byte aligned");
+  constexpr int rows_per_wg = kDenseLogitThreads / 16;
+  const dim3 grid((unsigned)((n_rows + rows_per_wg - 1) / rows_per_wg), (unsigned)(bs * n_kv_heads));
+  if (dtype == PKV_DTYPE_BF16)
+    hipLaunchKernelGGL(pkv_dense_logits_kernel<true>, grid, dim3(kDenseLogitThreads), 0, (hipStream_t)stream, q,
+                       n_kv_heads, group, k, k_stride_b, k_stride_h, n_rows, scale, out, out_stride);
+  else
+    hipLaunchKernelGGL(pkv_dense_logits_kernel<false>, grid, dim3(kDenseLogitThreads), 0, (hipStream_t)stream, q,
+                       n_kv_heads, group, k, k_stride_b, k_stride_h, n_rows, scale, out, out_stride);
+  PKV_LAUNCH_CHECK("pkv_dense_logits_kernel");
   return PKV_OK;
 }

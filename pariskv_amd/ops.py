@@ -318,12 +318,15 @@ def rerank4(coarse_indices: torch.Tensor, key_4bit: torch.Tensor, key_block_weig
 
 def adaptive_topk(sl_logits: torch.Tensor, sl_vnorm: torch.Tensor, cand_scores: torch.Tensor, cand_scale: float,
                   cand_ids: torch.Tensor, threshold: float, k_out: int, cand_vnorm: Optional[torch.Tensor] = None,
-                  value_norm: Optional[torch.Tensor] = None, vn_offset: int = 0):
+                  value_norm: Optional[torch.Tensor] = None, vn_offset: int = 0, k_min: int = 0, k_max: int = 0,
+                  row_keys_base: Optional[int] = None):
     """Adaptive top-k by value-weighted attention mass.
 
     sl_logits / sl_vnorm fp32 [bs,H,sl] (last dim contiguous); cand_scores fp32 or bf16 [bs,H,C] contiguous
     (logit = score * cand_scale); cand_ids int64 [bs,H,C]; candidate value norms either ``cand_vnorm`` fp32 [bs,H,C]
     or gathered from ``value_norm`` fp32 [bs,H,cap] at ``cand_ids + vn_offset``.
+    ``k_max > 0`` clamps k to [k_min, k_max] inside the kernel; ``row_keys_base`` asks for a third result,
+    int32 [bs,H] = row_keys_base + k (the per-row key count of the attention that follows).
     Returns (adaptive_k int64 [bs,H], topk_ids int64 [bs,H,k_out])."""
     _cuda(sl_logits, sl_vnorm, cand_scores, cand_ids, cand_vnorm, value_norm)
     bs, H, Cn = cand_scores.shape
@@ -346,14 +349,40 @@ def adaptive_topk(sl_logits: torch.Tensor, sl_vnorm: torch.Tensor, cand_scores: 
     dev = cand_scores.device
     ak = torch.empty(bs, H, dtype=torch.int64, device=dev)
     ids = torch.empty(bs, H, k_out, dtype=torch.int64, device=dev)
+    row_keys = None if row_keys_base is None else torch.empty(bs, H, dtype=torch.int32, device=dev)
     nbytes = _lib.lib().pkv_adaptive_topk_ws_bytes(rows, Cn, k_out)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     row_stride = lambda t: t.stride(1) if H > 1 else (t.stride(0) if bs > 1 else max(1, sl))
     _lib.check(_lib.lib().pkv_adaptive_topk(
         _p(sl_logits), row_stride(sl_logits), _p(sl_vnorm), row_stride(sl_vnorm), sl, _p(cand_scores),
         _dt(cand_scores.dtype), float(cand_scale), _p(cand_vnorm), _p(value_norm), vn_stride, vn_offset, _p(cand_ids), Cn,
-        float(threshold), k_out, rows, _p(ak), _p(ids), _p(ws), nbytes, _stream(cand_scores)))
-    return ak, ids
+        float(threshold), k_out, rows, _p(ak), _p(ids), int(k_min), int(k_max), _p(row_keys),
+        int(row_keys_base or 0), _p(ws), nbytes, _stream(cand_scores)))
+    return (ak, ids) if row_keys is None else (ak, ids, row_keys)
+
+
+def adaptive_topk_ws_bytes(rows: int, n_cand: int, k_out: int) -> int:
+    return int(_lib.lib().pkv_adaptive_topk_ws_bytes(rows, n_cand, k_out))
+
+
+def dense_logits(queries: torch.Tensor, keys: torch.Tensor, n_rows: int, scale: float,
+                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Logits of the first ``n_rows`` rows of ``keys`` [bs,H,rows,128] (contiguous rows) against the mean of each KV
+    head's query group: float32 [bs,H,n_rows] = dtype(mean_g(q) . k) * scale
+    (cache_hub/polar_cache_adaptivek_varlen.py:1418-1419, :1731).  queries: contiguous [bs,1,H*G,128]."""
+    _cuda(queries, keys)
+    bs, H, rows, D = keys.shape
+    _need(D == HEAD_DIM and keys.stride(3) == 1 and keys.stride(2) == D and 0 < n_rows <= rows and
+          keys.dtype == queries.dtype, "keys: [bs,H,rows,128] with contiguous rows, dtype of the queries")
+    _need(queries.is_contiguous() and queries.numel() % (bs * H * D) == 0, "queries must be contiguous [bs,1,Hq,128]")
+    G = queries.numel() // (bs * H * D)
+    if out is None:
+        out = torch.empty(bs, H, n_rows, dtype=torch.float32, device=keys.device)
+    _need(out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape[:2]) == (bs, H) and
+          out.shape[2] >= n_rows, "out: contiguous fp32 [bs,H,>=n_rows]")
+    _lib.check(_lib.lib().pkv_dense_logits(_p(queries), _dt(queries.dtype), bs, H, G, _p(keys), keys.stride(0),
+                                           keys.stride(1), n_rows, float(scale), _p(out), out.shape[2], _stream(keys)))
+    return out
 
 
 # ------------------------------------------------------------------ gathers
@@ -396,10 +425,12 @@ def gather_hbm(src_k, src_v, idx, dst_k, dst_v, idx_offset: int = 0, dst_row0: i
     _gather(_lib.lib().pkv_gather_hbm, src_k, src_v, idx, dst_k, dst_v, idx_offset, dst_row0)
 
 
-def append_kv(key_states, value_states, dst_k, dst_v, slot: int) -> None:
+def append_kv(key_states, value_states, dst_k, dst_v, slot: int, vnorm: Optional[torch.Tensor] = None) -> None:
     """dst_k[:, :, slot, :] = key_states[:, 0] and the same for values, in one launch
     (decode_update_kv_cache, cache_hub/polar_cache.py:848-856).  key_states/value_states [bs,1,Hkv,D];
-    dst_k/dst_v [bs,Hkv,rows,D] with contiguous rows."""
+    dst_k/dst_v [bs,Hkv,rows,D] with contiguous rows.  ``vnorm`` (fp32 [bs,Hkv,rows], last dim contiguous) also
+    receives ``||value_states[b,0,h]||`` at ``[b,h,slot]``, computed in the K/V dtype
+    (cache_hub/polar_cache_adaptivek_varlen.py:1179)."""
     bs, one, H, D = key_states.shape
     es = key_states.element_size()
     _need(one == 1 and value_states.shape == key_states.shape and key_states.stride(3) == 1 and
@@ -410,10 +441,16 @@ def append_kv(key_states, value_states, dst_k, dst_v, slot: int) -> None:
           dst_k.stride(2) == D and tuple(dst_k.shape[:2]) == (bs, H) and dst_k.shape[3] == D,
           "dst_k, dst_v: [bs,Hkv,rows,D] with contiguous rows")
     _need(key_states.is_cuda and dst_k.is_cuda, "append: tensors must be on the GPU")
+    vn_b = vn_h = 0
+    if vnorm is not None:
+        _need(vnorm.is_cuda and vnorm.dtype == torch.float32 and tuple(vnorm.shape[:2]) == (bs, H) and
+              vnorm.stride(2) == 1 and vnorm.shape[2] > slot, "vnorm: fp32 [bs,Hkv,rows] with contiguous rows")
+        vn_b, vn_h = vnorm.stride(0), vnorm.stride(1)
     _lib.check(_lib.lib().pkv_append_kv(
         key_states.data_ptr(), key_states.stride(0) * es, key_states.stride(2) * es,
-        value_states.data_ptr(), value_states.stride(0) * es, value_states.stride(2) * es, dst_k.data_ptr(), dst_v.data_ptr(), dst_k.stride(0) * es, dst_k.stride(1) * es, dst_k.shape[2], slot, bs, H,
-        D * es, _stream(dst_k)))
+        value_states.data_ptr(), value_states.stride(0) * es, value_states.stride(2) * es, dst_k.data_ptr(),
+        dst_v.data_ptr(), dst_k.stride(0) * es, dst_k.stride(1) * es, dst_k.shape[2], slot, bs, H, D * es,
+        _p(vnorm), vn_b, vn_h, _stream(dst_k)))
 
 
 def offload_rows(src_k, src_v, dst_k_cpu, dst_v_cpu, dst_row0: int, stream=None) -> None:
@@ -638,6 +675,32 @@ class BoundStep:
         return out
 
 
+class BoundAdaptiveStep:
+    """:class:`BoundStep` for the adaptive-k step (pkv_adaptive_decode_step): three argument blocks, validated once.
+    The caller patches what moves with every token (``ad.dense_rows``, ``ad.row_keys_base``, ``segs[0].n_rows``)."""
+
+    __slots__ = ("a", "ad", "aa", "segs", "keep", "_ra", "_rad", "_raa", "_ws", "_ws_bytes", "_fn", "_numel", "_dtype")
+
+    def __init__(self, plan, a, ad, aa, keep, q):
+        self.a, self.ad, self.aa, self.segs, self.keep = a, ad, aa, aa.segments, keep
+        self._ra, self._rad, self._raa = C.byref(a), C.byref(ad), C.byref(aa)
+        self._ws, self._ws_bytes = _p(plan.ws), plan.ws.numel()
+        self._fn = _lib.lib().pkv_adaptive_decode_step
+        self._numel, self._dtype = q.numel(), q.dtype
+
+    def launch(self, q: torch.Tensor) -> torch.Tensor:
+        """q: contiguous [bs,1,Hq,128] of the bound dtype.  Returns the attention output, shaped like q."""
+        _need(q.is_cuda and q.is_contiguous() and q.numel() == self._numel and q.dtype == self._dtype,
+              "queries must be contiguous [bs,1,Hq,128] of the cache dtype")
+        out = torch.empty_like(q)
+        self.a.q, self.aa.out = q.data_ptr(), out.data_ptr()
+        rc = self._fn(self._ra, self._ws, self._ws_bytes, self._rad, self._raa,
+                      torch.cuda.current_stream(q.device).cuda_stream)
+        if rc != 0:
+            _lib.check(rc)
+        return out
+
+
 class RetrievePlan:
     """Persistent workspace + argument block for :func:`pkv_retrieve` on key-major storage."""
 
@@ -722,6 +785,56 @@ class RetrievePlan:
         aa, _ = att.c_args(queries, segments, out=queries)  # out is patched at every launch
         keep = (signs, centers, cluster_counts, codes_km, nib_km, w_km, out_ids, gather, att, segments, self.ws)
         return BoundStep(self, a, aa, keep, queries)
+
+    def bind_adaptive(self, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts,
+                      n_cand, adaptive: dict, att, segments):
+        """The adaptive-k step of one layer as a :class:`BoundAdaptiveStep`.  ``adaptive``: dense_k [bs,H,rows,128],
+        dense_rows, dense_vnorm fp32 [bs,H,rows], dense_logits fp32 [bs,H,>=rows] scratch, scale, value_norm fp32
+        [bs,H,cap], vn_offset, threshold, k_out, k_min, k_max, adaptive_k int64 [bs,H], topk_ids int64 (>= bs*H*k_out
+        elements), row_keys int32 [bs,H], row_keys_base, ws uint8 (pkv_adaptive_topk_ws_bytes), src_k / src_v pinned
+        CPU [bs,H,len,128], dst_k / dst_v GPU [bs,H,>=k_out,128].  ``segments`` are the attention's; its per-row key
+        count is ``row_keys``."""
+        a = self._fill(queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, 1,
+                       None, None, None, True)
+        d = adaptive
+        bs, H = self.bs, self.H
+        dk, dvn, dl, vn = d["dense_k"], d["dense_vnorm"], d["dense_logits"], d["value_norm"]
+        ak, ids, rk, ws = d["adaptive_k"], d["topk_ids"], d["row_keys"], d["ws"]
+        sk, sv, tk, tv = d["src_k"], d["src_v"], d["dst_k"], d["dst_v"]
+        k_out = int(d["k_out"])
+        _cuda(dk, dvn, dl, vn, ak, ids, rk, ws, tk, tv)
+        _need(dk.dtype == queries.dtype and tuple(dk.shape[:2]) == (bs, H) and dk.shape[3] == HEAD_DIM and
+              dk.stride(3) == 1 and dk.stride(2) == HEAD_DIM, "dense_k: [bs,H,rows,128] with contiguous rows")
+        for t in (dvn, dl, vn):
+            _need(t.dtype == torch.float32 and t.is_contiguous() and tuple(t.shape[:2]) == (bs, H),
+                  "dense_vnorm / dense_logits / value_norm: contiguous fp32 [bs,H,*]")
+        _need(0 < int(d["dense_rows"]) <= min(dl.shape[2], dvn.shape[2], dk.shape[2]),
+              "dense_rows exceeds dense_k / dense_logits / dense_vnorm")
+        _need(0 < k_out <= n_cand, "k_out must be in (0, n_cand]")
+        _need(ak.dtype == torch.int64 and ak.is_contiguous() and ak.numel() == bs * H and ids.dtype == torch.int64 and
+              ids.is_contiguous() and ids.numel() >= bs * H * k_out and rk.dtype == torch.int32 and rk.is_contiguous() and
+              rk.numel() == bs * H, "adaptive_k / topk_ids / row_keys: contiguous int64 / int64 / int32 of the step's size")
+        need = _lib.lib().pkv_adaptive_topk_ws_bytes(self.rows, n_cand, k_out)
+        _need(ws.dtype == torch.uint8 and ws.is_contiguous() and ws.numel() >= need, "adaptive workspace too small")
+        _need(sk.is_cpu and sv.is_cpu and sk.is_pinned() and sv.is_pinned() and sk.is_contiguous() and sv.is_contiguous() and
+              sk.shape == sv.shape and tuple(sk.shape[:2]) == (bs, H) and sk.dtype == queries.dtype,
+              "src_k / src_v: contiguous pinned CPU [bs,H,len,128] of the query dtype")
+        _need(tk.is_contiguous() and tv.is_contiguous() and tk.shape == tv.shape and tuple(tk.shape[:2]) == (bs, H) and
+              tk.shape[2] >= k_out and tk.dtype == queries.dtype, "dst_k / dst_v: contiguous GPU [bs,H,>=k_out,128]")
+        ad = _lib.AdaptiveArgs()
+        ad.dense_k, ad.dense_stride_b, ad.dense_stride_h, ad.dense_rows = dk.data_ptr(), dk.stride(0), dk.stride(1), int(d["dense_rows"])
+        ad.dense_vnorm, ad.dense_vnorm_stride = dvn.data_ptr(), dvn.shape[2]
+        ad.dense_logits, ad.dense_logits_stride = dl.data_ptr(), dl.shape[2]
+        ad.scale, ad.value_norm, ad.vn_stride, ad.vn_offset = float(d["scale"]), vn.data_ptr(), vn.shape[2], int(d["vn_offset"])
+        ad.threshold, ad.k_out, ad.k_min, ad.k_max = float(d["threshold"]), k_out, int(d["k_min"]), int(d["k_max"])
+        ad.adaptive_k, ad.topk_ids, ad.row_keys, ad.row_keys_base = ak.data_ptr(), ids.data_ptr(), rk.data_ptr(), int(d["row_keys_base"])
+        ad.ws, ad.ws_bytes = ws.data_ptr(), ws.numel()
+        ad.src_k, ad.src_v, ad.src_len, ad.idx_offset = sk.data_ptr(), sv.data_ptr(), sk.shape[2], int(d.get("idx_offset", 0))
+        ad.dst_k, ad.dst_v, ad.dst_len, ad.dst_row0 = tk.data_ptr(), tv.data_ptr(), tk.shape[2], 0
+        ad.row_bytes = HEAD_DIM * sk.element_size()
+        aa, _ = att.c_args(queries, segments, out=queries, row_keys=rk)  # out is patched at every launch
+        keep = (signs, centers, cluster_counts, codes_km, nib_km, w_km, d, att, segments, self.ws)
+        return BoundAdaptiveStep(self, a, ad, aa, keep, queries)
 
     def view(self, name: str, n_keys: int, n_cand: int, k: int, dtype: torch.dtype) -> torch.Tensor:
         """An intermediate of the last :meth:`run` (qhat, qnorm, lut, cnt_u8, chunk_hist, cand, scores)."""

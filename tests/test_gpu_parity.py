@@ -1163,6 +1163,80 @@ def test_append_kv_equals_indexed_assignment(ops):
         ops.append_kv(fused[:, :, :H], fused[:, :, H:2 * H + 1], dk, dv, 0)
 
 
+def test_append_kv_value_norm(ops):
+    """The value norm written by pkv_append_kv (adaptive-k bookkeeping, reference polar_cache_adaptivek_varlen.py:1179):
+    bit-equal to the oracle's fixed-order restatement, within one step of the dtype of torch's vector_norm; the other
+    slots of the norm table stay untouched."""
+    g = torch.Generator().manual_seed(8)
+    bs, H, cap, D = 3, 4, 21, 128
+    for dtype, odt, rtol in ((torch.bfloat16, O.BF16, 2.0 ** -7), (torch.float32, O.F32, 2e-6)):
+        dk = torch.zeros(bs, H, cap, D, dtype=dtype, device=DEV)
+        dv = torch.zeros_like(dk)
+        table = torch.full((bs + 1, H, cap + 3), -1.0, device=DEV)
+        vn = table[1:]                                         # a batch slice: strided rows
+        fused = (torch.randn(bs, 1, 3 * H, D, generator=g) * torch.rand(bs, 1, 3 * H, 1, generator=g) * 4).to(dtype).to(DEV)
+        for slot, (k1, v1) in ((5, (fused[:, :, :H], fused[:, :, 2 * H:])), (cap - 1, (fused[:, :, H:2 * H], fused[:, :, :H]))):
+            ops.append_kv(k1, v1, dk, dv, slot, vnorm=vn)
+            torch.cuda.synchronize()
+            assert torch.equal(dv[:, :, slot], v1[:, 0]) and torch.equal(dk[:, :, slot], k1[:, 0])
+            want = O.value_norm(v1[:, 0].float().cpu().numpy().reshape(-1, D), odt).reshape(bs, H)
+            assert np.array_equal(vn[:, :, slot].cpu().numpy(), want)
+            ref = torch.linalg.vector_norm(v1[:, 0], dim=-1).float()
+            assert torch.allclose(vn[:, :, slot], ref, rtol=rtol, atol=0)
+        untouched = torch.ones(cap + 3, dtype=torch.bool)
+        untouched[[5, cap - 1]] = False
+        assert (vn[:, :, untouched] == -1).all() and (table[0] == -1).all()
+    with pytest.raises(RuntimeError, match="vnorm"):
+        ops.append_kv(fused[:, :, :H], fused[:, :, H:2 * H], dk, dv, 0, vnorm=vn[:, :, :0])
+
+
+@pytest.mark.parametrize("bs,H,G,rows,n", [(1, 8, 4, 700, 700), (2, 2, 7, 100, 33), (3, 1, 1, 17, 17), (1, 4, 12, 2000, 1999)])
+def test_dense_logits_match_oracle(ops, bs, H, G, rows, n):
+    """pkv_dense_logits (reference polar_cache_adaptivek_varlen.py:1418-1419 + :1731): bit-equal to the oracle's
+    fixed-order restatement in both rounding chains, and within one bf16 step / 2e-6 of the torch expressions; rows
+    beyond n and the padding of a longer output row are not written."""
+    g = torch.Generator().manual_seed(bs * 100 + G)
+    scale = 1.0 / math.sqrt(128)
+    for dtype, odt, rtol in ((torch.bfloat16, O.BF16, 2.0 ** -7), (torch.float32, O.F32, 2e-6)):
+        q = torch.randn(bs, 1, H * G, 128, generator=g).to(dtype).to(DEV)
+        store = (torch.randn(bs + 1, H, rows, 128, generator=g) * 1.5).to(dtype).to(DEV)
+        k = store[1:]                                           # strided batch
+        out = torch.full((bs, H, rows + 5), 7.0, device=DEV)
+        got = ops.dense_logits(q, k, n, scale, out=out)
+        torch.cuda.synchronize()
+        assert got.data_ptr() == out.data_ptr() and (out[:, :, n:] == 7.0).all()
+        qc, kc = q.float().cpu().numpy().reshape(bs, H, G, 128), k.float().cpu().numpy()
+        for b in range(bs):
+            for h in range(H):
+                want = O.dense_logits(qc[b, h], kc[b, h, :n], scale, odt)
+                assert np.array_equal(out[b, h, :n].cpu().numpy(), want), (b, h)
+        ref = torch.einsum("bhd,bhkd->bhk", q[:, 0].view(bs, H, G, 128).mean(dim=2), k[:, :, :n]).to(torch.float32) * scale
+        assert torch.allclose(out[:, :, :n], ref, rtol=rtol, atol=rtol * float(ref.abs().max()))
+        fresh = ops.dense_logits(q, k, n, scale)
+        assert fresh.shape == (bs, H, n) and torch.equal(fresh, out[:, :, :n])
+    with pytest.raises(RuntimeError):
+        ops.dense_logits(q, k, rows + 1, scale)
+
+
+def test_adaptive_topk_clamp_and_row_keys(ops):
+    """The clamp of k (reference polar_cache_adaptivek_varlen.py:1759) and the per-row key count folded into the
+    adaptive-k kernels, on the one-workgroup and the multi-workgroup path: equal to clamping the unclamped result."""
+    for Cn, k_out in ((3000, 800), (20000, 800)):
+        bs, H, sl = 2, 3, 200
+        q, slk, slv, cs, ci, cv, scale = _adaptive_recipe(bs, H, sl, Cn, 23)
+        sl_logits = (torch.einsum("bhd,bhkd->bhk", q, slk).float() * scale).to(DEV)
+        args = (sl_logits, slv.to(DEV), cs.to(DEV), scale, ci.to(DEV))
+        for thr in (0.3, 0.9, 0.9999):
+            ak0, ids0 = ops.adaptive_topk(*args, thr, k_out, cand_vnorm=cv.to(DEV))
+            ak1, ids1, rk = ops.adaptive_topk(*args, thr, k_out, cand_vnorm=cv.to(DEV), k_min=100, k_max=500, row_keys_base=sl + 7)
+            assert torch.equal(ids0, ids1)
+            assert torch.equal(ak1, ak0.clamp(min=100, max=500))
+            assert rk.dtype == torch.int32 and torch.equal(rk.long(), ak1 + sl + 7)
+        assert len({int(v) for v in ak0.flatten()} | {int(v) for v in ak1.flatten()}) > 1
+    with pytest.raises(RuntimeError, match="clamp"):
+        ops.adaptive_topk(*args, 0.9, k_out, cand_vnorm=cv.to(DEV), k_min=600, k_max=500)
+
+
 def test_offload_rows_equals_sliced_copy(ops):
     """pkv_offload_rows against the sliced copy_ it replaces (reference polar_cache.py:457-471, :778-799): rows read in
     place from the model's [bs,seq,h,d] layout and from a partly filled staging buffer, into a batch slice of the pinned

@@ -221,6 +221,35 @@ def test_adaptive_topk_edge_cases(oracle):
     assert k == 10 and np.array_equal(idx, np.arange(100)[::-1][:10])  # ties: candidate position ascending
 
 
+def test_dense_logits_and_value_norm_match_torch_forms(oracle):
+    """The two numpy restatements that feed adaptive-k (reference polar_cache_adaptivek_varlen.py:1418-1419, :1731,
+    :1179) against the torch expressions the reference evaluates and against float64: exact up to the last rounding
+    (one bf16 step in the bf16 chain, 1e-6 relative in fp32), and invariant facts a slip would break."""
+    g = torch.Generator().manual_seed(17)
+    G, n = 4, 300
+    for dtype, tdt, rtol in ((oracle.BF16, torch.bfloat16, 2.0 ** -7), (oracle.F32, torch.float32, 2e-6)):
+        q = torch.randn(G, 128, generator=g).to(tdt)
+        k = (torch.randn(n, 128, generator=g) * 2).to(tdt)
+        v = (torch.randn(n, 128, generator=g) * torch.rand(n, 1, generator=g) * 3).to(tdt)
+        scale = 1.0 / math.sqrt(128)
+        got = oracle.dense_logits(q.float().numpy(), k.float().numpy(), scale, dtype)
+        ref = (torch.einsum("d,kd->k", q.mean(dim=0), k).to(torch.float32) * scale).numpy()
+        f64 = (k.double() @ q.double().mean(dim=0)).numpy() * scale
+        assert np.allclose(got, ref, rtol=rtol, atol=rtol * np.abs(f64).max())
+        assert np.allclose(got, f64, rtol=rtol, atol=rtol * np.abs(f64).max())
+        vn = oracle.value_norm(v.float().numpy(), dtype)
+        vref = torch.linalg.vector_norm(v, dim=-1).float().numpy()
+        assert np.allclose(vn, vref, rtol=rtol)
+        assert np.allclose(vn, np.linalg.norm(v.double().numpy(), axis=1), rtol=rtol)
+        # a query group of four identical heads is that head (4a / 4 is exact); one-hot rows pick out single dimensions
+        same = oracle.dense_logits(np.repeat(q[:1].float().numpy(), 4, axis=0), k.float().numpy(), 1.0, dtype)
+        assert np.array_equal(same, oracle.dense_logits(q[:1].float().numpy(), k.float().numpy(), 1.0, dtype))
+        eye = np.eye(128, dtype=np.float32) * 3.0
+        assert np.array_equal(oracle.dense_logits(q[:1].float().numpy(), eye, 1.0, dtype),
+                              oracle.bf16_round(q[0].float().numpy() * 3.0) if dtype == oracle.BF16 else q[0].numpy() * 3.0)
+        assert np.array_equal(oracle.value_norm(eye, dtype), np.full(128, 3.0, np.float32))
+
+
 def test_retrieve_row_composes_the_stages(oracle, signs):
     n, C, K = 4096, 512, 128
     keys = oracle.synth_keys(n, seed=0)
