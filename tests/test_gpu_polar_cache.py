@@ -167,18 +167,21 @@ def test_single_sample_prefill_and_constructor_errors():
         polar_cache([0], 1, 1, 100, 2, 4, 64, torch.bfloat16, {0: DEV}, 8, 4, 32)
 
 
-def test_adaptive_k_cache_decode_loop():
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_adaptive_k_cache_decode_loop(dtype):
     """Adaptive-k variant (reference polar_cache_adaptivek_varlen.py): value-norm caches follow the K/V slots
     through prefill, decode writes and index refreshes; per-row k and the selected set equal the CPU oracle's on
-    the cache's own index; attention equals an fp32 softmax over sink ++ each row's own selection ++ dense tail."""
+    the cache's own index; attention equals an fp32 softmax over sink ++ each row's own selection ++ dense tail.
+    In bfloat16 (the reference's dtype) and in float32 (the fp32 chains of every kernel on the step)."""
     from pariskv_amd.cache_hub.polar_cache_adaptivek_varlen import polar_cache as adaptive_cache
 
+    odt, step_tol = (O.BF16, 2.0 ** -7) if dtype == torch.bfloat16 else (O.F32, 2e-6)
     bs, Hkv, Hq, layers, S, steps = 2, 2, 8, 2, 3000, 40
     sink, local, I = 4, 64, 16
     G = Hq // Hkv
     thr = 0.6
     cache = adaptive_cache(valid_start=[0] * bs, layer_num=layers, batch_size=bs, max_length=S + steps + 10,
-                           num_key_value_heads=Hkv, num_heads=Hq, head_dim=128, dtype=torch.bfloat16,
+                           num_key_value_heads=Hkv, num_heads=Hq, head_dim=128, dtype=dtype,
                            layer_mapping={i: DEV for i in range(layers)}, max_new_length=steps + 10, sink_size=sink,
                            local_size=local, core=1, nprobe=1, cache_unit_size=1, cache_cluster_num=1, num_gpus=1,
                            model_size=7, final_topk=100, dynamic_update_interval=I, full_attention_threshold=100,
@@ -188,9 +191,16 @@ def test_adaptive_k_cache_decode_loop():
         adaptive_cache([0], 1, 1, 100, 2, 4, 128, torch.bfloat16, {0: DEV}, 8, 4, 32, enable_offload=False)
     gen = torch.Generator().manual_seed(3)
     hist_k, hist_v = [None] * layers, [None] * layers
+
+    def synth(n):  # values of the cache dtype (fp32: not representable in bf16)
+        k, v = _synth_kv(gen, bs, n, Hkv)
+        if dtype == torch.float32:
+            k, v = k.float() * (1 + 1e-3 * torch.rand(k.shape, generator=gen)), v.float() * (1 + 1e-3 * torch.rand(v.shape, generator=gen))
+        return k, v
+
     for l in range(layers):
-        k, v = _synth_kv(gen, bs, S, Hkv)
-        v = v * (0.25 + 2.0 * torch.rand(bs, S, Hkv, 1, generator=gen)).to(torch.bfloat16)  # uneven value norms
+        k, v = synth(S)
+        v = v * (0.25 + 2.0 * torch.rand(bs, S, Hkv, 1, generator=gen)).to(dtype)  # uneven value norms
         hist_k[l], hist_v[l] = k, v
         cache.prefill_update_kv_cache(None, k.to(DEV), v.to(DEV), l, 0)
     signs = O.srht_signs(42)
@@ -198,10 +208,10 @@ def test_adaptive_k_cache_decode_loop():
     seen_k = set()
     for step in range(steps):
         for l in range(layers):
-            k1, v1 = _synth_kv(gen, bs, 1, Hkv)
+            k1, v1 = synth(1)
             # queries near a handful of recent keys make the attention mass concentrate, so k varies by row
             q = (hist_k[l][:, -3:].float().mean(dim=1).repeat_interleave(G, dim=1) * 0.3
-                 + 0.5 * torch.randn(bs, Hq, 128, generator=gen)).to(torch.bfloat16).view(bs, 1, Hq, 128)
+                 + 0.5 * torch.randn(bs, Hq, 128, generator=gen)).to(dtype).view(bs, 1, Hq, 128)
             hist_k[l] = torch.cat([hist_k[l], k1], dim=1)
             hist_v[l] = torch.cat([hist_v[l], v1], dim=1)
             cache.decode_update_kv_cache(k1.to(DEV), v1.to(DEV), l)
@@ -217,14 +227,14 @@ def test_adaptive_k_cache_decode_loop():
             # value norms: retrieval zone by absolute position, dense rows by GPU slot
             vn_ref = torch.linalg.vector_norm(hist_v[l], dim=-1).float().permute(0, 2, 1)      # [bs, H, total]
             assert torch.allclose(cache.value_norm_gpu[l][:, :, sink:sink + n_keys].cpu(), vn_ref[:, :, sink:sink + n_keys],
-                                  rtol=2.0 ** -7, atol=0)
-            assert torch.equal(cache.value_norm_gpu[l][:, :, sink:S - local].cpu(),
-                               vn_ref[:, :, sink:S - local])   # rows encoded at prefill: torch's own norm
+                                  rtol=step_tol, atol=0)
+            if dtype == torch.bfloat16:  # rows encoded at prefill: torch's own norm
+                assert torch.equal(cache.value_norm_gpu[l][:, :, sink:S - local].cpu(), vn_ref[:, :, sink:S - local])
             dense_pos = torch.cat([torch.arange(sink), torch.arange(sink + n_keys, total)])
             assert sl_end == len(dense_pos)
             # dense rows written at decode time carry the append kernel's norm: torch's within one bf16 step (bit
             # parity of that kernel with the oracle's restatement is a test of its own)
-            assert torch.allclose(cache._sl_vnorm_cache[l][:, :, :sl_end].cpu(), vn_ref[:, :, dense_pos], rtol=2.0 ** -7, atol=0)
+            assert torch.allclose(cache._sl_vnorm_cache[l][:, :, :sl_end].cpu(), vn_ref[:, :, dense_pos], rtol=step_tol, atol=0)
             codes = cache._codes_km[l].cpu().numpy()
             nib = cache._nib_km[l].cpu().numpy()
             w = cache._w_km[l].float().cpu().numpy()
@@ -238,13 +248,13 @@ def test_adaptive_k_cache_decode_loop():
                 ref = torch.empty(Hq, 128)
                 for h in range(Hkv):
                     zone = slice(sink, sink + n_keys)
-                    qh, qn = O.query_prep(q[b, 0, h * G:(h + 1) * G].float().numpy(), signs, O.BF16)
-                    lut = O.tier_lut(O.rank_centroids(qh, O.BF16), cc[b, h], tiers)
+                    qh, qn = O.query_prep(q[b, 0, h * G:(h + 1) * G].float().numpy(), signs, odt)
+                    lut = O.tier_lut(O.rank_centroids(qh, odt), cc[b, h], tiers)
                     cand_ref, _ = O.select_candidates(O.collision_count(codes[b, h][zone], lut), n_cand)
                     sc = O.rerank(cand_ref, nib[b, h][zone].reshape(-1, 16, 4), w[b, h][zone], qh, qn)
                     vn = cache.value_norm_gpu[l][b, h].cpu().numpy()[cand_ref + sink]
                     cap_k = min(cache._HARDCODED_MAX_K, n_cand)
-                    sl_logits = O.dense_logits(q[b, 0, h * G:(h + 1) * G].float().numpy(), dense_keys[b, h], scale, O.BF16)
+                    sl_logits = O.dense_logits(q[b, 0, h * G:(h + 1) * G].float().numpy(), dense_keys[b, h], scale, odt)
                     k_ref, ids_ref = O.adaptive_topk(sl_logits, sl_vnorm[b, h], sc * np.float32(scale), vn, cand_ref,
                                                      thr, cap_k)
                     k_ref = min(max(k_ref, min(cache._HARDCODED_MIN_K, cap_k)), cap_k)
@@ -261,8 +271,12 @@ def test_adaptive_k_cache_decode_loop():
                 cand, scores = cache._plan.run_candidates(qd, cache._srht_signs, cache._mag_centers, cache.cluster_key_counts_gpu[l],
                                                           cache._codes_km[l], cache._nib_km[l], cache._w_km[l], sink, n_keys,
                                                           tiers, n_cand)
+                qv = qd[:, 0].view(bs, Hkv, G, 128).float()
+                q_avg = qv[:, :, 0]
+                for gi in range(1, G):  # the group mean with the heads added in order (fp32 sums are order-dependent)
+                    q_avg = q_avg + qv[:, :, gi]
                 k_form, packed, global_k = cache._compute_adaptive_topk(
-                    qd[:, 0].view(bs, Hkv, G, 128).mean(dim=2), cache.unified_keys_gpu[l][:, :, :sl_end],
+                    (q_avg / G).to(dtype), cache.unified_keys_gpu[l][:, :, :sl_end],
                     cache._sl_vnorm_cache[l][:, :, :sl_end], scores, cand, l, thr)
                 assert np.array_equal(k_form.cpu().numpy(), ak) and global_k == int(ak.max())
                 cap_k = min(cache._HARDCODED_MAX_K, n_cand)
