@@ -58,6 +58,24 @@ def test_host_side_argument_errors_without_gpu():
     assert L.pkv_retrieve_ws_bytes(32, 100, 200, 10) == 0  # n_cand > n_keys
     with pytest.raises(RuntimeError, match="pariskv_hip error"):
         _lib.check(L.pkv_gather_cpu(None, None, None, None, None, 1, 1, 1, 1, 1, 2, 1))
+    assert L.pkv_adaptive_decode_step(None, None, 0, None, None, None) == _lib.EINVAL
+    a, ad, aa = _lib.RetrieveArgs(), _lib.AdaptiveArgs(), _lib.AttnArgs()
+    a.out_ids = 8  # a final top-k was asked for: not the candidates-only form
+    assert L.pkv_adaptive_decode_step(a, None, 0, ad, aa, None) == _lib.EINVAL
+    assert b"candidates-only" in L.pkv_last_error()
+    assert L.pkv_dense_logits(None, 1, 1, 1, 1, None, 0, 0, 1, 1.0, None, 1, None) == _lib.EINVAL
+    assert L.pkv_adaptive_topk(None, 0, None, 0, 0, None, 0, 1.0, None, None, 0, 0, None, 10, 0.9, 5, 1, None, None,
+                               6, 5, None, 0, None, 0, None) == _lib.EINVAL
+    assert b"clamp" in L.pkv_last_error()
+
+
+def test_struct_mirrors_have_the_library_sizes():
+    from pariskv_amd import _lib
+
+    L = _lib.lib()
+    for which, mirror in enumerate((_lib.AttnSegment, _lib.AttnArgs, _lib.RetrieveArgs, _lib.AdaptiveArgs)):
+        assert L.pkv_struct_bytes(which) == ctypes.sizeof(mirror) > 0
+    assert L.pkv_struct_bytes(4) == 0
 
 
 def test_gather_cpu_host_function():
