@@ -57,6 +57,11 @@ def main():
                          "--topk 100 --steps 256), end-to-end decode tokens/s")
     ap.add_argument("--no-offload", action="store_true", help="decode-loop: keep K/V in HBM (config 2's mode)")
     ap.add_argument("--adaptive", action="store_true", help="decode-loop: the adaptive-k cache class (config 4's mode)")
+    ap.add_argument("--adaptive-k-range", type=int, nargs=2, default=[256, 2048], metavar=("MIN", "MAX"),
+                    help="decode-loop --adaptive: clamp of k (config 4: 256 2048; the reference's built-in caps: 100 800)")
+    ap.add_argument("--adaptive-threshold", type=float, default=0.95, help="decode-loop --adaptive: mass threshold")
+    ap.add_argument("--key-drift", type=float, default=0.0,
+                    help="decode-loop: rotate the key mean by this many degrees per 1K tokens (config 4: 0.5)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (rows would shard across GPUs by (batch, kv-head))",
@@ -128,24 +133,35 @@ def main():
             from pariskv_amd.cache_hub.polar_cache import polar_cache
 
         S, T = N, args.steps
+        extra = {}
+        if args.adaptive:  # the class takes its caps from the environment, like the reference
+            os.environ["ADAPTIVE_TOPK_MIN_K"], os.environ["ADAPTIVE_TOPK_MAX_K"] = (str(v) for v in args.adaptive_k_range)
+            extra["adaptive_topk_threshold"] = args.adaptive_threshold
         cache = polar_cache(valid_start=[0] * bs, layer_num=L, batch_size=bs, max_length=S + T + 8, num_key_value_heads=H,
                             num_heads=H * G, head_dim=D, dtype=torch.bfloat16, layer_mapping={i: dev for i in range(L)},
                             max_new_length=T + 8, sink_size=64, local_size=512, core=1, nprobe=1, cache_unit_size=1,
                             cache_cluster_num=1, num_gpus=1, model_size=8, final_topk=K, dynamic_update_interval=1024,
-                            full_attention_threshold=2000, enable_offload=not args.no_offload)
+                            full_attention_threshold=2000, enable_offload=not args.no_offload, **extra)
         g = torch.Generator(device=dev).manual_seed(0)
         t0 = time.perf_counter()
         for l in range(L):
             k = torch.randn(bs, S, H, D, generator=g, device=dev, dtype=torch.bfloat16)
             k[..., [7, 31, 64, 101]] *= 10.0
+            if args.key_drift:  # key mean of norm 2 turning in the plane of dims (0, 1)
+                ang = torch.arange(S, device=dev, dtype=torch.float32) * (args.key_drift * math.pi / 180.0 / 1000.0)
+                k[..., 0] += (2.0 * torch.cos(ang)).to(torch.bfloat16)[None, :, None]
+                k[..., 1] += (2.0 * torch.sin(ang)).to(torch.bfloat16)[None, :, None]
             v = torch.randn(bs, S, H, D, generator=g, device=dev, dtype=torch.bfloat16)
             cache.prefill_update_kv_cache(None, k, v, l, 0)
+            kmean = k[:, -1024:].float().mean(dim=1)  # [bs, H, D]
             del k, v
         torch.cuda.synchronize()
         t_prefill = time.perf_counter() - t0
         k1 = torch.randn(T, bs, 1, H, D, generator=g, device=dev, dtype=torch.bfloat16)
         v1 = torch.randn(T, bs, 1, H, D, generator=g, device=dev, dtype=torch.bfloat16)
-        q = torch.randn(bs, 1, H * G, D, generator=g, device=dev, dtype=torch.bfloat16)
+        # queries = mean of the recent keys of the head + N(0, 0.5), one per query head
+        q = (kmean.repeat_interleave(G, dim=1) + 0.5 * torch.randn(bs, H * G, D, generator=g, device=dev)
+             ).to(torch.bfloat16).view(bs, 1, H * G, D)
         torch.cuda.synchronize()
         tok_us, issue = [], []
         for t in range(T):
@@ -158,7 +174,12 @@ def main():
             tok_us.append((time.perf_counter() - a) * 1e6)
             issue.append((b - a) * 1e6)
         body = sorted(tok_us[8:])
+        if args.adaptive:
+            ak = cache.last_adaptive_k.flatten().tolist()
+            adaptive_info = {"k_range": args.adaptive_k_range, "threshold": args.adaptive_threshold,
+                             "k_of_last_step": [min(ak), max(ak)]}
         print(json.dumps({"only": "decode-loop", "cache": "adaptive-k" if args.adaptive else "fixed-k",
+                          **({"adaptive": adaptive_info} if args.adaptive else {}), "key_drift_deg_per_1k": args.key_drift,
                           "offload": not args.no_offload, "layers": L, "batch": bs, "prompt": S,
                           "generated": T, "final_topk": K, "prefill_s": round(t_prefill, 2),
                           "us_per_layer_step_median": round(body[len(body) // 2] / L, 1),
