@@ -324,6 +324,16 @@ int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, const float *sl
                       int64_t *adaptive_k, int64_t *topk_ids, int64_t k_min, int64_t k_max,
                       int32_t *row_keys, int64_t row_keys_base, void *ws, size_t ws_bytes, void *stream);
 
+/* uniform_k[r] = max over the rows of adaptive_k (device int64 [rows] each);
+ * row_keys (optional, device int32 [rows]) = row_keys_base + that maximum.  The
+ * dense form of the adaptive step: every (batch, kv-head) row keeps as many ids
+ * as the greediest one, which is how
+ * cache_hub/polar_cache_atten_value_indices_adaptive_k.py:1585-1589, 1462-1499
+ * sizes its gather and attention (global_k = adaptive_k.max().item()) - here
+ * without the host read. */
+int pkv_uniform_k(const int64_t *adaptive_k, int rows, int64_t *uniform_k, int32_t *row_keys,
+                  int64_t row_keys_base, void *stream);
+
 /* Logits of the dense (sink / local / update buffer) rows against the mean of
  * each KV head's query group: replaces query.mean over the group plus
  * torch.einsum("bhd,bhkd->bhk") .to(float32) * scale
@@ -500,6 +510,8 @@ typedef struct pkv_adaptive_args {
   int64_t *topk_ids;              /* [bs*n_kv_heads][k_out] */
   int32_t *row_keys;              /* [bs*n_kv_heads]; also passed to the attention */
   int64_t row_keys_base;
+  int64_t *uniform_k;             /* NULL, or [bs*n_kv_heads]: pkv_uniform_k runs after the adaptive stage and the
+                                     gather and row_keys use max(adaptive_k) for every row (the dense form) */
   void *ws;                       /* pkv_adaptive_topk_ws_bytes(rows, n_cand, k_out) */
   size_t ws_bytes;
   const void *src_k, *src_v;      /* pinned host K/V stores [bs][h][src_len] rows */

@@ -61,7 +61,7 @@ class AdaptiveArgs(C.Structure):
         ("scale", C.c_float), ("value_norm", _vp), ("vn_stride", _i64), ("vn_offset", _i64),
         ("threshold", C.c_float), ("k_out", _i64), ("k_min", _i64), ("k_max", _i64),
         ("adaptive_k", _vp), ("topk_ids", _vp), ("row_keys", _vp), ("row_keys_base", _i64),
-        ("ws", _vp), ("ws_bytes", _sz),
+        ("uniform_k", _vp), ("ws", _vp), ("ws_bytes", _sz),
         ("src_k", _vp), ("src_v", _vp), ("src_len", _i64), ("idx_offset", _i64),
         ("dst_k", _vp), ("dst_v", _vp), ("dst_len", _i64), ("dst_row0", _i64), ("row_bytes", _i),
     ]
@@ -107,6 +107,7 @@ PROTOTYPES = {
     "pkv_adaptive_topk_ws_bytes": (_sz, [_i, _i64, _i64]),
     "pkv_adaptive_topk": (_i, [_vp, _i64, _vp, _i64, _i64, _vp, _i, C.c_float, _vp, _vp, _i64, _i64, _vp, _i64,
                                C.c_float, _i64, _i, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
+    "pkv_uniform_k": (_i, [_vp, _i, _vp, _vp, _i64, _vp]),
     "pkv_dense_logits": (_i, [_vp, _i, _i, _i, _i, _vp, _i64, _i64, _i64, C.c_float, _vp, _i64, _vp]),
     "pkv_decode_attention_ws_bytes": (_sz, [_i, _i, _i, _i64]),
     "pkv_decode_attention": (_i, [_vp, _i, _i, _i, _i, C.POINTER(AttnSegment), _i, _vp, C.c_float, _vp, _vp, _sz, _vp]),

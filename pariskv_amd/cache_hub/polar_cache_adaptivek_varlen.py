@@ -55,25 +55,32 @@ class polar_cache(_polar_cache_base):
         # the caps the reference actually applies (:255-257): environment overrides with the same names
         self._HARDCODED_MAX_K = int(os.environ.get("ADAPTIVE_TOPK_MAX_K", "800"))
         self._HARDCODED_MIN_K = int(os.environ.get("ADAPTIVE_TOPK_MIN_K", "100"))
-        self._adaptive_topk_buffer_cap = self._HARDCODED_MAX_K
-        self._attn_scale = 1.0 / math.sqrt(self.head_dim)
+        self._init_adaptive_state(self._HARDCODED_MAX_K, uniform_k=False)
 
+    def _init_adaptive_state(self, buffer_cap: int, uniform_k: bool) -> None:
+        """Value-norm caches, the gathered-row buffer of ``buffer_cap`` rows and the operands of the fused step that
+        all layers share.  ``uniform_k``: every row gathers and attends to max(adaptive_k) ids (the dense form of
+        polar_cache_atten_value_indices_adaptive_k.py) instead of its own k."""
+        self._adaptive_topk_buffer_cap = buffer_cap
+        self._attn_scale = 1.0 / math.sqrt(self.head_dim)
+        layer_num = len(self._zones)
         dev, bs, H = self.device, self.batch_size, self.kv_head
         self._sl_vnorm_cache = [torch.zeros((bs, H, self.gpu_kv_capacity), dtype=torch.float32, device=dev)
                                 for _ in range(layer_num)]
         self.value_norm_gpu = [torch.zeros((bs, H, self.unified_kv_capacity), dtype=torch.float32, device=dev)
                                for _ in range(layer_num)]
-        cap = max(1, self._adaptive_topk_buffer_cap)
-        self._topk_k = torch.zeros((bs, H, cap, self.head_dim), dtype=self.dtype, device=dev)
-        self._topk_v = torch.zeros((bs, H, cap, self.head_dim), dtype=self.dtype, device=dev)
-        # operands of the fused step that all layers share
+        cap = max(1, buffer_cap)
         self._dense_logits = torch.empty((bs, H, self.gpu_kv_capacity), dtype=torch.float32, device=dev)
         self._adaptive_k = torch.zeros((bs, H), dtype=torch.int64, device=dev)
+        self._uniform_k = torch.zeros((bs, H), dtype=torch.int64, device=dev) if uniform_k else None
         self._topk_ids = torch.zeros((bs * H * cap,), dtype=torch.int64, device=dev)
         self._row_keys = torch.zeros((bs, H), dtype=torch.int32, device=dev)
         self._adk_ws = None
         self._adaptive_bound = [None] * layer_num  # per layer: (n_keys, ops.BoundAdaptiveStep, topk_cap)
         self.last_adaptive_k = None  # [bs, H] int64 of the most recent retrieval step
+        if self.enable_offload:
+            self._topk_k = torch.zeros((bs, H, cap, self.head_dim), dtype=self.dtype, device=dev)
+            self._topk_v = torch.zeros((bs, H, cap, self.head_dim), dtype=self.dtype, device=dev)
 
     # ------------------------------------------------------------ ratios
     def _get_adaptive_ratios(self, retrieval_len):
@@ -187,7 +194,7 @@ class polar_cache(_polar_cache_base):
                         dense_logits=self._dense_logits, scale=self._attn_scale, value_norm=self.value_norm_gpu[layer_idx],
                         vn_offset=self.sink_size, threshold=self.adaptive_topk_threshold, k_out=topk_cap, k_min=k_min,
                         k_max=k_max, adaptive_k=self._adaptive_k, topk_ids=self._topk_ids, row_keys=self._row_keys,
-                        row_keys_base=sl_end, ws=self._adk_ws, src_k=self.unified_keys_cpu[layer_idx],
+                        row_keys_base=sl_end, uniform_k=self._uniform_k, ws=self._adk_ws, src_k=self.unified_keys_cpu[layer_idx],
                         src_v=self.unified_values_cpu[layer_idx], dst_k=self._topk_k, dst_v=self._topk_v)
         segments = [(kg, vg, 0, sl_end), (self._topk_k, self._topk_v, 0, topk_cap)]
         bound = self._plan.bind_adaptive(q, self._srht_signs, self._mag_centers, self.cluster_key_counts_gpu[layer_idx],

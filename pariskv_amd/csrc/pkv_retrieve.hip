@@ -200,7 +200,12 @@ extern "C" int pkv_adaptive_decode_step(const pkv_retrieve_args *retrieve, void 
                          ad->vn_offset, cand, retrieve->n_cand, ad->threshold, ad->k_out, rows, ad->adaptive_k,
                          ad->topk_ids, ad->k_min, ad->k_max, ad->row_keys, ad->row_keys_base, ad->ws, ad->ws_bytes, stream);
   if (rc) return rc;
-  rc = pkv_gather_uva_ragged(ad->src_k, ad->src_v, ad->src_len, ad->topk_ids, ad->k_out, ad->adaptive_k, ad->idx_offset,
+  if (ad->uniform_k) {
+    rc = pkv_uniform_k(ad->adaptive_k, rows, ad->uniform_k, ad->row_keys, ad->row_keys_base, stream);
+    if (rc) return rc;
+  }
+  rc = pkv_gather_uva_ragged(ad->src_k, ad->src_v, ad->src_len, ad->topk_ids, ad->k_out,
+                             ad->uniform_k ? ad->uniform_k : ad->adaptive_k, ad->idx_offset,
                              ad->dst_k, ad->dst_v, ad->dst_len, ad->dst_row0, retrieve->bs, retrieve->n_kv_heads,
                              ad->row_bytes, stream);
   if (rc) return rc;

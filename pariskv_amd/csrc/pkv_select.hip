@@ -1258,6 +1258,32 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adk_finish_kernel(
                 adaptive_k + row, topk_ids + (int64_t)row * k_out, cl, row, (float *)s_hist, &s_counter);
 }
 
+// uniform_k[r] = max over all rows of adaptive_k, row_keys[r] = base + that maximum: the dense form of the
+// adaptive-k step, where every row keeps as many ids as the greediest one
+// (polar_cache_atten_value_indices_adaptive_k.py:1462-1499 sizes its gather and attention by max(adaptive_k)).
+// One workgroup of 1024 threads.
+__global__ __launch_bounds__(kTopkThreads) void pkv_uniform_k_kernel(const int64_t *__restrict__ adaptive_k, int rows,
+                                                                    int64_t *__restrict__ uniform_k,
+                                                                    int32_t *__restrict__ row_keys, int64_t base) {
+  __shared__ int64_t s_max[kTopkThreads / PKV_WAVE];
+  int64_t m = 0;
+  for (int r = threadIdx.x; r < rows; r += kTopkThreads) m = adaptive_k[r] > m ? adaptive_k[r] : m;
+#pragma unroll
+  for (int o = PKV_WAVE / 2; o > 0; o >>= 1) {
+    const int64_t other = __shfl_xor(m, o, PKV_WAVE);
+    m = other > m ? other : m;
+  }
+  if (pkv_lane() == 0) s_max[threadIdx.x / PKV_WAVE] = m;
+  __syncthreads();
+  m = s_max[0];
+#pragma unroll
+  for (int w = 1; w < kTopkThreads / PKV_WAVE; ++w) m = s_max[w] > m ? s_max[w] : m;
+  for (int r = threadIdx.x; r < rows; r += kTopkThreads) {
+    uniform_k[r] = m;
+    if (row_keys) row_keys[r] = (int32_t)(base + m);
+  }
+}
+
 // Logits of the dense (sink / local / buffer) rows against the group-mean query
 // (polar_cache_adaptivek_varlen.py:1418-1419, :1731): out[(b,h)][r] = dtype(mean_g q . K[r]) widened to fp32,
 // times scale.  16 lanes per key row, 8 dims per lane: a lane adds its 8 products in order, the 16 partial
@@ -1598,5 +1624,14 @@ extern "C" int pkv_dense_logits(const void *q, int dtype, int bs, int n_kv_heads
     hipLaunchKernelGGL(pkv_dense_logits_kernel<false>, grid, dim3(kDenseLogitThreads), 0, (hipStream_t)stream, q,
                        n_kv_heads, group, k, k_stride_b, k_stride_h, n_rows, scale, out, out_stride);
   PKV_LAUNCH_CHECK("pkv_dense_logits_kernel");
+  return PKV_OK;
+}
+
+extern "C" int pkv_uniform_k(const int64_t *adaptive_k, int rows, int64_t *uniform_k, int32_t *row_keys,
+                             int64_t row_keys_base, void *stream) {
+  PKV_REQUIRE(adaptive_k && uniform_k && rows > 0, "pkv_uniform_k: bad arguments");
+  hipLaunchKernelGGL(pkv_uniform_k_kernel, dim3(1), dim3(kTopkThreads), 0, (hipStream_t)stream, adaptive_k, rows,
+                     uniform_k, row_keys, row_keys_base);
+  PKV_LAUNCH_CHECK("pkv_uniform_k_kernel");
   return PKV_OK;
 }

@@ -361,6 +361,20 @@ def adaptive_topk(sl_logits: torch.Tensor, sl_vnorm: torch.Tensor, cand_scores: 
     return (ak, ids) if row_keys is None else (ak, ids, row_keys)
 
 
+def uniform_k(adaptive_k: torch.Tensor, row_keys_base: Optional[int] = None):
+    """max over all (batch, kv-head) rows of ``adaptive_k`` (int64 [bs,H]) broadcast to every row, on the GPU: the
+    ``global_k`` of cache_hub/polar_cache_atten_value_indices_adaptive_k.py:1585 without its host read.  Returns the
+    int64 [bs,H] tensor, and with ``row_keys_base`` also int32 [bs,H] = base + max."""
+    _cuda(adaptive_k)
+    _need(adaptive_k.dtype == torch.int64 and adaptive_k.is_contiguous() and adaptive_k.numel() > 0,
+          "adaptive_k: contiguous int64")
+    out = torch.empty_like(adaptive_k)
+    rk = None if row_keys_base is None else torch.empty(adaptive_k.shape, dtype=torch.int32, device=adaptive_k.device)
+    _lib.check(_lib.lib().pkv_uniform_k(_p(adaptive_k), adaptive_k.numel(), _p(out), _p(rk), int(row_keys_base or 0),
+                                        _stream(adaptive_k)))
+    return out if rk is None else (out, rk)
+
+
 def adaptive_topk_ws_bytes(rows: int, n_cand: int, k_out: int) -> int:
     return int(_lib.lib().pkv_adaptive_topk_ws_bytes(rows, n_cand, k_out))
 
@@ -378,10 +392,11 @@ def dense_logits(queries: torch.Tensor, keys: torch.Tensor, n_rows: int, scale: 
     G = queries.numel() // (bs * H * D)
     if out is None:
         out = torch.empty(bs, H, n_rows, dtype=torch.float32, device=keys.device)
-    _need(out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape[:2]) == (bs, H) and
-          out.shape[2] >= n_rows, "out: contiguous fp32 [bs,H,>=n_rows]")
+    _need(out.is_cuda and out.dtype == torch.float32 and tuple(out.shape[:2]) == (bs, H) and out.shape[2] >= n_rows and
+          out.stride(2) == 1 and out.stride(1) >= n_rows and (bs == 1 or out.stride(0) == H * out.stride(1)),
+          "out: fp32 [bs,H,>=n_rows] with contiguous rows at one uniform stride")
     _lib.check(_lib.lib().pkv_dense_logits(_p(queries), _dt(queries.dtype), bs, H, G, _p(keys), keys.stride(0),
-                                           keys.stride(1), n_rows, float(scale), _p(out), out.shape[2], _stream(keys)))
+                                           keys.stride(1), n_rows, float(scale), _p(out), out.stride(1), _stream(keys)))
     return out
 
 
@@ -791,7 +806,8 @@ class RetrievePlan:
         """The adaptive-k step of one layer as a :class:`BoundAdaptiveStep`.  ``adaptive``: dense_k [bs,H,rows,128],
         dense_rows, dense_vnorm fp32 [bs,H,rows], dense_logits fp32 [bs,H,>=rows] scratch, scale, value_norm fp32
         [bs,H,cap], vn_offset, threshold, k_out, k_min, k_max, adaptive_k int64 [bs,H], topk_ids int64 (>= bs*H*k_out
-        elements), row_keys int32 [bs,H], row_keys_base, ws uint8 (pkv_adaptive_topk_ws_bytes), src_k / src_v pinned
+        elements), row_keys int32 [bs,H], row_keys_base, optional uniform_k int64 [bs,H] (then every row gathers and
+        attends to max(adaptive_k) ids), ws uint8 (pkv_adaptive_topk_ws_bytes), src_k / src_v pinned
         CPU [bs,H,len,128], dst_k / dst_v GPU [bs,H,>=k_out,128].  ``segments`` are the attention's; its per-row key
         count is ``row_keys``."""
         a = self._fill(queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, 1,
@@ -828,6 +844,11 @@ class RetrievePlan:
         ad.scale, ad.value_norm, ad.vn_stride, ad.vn_offset = float(d["scale"]), vn.data_ptr(), vn.shape[2], int(d["vn_offset"])
         ad.threshold, ad.k_out, ad.k_min, ad.k_max = float(d["threshold"]), k_out, int(d["k_min"]), int(d["k_max"])
         ad.adaptive_k, ad.topk_ids, ad.row_keys, ad.row_keys_base = ak.data_ptr(), ids.data_ptr(), rk.data_ptr(), int(d["row_keys_base"])
+        uk = d.get("uniform_k")
+        if uk is not None:
+            _cuda(uk)
+            _need(uk.dtype == torch.int64 and uk.is_contiguous() and uk.numel() == bs * H, "uniform_k: contiguous int64 [bs,H]")
+            ad.uniform_k = uk.data_ptr()
         ad.ws, ad.ws_bytes = ws.data_ptr(), ws.numel()
         ad.src_k, ad.src_v, ad.src_len, ad.idx_offset = sk.data_ptr(), sv.data_ptr(), sk.shape[2], int(d.get("idx_offset", 0))
         ad.dst_k, ad.dst_v, ad.dst_len, ad.dst_row0 = tk.data_ptr(), tv.data_ptr(), tk.shape[2], 0

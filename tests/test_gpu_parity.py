@@ -1237,6 +1237,18 @@ def test_adaptive_topk_clamp_and_row_keys(ops):
         ops.adaptive_topk(*args, 0.9, k_out, cand_vnorm=cv.to(DEV), k_min=600, k_max=500)
 
 
+def test_uniform_k_is_the_row_maximum(ops):
+    """pkv_uniform_k: max over all rows, broadcast, plus the attention's key count (the reference reads
+    adaptive_k.max().item() on the host, polar_cache_atten_value_indices_adaptive_k.py:1585)."""
+    g = torch.Generator().manual_seed(2)
+    for shape in ((1, 1), (2, 3), (8, 8), (40, 64)):   # up to 2560 rows: more than one pass of the 1024 threads
+        ak = torch.randint(1, 5000, shape, generator=g).to(DEV)
+        uk, rk = ops.uniform_k(ak, row_keys_base=77)
+        assert uk.shape == ak.shape and (uk == ak.max()).all()
+        assert rk.dtype == torch.int32 and (rk == int(ak.max()) + 77).all()
+        assert torch.equal(ops.uniform_k(ak), uk)
+
+
 def test_offload_rows_equals_sliced_copy(ops):
     """pkv_offload_rows against the sliced copy_ it replaces (reference polar_cache.py:457-471, :778-799): rows read in
     place from the model's [bs,seq,h,d] layout and from a partly filled staging buffer, into a batch slice of the pinned

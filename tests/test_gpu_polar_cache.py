@@ -286,6 +286,95 @@ def test_adaptive_k_cache_decode_loop(dtype):
     assert len(seen_k) >= 3, f"k should vary across rows and steps, saw {sorted(seen_k)}"
 
 
+@pytest.mark.parametrize("offload", [True, False])
+def test_dense_adaptive_k_cache_decode_loop(offload):
+    """Dense-form adaptive-k variant (reference polar_cache_atten_value_indices_adaptive_k.py), both storage modes:
+    per-row k (capped by adaptive_topk_max_k, no lower clamp) equals the CPU oracle's on the cache's own index, and the
+    attention equals an fp32 softmax over sink ++ the first max-over-rows(k) ids of each row's benefit order ++ dense
+    tail, which is the set the reference attends to (:1462-1499, :1585-1589)."""
+    from pariskv_amd.cache_hub.polar_cache_atten_value_indices_adaptive_k import polar_cache as dense_adaptive_cache
+
+    bs, Hkv, Hq, S, steps = 2, 2, 8, 3000, 40
+    sink, local, I, thr, max_k = 4, 64, 16, 0.6, 250
+    G = Hq // Hkv
+    cache = dense_adaptive_cache(valid_start=[0] * bs, layer_num=1, batch_size=bs, max_length=S + steps + 10,
+                                 num_key_value_heads=Hkv, num_heads=Hq, head_dim=128, dtype=torch.bfloat16,
+                                 layer_mapping={0: DEV}, max_new_length=steps + 10, sink_size=sink, local_size=local, core=1,
+                                 nprobe=1, cache_unit_size=1, cache_cluster_num=1, num_gpus=1, model_size=7, final_topk=100,
+                                 dynamic_update_interval=I, full_attention_threshold=100, enable_offload=offload,
+                                 adaptive_topk_threshold=thr, adaptive_topk_max_k=max_k)
+    gen = torch.Generator().manual_seed(5)
+    hk, hv = _synth_kv(gen, bs, S, Hkv)
+    hv = hv * (0.25 + 2.0 * torch.rand(bs, S, Hkv, 1, generator=gen)).to(torch.bfloat16)
+    cache.prefill_update_kv_cache(None, hk.to(DEV), hv.to(DEV), 0, 0)
+    signs = O.srht_signs(42)
+    scale = 1.0 / math.sqrt(128)
+    seen_k, uneven = set(), False
+    for step in range(steps):
+        k1, v1 = _synth_kv(gen, bs, 1, Hkv)
+        q = (hk[:, -3:].float().mean(dim=1).repeat_interleave(G, dim=1) * 0.3
+             + 0.5 * torch.randn(bs, Hq, 128, generator=gen)).to(torch.bfloat16).view(bs, 1, Hq, 128)
+        hk, hv = torch.cat([hk, k1], dim=1), torch.cat([hv, v1], dim=1)
+        cache.decode_update_kv_cache(k1.to(DEV), v1.to(DEV), 0)
+        out = cache.compute(q.to(DEV), 0)
+        if step % 6 != 0 and step not in (I - 1, I, 2 * I - 1):
+            continue
+        torch.cuda.synchronize()
+        total = S + step + 1
+        z = cache._zones[0]
+        n_keys, n_cand, _, tiers = cache.retrieval_shape(0)
+        assert n_keys == z.encoded and z.seq_len == total
+        dense_pos = torch.cat([torch.arange(sink), torch.arange(sink + n_keys, total)])
+        vn_ref = torch.linalg.vector_norm(hv, dim=-1).float().permute(0, 2, 1)
+        norms = cache._sl_vnorm_cache[0].cpu()
+        sl_vnorm = (norms[:, :, :len(dense_pos)] if offload else norms[:, :, dense_pos]).numpy()
+        assert np.allclose(sl_vnorm, vn_ref[:, :, dense_pos].numpy(), rtol=2.0 ** -7, atol=0)
+        value_norm = cache.value_norm_gpu[0].cpu().numpy()
+        assert np.allclose(value_norm[:, :, sink:sink + n_keys], vn_ref[:, :, sink:sink + n_keys].numpy(), rtol=2.0 ** -7, atol=0)
+        codes, nib = cache._codes_km[0].cpu().numpy(), cache._nib_km[0].cpu().numpy()
+        w, cc = cache._w_km[0].float().cpu().numpy(), cache.cluster_key_counts_gpu[0].cpu().numpy()
+        ak = cache.last_adaptive_k.cpu().numpy()
+        cap_k = min(max_k, n_cand)
+        ids_ref = np.zeros((bs, Hkv, cap_k), np.int64)
+        for b in range(bs):
+            for h in range(Hkv):
+                zone = slice(sink, sink + n_keys)
+                qh, qn = O.query_prep(q[b, 0, h * G:(h + 1) * G].float().numpy(), signs, O.BF16)
+                lut = O.tier_lut(O.rank_centroids(qh, O.BF16), cc[b, h], tiers)
+                cand_ref, _ = O.select_candidates(O.collision_count(codes[b, h][zone], lut), n_cand)
+                sc = O.rerank(cand_ref, nib[b, h][zone].reshape(-1, 16, 4), w[b, h][zone], qh, qn)
+                sl_logits = O.dense_logits(q[b, 0, h * G:(h + 1) * G].float().numpy(), hk[b, dense_pos, h].float().numpy(),
+                                           scale, O.BF16)
+                k_ref, ids_ref[b, h] = O.adaptive_topk(sl_logits, sl_vnorm[b, h], sc * np.float32(scale),
+                                                       value_norm[b, h][cand_ref + sink], cand_ref, thr, cap_k)
+                assert int(ak[b, h]) == k_ref, f"step {step} row {(b, h)}: k {ak[b, h]} vs {k_ref}"
+                seen_k.add(k_ref)
+        global_k = int(ak.max())
+        uneven = uneven or int(ak.min()) < global_k
+        for b in range(bs):
+            K, V = hk[b].permute(1, 0, 2), hv[b].permute(1, 0, 2)
+            ref = torch.empty(Hq, 128)
+            for h in range(Hkv):
+                sel = torch.cat([torch.arange(sink), torch.from_numpy(ids_ref[b, h, :global_k]) + sink,
+                                 torch.arange(sink + n_keys, total)])
+                ref[h * G:(h + 1) * G] = _ref_attention(q[b, 0, h * G:(h + 1) * G], K[h:h + 1, sel], V[h:h + 1, sel], G=G * 10)
+            err = (out[b, 0].float().cpu() - ref).abs().max().item()
+            assert err < 2e-2, f"attention differs by {err} at step {step}"
+        if step == 36:  # the reference's method form (:1508-1589)
+            qd = q.to(DEV)
+            cand, scores = cache._plan.run_candidates(qd, cache._srht_signs, cache._mag_centers, cache.cluster_key_counts_gpu[0],
+                                                      cache._codes_km[0], cache._nib_km[0], cache._w_km[0], sink, n_keys,
+                                                      tiers, n_cand)
+            dense_k = torch.from_numpy(np.stack([[hk[b, dense_pos, h].float().numpy() for h in range(Hkv)]
+                                                 for b in range(bs)])).to(torch.bfloat16).to(DEV)
+            k_form, idx_form, gk = cache._compute_adaptive_topk(
+                qd[:, 0].view(bs, Hkv, G, 128).float().mean(dim=2).to(torch.bfloat16), dense_k,
+                torch.from_numpy(sl_vnorm).to(DEV), scores, cand, 0, thr)
+            assert np.array_equal(k_form.cpu().numpy(), ak) and gk == global_k
+            assert np.array_equal(idx_form.cpu().numpy(), ids_ref[:, :, :global_k])
+    assert len(seen_k) >= 3 and uneven, f"k should vary across rows and steps, saw {sorted(seen_k)}"
+
+
 def test_reference_multibatch_smoke_shape():
     """The reference's own integration smoke (tests/test_multibatch_smoke.py:23-117): batch 8 in lockstep, 28 layers,
     4 KV heads x GQA 8, prefill 20480, 50 decode steps, sink 128 / local 256, refresh every 128 tokens, offload on,
