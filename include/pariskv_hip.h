@@ -461,6 +461,11 @@ typedef struct pkv_retrieve_args {
    * 1: the same k ids in an unspecified but fixed order (a function of the inputs only), for callers that
    *    use them as a set, as polar_cache.compute does (gather + attention): the final sort is left out. */
   int any_order;
+  /* Bytes from one key's 64 nibble bytes (16 weights) to the next key's; 0 = packed arrays (64 / 32).  A key's
+   * nibbles and weights are only ever read together (by the rerank, for candidates scattered over the zone) and
+   * HBM is fetched in 128-byte lines, so keeping both in one 128-byte-aligned record per key (nib = record,
+   * weight = record + 64, both strides 128) halves the traffic of that gather. */
+  int64_t nib_key_stride, weight_key_stride;
 } pkv_retrieve_args;
 
 size_t pkv_retrieve_ws_bytes(int rows, int64_t n_keys, int64_t n_cand, int64_t k);

@@ -48,7 +48,7 @@ class RetrieveArgs(C.Structure):
         ("src_k", _vp), ("src_v", _vp), ("gather_from_host", _i),
         ("src_len", _i64), ("idx_offset", _i64),
         ("dst_k", _vp), ("dst_v", _vp), ("dst_len", _i64), ("dst_row0", _i64),
-        ("row_bytes", _i), ("any_order", _i),
+        ("row_bytes", _i), ("any_order", _i), ("nib_key_stride", _i64), ("weight_key_stride", _i64),
     ]
 
 

@@ -78,9 +78,10 @@ PKV_INTERNAL int pkv_launch_select(const uint8_t *cnt_u8, int64_t cnt_stride, co
                                    int64_t *out, hipStream_t s);
 PKV_INTERNAL int pkv_launch_select_rerank(const uint8_t *cnt_u8, int64_t cnt_stride, const uint32_t *row_suf,
                                           const uint16_t *chunk_suf, int chunk_keys, int bs, int n_kv_heads, int64_t n_keys, int64_t k,
-                                          const uint8_t *nib, int64_t ns_b, int64_t ns_h, const uint16_t *weight,
-                                          int64_t ws_b, int64_t ws_h, const float *qhat, const float *qnorm,
-                                          const float *centers, int64_t *cand, float *scores, hipStream_t s);
+                                          const uint8_t *nib, int64_t ns_b, int64_t ns_h, int64_t ns_key,
+                                          const uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key,
+                                          const float *qhat, const float *qnorm, const float *centers, int64_t *cand,
+                                          float *scores, hipStream_t s);
 PKV_INTERNAL int pkv_launch_rerank(const int64_t *cand, int bs, int n_kv_heads, int64_t n_cand, int64_t n_keys,
                                    const uint8_t *nib, int64_t ns_b, int64_t ns_h, int64_t ns_key, int64_t ns_sub,
                                    const uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key,
@@ -316,7 +317,8 @@ __device__ __forceinline__ float pkv_block_dot(const float *__restrict__ s_prod,
   return t;
 }
 
-// Score of one key stored key-major: 64 B of nibbles at np, 16 bf16 weights at wp (both 16-byte aligned).
+// Score of one key stored key-major: 64 B of nibbles at np, 16 bf16 weights at wp (both 16-byte aligned; in the
+// cache's layout the two sit in one 128-byte record, so a candidate costs one HBM line).
 // Order: dims 0..7 inside a block, blocks 0..15, then * ||q||; multiply and add rounded separately.
 // The four 16-byte groups are walked by a rolled loop that rotates the data registers, so that only one
 // group's 32 table reads are in flight at a time (fully unrolled, the scheduler hoists all 128 reads and

@@ -28,7 +28,8 @@ __device__ __forceinline__ void store_v4b(uint16_t *__restrict__ v4b, int64_t ro
   *(pkv_u32x4 *)(v4b + (((row * 16 + blk) * n_cand) + i) * 8) = o;
 }
 
-// KEYMAJOR: nib [key][64] bytes, weight [key][16] bf16, both 16-byte aligned.
+// KEYMAJOR: 64 contiguous nibble bytes and 16 contiguous bf16 weights per key, both 16-byte aligned
+// (key strides ns_key bytes / ws_key elements: 64 / 16 when packed, 128 / 64 inside a 128-byte record).
 // Otherwise: nib addressed by (ns_key, ns_sub) in bytes (4-byte aligned words),
 // weight by (ws_key, ws_sub) in elements.
 template <bool KEYMAJOR, bool V4B>
@@ -60,8 +61,8 @@ __global__ __launch_bounds__(kRerankThreads) void pkv_rerank_kernel(
   const uint16_t *wrow = weight + (int64_t)b * ws_b + (int64_t)h * ws_h;
   float s = 0.f;
   if (KEYMAJOR) {
-    const pkv_u32x4 *np = (const pkv_u32x4 *)(nrow + key * 64);
-    const pkv_u32x4 *wp = (const pkv_u32x4 *)(wrow + key * 16);
+    const pkv_u32x4 *np = (const pkv_u32x4 *)(nrow + key * ns_key);
+    const pkv_u32x4 *wp = (const pkv_u32x4 *)(wrow + key * ws_key);
     pkv_u32x4 nv[4], wv[2];
 #pragma unroll
     for (int u = 0; u < 4; ++u) nv[u] = np[u];
@@ -103,7 +104,8 @@ int pkv_launch_rerank(const int64_t *cand, int bs, int n_kv_heads, int64_t n_can
               (long long)n_keys);
   PKV_REQUIRE(!v4b || pkv_aligned(v4b, 16), "v4b must be 16-byte aligned");
   dim3 grid((unsigned)((n_cand + kRerankThreads - 1) / kRerankThreads), (unsigned)(bs * n_kv_heads));
-  const bool keymajor = ns_sub == 4 && ns_key == 64 && ws_sub == 1 && ws_key == 16 && pkv_aligned(nib, 16) &&
+  const bool keymajor = ns_sub == 4 && ns_key >= 64 && ns_key % 16 == 0 && ws_sub == 1 && ws_key >= 16 &&
+                        ws_key % 8 == 0 && pkv_aligned(nib, 16) &&
                         pkv_aligned(weight, 16) && ns_b % 16 == 0 && ns_h % 16 == 0 && ws_b % 8 == 0 && ws_h % 8 == 0;
   if (!keymajor)
     PKV_REQUIRE(pkv_aligned(nib, 4) && ns_b % 4 == 0 && ns_h % 4 == 0 && ns_key % 4 == 0 && ns_sub % 4 == 0,

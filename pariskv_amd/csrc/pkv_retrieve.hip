@@ -123,25 +123,31 @@ extern "C" int pkv_retrieve(const pkv_retrieve_args *a, void *ws, size_t ws_byte
   for (int i = 0; i < a->n_tiers; ++i) t.t[i] = a->tier_counts[i];
 
   const int H = a->n_kv_heads;
+  // bytes from one key's nibbles / weights to the next key's: packed arrays, or both inside one wider record
+  const int64_t nk = a->nib_key_stride ? a->nib_key_stride : 64;
+  const int64_t wk = (a->weight_key_stride ? a->weight_key_stride : 32) / 2;  // in bf16 elements
+  PKV_REQUIRE(nk >= 64 && nk % 16 == 0 && wk >= 16 && wk % 8 == 0,
+              "key strides of %lld / %lld bytes: nibbles need >= 64, weights >= 32, multiples of 16",
+              (long long)a->nib_key_stride, (long long)a->weight_key_stride);
   int rc = pkv_launch_query_prep_lut(a->q, a->dtype, a->bs, H, a->group, a->signs, a->cluster_counts,
                                      (int64_t)H * 4096, 4096, t, qhat, qnorm, lut, nullptr, rowsuf, s);
   if (rc) return rc;
   const uint8_t *codes = a->codes + a->key0 * 16;
-  const uint8_t *nib = a->nib + a->key0 * 64;
-  const uint16_t *weight = a->weight + a->key0 * 16;
+  const uint8_t *nib = a->nib + a->key0 * nk;
+  const uint16_t *weight = a->weight + a->key0 * wk;
   if (a->n_cand == a->n_keys) {
     rc = pkv_launch_identity_fill(cand, a->n_keys, a->n_cand, rows, s);
     if (rc) return rc;
-    rc = pkv_launch_rerank(cand, a->bs, H, a->n_cand, a->n_keys, nib, (int64_t)H * a->cap * 64, a->cap * 64, 64, 4,
-                           weight, (int64_t)H * a->cap * 16, a->cap * 16, 16, 1, qhat, qnorm, a->centers, scores,
+    rc = pkv_launch_rerank(cand, a->bs, H, a->n_cand, a->n_keys, nib, (int64_t)H * a->cap * nk, a->cap * nk, nk, 4,
+                           weight, (int64_t)H * a->cap * wk, a->cap * wk, wk, 1, qhat, qnorm, a->centers, scores,
                            nullptr, s);
   } else {
     rc = pkv_launch_scan(codes, (int64_t)H * a->cap * 16, a->cap * 16, 16, 1, a->bs, H, a->n_keys, lut, cnt,
                          w.cnt_stride, nullptr, rowsuf, hist, w.chunk_keys, s);
     if (rc) return rc;
     rc = pkv_launch_select_rerank(cnt, w.cnt_stride, rowsuf, hist, w.chunk_keys, a->bs, H, a->n_keys, a->n_cand, nib,
-                                  (int64_t)H * a->cap * 64, a->cap * 64, weight, (int64_t)H * a->cap * 16, a->cap * 16,
-                                  qhat, qnorm, a->centers, cand, scores, s);
+                                  (int64_t)H * a->cap * nk, a->cap * nk, nk, weight, (int64_t)H * a->cap * wk, a->cap * wk,
+                                  wk, qhat, qnorm, a->centers, cand, scores, s);
   }
   if (rc) return rc;
   if (!a->out_ids) return PKV_OK;  // candidates only: the caller reads them out of the workspace

@@ -162,9 +162,9 @@ __global__ __launch_bounds__(kSelThreads) void pkv_select_kernel(const uint8_t *
 __global__ __launch_bounds__(kSelThreads) void pkv_select_rerank_kernel(
     const uint8_t *__restrict__ cnt, int64_t cnt_stride, const uint32_t *__restrict__ row_suf,
     const uint16_t *__restrict__ chunk_suf, int chunk_keys, int n_kv_heads, int64_t n_keys, int64_t k,
-    const uint8_t *__restrict__ nib, int64_t ns_b, int64_t ns_h, const uint16_t *__restrict__ weight, int64_t ws_b,
-    int64_t ws_h, const float *__restrict__ qhat, const float *__restrict__ qnorm, const float *__restrict__ centers,
-    int64_t *__restrict__ out, float *__restrict__ scores) {
+    const uint8_t *__restrict__ nib, int64_t ns_b, int64_t ns_h, int ns_key, const uint16_t *__restrict__ weight,
+    int64_t ws_b, int64_t ws_h, int ws_key, const float *__restrict__ qhat, const float *__restrict__ qnorm,
+    const float *__restrict__ centers, int64_t *__restrict__ out, float *__restrict__ scores) {
   const int row = blockIdx.y;
   const int chunk = blockIdx.x;
   const int tid = threadIdx.x;
@@ -233,7 +233,7 @@ __global__ __launch_bounds__(kSelThreads) void pkv_select_rerank_kernel(
       if (pos >= 0) {
         const int64_t key = blk0 + s_list_key[j];
         orow[pos] = key;
-        srow[pos] = pkv_rerank_keymajor(s_prod, (const pkv_u32x4 *)(nrow + key * 64), (const pkv_u32x4 *)(wrow + key * 16), qn);
+        srow[pos] = pkv_rerank_keymajor(s_prod, (const pkv_u32x4 *)(nrow + key * ns_key), (const pkv_u32x4 *)(wrow + key * ws_key), qn);
       }
     }
     __syncthreads();  // the list is rewritten by the next iteration
@@ -1353,20 +1353,23 @@ int pkv_launch_select(const uint8_t *cnt_u8, int64_t cnt_stride, const uint32_t 
 int pkv_launch_select_rerank(const uint8_t *cnt_u8, int64_t cnt_stride, const uint32_t *row_suf,
                              const uint16_t *chunk_suf, int chunk_keys, int bs,
                              int n_kv_heads, int64_t n_keys, int64_t k, const uint8_t *nib, int64_t ns_b, int64_t ns_h,
-                             const uint16_t *weight, int64_t ws_b, int64_t ws_h, const float *qhat, const float *qnorm,
-                             const float *centers, int64_t *cand, float *scores, hipStream_t s) {
+                             int64_t ns_key, const uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key,
+                             const float *qhat, const float *qnorm, const float *centers, int64_t *cand, float *scores,
+                             hipStream_t s) {
   PKV_REQUIRE(k >= 1 && k < n_keys && k < ((int64_t)1 << 31), "select needs 1 <= k < n_keys (k=%lld n=%lld)", (long long)k,
               (long long)n_keys);
   PKV_REQUIRE(cnt_stride % 16 == 0 && cnt_stride >= n_keys && pkv_aligned(cnt_u8, 16),
               "count rows must be 16-byte aligned and padded");
   PKV_REQUIRE(pkv_aligned(nib, 16) && pkv_aligned(weight, 16) && ns_b % 16 == 0 && ns_h % 16 == 0 && ws_b % 8 == 0 &&
-                  ws_h % 8 == 0,
-              "key-major nibbles / weights must be 16-byte aligned");
+                  ws_h % 8 == 0 && ns_key >= 64 && ns_key % 16 == 0 && ws_key >= 16 && ws_key % 8 == 0 &&
+                  ns_key < (1 << 20) && ws_key < (1 << 20),
+              "key-major nibbles / weights must be 16-byte aligned, 64 bytes / 16 weights per key");
   const int64_t n_chunks = (n_keys + chunk_keys - 1) / chunk_keys;
   dim3 grid((unsigned)n_chunks, (unsigned)(bs * n_kv_heads));
   hipLaunchKernelGGL(pkv_select_rerank_kernel, grid, dim3(kSelThreads), 0, s, cnt_u8, cnt_stride, row_suf, chunk_suf,
                      chunk_keys,
-                     n_kv_heads, n_keys, k, nib, ns_b, ns_h, weight, ws_b, ws_h, qhat, qnorm, centers, cand, scores);
+                     n_kv_heads, n_keys, k, nib, ns_b, ns_h, (int)ns_key, weight, ws_b, ws_h, (int)ws_key, qhat, qnorm,
+                     centers, cand, scores);
   PKV_LAUNCH_CHECK("pkv_select_rerank_kernel");
   return PKV_OK;
 }

@@ -19,6 +19,7 @@ import torch
 from . import _lib
 
 B_SUB, M_SUB, K_CLUSTERS, HEAD_DIM = 16, 8, 256, 128
+RERANK_RECORD_BYTES = 128  # one key's 64 nibble bytes + 16 bf16 weights, padded to an HBM line
 TIER_RATIOS = (0.05, 0.15, 0.30, 0.50, 0.75, 1.0)  # cache_hub/polar_cache.py:1221
 # cache_hub/polar_cache.py:188-193 rounded to bf16
 MAG_THRESHOLDS = (0.08447265625, 0.169921875, 0.2578125, 0.349609375, 0.44921875, 0.55859375, 0.69140625)
@@ -84,10 +85,15 @@ def alloc_keymajor(bs: int, heads: int, cap: int, device):
 
     Returns ``(codes_km [bs,H,cap,16] u8, nib_km [bs,H,cap,64] u8, w_km [bs,H,cap,16] bf16,
     codebook [bs,H,16,cap], key_4bit [bs,H,16,cap,4], key_block_weight [bs,H,16,cap])``;
-    the last three are permuted views of the first three."""
+    the last three are permuted views of the first three.  The codes are one packed array (the collision scan
+    streams them); a key's nibbles and weights share one 128-byte-aligned record (bytes 0-63 and 64-95): the
+    rerank reads both for candidates scattered over the zone, HBM comes in 128-byte lines, and two packed arrays
+    would cost two lines per candidate."""
     codes = torch.zeros(bs, heads, cap, B_SUB, dtype=torch.uint8, device=device)
-    nib = torch.zeros(bs, heads, cap, B_SUB * 4, dtype=torch.uint8, device=device)
-    w = torch.zeros(bs, heads, cap, B_SUB, dtype=torch.bfloat16, device=device)
+    rec = torch.zeros(bs, heads, cap, RERANK_RECORD_BYTES, dtype=torch.uint8, device=device)
+    _need(rec.data_ptr() % RERANK_RECORD_BYTES == 0, "allocator returned a buffer that is not 128-byte aligned")
+    nib = rec[..., :B_SUB * 4]
+    w = rec[..., B_SUB * 4:B_SUB * 4 + B_SUB * 2].view(torch.bfloat16)
     return (codes, nib, w, codes.permute(0, 1, 3, 2), nib.view(bs, heads, cap, B_SUB, 4).permute(0, 1, 3, 2, 4),
             w.permute(0, 1, 3, 2))
 
@@ -752,9 +758,12 @@ class RetrievePlan:
         a.q, a.dtype, a.bs, a.n_kv_heads, a.group = q.data_ptr(), _dt(q.dtype), self.bs, self.H, self.group
         a.signs, a.centers, a.cluster_counts = signs.data_ptr(), centers.data_ptr(), cluster_counts.data_ptr()
         _need(cluster_counts.is_contiguous(), "cluster_counts must be contiguous")
-        for t in (codes_km, nib_km, w_km):
-            _need(t.is_contiguous() and t.shape[2] == self.cap, "key-major storage must be contiguous [bs,H,cap,*]")
+        _need(codes_km.is_contiguous() and codes_km.shape[2] == self.cap, "codes must be contiguous [bs,H,cap,16]")
+        for t in (nib_km, w_km):  # packed, or views into a wider per-key record
+            _need(t.shape[2] == self.cap and t.stride(3) == 1 and t.stride(1) == self.cap * t.stride(2) and
+                  t.stride(0) == self.H * t.stride(1), "key-major nibbles / weights: [bs,H,cap,*] rows at one uniform key stride")
         a.codes, a.nib, a.weight = codes_km.data_ptr(), nib_km.data_ptr(), w_km.data_ptr()
+        a.nib_key_stride, a.weight_key_stride = nib_km.stride(2), w_km.stride(2) * w_km.element_size()
         a.cap, a.key0, a.n_keys = self.cap, key0, n_keys
         for i, t in enumerate(tier_counts):
             a.tier_counts[i] = int(t)
