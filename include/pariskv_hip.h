@@ -306,7 +306,9 @@ int pkv_host_device_pointer(const void *host_ptr, void **dev_ptr);
  * [rows][n_cand] of cand_dtype (PKV_DTYPE_F32 with cand_scale 1 for prescaled
  * logits; PKV_DTYPE_BF16 with the attention scale for raw rerank scores).
  * Candidate value norm = cand_vnorm[row][i], or, when cand_vnorm is NULL,
- * value_norm[row*vn_stride + cand_ids[row][i] + vn_offset].
+ * value_norm[row*vn_stride + (cand_ids[row][i] + vn_offset)*vn_pos_stride]
+ * (vn_pos_stride 0 or 1: packed rows; larger when the norms sit inside wider
+ * per-key records; a row then holds vn_stride / vn_pos_stride positions).
  * benefit = exp(logit - max) * ||v||; adaptive_k[row] = smallest k <= k_out with
  * dense_benefit + sum of the k largest candidate benefits >= threshold * total
  * (k_out if never, 1 if total <= 0); topk_ids int64 [rows][k_out] = cand_ids in
@@ -320,7 +322,7 @@ size_t pkv_adaptive_topk_ws_bytes(int rows, int64_t n_cand, int64_t k_out);
 int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, const float *sl_vnorm, int64_t slv_stride,
                       int64_t sl, const void *cand_scores, int cand_dtype, float cand_scale,
                       const float *cand_vnorm, const float *value_norm, int64_t vn_stride, int64_t vn_offset,
-                      const int64_t *cand_ids, int64_t n_cand, float threshold, int64_t k_out, int rows,
+                      int64_t vn_pos_stride, const int64_t *cand_ids, int64_t n_cand, float threshold, int64_t k_out, int rows,
                       int64_t *adaptive_k, int64_t *topk_ids, int64_t k_min, int64_t k_max,
                       int32_t *row_keys, int64_t row_keys_base, void *ws, size_t ws_bytes, void *stream);
 
@@ -466,6 +468,12 @@ typedef struct pkv_retrieve_args {
    * HBM is fetched in 128-byte lines, so keeping both in one 128-byte-aligned record per key (nib = record,
    * weight = record + 64, both strides 128) halves the traffic of that gather. */
   int64_t nib_key_stride, weight_key_stride;
+  /* > 0: byte offset (multiple of 4, inside the nibble record, i.e. < nib_key_stride) of one fp32 word per key
+   * that the fused select+rerank copies out for every candidate, into the workspace segment "cand_record_word"
+   * ([R][n_cand] floats, same order as "cand").  The adaptive-k caches keep a key's value norm there, so that
+   * it arrives with the candidate's HBM line instead of through a second scattered read
+   * (cache_hub/polar_cache_adaptivek_varlen.py:1741-1753 gathers value_norm_gpu at cand_idx + sink). */
+  int64_t record_word_offset;
 } pkv_retrieve_args;
 
 size_t pkv_retrieve_ws_bytes(int rows, int64_t n_keys, int64_t n_cand, int64_t k);
@@ -507,8 +515,8 @@ typedef struct pkv_adaptive_args {
   float *dense_logits;            /* scratch [bs*n_kv_heads][dense_logits_stride] */
   int64_t dense_logits_stride;
   float scale;                    /* attention scale: logits of dense rows and of candidates */
-  const float *value_norm;        /* [bs*n_kv_heads][vn_stride], candidate id + vn_offset */
-  int64_t vn_stride, vn_offset;
+  const float *value_norm;        /* row r, position p at value_norm[r*vn_stride + p*vn_pos_stride]; p = candidate id + vn_offset */
+  int64_t vn_stride, vn_offset, vn_pos_stride;  /* vn_pos_stride 0 or 1: packed rows */
   float threshold;
   int64_t k_out, k_min, k_max;
   int64_t *adaptive_k;            /* [bs*n_kv_heads] */
@@ -531,7 +539,7 @@ int pkv_adaptive_decode_step(const pkv_retrieve_args *retrieve, void *ws, size_t
 
 /* Names and device pointers of the intermediates inside a pkv_retrieve
  * workspace (for tests and profiling): qhat, qnorm, lut, cnt_u8,
- * chunk_suffix_hist, row_suffix_hist, cand, scores.  Returns PKV_EINVAL for an unknown name. */
+ * chunk_suffix_hist, row_suffix_hist, cand, scores, cand_record_word.  Returns PKV_EINVAL for an unknown name. */
 int pkv_retrieve_ws_view(void *ws, int rows, int64_t n_keys, int64_t n_cand, int64_t k,
                          const char *name, void **ptr, size_t *bytes);
 

@@ -49,6 +49,7 @@ class RetrieveArgs(C.Structure):
         ("src_len", _i64), ("idx_offset", _i64),
         ("dst_k", _vp), ("dst_v", _vp), ("dst_len", _i64), ("dst_row0", _i64),
         ("row_bytes", _i), ("any_order", _i), ("nib_key_stride", _i64), ("weight_key_stride", _i64),
+        ("record_word_offset", _i64),
     ]
 
 
@@ -58,7 +59,7 @@ class AdaptiveArgs(C.Structure):
     _fields_ = [
         ("dense_k", _vp), ("dense_stride_b", _i64), ("dense_stride_h", _i64), ("dense_rows", _i64),
         ("dense_vnorm", _vp), ("dense_vnorm_stride", _i64), ("dense_logits", _vp), ("dense_logits_stride", _i64),
-        ("scale", C.c_float), ("value_norm", _vp), ("vn_stride", _i64), ("vn_offset", _i64),
+        ("scale", C.c_float), ("value_norm", _vp), ("vn_stride", _i64), ("vn_offset", _i64), ("vn_pos_stride", _i64),
         ("threshold", C.c_float), ("k_out", _i64), ("k_min", _i64), ("k_max", _i64),
         ("adaptive_k", _vp), ("topk_ids", _vp), ("row_keys", _vp), ("row_keys_base", _i64),
         ("uniform_k", _vp), ("ws", _vp), ("ws_bytes", _sz),
@@ -105,7 +106,7 @@ PROTOTYPES = {
     "pkv_host_free": (_i, [_vp]),
     "pkv_host_device_pointer": (_i, [_vp, C.POINTER(_vp)]),
     "pkv_adaptive_topk_ws_bytes": (_sz, [_i, _i64, _i64]),
-    "pkv_adaptive_topk": (_i, [_vp, _i64, _vp, _i64, _i64, _vp, _i, C.c_float, _vp, _vp, _i64, _i64, _vp, _i64,
+    "pkv_adaptive_topk": (_i, [_vp, _i64, _vp, _i64, _i64, _vp, _i, C.c_float, _vp, _vp, _i64, _i64, _i64, _vp, _i64,
                                C.c_float, _i64, _i, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
     "pkv_uniform_k": (_i, [_vp, _i, _vp, _vp, _i64, _vp]),
     "pkv_dense_logits": (_i, [_vp, _i, _i, _i, _i, _vp, _i64, _i64, _i64, C.c_float, _vp, _i64, _vp]),

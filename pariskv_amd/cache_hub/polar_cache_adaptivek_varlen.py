@@ -67,8 +67,9 @@ class polar_cache(_polar_cache_base):
         dev, bs, H = self.device, self.batch_size, self.kv_head
         self._sl_vnorm_cache = [torch.zeros((bs, H, self.gpu_kv_capacity), dtype=torch.float32, device=dev)
                                 for _ in range(layer_num)]
-        self.value_norm_gpu = [torch.zeros((bs, H, self.unified_kv_capacity), dtype=torch.float32, device=dev)
-                               for _ in range(layer_num)]
+        # value norm by absolute position: the spare fp32 word of each key's rerank record, so that a candidate's
+        # norm is in the HBM line the rerank fetches anyway (the reference keeps a separate [bs,H,cap] tensor)
+        self.value_norm_gpu = [ops.record_value_norm_view(self._nib_km[l]) for l in range(layer_num)]
         cap = max(1, buffer_cap)
         self._dense_logits = torch.empty((bs, H, self.gpu_kv_capacity), dtype=torch.float32, device=dev)
         self._adaptive_k = torch.zeros((bs, H), dtype=torch.int64, device=dev)
@@ -192,7 +193,7 @@ class polar_cache(_polar_cache_base):
             self._adk_ws = torch.empty(need, dtype=torch.uint8, device=self.device)
         adaptive = dict(dense_k=kg, dense_rows=sl_end, dense_vnorm=self._sl_vnorm_cache[layer_idx],
                         dense_logits=self._dense_logits, scale=self._attn_scale, value_norm=self.value_norm_gpu[layer_idx],
-                        vn_offset=self.sink_size, threshold=self.adaptive_topk_threshold, k_out=topk_cap, k_min=k_min,
+                        vn_offset=self.sink_size, record_word_offset=ops.RECORD_VALUE_NORM_OFFSET, threshold=self.adaptive_topk_threshold, k_out=topk_cap, k_min=k_min,
                         k_max=k_max, adaptive_k=self._adaptive_k, topk_ids=self._topk_ids, row_keys=self._row_keys,
                         row_keys_base=sl_end, uniform_k=self._uniform_k, ws=self._adk_ws, src_k=self.unified_keys_cpu[layer_idx],
                         src_v=self.unified_values_cpu[layer_idx], dst_k=self._topk_k, dst_v=self._topk_v)

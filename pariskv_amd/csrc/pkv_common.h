@@ -81,7 +81,8 @@ PKV_INTERNAL int pkv_launch_select_rerank(const uint8_t *cnt_u8, int64_t cnt_str
                                           const uint8_t *nib, int64_t ns_b, int64_t ns_h, int64_t ns_key,
                                           const uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key,
                                           const float *qhat, const float *qnorm, const float *centers, int64_t *cand,
-                                          float *scores, hipStream_t s);
+                                          float *scores, hipStream_t s, int64_t extra_off = 0,
+                                          float *extra_out = nullptr);
 PKV_INTERNAL int pkv_launch_rerank(const int64_t *cand, int bs, int n_kv_heads, int64_t n_cand, int64_t n_keys,
                                    const uint8_t *nib, int64_t ns_b, int64_t ns_h, int64_t ns_key, int64_t ns_sub,
                                    const uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key,

@@ -13,7 +13,7 @@ PKV_INTERNAL int pkv_launch_identity_fill(int64_t *out, int64_t len, int64_t k, 
 namespace {
 
 struct WsLayout {
-  size_t qhat, qnorm, lut, cnt, hist, rowsuf, cand, scores, topk, topk_bytes, total;
+  size_t qhat, qnorm, lut, cnt, hist, rowsuf, cand, scores, cand_extra, topk, topk_bytes, total;
   int64_t cnt_stride;
   int chunk_keys;
   int64_t n_chunks;
@@ -38,6 +38,7 @@ WsLayout layout(int rows, int64_t n_keys, int64_t n_cand, int64_t k) {
   w.rowsuf = take((size_t)rows * 128 * sizeof(uint32_t));
   w.cand = take((size_t)rows * (size_t)n_cand * sizeof(int64_t));
   w.scores = take((size_t)rows * (size_t)n_cand * sizeof(float));
+  w.cand_extra = take((size_t)rows * (size_t)n_cand * sizeof(float));  // record word passed through per candidate
   w.topk_bytes = pkv_topk_ws_bytes_impl(rows, n_cand, k);  // lists of the multi-workgroup top-k (wide rows only)
   w.topk = take(w.topk_bytes);
   w.total = off;
@@ -77,6 +78,8 @@ extern "C" int pkv_retrieve_ws_view(void *ws, int rows, int64_t n_keys, int64_t 
     *ptr = base + w.cand, *bytes = (size_t)rows * (size_t)n_cand * 8;
   } else if (!strcmp(name, "scores")) {
     *ptr = base + w.scores, *bytes = (size_t)rows * (size_t)n_cand * 4;
+  } else if (!strcmp(name, "cand_record_word")) {
+    *ptr = base + w.cand_extra, *bytes = (size_t)rows * (size_t)n_cand * 4;
   } else {
     pkv_set_error("unknown workspace segment '%s'", name);
     return PKV_EINVAL;
@@ -147,7 +150,8 @@ extern "C" int pkv_retrieve(const pkv_retrieve_args *a, void *ws, size_t ws_byte
     if (rc) return rc;
     rc = pkv_launch_select_rerank(cnt, w.cnt_stride, rowsuf, hist, w.chunk_keys, a->bs, H, a->n_keys, a->n_cand, nib,
                                   (int64_t)H * a->cap * nk, a->cap * nk, nk, weight, (int64_t)H * a->cap * wk, a->cap * wk,
-                                  wk, qhat, qnorm, a->centers, cand, scores, s);
+                                  wk, qhat, qnorm, a->centers, cand, scores, s, a->record_word_offset,
+                                  a->record_word_offset > 0 ? (float *)(base + w.cand_extra) : nullptr);
   }
   if (rc) return rc;
   if (!a->out_ids) return PKV_OK;  // candidates only: the caller reads them out of the workspace
@@ -197,13 +201,17 @@ extern "C" int pkv_adaptive_decode_step(const pkv_retrieve_args *retrieve, void 
   const WsLayout w = layout(rows, retrieve->n_keys, retrieve->n_cand, retrieve->k);
   const int64_t *cand = (const int64_t *)((char *)ws + w.cand);
   const float *scores = (const float *)((char *)ws + w.scores);
+  // the candidates' value norms came out of the rerank with the scores when the caller keeps them in the key
+  // records (not on the all-keys-are-candidates path, which reranks without the fused kernel)
+  const bool norms_emitted = retrieve->record_word_offset > 0 && retrieve->n_cand != retrieve->n_keys;
+  const float *cand_vnorm = norms_emitted ? (const float *)((char *)ws + w.cand_extra) : nullptr;
   rc = pkv_dense_logits(retrieve->q, retrieve->dtype, retrieve->bs, retrieve->n_kv_heads, retrieve->group, ad->dense_k,
                         ad->dense_stride_b, ad->dense_stride_h, ad->dense_rows, ad->scale, ad->dense_logits,
                         ad->dense_logits_stride, stream);
   if (rc) return rc;
   rc = pkv_adaptive_topk(ad->dense_logits, ad->dense_logits_stride, ad->dense_vnorm, ad->dense_vnorm_stride,
-                         ad->dense_rows, scores, PKV_DTYPE_F32, ad->scale, nullptr, ad->value_norm, ad->vn_stride,
-                         ad->vn_offset, cand, retrieve->n_cand, ad->threshold, ad->k_out, rows, ad->adaptive_k,
+                         ad->dense_rows, scores, PKV_DTYPE_F32, ad->scale, cand_vnorm, ad->value_norm, ad->vn_stride,
+                         ad->vn_offset, ad->vn_pos_stride, cand, retrieve->n_cand, ad->threshold, ad->k_out, rows, ad->adaptive_k,
                          ad->topk_ids, ad->k_min, ad->k_max, ad->row_keys, ad->row_keys_base, ad->ws, ad->ws_bytes, stream);
   if (rc) return rc;
   if (ad->uniform_k) {

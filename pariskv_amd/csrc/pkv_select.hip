@@ -159,12 +159,15 @@ __global__ __launch_bounds__(kSelThreads) void pkv_select_kernel(const uint8_t *
 // candidates of its chunk as above, parks them in LDS and scores them right away, so the candidate
 // list is never re-read and one launch disappears from the decode step.
 // out/scores: [rows][k]; position p of a row holds the candidate's key index and its score.
+// extra_out (optional, [rows][k]): the fp32 word at byte extra_off of the candidate's record, e.g. the value
+// norm the adaptive-k stage weighs it with.
 __global__ __launch_bounds__(kSelThreads) void pkv_select_rerank_kernel(
     const uint8_t *__restrict__ cnt, int64_t cnt_stride, const uint32_t *__restrict__ row_suf,
     const uint16_t *__restrict__ chunk_suf, int chunk_keys, int n_kv_heads, int64_t n_keys, int64_t k,
     const uint8_t *__restrict__ nib, int64_t ns_b, int64_t ns_h, int ns_key, const uint16_t *__restrict__ weight,
     int64_t ws_b, int64_t ws_h, int ws_key, const float *__restrict__ qhat, const float *__restrict__ qnorm,
-    const float *__restrict__ centers, int64_t *__restrict__ out, float *__restrict__ scores) {
+    const float *__restrict__ centers, int64_t *__restrict__ out, float *__restrict__ scores, int extra_off,
+    float *__restrict__ extra_out) {
   const int row = blockIdx.y;
   const int chunk = blockIdx.x;
   const int tid = threadIdx.x;
@@ -234,6 +237,8 @@ __global__ __launch_bounds__(kSelThreads) void pkv_select_rerank_kernel(
         const int64_t key = blk0 + s_list_key[j];
         orow[pos] = key;
         srow[pos] = pkv_rerank_keymajor(s_prod, (const pkv_u32x4 *)(nrow + key * ns_key), (const pkv_u32x4 *)(wrow + key * ws_key), qn);
+        // one more fp32 word of the key's record (same HBM line), passed through for the caller
+        if (extra_out) extra_out[(int64_t)row * k + pos] = *(const float *)(nrow + key * ns_key + extra_off);
       }
     }
     __syncthreads();  // the list is rewritten by the next iteration
@@ -1058,7 +1063,7 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adaptive_topk_kernel(
     const float *__restrict__ sl_logits, int64_t sl_stride, const float *__restrict__ sl_vnorm, int64_t slv_stride,
     int64_t sl, const void *__restrict__ cand_scores, int cand_dtype, float cand_scale,
     const float *__restrict__ cand_vnorm, const float *__restrict__ value_norm, int64_t vn_stride, int64_t vn_offset,
-    const int64_t *__restrict__ cand_ids, int n_cand, float threshold, int64_t k_out, int P,
+    int64_t vn_pos_stride, const int64_t *__restrict__ cand_ids, int n_cand, float threshold, int64_t k_out, int P,
     int64_t *__restrict__ adaptive_k, int64_t *__restrict__ topk_ids, AdkClamp cl) {
   extern __shared__ uint64_t s_keys[];
   __shared__ float s_part[16];
@@ -1075,7 +1080,7 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adaptive_topk_kernel(
   for (int e = 0; e < EIN; ++e) {
     const int i = tid + e * kTopkThreads, ii = i < n_cand ? i : n_cand - 1;  // clamped: the loads carry no branch
     const float lg = cand_logit(r.cs, cand_dtype, cand_scale, ii);
-    const float vv = r.cv ? r.cv[ii] : r.vn[vn_index(r.ci[ii] + vn_offset, vn_stride)];
+    const float vv = r.cv ? r.cv[ii] : r.vn[vn_index(r.ci[ii] + vn_offset, vn_stride / vn_pos_stride) * vn_pos_stride];
     logit[e] = i < n_cand ? lg : -__uint_as_float(0x7f800000u);
     vnorm[e] = i < n_cand ? vv : 0.f;
   }
@@ -1135,7 +1140,8 @@ constexpr int kAdkPartThreads = 256;
 __global__ __launch_bounds__(kAdkPartThreads) void pkv_adk_max_gather_kernel(
     const float *__restrict__ sl_logits, int64_t sl_stride, int64_t sl, const void *__restrict__ cand_scores,
     int cand_dtype, float cand_scale, const float *__restrict__ value_norm, int64_t vn_stride, int64_t vn_offset,
-    const int64_t *__restrict__ cand_ids, int64_t n_cand, float *__restrict__ ws_max, float *__restrict__ ws_vn,
+    int64_t vn_pos_stride, const int64_t *__restrict__ cand_ids, int64_t n_cand, float *__restrict__ ws_max,
+    float *__restrict__ ws_vn,
     uint32_t *__restrict__ ctl) {
   __shared__ float s_part[kAdkPartThreads / PKV_WAVE];
   const int row = blockIdx.y, part = blockIdx.x, tid = threadIdx.x;
@@ -1148,7 +1154,7 @@ __global__ __launch_bounds__(kAdkPartThreads) void pkv_adk_max_gather_kernel(
 #pragma unroll
     for (int e = 0; e < E; ++e) {
       const int64_t i = (int64_t)part * kAdkPart + e * kAdkPartThreads + tid;
-      vv[e] = vn[vn_index(ci[i < n_cand ? i : n_cand - 1] + vn_offset, vn_stride)];
+      vv[e] = vn[vn_index(ci[i < n_cand ? i : n_cand - 1] + vn_offset, vn_stride / vn_pos_stride) * vn_pos_stride];
     }
 #pragma unroll
     for (int e = 0; e < E; ++e) {
@@ -1355,7 +1361,10 @@ int pkv_launch_select_rerank(const uint8_t *cnt_u8, int64_t cnt_stride, const ui
                              int n_kv_heads, int64_t n_keys, int64_t k, const uint8_t *nib, int64_t ns_b, int64_t ns_h,
                              int64_t ns_key, const uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key,
                              const float *qhat, const float *qnorm, const float *centers, int64_t *cand, float *scores,
-                             hipStream_t s) {
+                             hipStream_t s, int64_t extra_off, float *extra_out) {
+  PKV_REQUIRE(!extra_out || (extra_off >= 0 && extra_off % 4 == 0 && extra_off + 4 <= ns_key),
+              "the extra word must lie inside the key's record (offset %lld, record %lld bytes)", (long long)extra_off,
+              (long long)ns_key);
   PKV_REQUIRE(k >= 1 && k < n_keys && k < ((int64_t)1 << 31), "select needs 1 <= k < n_keys (k=%lld n=%lld)", (long long)k,
               (long long)n_keys);
   PKV_REQUIRE(cnt_stride % 16 == 0 && cnt_stride >= n_keys && pkv_aligned(cnt_u8, 16),
@@ -1369,7 +1378,7 @@ int pkv_launch_select_rerank(const uint8_t *cnt_u8, int64_t cnt_stride, const ui
   hipLaunchKernelGGL(pkv_select_rerank_kernel, grid, dim3(kSelThreads), 0, s, cnt_u8, cnt_stride, row_suf, chunk_suf,
                      chunk_keys,
                      n_kv_heads, n_keys, k, nib, ns_b, ns_h, (int)ns_key, weight, ws_b, ws_h, (int)ws_key, qhat, qnorm,
-                     centers, cand, scores);
+                     centers, cand, scores, (int)extra_off, extra_out);
   PKV_LAUNCH_CHECK("pkv_select_rerank_kernel");
   return PKV_OK;
 }
@@ -1550,7 +1559,8 @@ extern "C" size_t pkv_adaptive_topk_ws_bytes(int rows, int64_t n_cand, int64_t k
 extern "C" int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, const float *sl_vnorm, int64_t slv_stride,
                                  int64_t sl, const void *cand_scores, int cand_dtype, float cand_scale,
                                  const float *cand_vnorm, const float *value_norm, int64_t vn_stride, int64_t vn_offset,
-                                 const int64_t *cand_ids, int64_t n_cand, float threshold, int64_t k_out, int rows,
+                                 int64_t vn_pos_stride, const int64_t *cand_ids, int64_t n_cand, float threshold,
+                                 int64_t k_out, int rows,
                                  int64_t *adaptive_k, int64_t *topk_ids, int64_t k_min, int64_t k_max,
                                  int32_t *row_keys, int64_t row_keys_base, void *ws, size_t ws_bytes, void *stream) {
   PKV_REQUIRE(k_max <= 0 || (k_min >= 0 && k_min <= k_max), "pkv_adaptive_topk: clamp [%lld, %lld] is empty",
@@ -1559,7 +1569,9 @@ extern "C" int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, cons
   PKV_REQUIRE(cand_scores && cand_ids && adaptive_k && topk_ids && (cand_vnorm || value_norm),
               "pkv_adaptive_topk: null pointer");
   PKV_REQUIRE(sl >= 0 && (sl == 0 || (sl_logits && sl_vnorm)), "pkv_adaptive_topk: dense logits missing");
-  PKV_REQUIRE(cand_vnorm || vn_stride > 0, "pkv_adaptive_topk: value_norm needs its row length (vn_stride)");
+  if (vn_pos_stride <= 0) vn_pos_stride = 1;
+  PKV_REQUIRE(cand_vnorm || (vn_stride > 0 && vn_stride % vn_pos_stride == 0),
+              "pkv_adaptive_topk: value_norm needs its row stride (vn_stride), a multiple of the position stride");
   PKV_REQUIRE(cand_dtype == PKV_DTYPE_F32 || cand_dtype == PKV_DTYPE_BF16, "unknown candidate score dtype %d", cand_dtype);
   PKV_REQUIRE(rows > 0 && rows <= 65535 && n_cand > 0 && n_cand < ((int64_t)1 << 31) && k_out > 0 && k_out <= n_cand,
               "need 0 < k_out <= n_cand (k_out=%lld n_cand=%lld rows=%d)", (long long)k_out, (long long)n_cand, rows);
@@ -1571,8 +1583,8 @@ extern "C" int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, cons
 #define PKV_ADK(EIN)                                                                                                  \
   hipLaunchKernelGGL((pkv_adaptive_topk_kernel<EIN>), dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes(P), s,      \
                      sl_logits, sl_stride, sl_vnorm, slv_stride, sl, cand_scores, cand_dtype, cand_scale, cand_vnorm, \
-                     value_norm, vn_stride, vn_offset, cand_ids, (int)n_cand, threshold, k_out, P, adaptive_k, topk_ids, \
-                     cl)
+                     value_norm, vn_stride, vn_offset, vn_pos_stride, cand_ids, (int)n_cand, threshold, k_out, P,     \
+                     adaptive_k, topk_ids, cl)
     if (ein <= 1) PKV_ADK(1); else if (ein == 2) PKV_ADK(2); else if (ein == 4) PKV_ADK(4); else PKV_ADK(8);
 #undef PKV_ADK
     PKV_LAUNCH_CHECK("pkv_adaptive_topk_kernel");
@@ -1593,7 +1605,7 @@ extern "C" int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, cons
   const dim3 grid((unsigned)n_slices, (unsigned)rows);
   hipLaunchKernelGGL(pkv_adk_max_gather_kernel, dim3((unsigned)n_parts, (unsigned)rows), dim3(kAdkPartThreads), 0, s,
                      sl_logits, sl_stride, sl, cand_scores, cand_dtype, cand_scale, cand_vnorm ? nullptr : value_norm,
-                     vn_stride, vn_offset, cand_ids, n_cand, smax, gathered, ctl);
+                     vn_stride, vn_offset, vn_pos_stride, cand_ids, n_cand, smax, gathered, ctl);
   PKV_LAUNCH_CHECK("pkv_adk_max_gather_kernel");
   hipLaunchKernelGGL(pkv_adk_benefit_kernel, grid, dim3(kTopkThreads), 0, s, cand_scores, cand_dtype, cand_scale,
                      cand_vnorm ? cand_vnorm : gathered, n_cand, smax, n_parts, ben, ssum, ctl);

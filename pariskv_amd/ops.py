@@ -20,6 +20,7 @@ from . import _lib
 
 B_SUB, M_SUB, K_CLUSTERS, HEAD_DIM = 16, 8, 256, 128
 RERANK_RECORD_BYTES = 128  # one key's 64 nibble bytes + 16 bf16 weights, padded to an HBM line
+RECORD_VALUE_NORM_OFFSET = 96  # spare bytes of the record: one fp32 word for the adaptive-k caches
 TIER_RATIOS = (0.05, 0.15, 0.30, 0.50, 0.75, 1.0)  # cache_hub/polar_cache.py:1221
 # cache_hub/polar_cache.py:188-193 rounded to bf16
 MAG_THRESHOLDS = (0.08447265625, 0.169921875, 0.2578125, 0.349609375, 0.44921875, 0.55859375, 0.69140625)
@@ -96,6 +97,17 @@ def alloc_keymajor(bs: int, heads: int, cap: int, device):
     w = rec[..., B_SUB * 4:B_SUB * 4 + B_SUB * 2].view(torch.bfloat16)
     return (codes, nib, w, codes.permute(0, 1, 3, 2), nib.view(bs, heads, cap, B_SUB, 4).permute(0, 1, 3, 2, 4),
             w.permute(0, 1, 3, 2))
+
+
+def record_value_norm_view(nib_km: torch.Tensor) -> torch.Tensor:
+    """fp32 [bs,H,cap] view of the word at byte 96 of every key's record, given the record's nibble view from
+    :func:`alloc_keymajor`.  The adaptive-k caches keep ``value_norm_gpu`` there: the fused select+rerank then
+    passes a candidate's value norm through with the HBM line it reads anyway."""
+    bs, H, cap, _ = nib_km.shape
+    _need(nib_km.dtype == torch.uint8 and nib_km.stride(2) == RERANK_RECORD_BYTES and nib_km.stride(3) == 1,
+          "expected the nibble view of 128-byte key records")
+    rec = nib_km.as_strided((bs, H, cap, RERANK_RECORD_BYTES), nib_km.stride(), nib_km.storage_offset())
+    return rec[..., RECORD_VALUE_NORM_OFFSET:RECORD_VALUE_NORM_OFFSET + 4].view(torch.float32).squeeze(-1)
 
 
 # ------------------------------------------------------------------- append
@@ -347,11 +359,14 @@ def adaptive_topk(sl_logits: torch.Tensor, sl_vnorm: torch.Tensor, cand_scores: 
     if cand_vnorm is not None:
         _need(cand_vnorm.dtype == torch.float32 and cand_vnorm.is_contiguous() and tuple(cand_vnorm.shape) == (bs, H, Cn),
               "cand_vnorm must be contiguous fp32 [bs,H,C]")
-        vn_stride = 0
+        vn_stride = vn_pos = 0
     else:
-        _need(value_norm is not None and value_norm.dtype == torch.float32 and value_norm.is_contiguous() and
-              tuple(value_norm.shape[:2]) == (bs, H), "value_norm must be contiguous fp32 [bs,H,cap]")
-        vn_stride = value_norm.shape[2]
+        _need(value_norm is not None and value_norm.dtype == torch.float32 and value_norm.dim() == 3 and
+              tuple(value_norm.shape[:2]) == (bs, H) and value_norm.stride(2) >= 1 and
+              value_norm.stride(1) == value_norm.shape[2] * value_norm.stride(2) and
+              (bs == 1 or value_norm.stride(0) == H * value_norm.stride(1)),
+              "value_norm must be fp32 [bs,H,cap] with one uniform position stride")
+        vn_stride, vn_pos = value_norm.stride(1), value_norm.stride(2)
     dev = cand_scores.device
     ak = torch.empty(bs, H, dtype=torch.int64, device=dev)
     ids = torch.empty(bs, H, k_out, dtype=torch.int64, device=dev)
@@ -361,7 +376,8 @@ def adaptive_topk(sl_logits: torch.Tensor, sl_vnorm: torch.Tensor, cand_scores: 
     row_stride = lambda t: t.stride(1) if H > 1 else (t.stride(0) if bs > 1 else max(1, sl))
     _lib.check(_lib.lib().pkv_adaptive_topk(
         _p(sl_logits), row_stride(sl_logits), _p(sl_vnorm), row_stride(sl_vnorm), sl, _p(cand_scores),
-        _dt(cand_scores.dtype), float(cand_scale), _p(cand_vnorm), _p(value_norm), vn_stride, vn_offset, _p(cand_ids), Cn,
+        _dt(cand_scores.dtype), float(cand_scale), _p(cand_vnorm), _p(value_norm), vn_stride, vn_offset, vn_pos,
+        _p(cand_ids), Cn,
         float(threshold), k_out, rows, _p(ak), _p(ids), int(k_min), int(k_max), _p(row_keys),
         int(row_keys_base or 0), _p(ws), nbytes, _stream(cand_scores)))
     return (ak, ids) if row_keys is None else (ak, ids, row_keys)
@@ -745,7 +761,7 @@ class RetrievePlan:
         return cand, scores
 
     def _fill(self, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, k,
-              out_ids, out_scores, gather, candidates_only, any_order=False):
+              out_ids, out_scores, gather, candidates_only, any_order=False, record_word_offset=0):
         """Validate one retrieval's operands and return its C argument block."""
         lib = _lib.lib()
         need = lib.pkv_retrieve_ws_bytes(self.rows, n_keys, n_cand, k)
@@ -764,6 +780,9 @@ class RetrievePlan:
                   t.stride(0) == self.H * t.stride(1), "key-major nibbles / weights: [bs,H,cap,*] rows at one uniform key stride")
         a.codes, a.nib, a.weight = codes_km.data_ptr(), nib_km.data_ptr(), w_km.data_ptr()
         a.nib_key_stride, a.weight_key_stride = nib_km.stride(2), w_km.stride(2) * w_km.element_size()
+        _need(record_word_offset == 0 or (record_word_offset % 4 == 0 and 64 <= record_word_offset <= nib_km.stride(2) - 4),
+              "record_word_offset must name a 4-byte word of the key record outside its nibbles")
+        a.record_word_offset = int(record_word_offset)
         a.cap, a.key0, a.n_keys = self.cap, key0, n_keys
         for i, t in enumerate(tier_counts):
             a.tier_counts[i] = int(t)
@@ -814,14 +833,15 @@ class RetrievePlan:
                       n_cand, adaptive: dict, att, segments):
         """The adaptive-k step of one layer as a :class:`BoundAdaptiveStep`.  ``adaptive``: dense_k [bs,H,rows,128],
         dense_rows, dense_vnorm fp32 [bs,H,rows], dense_logits fp32 [bs,H,>=rows] scratch, scale, value_norm fp32
-        [bs,H,cap], vn_offset, threshold, k_out, k_min, k_max, adaptive_k int64 [bs,H], topk_ids int64 (>= bs*H*k_out
+        [bs,H,cap] (packed, or the :func:`record_value_norm_view` with ``record_word_offset`` = its byte offset: the
+        rerank then hands the candidates' norms over and no second gather runs), vn_offset, threshold, k_out, k_min, k_max, adaptive_k int64 [bs,H], topk_ids int64 (>= bs*H*k_out
         elements), row_keys int32 [bs,H], row_keys_base, optional uniform_k int64 [bs,H] (then every row gathers and
         attends to max(adaptive_k) ids), ws uint8 (pkv_adaptive_topk_ws_bytes), src_k / src_v pinned
         CPU [bs,H,len,128], dst_k / dst_v GPU [bs,H,>=k_out,128].  ``segments`` are the attention's; its per-row key
         count is ``row_keys``."""
-        a = self._fill(queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, 1,
-                       None, None, None, True)
         d = adaptive
+        a = self._fill(queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, 1,
+                       None, None, None, True, record_word_offset=int(d.get("record_word_offset", 0)))
         bs, H = self.bs, self.H
         dk, dvn, dl, vn = d["dense_k"], d["dense_vnorm"], d["dense_logits"], d["value_norm"]
         ak, ids, rk, ws = d["adaptive_k"], d["topk_ids"], d["row_keys"], d["ws"]
@@ -830,9 +850,16 @@ class RetrievePlan:
         _cuda(dk, dvn, dl, vn, ak, ids, rk, ws, tk, tv)
         _need(dk.dtype == queries.dtype and tuple(dk.shape[:2]) == (bs, H) and dk.shape[3] == HEAD_DIM and
               dk.stride(3) == 1 and dk.stride(2) == HEAD_DIM, "dense_k: [bs,H,rows,128] with contiguous rows")
-        for t in (dvn, dl, vn):
+        for t in (dvn, dl):
             _need(t.dtype == torch.float32 and t.is_contiguous() and tuple(t.shape[:2]) == (bs, H),
-                  "dense_vnorm / dense_logits / value_norm: contiguous fp32 [bs,H,*]")
+                  "dense_vnorm / dense_logits: contiguous fp32 [bs,H,*]")
+        _need(vn.dtype == torch.float32 and vn.dim() == 3 and tuple(vn.shape[:2]) == (bs, H) and vn.stride(2) >= 1 and
+              vn.stride(1) == vn.shape[2] * vn.stride(2) and (bs == 1 or vn.stride(0) == H * vn.stride(1)),
+              "value_norm: fp32 [bs,H,cap] with one uniform position stride")
+        if d.get("record_word_offset", 0):  # the norms the rerank passes through must be the ones value_norm names
+            _need(vn.data_ptr() == nib_km.data_ptr() + int(d["record_word_offset"]) and
+                  vn.stride(2) * 4 == nib_km.stride(2) and int(d["vn_offset"]) == key0,
+                  "record_word_offset: value_norm must be the view of that word of the key records")
         _need(0 < int(d["dense_rows"]) <= min(dl.shape[2], dvn.shape[2], dk.shape[2]),
               "dense_rows exceeds dense_k / dense_logits / dense_vnorm")
         _need(0 < k_out <= n_cand, "k_out must be in (0, n_cand]")
@@ -850,7 +877,8 @@ class RetrievePlan:
         ad.dense_k, ad.dense_stride_b, ad.dense_stride_h, ad.dense_rows = dk.data_ptr(), dk.stride(0), dk.stride(1), int(d["dense_rows"])
         ad.dense_vnorm, ad.dense_vnorm_stride = dvn.data_ptr(), dvn.shape[2]
         ad.dense_logits, ad.dense_logits_stride = dl.data_ptr(), dl.shape[2]
-        ad.scale, ad.value_norm, ad.vn_stride, ad.vn_offset = float(d["scale"]), vn.data_ptr(), vn.shape[2], int(d["vn_offset"])
+        ad.scale, ad.value_norm, ad.vn_stride, ad.vn_offset = float(d["scale"]), vn.data_ptr(), vn.stride(1), int(d["vn_offset"])
+        ad.vn_pos_stride = vn.stride(2)
         ad.threshold, ad.k_out, ad.k_min, ad.k_max = float(d["threshold"]), k_out, int(d["k_min"]), int(d["k_max"])
         ad.adaptive_k, ad.topk_ids, ad.row_keys, ad.row_keys_base = ak.data_ptr(), ids.data_ptr(), rk.data_ptr(), int(d["row_keys_base"])
         uk = d.get("uniform_k")

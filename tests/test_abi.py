@@ -64,7 +64,7 @@ def test_host_side_argument_errors_without_gpu():
     assert L.pkv_adaptive_decode_step(a, None, 0, ad, aa, None) == _lib.EINVAL
     assert b"candidates-only" in L.pkv_last_error()
     assert L.pkv_dense_logits(None, 1, 1, 1, 1, None, 0, 0, 1, 1.0, None, 1, None) == _lib.EINVAL
-    assert L.pkv_adaptive_topk(None, 0, None, 0, 0, None, 0, 1.0, None, None, 0, 0, None, 10, 0.9, 5, 1, None, None,
+    assert L.pkv_adaptive_topk(None, 0, None, 0, 0, None, 0, 1.0, None, None, 0, 0, 0, None, 10, 0.9, 5, 1, None, None,
                                6, 5, None, 0, None, 0, None) == _lib.EINVAL
     assert b"clamp" in L.pkv_last_error()
 

@@ -286,6 +286,65 @@ def test_adaptive_k_cache_decode_loop(dtype):
     assert len(seen_k) >= 3, f"k should vary across rows and steps, saw {sorted(seen_k)}"
 
 
+def test_adaptive_k_cache_with_more_than_8192_candidates():
+    """The fused adaptive step where a row has more candidates than one workgroup holds (multi-workgroup adaptive-k
+    kernels, value norms handed over by the rerank): 170 K-token prompt, 8.5 K candidates per row; k and the selected
+    set against the CPU oracle on the cache's own index."""
+    from pariskv_amd.cache_hub.polar_cache_adaptivek_varlen import polar_cache as adaptive_cache
+
+    bs, Hkv, Hq, S, steps = 1, 2, 8, 170_000, 3
+    sink, local, thr = 4, 64, 0.7
+    G = Hq // Hkv
+    cache = adaptive_cache(valid_start=[0] * bs, layer_num=1, batch_size=bs, max_length=S + steps + 10,
+                           num_key_value_heads=Hkv, num_heads=Hq, head_dim=128, dtype=torch.bfloat16, layer_mapping={0: DEV},
+                           max_new_length=steps + 10, sink_size=sink, local_size=local, core=1, nprobe=1, cache_unit_size=1,
+                           cache_cluster_num=1, num_gpus=1, model_size=7, final_topk=100, dynamic_update_interval=16,
+                           full_attention_threshold=100, enable_offload=True, adaptive_topk_threshold=thr)
+    gen = torch.Generator().manual_seed(11)
+    hk, hv = _synth_kv(gen, bs, S, Hkv)
+    hv = hv * (0.25 + 2.0 * torch.rand(bs, S, Hkv, 1, generator=gen)).to(torch.bfloat16)
+    cache.prefill_update_kv_cache(None, hk.to(DEV), hv.to(DEV), 0, 0)
+    signs = O.srht_signs(42)
+    scale = 1.0 / math.sqrt(128)
+    for step in range(steps):
+        k1, v1 = _synth_kv(gen, bs, 1, Hkv)
+        q = (hk[:, -3:].float().mean(dim=1).repeat_interleave(G, dim=1) * 0.3
+             + 0.5 * torch.randn(bs, Hq, 128, generator=gen)).to(torch.bfloat16).view(bs, 1, Hq, 128)
+        hk, hv = torch.cat([hk, k1], dim=1), torch.cat([hv, v1], dim=1)
+        cache.decode_update_kv_cache(k1.to(DEV), v1.to(DEV), 0)
+        out = cache.compute(q.to(DEV), 0)
+    torch.cuda.synchronize()
+    total = S + steps
+    z = cache._zones[0]
+    n_keys, n_cand, _, tiers = cache.retrieval_shape(0)
+    assert n_cand > 8192 and n_keys == z.encoded
+    sl_end = z.gpu_prefix_rows
+    dense_keys = cache.unified_keys_gpu[0][:, :, :sl_end].float().cpu().numpy()
+    sl_vnorm = cache._sl_vnorm_cache[0][:, :, :sl_end].cpu().numpy()
+    value_norm = cache.value_norm_gpu[0].cpu().numpy()
+    codes, nib = cache._codes_km[0].cpu().numpy(), cache._nib_km[0].cpu().numpy()
+    w, cc = cache._w_km[0].float().cpu().numpy(), cache.cluster_key_counts_gpu[0].cpu().numpy()
+    ak = cache.last_adaptive_k.cpu().numpy()
+    cap_k = min(cache._HARDCODED_MAX_K, n_cand)
+    ids_gpu = cache._topk_ids[:bs * Hkv * cap_k].view(bs, Hkv, cap_k).cpu().numpy()
+    K, V = hk[0].permute(1, 0, 2), hv[0].permute(1, 0, 2)
+    ref = torch.empty(Hq, 128)
+    for h in range(Hkv):
+        zone = slice(sink, sink + n_keys)
+        qh, qn = O.query_prep(q[0, 0, h * G:(h + 1) * G].float().numpy(), signs, O.BF16)
+        lut = O.tier_lut(O.rank_centroids(qh, O.BF16), cc[0, h], tiers)
+        cand_ref, _ = O.select_candidates(O.collision_count(codes[0, h][zone], lut), n_cand)
+        sc = O.rerank(cand_ref, nib[0, h][zone].reshape(-1, 16, 4), w[0, h][zone], qh, qn)
+        sl_logits = O.dense_logits(q[0, 0, h * G:(h + 1) * G].float().numpy(), dense_keys[0, h], scale, O.BF16)
+        k_ref, ids_ref = O.adaptive_topk(sl_logits, sl_vnorm[0, h], sc * np.float32(scale), value_norm[0, h][cand_ref + sink],
+                                         cand_ref, thr, cap_k)
+        k_ref = min(max(k_ref, min(cache._HARDCODED_MIN_K, cap_k)), cap_k)
+        assert int(ak[0, h]) == k_ref and np.array_equal(ids_gpu[0, h], ids_ref), (h, int(ak[0, h]), k_ref)
+        sel = torch.cat([torch.arange(sink), torch.from_numpy(ids_ref[:k_ref]) + sink, torch.arange(sink + n_keys, total)])
+        ref[h * G:(h + 1) * G] = _ref_attention(q[0, 0, h * G:(h + 1) * G], K[h:h + 1, sel], V[h:h + 1, sel], G=G * 10)
+    assert (out[0, 0].float().cpu() - ref).abs().max().item() < 2e-2
+
+
 @pytest.mark.parametrize("offload", [True, False])
 def test_dense_adaptive_k_cache_decode_loop(offload):
     """Dense-form adaptive-k variant (reference polar_cache_atten_value_indices_adaptive_k.py), both storage modes:
