@@ -425,7 +425,8 @@ def dense_logits(queries: torch.Tensor, keys: torch.Tensor, n_rows: int, scale: 
 # ------------------------------------------------------------------ gathers
 
 
-def _gather(fn, src_k, src_v, idx, dst_k, dst_v, idx_offset, dst_row0):
+def _gather(fn, src_k, src_v, idx, dst_k, dst_v, idx_offset, dst_row0, row_counts=None):
+    """Shared checks and call of the gather entry points; ``row_counts`` only for the ragged one."""
     bs, H, src_len, D = src_k.shape
     _need(src_k.shape == src_v.shape and dst_k.shape == dst_v.shape, "K/V shape mismatch")
     _need(src_k.dtype == src_v.dtype == dst_k.dtype == dst_v.dtype, "K/V dtype mismatch")
@@ -436,8 +437,9 @@ def _gather(fn, src_k, src_v, idx, dst_k, dst_v, idx_offset, dst_row0):
     _need(dst_k.is_cuda and dst_v.is_cuda and tuple(dst_k.shape[:2]) == (bs, H) and dst_k.shape[3] == D, "dst shape mismatch")
     k = idx.shape[2]
     row_bytes = D * src_k.element_size()
-    _lib.check(fn(_p(src_k), _p(src_v), src_len, _p(idx), k, idx_offset, _p(dst_k), _p(dst_v), dst_k.shape[2], dst_row0,
-                  bs, H, row_bytes, _stream(dst_k)))
+    counts = () if row_counts is None else (_p(row_counts),)
+    _lib.check(fn(_p(src_k), _p(src_v), src_len, _p(idx), k, *counts, idx_offset, _p(dst_k), _p(dst_v), dst_k.shape[2],
+                  dst_row0, bs, H, row_bytes, _stream(dst_k)))
 
 
 def gather_uva(src_k, src_v, idx, dst_k, dst_v, idx_offset: int = 0, dst_row0: int = 0) -> None:
@@ -452,9 +454,7 @@ def gather_uva_ragged(src_k, src_v, idx, row_counts, dst_k, dst_v, idx_offset: i
     _need(src_k.is_cpu and src_v.is_cpu and src_k.is_pinned() and src_v.is_pinned(), "src must be pinned CPU tensors")
     _need(row_counts.is_cuda and row_counts.dtype == torch.int64 and row_counts.is_contiguous() and
           row_counts.numel() == idx.shape[0] * idx.shape[1], "row_counts: contiguous int64 [bs,H] on the GPU")
-    fn = _lib.lib().pkv_gather_uva_ragged
-    _gather(lambda sk, sv, sl, ix, k, *rest: fn(sk, sv, sl, ix, k, _p(row_counts), *rest), src_k, src_v, idx, dst_k, dst_v,
-            idx_offset, dst_row0)
+    _gather(_lib.lib().pkv_gather_uva_ragged, src_k, src_v, idx, dst_k, dst_v, idx_offset, dst_row0, row_counts=row_counts)
 
 
 def gather_hbm(src_k, src_v, idx, dst_k, dst_v, idx_offset: int = 0, dst_row0: int = 0) -> None:
