@@ -479,6 +479,27 @@ typedef struct pkv_retrieve_args {
 size_t pkv_retrieve_ws_bytes(int rows, int64_t n_keys, int64_t n_cand, int64_t k);
 int pkv_retrieve(const pkv_retrieve_args *args, void *ws, size_t ws_bytes, void *stream);
 
+/* pkv_retrieve for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc): the
+ * same launches on `stream`, same results, but the workspace is a fixed
+ * PKV_NOALLOC_SCRATCH_BYTES array inside the library's device code, one copy per
+ * GPU, held until the process ends.  The call allocates and frees nothing.
+ * No counterpart in the reference (its kernels allocate their outputs and
+ * temporaries with torch::zeros on every call).
+ *   - The GPU of `stream` must be the calling thread's current device.
+ *   - Shapes whose workspace (pkv_retrieve_ws_bytes) exceeds the array are
+ *     rejected with PKV_ENOMEM and a message naming both sizes;
+ *     pkv_retrieve_noalloc_max_bytes() returns the array's size.
+ *   - args->out_ids must be non-NULL (the candidates-only form returns its
+ *     results in the workspace, which is not the caller's here).
+ *   - All calls on one GPU share that GPU's array, which keeps the previous
+ *     call's contents; every segment that must start at zero is cleared by the
+ *     kernels themselves.  Calls that overlap in time on one GPU (two streams,
+ *     two threads) race on it: serialise them, or use pkv_retrieve. */
+#define PKV_NOALLOC_SCRATCH_BYTES (32u << 20)
+size_t pkv_retrieve_noalloc_max_bytes(void);
+int pkv_retrieve_noalloc(const pkv_retrieve_args *args, void *stream);
+
 /* The whole decode step of one layer from one host call: pkv_retrieve (with its
  * gather) followed by pkv_decode_attention over the attended set, on the same
  * stream - polar_cache.compute (cache_hub/polar_cache.py:1002-1107) after the

@@ -117,6 +117,8 @@ PROTOTYPES = {
     "pkv_silu_mul": (_i, [_vp, _i64, _i, _i, _vp, _vp]),
     "pkv_retrieve_ws_bytes": (_sz, [_i, _i64, _i64, _i64]),
     "pkv_retrieve": (_i, [C.POINTER(RetrieveArgs), _vp, _sz, _vp]),
+    "pkv_retrieve_noalloc_max_bytes": (_sz, []),
+    "pkv_retrieve_noalloc": (_i, [C.POINTER(RetrieveArgs), _vp]),
     "pkv_decode_step": (_i, [C.POINTER(RetrieveArgs), _vp, _sz, C.POINTER(AttnArgs), _vp]),
     "pkv_adaptive_decode_step": (_i, [C.POINTER(RetrieveArgs), _vp, _sz, C.POINTER(AdaptiveArgs), C.POINTER(AttnArgs), _vp]),
     "pkv_retrieve_ws_view": (_i, [_vp, _i, _i64, _i64, _i64, C.c_char_p, C.POINTER(_vp), C.POINTER(_sz)]),

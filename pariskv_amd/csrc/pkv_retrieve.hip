@@ -8,6 +8,8 @@
 // :1207-1231, :1244-1304 and the gather at :1075-1095.
 #include "pkv_common.h"
 
+#include <mutex>
+
 PKV_INTERNAL int pkv_launch_identity_fill(int64_t *out, int64_t len, int64_t k, int rows, hipStream_t s);
 
 namespace {
@@ -87,7 +89,7 @@ extern "C" int pkv_retrieve_ws_view(void *ws, int rows, int64_t n_keys, int64_t 
   return PKV_OK;
 }
 
-extern "C" int pkv_retrieve(const pkv_retrieve_args *a, void *ws, size_t ws_bytes, void *stream) {
+static int retrieve_impl(const pkv_retrieve_args *a, void *ws, size_t ws_bytes, void *stream) {
   PKV_REQUIRE(a != nullptr, "pkv_retrieve: null args");
   PKV_REQUIRE(a->q && a->signs && a->centers && a->cluster_counts && a->codes && a->nib && a->weight,
               "pkv_retrieve: null pointer");
@@ -173,6 +175,64 @@ extern "C" int pkv_retrieve(const pkv_retrieve_args *a, void *ws, size_t ws_byte
                            a->dst_row0, rows, a->row_bytes, s);
   }
   return rc;
+}
+
+extern "C" int pkv_retrieve(const pkv_retrieve_args *a, void *ws, size_t ws_bytes, void *stream) {
+  return retrieve_impl(a, ws, ws_bytes, stream);
+}
+
+// ---- the same retrieval for callers that cannot allocate: the workspace is a fixed array of the library ----
+
+// Scratch of the no-allocation entry point: the segments pkv_retrieve lays out in its caller's workspace
+// (rotated query, vote table, vote counts, chunk histograms, candidate list, scores, lists of the wide top-k).
+// One copy per GPU, held from the load of the library's code object on that GPU until the process ends.
+static __device__ __align__(256) unsigned char scratch[PKV_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices];  // per device: the address of that GPU's copy of `scratch`
+
+// Device address of the calling thread's current GPU's scratch array (looked up once per device).
+int scratch_for_current_device(void **out) {
+  int dev = -1;
+  PKV_HIP(hipGetDevice(&dev));
+  PKV_REQUIRE(dev >= 0 && dev < kMaxDevices, "device ordinal %d outside [0,%d)", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    PKV_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    PKV_REQUIRE(p != nullptr && pkv_aligned(p, 256), "the scratch array of device %d has no usable address", dev);
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return PKV_OK;
+}
+}  // namespace
+
+extern "C" size_t pkv_retrieve_noalloc_max_bytes(void) { return (size_t)PKV_NOALLOC_SCRATCH_BYTES; }
+
+extern "C" int pkv_retrieve_noalloc(const pkv_retrieve_args *a, void *stream) {
+  PKV_REQUIRE(a != nullptr, "pkv_retrieve_noalloc: null args");
+  PKV_REQUIRE(a->out_ids != nullptr,
+              "pkv_retrieve_noalloc: the candidates-only form (out_ids == NULL) leaves its results in the workspace, "
+              "which here is the library's own scratch; use pkv_retrieve");
+  const int rows = a->bs * a->n_kv_heads;
+  PKV_REQUIRE(a->bs > 0 && a->n_kv_heads > 0 && shape_ok(rows, a->n_keys, a->n_cand, a->k),
+              "need 0 < k <= n_cand <= n_keys <= 2^24 (k=%lld n_cand=%lld n_keys=%lld rows=%d)", (long long)a->k,
+              (long long)a->n_cand, (long long)a->n_keys, rows);
+  const size_t need = layout(rows, a->n_keys, a->n_cand, a->k).total;
+  if (need > (size_t)PKV_NOALLOC_SCRATCH_BYTES) {
+    pkv_set_error("pkv_retrieve_noalloc: this shape needs %zu bytes of scratch, the fixed array holds %zu "
+                  "(rows=%d n_keys=%lld n_cand=%lld k=%lld); use pkv_retrieve with a workspace of the caller's",
+                  need, (size_t)PKV_NOALLOC_SCRATCH_BYTES, rows, (long long)a->n_keys, (long long)a->n_cand,
+                  (long long)a->k);
+    return PKV_ENOMEM;
+  }
+  void *ws = nullptr;
+  const int rc = scratch_for_current_device(&ws);
+  if (rc) return rc;
+  return retrieve_impl(a, ws, (size_t)PKV_NOALLOC_SCRATCH_BYTES, stream);
 }
 
 extern "C" int pkv_decode_step(const pkv_retrieve_args *retrieve, void *ws, size_t ws_bytes,

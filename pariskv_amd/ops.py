@@ -738,6 +738,60 @@ class BoundAdaptiveStep:
         return out
 
 
+def _retrieve_args(bs, H, group, cap, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys,
+                   tier_counts, n_cand, k, out_ids, out_scores, gather, candidates_only, any_order=False,
+                   record_word_offset=0):
+    """Validate one retrieval's operands (key-major storage of ``cap`` keys per row) and return its C argument block."""
+    q = queries.reshape(bs, -1, HEAD_DIM)
+    _need(q.is_contiguous() and q.shape[1] == H * group, "queries must be contiguous [bs,1,Hq,128]")
+    a = _lib.RetrieveArgs()
+    a.q, a.dtype, a.bs, a.n_kv_heads, a.group = q.data_ptr(), _dt(q.dtype), bs, H, group
+    a.signs, a.centers, a.cluster_counts = signs.data_ptr(), centers.data_ptr(), cluster_counts.data_ptr()
+    _need(cluster_counts.is_contiguous(), "cluster_counts must be contiguous")
+    _need(codes_km.is_contiguous() and codes_km.shape[2] == cap, "codes must be contiguous [bs,H,cap,16]")
+    for t in (nib_km, w_km):  # packed, or views into a wider per-key record
+        _need(t.shape[2] == cap and t.stride(3) == 1 and t.stride(1) == cap * t.stride(2) and
+              t.stride(0) == H * t.stride(1), "key-major nibbles / weights: [bs,H,cap,*] rows at one uniform key stride")
+    a.codes, a.nib, a.weight = codes_km.data_ptr(), nib_km.data_ptr(), w_km.data_ptr()
+    a.nib_key_stride, a.weight_key_stride = nib_km.stride(2), w_km.stride(2) * w_km.element_size()
+    _need(record_word_offset == 0 or (record_word_offset % 4 == 0 and 64 <= record_word_offset <= nib_km.stride(2) - 4),
+          "record_word_offset must name a 4-byte word of the key record outside its nibbles")
+    a.record_word_offset = int(record_word_offset)
+    a.cap, a.key0, a.n_keys = cap, key0, n_keys
+    for i, t in enumerate(tier_counts):
+        a.tier_counts[i] = int(t)
+    a.n_tiers, a.n_cand, a.k = len(tier_counts), n_cand, k
+    a.out_ids = None if candidates_only else out_ids.data_ptr()
+    a.out_scores = out_scores.data_ptr() if out_scores is not None else None
+    a.any_order = int(bool(any_order))
+    if gather is not None:
+        sk, sv, dk, dv = gather["src_k"], gather["src_v"], gather["dst_k"], gather["dst_v"]
+        a.src_k, a.src_v, a.gather_from_host = sk.data_ptr(), sv.data_ptr(), int(bool(gather["from_host"]))
+        a.src_len, a.idx_offset = sk.shape[2], int(gather.get("idx_offset", 0))
+        a.dst_k, a.dst_v, a.dst_len, a.dst_row0 = dk.data_ptr(), dv.data_ptr(), dk.shape[2], int(gather.get("dst_row0", 0))
+        a.row_bytes = sk.shape[3] * sk.element_size()
+    return a
+
+
+def retrieve_noalloc(queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, k,
+                     out_ids, out_scores=None, gather=None, any_order=False):
+    """One layer's retrieval through ``pkv_retrieve_noalloc``: the call of :meth:`RetrievePlan.run` for callers that may
+    not allocate device memory.  The workspace is a fixed array inside the library (one per GPU, shared by every call
+    on that GPU: overlapping calls race), so no plan is needed; ``out_ids`` int64 [bs,H,k] (and the optional
+    ``out_scores`` / gather destinations) are the caller's.  Shapes beyond ``pkv_retrieve_noalloc_max_bytes()`` raise."""
+    bs, H, cap = codes_km.shape[0], codes_km.shape[1], codes_km.shape[2]
+    group = queries.numel() // (bs * H * HEAD_DIM)
+    _cuda(queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, out_ids, out_scores)
+    _need(out_ids.dtype == torch.int64 and out_ids.is_contiguous() and out_ids.numel() == bs * H * k,
+          "out_ids: contiguous int64 [bs,H,k]")
+    _need(out_scores is None or (out_scores.dtype == torch.float32 and out_scores.is_contiguous() and
+                                 out_scores.numel() == bs * H * k), "out_scores: contiguous float32 [bs,H,k]")
+    a = _retrieve_args(bs, H, group, cap, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys,
+                       tier_counts, n_cand, k, out_ids, out_scores, gather, False, any_order)
+    _lib.check(_lib.lib().pkv_retrieve_noalloc(C.byref(a), _stream(codes_km)))
+    return out_ids
+
+
 class RetrievePlan:
     """Persistent workspace + argument block for :func:`pkv_retrieve` on key-major storage."""
 
@@ -762,41 +816,14 @@ class RetrievePlan:
 
     def _fill(self, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, k,
               out_ids, out_scores, gather, candidates_only, any_order=False, record_word_offset=0):
-        """Validate one retrieval's operands and return its C argument block."""
-        lib = _lib.lib()
-        need = lib.pkv_retrieve_ws_bytes(self.rows, n_keys, n_cand, k)
+        """Validate one retrieval's operands and return its C argument block (the workspace grows if it must)."""
+        need = _lib.lib().pkv_retrieve_ws_bytes(self.rows, n_keys, n_cand, k)
         _need(need > 0, "need 0 < k <= n_cand <= n_keys")
         if need > self.ws.numel():
             self.ws = torch.empty(int(need), dtype=torch.uint8, device=self.device)
-        q = queries.reshape(self.bs, -1, HEAD_DIM)
-        _need(q.is_contiguous() and q.shape[1] == self.H * self.group, "queries must be contiguous [bs,1,Hq,128]")
-        a = _lib.RetrieveArgs()
-        a.q, a.dtype, a.bs, a.n_kv_heads, a.group = q.data_ptr(), _dt(q.dtype), self.bs, self.H, self.group
-        a.signs, a.centers, a.cluster_counts = signs.data_ptr(), centers.data_ptr(), cluster_counts.data_ptr()
-        _need(cluster_counts.is_contiguous(), "cluster_counts must be contiguous")
-        _need(codes_km.is_contiguous() and codes_km.shape[2] == self.cap, "codes must be contiguous [bs,H,cap,16]")
-        for t in (nib_km, w_km):  # packed, or views into a wider per-key record
-            _need(t.shape[2] == self.cap and t.stride(3) == 1 and t.stride(1) == self.cap * t.stride(2) and
-                  t.stride(0) == self.H * t.stride(1), "key-major nibbles / weights: [bs,H,cap,*] rows at one uniform key stride")
-        a.codes, a.nib, a.weight = codes_km.data_ptr(), nib_km.data_ptr(), w_km.data_ptr()
-        a.nib_key_stride, a.weight_key_stride = nib_km.stride(2), w_km.stride(2) * w_km.element_size()
-        _need(record_word_offset == 0 or (record_word_offset % 4 == 0 and 64 <= record_word_offset <= nib_km.stride(2) - 4),
-              "record_word_offset must name a 4-byte word of the key record outside its nibbles")
-        a.record_word_offset = int(record_word_offset)
-        a.cap, a.key0, a.n_keys = self.cap, key0, n_keys
-        for i, t in enumerate(tier_counts):
-            a.tier_counts[i] = int(t)
-        a.n_tiers, a.n_cand, a.k = len(tier_counts), n_cand, k
-        a.out_ids = None if candidates_only else out_ids.data_ptr()
-        a.out_scores = out_scores.data_ptr() if out_scores is not None else None
-        a.any_order = int(bool(any_order))
-        if gather is not None:
-            sk, sv, dk, dv = gather["src_k"], gather["src_v"], gather["dst_k"], gather["dst_v"]
-            a.src_k, a.src_v, a.gather_from_host = sk.data_ptr(), sv.data_ptr(), int(bool(gather["from_host"]))
-            a.src_len, a.idx_offset = sk.shape[2], int(gather.get("idx_offset", 0))
-            a.dst_k, a.dst_v, a.dst_len, a.dst_row0 = dk.data_ptr(), dv.data_ptr(), dk.shape[2], int(gather.get("dst_row0", 0))
-            a.row_bytes = sk.shape[3] * sk.element_size()
-        return a
+        return _retrieve_args(self.bs, self.H, self.group, self.cap, queries, signs, centers, cluster_counts, codes_km,
+                              nib_km, w_km, key0, n_keys, tier_counts, n_cand, k, out_ids, out_scores, gather,
+                              candidates_only, any_order, record_word_offset)
 
     def run(self, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, k,
             out_ids=None, out_scores=None, gather=None, candidates_only=False, attention=None, any_order=False):
