@@ -11,7 +11,10 @@ under ``attn_hub/polar_attn.py``.  What differs inside:
   also gathers the selected K/V rows straight behind the dense prefix, so no
   ``torch.cat`` / ``torch.gather`` of K/V happens per step;
 * zone counters are per layer (see ``zones.py``);
-* the offload copy is ordered by stream events, not a host-blocking synchronize.
+* the offload copy is ordered by stream events, not a host-blocking synchronize;
+* K/V placement is per layer: with ``host_kv_budget_bytes`` the first layers keep their retrieval-zone K/V in pinned
+  host memory up to that many bytes and the remaining layers keep theirs in HBM (the reference has one global
+  ``enable_offload``, :213-237, and fails when the host cannot pin the whole store).
 """
 from __future__ import annotations
 
@@ -59,7 +62,8 @@ class polar_cache(KV_Cache):
                  cache_cluster_num: int = 0, num_gpus: int = 1, model_size: int = 0,
                  codebook_path: Optional[str] = None, final_topk: int = 100, dynamic_update_interval: int = 512,
                  full_attention_threshold: int = 2000, enable_offload: bool = True,
-                 collision_ratio: Optional[float] = None, candidate_ratio: Optional[float] = None) -> None:
+                 collision_ratio: Optional[float] = None, candidate_ratio: Optional[float] = None,
+                 host_kv_budget_bytes=None) -> None:
         super().__init__(layer_num, batch_size, max_length, num_key_value_heads, num_heads, head_dim, dtype,
                          layer_mapping, num_gpus, model_size)
         if head_dim != ops.HEAD_DIM:
@@ -94,32 +98,58 @@ class polar_cache(KV_Cache):
         self._srht_signs = ops.srht_signs(dev, seed=42)
         self._mag_centers = ops.mag_centers(dev)
         self.unified_kv_capacity = self.input_length + self.max_new_length
-        self._zones = [LayerZones(sink_size, local_size, I, enable_offload) for _ in range(layer_num)]
 
+        # ---- K/V placement, per layer (the reference: one global switch, polar_cache.py:213-237) ----
+        # A layer either offloads its retrieval zone to pinned host memory (GPU rows: [sink | local | update buffer |
+        # gathered top-k (transient)]) or keeps every token at its absolute position in HBM.  With enable_offload and no
+        # budget every layer offloads, as in the reference.  host_kv_budget_bytes = N: layers offload, in order, while
+        # the pinned total stays within N bytes; "auto": until the host refuses to pin more.  The others stay in HBM.
+        self.cpu_kv_capacity = max(1, self.unified_kv_capacity - sink_size - local_size)
+        self.gpu_kv_capacity = sink_size + local_size + I if enable_offload else self.unified_kv_capacity
+        layer_host_bytes = 2 * bs * H * self.cpu_kv_capacity * D * torch.empty((), dtype=dtype).element_size()
+        self.unified_keys_cpu = [None] * layer_num if enable_offload else None
+        self.unified_values_cpu = [None] * layer_num if enable_offload else None
+        self.cpu_valid_end = [0] * layer_num if enable_offload else None
+        self._layer_offload = [False] * layer_num
+        self._offload_keys_buffer = [None] * layer_num
+        self._offload_values_buffer = [None] * layer_num
         if enable_offload:
-            # GPU rows: [sink | local | update buffer | gathered top-k (transient)]
-            self.gpu_kv_capacity = sink_size + local_size + I
-            rows = self.gpu_kv_capacity + final_topk
-            self.cpu_kv_capacity = max(1, self.unified_kv_capacity - sink_size - local_size)
             self._copy_stream = torch.cuda.Stream(device=dev)
             self._copy_events = [torch.cuda.Event() for _ in range(layer_num)]
             self._offload_inflight = [False] * layer_num
-            self.unified_keys_cpu = [ops.alloc_pinned((bs, H, self.cpu_kv_capacity, D), dtype)
-                                     for _ in range(layer_num)]
-            self.unified_values_cpu = [ops.alloc_pinned((bs, H, self.cpu_kv_capacity, D), dtype)
-                                       for _ in range(layer_num)]
-            self.cpu_valid_end = [0] * layer_num
-            self._offload_keys_buffer = [torch.empty((bs, H, I, D), dtype=dtype, device=dev) for _ in range(layer_num)]
-            self._offload_values_buffer = [torch.empty((bs, H, I, D), dtype=dtype, device=dev) for _ in range(layer_num)]
-        else:
-            # GPU rows: every token at its absolute position
-            self.gpu_kv_capacity = self.unified_kv_capacity
-            rows = self.unified_kv_capacity
-            self.unified_keys_cpu = None
-            self.unified_values_cpu = None
-            self.cpu_valid_end = None
-        self.unified_keys_gpu = [torch.zeros((bs, H, rows, D), dtype=dtype, device=dev) for _ in range(layer_num)]
-        self.unified_values_gpu = [torch.zeros((bs, H, rows, D), dtype=dtype, device=dev) for _ in range(layer_num)]
+            budget = host_kv_budget_bytes
+            if budget is not None and budget != "auto":
+                budget = int(budget)
+            pinned = 0
+            for l in range(layer_num):
+                if isinstance(budget, int) and pinned + layer_host_bytes > budget:
+                    break
+                try:
+                    kc = ops.alloc_pinned((bs, H, self.cpu_kv_capacity, D), dtype)
+                    vc = ops.alloc_pinned((bs, H, self.cpu_kv_capacity, D), dtype)
+                except RuntimeError:
+                    if budget is None:
+                        raise  # the reference's behaviour: the whole store must fit
+                    kc = vc = None
+                    break
+                self.unified_keys_cpu[l], self.unified_values_cpu[l] = kc, vc
+                self._layer_offload[l] = True
+                pinned += layer_host_bytes
+                self._offload_keys_buffer[l] = torch.empty((bs, H, I, D), dtype=dtype, device=dev)
+                self._offload_values_buffer[l] = torch.empty((bs, H, I, D), dtype=dtype, device=dev)
+        self._gpu_rows = [(sink_size + local_size + I + final_topk) if off else self.unified_kv_capacity
+                          for off in self._layer_offload]
+        self.unified_keys_gpu = [torch.zeros((bs, H, r, D), dtype=dtype, device=dev) for r in self._gpu_rows]
+        self.unified_values_gpu = [torch.zeros((bs, H, r, D), dtype=dtype, device=dev) for r in self._gpu_rows]
+        self._zones = [LayerZones(sink_size, local_size, I, off) for off in self._layer_offload]
+        n_host = sum(self._layer_offload)
+        esz = torch.empty((), dtype=dtype).element_size()
+        self.kv_placement = {
+            "host_layers": n_host, "hbm_layers": layer_num - n_host,
+            "host_pinned_bytes": n_host * layer_host_bytes,
+            "hbm_kv_bytes": sum(2 * bs * H * r * D * esz for r in self._gpu_rows),
+            "host_kv_budget_bytes": host_kv_budget_bytes,
+        }
 
         # index metadata, addressed by absolute position (polar_cache.py:283-312)
         self.retrieval_zone_capacity = self.unified_kv_capacity
@@ -172,7 +202,7 @@ class polar_cache(KV_Cache):
 
     def _wait_offload(self, layer_idx: int) -> None:
         """Order the current stream after the layer's last host copy (GPU-side wait, no host block)."""
-        if self.enable_offload and self._offload_inflight[layer_idx]:
+        if self._layer_offload[layer_idx] and self._offload_inflight[layer_idx]:
             torch.cuda.current_stream(self.device).wait_event(self._copy_events[layer_idx])
             self._offload_inflight[layer_idx] = False
 
@@ -227,7 +257,7 @@ class polar_cache(KV_Cache):
         kg, vg = self.unified_keys_gpu[layer_idx], self.unified_values_gpu[layer_idx]
         last = (layer_idx == self.layer_num - 1) and (b1 == self.batch_size)
         if retrieval == 0:  # short prompt: everything stays dense on the GPU (:430-440)
-            n = min(n_tok, self.gpu_kv_capacity)
+            n = min(n_tok, self._gpu_rows[layer_idx])
             kg[b0:b1, :, :n] = k[:, :, :n].to(self.dtype)
             vg[b0:b1, :, :n] = v[:, :, :n].to(self.dtype)
             self._on_prefill(layer_idx, b0, b1, v, 0, n)
@@ -235,7 +265,7 @@ class polar_cache(KV_Cache):
                 self.context += n
             return key_states[:, vs:], value_states[:, vs:]
         S0, r_end = self.sink_size, self.sink_size + retrieval
-        if self.enable_offload:
+        if self._layer_offload[layer_idx]:
             kg[b0:b1, :, :S0] = k[:, :, :S0].to(self.dtype)
             vg[b0:b1, :, :S0] = v[:, :, :S0].to(self.dtype)
             kg[b0:b1, :, S0:S0 + local_len] = k[:, :, r_end:].to(self.dtype)
@@ -281,7 +311,7 @@ class polar_cache(KV_Cache):
         bs = self.batch_size
         self._encode(layer_idx, kg[:, :, r.gpu_row0:r.gpu_row0 + n], 0, bs, r.encode_abs0)
         self._on_refresh(layer_idx, r)
-        if not self.enable_offload:
+        if not self._layer_offload[layer_idx]:
             return
         self._wait_offload(layer_idx)  # staging buffers are free again
         sk, sv = self._offload_keys_buffer[layer_idx][:, :, :n], self._offload_values_buffer[layer_idx][:, :, :n]
@@ -335,7 +365,7 @@ class polar_cache(KV_Cache):
         """Dense fallback: every stored token (reference _get_full_kv_for_attention :701-737)."""
         z = self._zones[layer_idx]
         kg, vg = self.unified_keys_gpu[layer_idx], self.unified_values_gpu[layer_idx]
-        if not self.enable_offload:
+        if not self._layer_offload[layer_idx]:
             return kg[:, :, :z.seq_len], vg[:, :, :z.seq_len]
         n = z.gpu_prefix_rows
         if z.encoded == 0:
@@ -349,7 +379,7 @@ class polar_cache(KV_Cache):
     def retrieval_shape(self, layer_idx):
         """(n_keys, n_cand, k, tier_counts) the next retrieval of this layer will use."""
         z = self._zones[layer_idx]
-        n_keys = self.cpu_valid_end[layer_idx] if self.enable_offload else z.encoded
+        n_keys = self.cpu_valid_end[layer_idx] if self._layer_offload[layer_idx] else z.encoded
         cand_ratio, coll_ratio = self._get_adaptive_ratios(n_keys)
         n_cand = min(n_keys, max(1, int(math.ceil(n_keys * cand_ratio))))        # :1239-1240
         k = min(self.final_topk, n_cand)                                          # :1300
@@ -360,7 +390,8 @@ class polar_cache(KV_Cache):
         """Decode attention for one token: [bs,1,Hq,D] -> [bs,1,Hq,D] (:1002-1107)."""
         z = self._zones[layer_idx]
         total = z.seq_len
-        n_keys = (self.cpu_valid_end[layer_idx] if self.enable_offload else z.encoded)
+        offload = self._layer_offload[layer_idx]
+        n_keys = self.cpu_valid_end[layer_idx] if offload else z.encoded
         min_total = max(self.FULL_ATTENTION_THRESHOLD, self.sink_size + self.local_size + self.final_topk * 2)
         if total < min_total or n_keys <= 0:
             k, v = self._full_kv(layer_idx)
@@ -373,7 +404,7 @@ class polar_cache(KV_Cache):
             step = self._bind_step(layer_idx, q, n_keys)
         _, bound, topk, out_ids, local_seg = step
         # what moves with every token: where the gathered rows go / how long the dense tail is
-        if self.enable_offload:
+        if offload:
             prefix = z.gpu_prefix_rows
             bound.a.dst_row0 = prefix
             bound.segs[0].n_rows = prefix + topk
@@ -391,7 +422,8 @@ class polar_cache(KV_Cache):
         n_keys, n_cand, topk, tiers = self.retrieval_shape(layer_idx)
         kg, vg = self.unified_keys_gpu[layer_idx], self.unified_values_gpu[layer_idx]
         local_seg = 0
-        if self.enable_offload:
+        offload = self._layer_offload[layer_idx]
+        if offload:
             prefix = z.gpu_prefix_rows
             gather = dict(src_k=self.unified_keys_cpu[layer_idx], src_v=self.unified_values_cpu[layer_idx], from_host=True,
                           idx_offset=0, dst_k=kg, dst_v=vg, dst_row0=prefix)
@@ -399,7 +431,7 @@ class polar_cache(KV_Cache):
         out_ids = self._out_ids[:, :, :topk]
         if not out_ids.is_contiguous():
             out_ids = torch.empty((self.batch_size, self.kv_head, topk), dtype=torch.int64, device=self.device)
-        if not self.enable_offload:
+        if not offload:
             # The reference gathers sink ++ top-k ++ local rows into a new tensor (:1089-1095).  Sink and local window
             # are always attended in place here.  The selected rows are either a segment addressed through the index
             # list the retrieval just wrote (nothing is copied, one launch fewer) or gathered into a small buffer

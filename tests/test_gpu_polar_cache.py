@@ -46,7 +46,8 @@ def _synth_kv(gen, bs, S, Hkv):
     return k.to(torch.bfloat16), v.to(torch.bfloat16)
 
 
-@pytest.mark.parametrize("offload,bs,Hkv", [(True, 2, 2), (False, 2, 2), (False, 4, 4)])  # 16 rows: selected rows attended in place
+# 16 rows: selected rows attended in place; "mixed": a host budget that holds one layer, the other stays in HBM
+@pytest.mark.parametrize("offload,bs,Hkv", [(True, 2, 2), (False, 2, 2), (False, 4, 4), ("mixed", 2, 2), ("mixed", 4, 4)])
 def test_decode_loop_matches_oracle_and_dense_reference(offload, bs, Hkv):
     from pariskv_amd.attn_hub import polar_decode_attn
 
@@ -54,7 +55,17 @@ def test_decode_loop_matches_oracle_and_dense_reference(offload, bs, Hkv):
     Hq, layers, S, steps = 4 * Hkv, 2, 3000, 70
     sink, local, I, topk = 4, 64, 32, 200
     G = Hq // Hkv
-    cache = _make_cache(offload, bs, Hkv, Hq, layers, S, steps + 10, sink, local, I, topk)
+    if offload == "mixed":
+        layer_bytes = 2 * bs * Hkv * (S + steps + 10 - sink - local) * 128 * 2
+        cache = _make_cache(True, bs, Hkv, Hq, layers, S, steps + 10, sink, local, I, topk,
+                            host_kv_budget_bytes=layer_bytes + layer_bytes // 2)
+        assert cache._layer_offload == [True, False]
+        assert cache.kv_placement["host_layers"] == 1 and cache.kv_placement["hbm_layers"] == 1
+        assert cache.kv_placement["host_pinned_bytes"] == layer_bytes
+        assert cache.unified_keys_cpu[1] is None and cache.unified_keys_gpu[1].shape[2] == S + steps + 10
+    else:
+        cache = _make_cache(offload, bs, Hkv, Hq, layers, S, steps + 10, sink, local, I, topk)
+        assert cache._layer_offload == [bool(offload)] * layers
     gen = torch.Generator().manual_seed(0)
     hist_k = [None] * layers
     hist_v = [None] * layers
