@@ -33,7 +33,63 @@ TIER_RATIOS = (0.05, 0.15, 0.30, 0.50, 0.75, 1.0)
 
 # HBM bytes moved by one collision-scan launch at this workload, from the two
 # rocprofv3 --pmc runs summarised in profiles/ (None until measured).
-SCAN_TRAFFIC_BYTES = 72834000  # profiles/scan_cfg3_hbm_traffic.md
+SCAN_TRAFFIC_BYTES = 72834000
+SCAN_TRAFFIC_SOURCE = "profiles/scan_cfg3_hbm_traffic.md"
+SCAN_KERNEL = "pkv_scan_keymajor_kernel"
+
+
+def model_decode(torch, dev, L, bs, S, T, K, warmup, offload, host_budget):
+    """BASELINE config 5: T decode tokens of a random-initialised Qwen3-8B-shaped decoder (L layers) at batch bs over a
+    synthetic S-token prompt held by polar_cache (sink 64, local 512, update buffer 1024, final_topk K); returns
+    decode tokens/s and where the K/V store was placed.  host_budget: bytes of pinned host memory the cache may use for
+    the offloaded K/V (None: all of it); layers beyond the budget keep their K/V in HBM."""
+    from pariskv_amd.cache_hub.polar_cache import polar_cache
+    from pariskv_amd.model_hub import QwenConfig, QwenModel
+
+    cfg = QwenConfig(num_layers=L)
+    H, D = cfg.num_key_value_heads, cfg.head_dim
+    cache = polar_cache(valid_start=[0] * bs, layer_num=L, batch_size=bs, max_length=S + T + 8,
+                        num_key_value_heads=H, num_heads=cfg.num_heads, head_dim=D,
+                        dtype=torch.bfloat16, layer_mapping={i: dev for i in range(L)}, max_new_length=T + 8,
+                        sink_size=64, local_size=512, core=1, nprobe=1, cache_unit_size=1, cache_cluster_num=1,
+                        num_gpus=1, model_size=8, final_topk=K, dynamic_update_interval=1024,
+                        full_attention_threshold=2000, enable_offload=offload,
+                        host_kv_budget_bytes=host_budget if offload else None)
+    g = torch.Generator(device=dev).manual_seed(0)
+    t0 = time.perf_counter()
+    # the prompt's K/V are synthetic (the prompt is not run through the model): keys ~ N(mean_t, 1) with four
+    # outlier channels and a mean that rotates by 0.5 degrees per 1K tokens in the (0, 1) plane; values ~ N(0, 1)
+    ang = torch.arange(S, device=dev, dtype=torch.float32) * (0.5 / 1000.0) * (math.pi / 180.0)
+    for l in range(L):
+        k = torch.randn(bs, S, H, D, generator=g, device=dev, dtype=torch.bfloat16)
+        k[..., 0] += ang.cos().to(torch.bfloat16)[None, :, None]
+        k[..., 1] += ang.sin().to(torch.bfloat16)[None, :, None]
+        k[..., [7, 31, 64, 101]] *= 10.0
+        v = torch.randn(bs, S, H, D, generator=g, device=dev, dtype=torch.bfloat16)
+        cache.prefill_update_kv_cache(None, k, v, l, 0)
+        del k, v
+    torch.cuda.synchronize()
+    t_prefill = time.perf_counter() - t0
+    model = QwenModel(cfg, cache, device=dev, max_positions=S + T + 8)
+    ids = torch.randint(0, cfg.vocab_size, (bs, 1), generator=g, device=dev)
+    for _ in range(warmup):
+        ids = model.decode_forward(ids).argmax(dim=-1)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(T - warmup):
+        ids = model.decode_forward(ids).argmax(dim=-1)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    n_tok = T - warmup
+    pl = cache.kv_placement
+    return {"model": "Qwen3-8B shape, random init, bf16", "layers": L, "batch": bs, "prompt": S, "generated": T,
+            "timed_tokens": n_tok, "offload": bool(offload), "final_topk": K,
+            "placement": {"host_layers": pl["host_layers"], "hbm_layers": pl["hbm_layers"],
+                          "host_pinned_GiB": round(pl["host_pinned_bytes"] / 2**30, 2),
+                          "hbm_kv_GiB": round(pl["hbm_kv_bytes"] / 2**30, 2),
+                          "host_budget_GiB": None if host_budget is None else round(host_budget / 2**30, 2)},
+            "cache_fill_s": round(t_prefill, 2), "ms_per_token": round(dt * 1e3 / n_tok, 3),
+            "decode_tokens_per_s": round(bs * n_tok / dt, 1), "us_per_layer": round(dt * 1e6 / n_tok / L, 1)}
 
 
 def main():
@@ -56,6 +112,10 @@ def main():
                          "random-initialised Qwen3-8B-shaped decoder (config 5: --layers 36 --batch 8 --context 65536 "
                          "--topk 100 --steps 256), end-to-end decode tokens/s")
     ap.add_argument("--no-offload", action="store_true", help="decode-loop: keep K/V in HBM (config 2's mode)")
+    ap.add_argument("--host-kv-budget-gib", type=float, default=56.0,
+                    help="model-decode / the default run's cfg5 leg: pinned host memory the cache may use for offloaded "
+                         "K/V; layers beyond it keep their K/V in HBM (0: no limit, every layer offloads)")
+    ap.add_argument("--no-cfg5", action="store_true", help="default run: leave out the config-5 decode leg")
     ap.add_argument("--adaptive", action="store_true", help="decode-loop: the adaptive-k cache class (config 4's mode)")
     ap.add_argument("--adaptive-k-range", type=int, nargs=2, default=[256, 2048], metavar=("MIN", "MAX"),
                     help="decode-loop --adaptive: clamp of k (config 4: 256 2048; the reference's built-in caps: 100 800)")
@@ -80,49 +140,9 @@ def main():
     lib = _lib.lib()
 
     if args.only == "model-decode":
-        from pariskv_amd.cache_hub.polar_cache import polar_cache
-        from pariskv_amd.model_hub import QwenConfig, QwenModel
-
-        S, T = N, args.steps
-        cfg = QwenConfig(num_layers=L)
-        cache = polar_cache(valid_start=[0] * bs, layer_num=L, batch_size=bs, max_length=S + T + 8,
-                            num_key_value_heads=cfg.num_key_value_heads, num_heads=cfg.num_heads, head_dim=cfg.head_dim,
-                            dtype=torch.bfloat16, layer_mapping={i: dev for i in range(L)}, max_new_length=T + 8,
-                            sink_size=64, local_size=512, core=1, nprobe=1, cache_unit_size=1, cache_cluster_num=1,
-                            num_gpus=1, model_size=8, final_topk=K, dynamic_update_interval=1024,
-                            full_attention_threshold=2000, enable_offload=not args.no_offload)
-        g = torch.Generator(device=dev).manual_seed(0)
-        t0 = time.perf_counter()
-        # the prompt's K/V are synthetic (the prompt is not run through the model): keys ~ N(mean_t, 1) with four
-        # outlier channels and a mean that rotates by 0.5 degrees per 1K tokens in the (0, 1) plane; values ~ N(0, 1)
-        ang = torch.arange(S, device=dev, dtype=torch.float32) * (0.5 / 1000.0) * (math.pi / 180.0)
-        for l in range(L):
-            k = torch.randn(bs, S, H, D, generator=g, device=dev, dtype=torch.bfloat16)
-            k[..., 0] += ang.cos().to(torch.bfloat16)[None, :, None]
-            k[..., 1] += ang.sin().to(torch.bfloat16)[None, :, None]
-            k[..., [7, 31, 64, 101]] *= 10.0
-            v = torch.randn(bs, S, H, D, generator=g, device=dev, dtype=torch.bfloat16)
-            cache.prefill_update_kv_cache(None, k, v, l, 0)
-            del k, v
-        torch.cuda.synchronize()
-        t_prefill = time.perf_counter() - t0
-        model = QwenModel(cfg, cache, device=dev, max_positions=S + T + 8)
-        ids = torch.randint(0, cfg.vocab_size, (bs, 1), generator=g, device=dev)
-        for _ in range(args.warmup):
-            ids = model.decode_forward(ids).argmax(dim=-1)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(T - args.warmup):
-            ids = model.decode_forward(ids).argmax(dim=-1)
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-        n_tok = T - args.warmup
-        print(json.dumps({"only": "model-decode", "model": "Qwen3-8B shape, random init, bf16", "layers": L, "batch": bs,
-                          "prompt": S, "generated": T, "timed_tokens": n_tok, "offload": not args.no_offload,
-                          "final_topk": K, "cache_fill_s": round(t_prefill, 2),
-                          "ms_per_token": round(dt * 1e3 / n_tok, 3),
-                          "decode_tokens_per_s": round(bs * n_tok / dt, 1),
-                          "us_per_layer": round(dt * 1e6 / n_tok / L, 1)}))
+        print(json.dumps({"only": "model-decode",
+                          **model_decode(torch, dev, L, bs, N, args.steps, K, args.warmup, not args.no_offload,
+                                         None if args.host_kv_budget_gib <= 0 else int(args.host_kv_budget_gib * 2**30))}))
         return
 
     if args.only == "decode-loop":
@@ -344,8 +364,16 @@ def main():
         if i >= args.warmup:
             scan_us.append(kus.value)
     scan_avg_us = sum(scan_us) / len(scan_us)
-    scan_bytes = R * N * (16 + 1)                     # 16 B of codes read + 1 B vote count written per key
+    scan_bytes = R * N * 16                           # algorithmic bytes of one launch: 16 B of sign codes per key
+    scan_bytes_with_counts = R * N * (16 + 1)         # ... plus the 1 B vote count it writes (an intermediate)
     achieved = scan_bytes / (scan_avg_us * 1e-6) / 1e9
+
+    # PCIe yardstick beside the gather: one plain pinned-host -> device copy of the gather's byte count
+    # (hipMemcpyAsync through the copy engines), same timing method
+    pin_src = torch.empty(R * 512 * K, dtype=torch.uint8, pin_memory=True)
+    pin_dst = torch.empty(R * 512 * K, dtype=torch.uint8, device=dev)
+    pin_dst.copy_(pin_src, non_blocking=True)
+    us_memcpy = timed(lambda i: pin_dst.copy_(pin_src, non_blocking=True), max(8, args.steps // 4))
 
     # yardstick beside the published peak: a read-only kernel with the scan's access pattern over the same arrays
     sink = torch.zeros(64, dtype=torch.int32, device=dev)
@@ -386,10 +414,18 @@ def main():
         "algorithmic_bytes": {"hbm_per_step": a_hbm, "pcie_per_step": a_pcie},
         "streaming_read_GBps_same_arrays": round(read_gbps, 1),
         "pcie_GBps_gather": round(a_pcie / (us_gather * 1e-6) / 1e9, 2),
-        "roofline": {"kernel": "pkv_scan_keymajor_kernel", "bound": "hbm", "achieved": round(achieved, 1),
+        "pcie_GBps_plain_memcpy_same_bytes": round(a_pcie / (us_memcpy * 1e-6) / 1e9, 2),
+        "roofline": {"kernel": SCAN_KERNEL, "bound": "hbm", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": SCAN_TRAFFIC_BYTES, "bytes_per_launch": scan_bytes,
-                     "avg_launch_us": round(scan_avg_us, 2)},
+                     "traffic": SCAN_TRAFFIC_BYTES,
+                     "traffic_source": "constant from " + SCAN_TRAFFIC_SOURCE + " (rocprofv3 --pmc FETCH_SIZE / "
+                                       "WRITE_SIZE of this command), not measured in this run",
+                     "bytes_per_launch": scan_bytes, "bytes_per_key": 16,
+                     "avg_launch_us": round(scan_avg_us, 2),
+                     "avg_launch_us_source": "begin/end timestamps of each dispatch (hipExtLaunchKernelGGL events); "
+                                             "the rocprofv3 --kernel-trace average in profiles/ is the cross-check",
+                     "GBps_counting_the_1B_vote_count_written": round(
+                         scan_bytes_with_counts / (scan_avg_us * 1e-6) / 1e9, 1)},
         "wall_s_timed_region": round(t_wall, 4),
     }
 
@@ -434,11 +470,62 @@ def main():
             times.append(time.perf_counter() - t0)
         times.sort()
         med = times[len(times) // 2]
+        # the same math as batched torch ops on the host (the form the reference's own torch code has), at the default
+        # intra-op thread count and at one thread (the reference pins torch.set_num_threads(1), polar_cache.py:320-326)
+        from oracle import torch_baseline as TB
+
+        tb = dict(q=ly["q"].cpu(), signs=signs.cpu(), cb=ly["codes"].permute(0, 1, 3, 2).contiguous().cpu(),
+                  k4=ly["nib"].view(bs, H, N, 16, 4).permute(0, 1, 3, 2, 4).contiguous().cpu(),
+                  kw=ly["w"].permute(0, 1, 3, 2).contiguous().cpu(), cc=ly["cc"].cpu())
+
+        def torch_layer_step():
+            return TB.retrieve_layer(tb["q"], tb["signs"], tb["cb"], tb["k4"], tb["kw"], tb["cc"], tiers, Cn, K, kcpu, vcpu)[0]
+
+        def time_torch(n_threads, budget_s):
+            torch.set_num_threads(n_threads)
+            ids = torch_layer_step()  # warm-up
+            ts = []
+            t_end = time.perf_counter() + budget_s
+            while len(ts) < 20 and (time.perf_counter() < t_end or len(ts) < 3):
+                t0 = time.perf_counter()
+                torch_layer_step()
+                ts.append(time.perf_counter() - t0)
+            ts.sort()
+            return ts[len(ts) // 2], len(ts), ids
+
+        default_threads = torch.get_num_threads()
+        t_def, n_def, tids = time_torch(default_threads, 10.0)
+        t_one, n_one, _ = time_torch(1, 12.0)
+        torch.set_num_threads(default_threads)
+        overlap = sum(len(np.intersect1d(tids.view(R, K)[r].numpy(), ref_ids[r])) for r in rows) / float(R * K)
         result["cpu_baseline"] = {"value": round(med * 1e6, 1), "unit": "us/layer/decode-step", "cores": 1, "kind": "port",
                                   "sample": f"all {R} rows of one layer at the full workload (C oracle, single thread, "
                                             f"host gather included), median of {len(times)} repetitions",
-                                  "host_cpus": os.cpu_count()}
+                                  "host_cpus": os.cpu_count(),
+                                  "torch_cpu_default_threads": {"value": round(t_def * 1e6, 1), "threads": default_threads,
+                                                                "repetitions": n_def},
+                                  "torch_cpu_one_thread": {"value": round(t_one * 1e6, 1), "threads": 1,
+                                                           "repetitions": n_one},
+                                  "torch_cpu_sample": f"the same {R} rows as batched torch ops on the reference's "
+                                                      f"subspace-major tensors (oracle/torch_baseline.py), host gather "
+                                                      f"included, median; final ids overlap with the C oracle's: "
+                                                      f"{overlap:.4f}"}
         result["parity_vs_oracle_on_bench_workload"] = bool(parity)
+
+    # ------------------------------------- config 5: end-to-end decode tokens/s
+    if not args.no_cfg5:
+        del layers, luts, kcpu, vcpu, dst_k, dst_v, cnt_ws, hist_ws, plan, gather
+        if not args.no_cpu_baseline:
+            del host, tb
+        import gc
+
+        gc.collect()
+        torch.cuda.empty_cache()
+        try:
+            result["cfg5"] = model_decode(torch, dev, 36, 8, 65536, 256, 100, 8, True, int(args.host_kv_budget_gib * 2**30)
+                                          if args.host_kv_budget_gib > 0 else None)
+        except Exception as e:  # an allocation the box cannot satisfy must not cost the record its headline line
+            result["cfg5"] = {"error": f"{type(e).__name__}: {e}"[:400]}
     print(json.dumps(result))
 
 

@@ -296,3 +296,31 @@ def test_attention_matches_torch_sdpa_and_closed_forms(oracle):
     kk[123] = 50.0 * q[2].numpy()
     out = O.attention(q[2:3].numpy(), kk, v.numpy())
     np.testing.assert_allclose(out[0], v[123].numpy(), atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [0, 1])  # oracle.F32, oracle.BF16
+def test_torch_cpu_baseline_selects_the_oracles_keys_up_to_ties(oracle, dtype):
+    """oracle/torch_baseline.py (the batched torch form timed as the CPU baseline) against the C oracle: the two break
+    ties differently (torch.topk / argsort vs the fixed rule) and the torch rerank rounds in the tensor dtype, so the
+    final id sets agree on all but a few boundary keys."""
+    import torch
+
+    import workloads as W
+    from oracle import torch_baseline as TB
+
+    w = W.make_workload("tb", 2, 2, 4, 6000, 600, 128, dtype, 0.3, seed0=1)
+    tdt = torch.bfloat16 if dtype == oracle.BF16 else torch.float32
+    q = torch.from_numpy(w.queries).to(tdt).view(w.bs, 1, w.H * w.G, 128)
+    cb = torch.from_numpy(w.codes.reshape(w.bs, w.H, w.N, 16)).permute(0, 1, 3, 2).contiguous()
+    k4 = torch.from_numpy(w.nib.reshape(w.bs, w.H, w.N, 16, 4)).permute(0, 1, 3, 2, 4).contiguous()
+    kw = torch.from_numpy(w.weight.reshape(w.bs, w.H, w.N, 16)).to(torch.bfloat16).permute(0, 1, 3, 2).contiguous()
+    cc = torch.from_numpy(w.cluster_counts.reshape(w.bs, w.H, 16, 256))
+    keys = torch.from_numpy(w.keys.reshape(w.bs, w.H, w.N, 128))
+    ids, gk, gv = TB.retrieve_layer(q, torch.from_numpy(w.signs), cb, k4, kw, cc, w.tiers, w.C, w.K, keys, keys)
+    assert ids.shape == (w.bs, w.H, w.K) and torch.equal(gk, gv)
+    same = 0
+    for r in range(w.R):
+        b, h = divmod(r, w.H)
+        same += len(np.intersect1d(ids[b, h].numpy(), W.oracle_stages(w, r)["final"]))
+        assert torch.equal(gk[b, h], keys[b, h][ids[b, h]])
+    assert same >= 0.95 * w.R * w.K
