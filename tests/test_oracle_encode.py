@@ -102,6 +102,8 @@ def test_encode_matches_library_restatement(oracle, signs, dtype_name):
     rel = np.abs(w - rw) / np.maximum(np.abs(rw), 1e-6)
     assert np.median(rel) == 0.0 or np.median(rel) < 1e-2
     assert rel[agree].max() <= 2 ** -7  # at most one bf16 ulp where the codes agree
+    # ... and bit-identical almost everywhere: what is left is the summation order inside torch's reductions
+    assert (w[agree] == rw[agree]).mean() >= 0.99
     # invariants
     assert w.min() > 0 and np.array_equal(oracle.bf16_round(w), w)
     assert ((nib & 0x07) <= 7).all()
@@ -129,6 +131,63 @@ def test_encode_exact_closed_form_cases(oracle):
     # zero key: no NaNs, codes 255 (0 >= 0), magnitude bucket 0, weight 0
     codes3, nib3, w3 = oracle.encode(np.zeros((1, 128), np.float32), ones, oracle.BF16)
     assert (codes3 == 255).all() and (nib3 == 0x88).all() and (w3 == 0).all()
+
+
+def _bf16(x):
+    """Round-to-nearest-even bf16 of float32 values, by integer arithmetic on the bit patterns."""
+    u = np.asarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    return u.astype(np.uint32).view(np.float32)
+
+
+# keys k[i] = ((i * a) mod (2b + 3) - (b + 1)) / 4 and the bf16 bit patterns of their 16 block weights
+_ALPHA_ROUNDING_KEYS = {
+    (1, 1): [0x3f8f, 0x3f19, 0x3f53, 0x3f8f, 0x3f75, 0x3f39, 0x3f8a, 0x3f32, 0x3f44, 0x3f89, 0x3fa8, 0x3fa6, 0x3f77, 0x3f71,
+             0x3fa8, 0x3fba],
+    (4, 4): [0x3fc9, 0x4058, 0x3fc0, 0x4014, 0x4007, 0x402f, 0x3f9a, 0x4053, 0x3ff3, 0x3fb7, 0x3fea, 0x403f, 0x401f, 0x3fc8,
+             0x402a, 0x4024],
+    (1, 7): [0x409d, 0x4076, 0x406d, 0x403e, 0x401d, 0x4056, 0x4040, 0x4061, 0x4081, 0x4081, 0x4065, 0x40a7, 0x403b, 0x4021,
+             0x404a, 0x3ff6],
+}
+
+
+@pytest.mark.parametrize("ab", sorted(_ALPHA_ROUNDING_KEYS))
+def test_block_weight_rounds_the_alpha_products_before_the_sum(oracle, signs, ab):
+    """polar_cache.py:972-976 in the bf16 chain: ``a_vals * abs_u`` is a bf16 tensor, so every product is rounded to
+    bf16 BEFORE the fp32 sum that gives alpha.  These constructed keys are ones where that rounding point shows in
+    the stored weight: summing the unrounded products changes the bf16 bits of at least three blocks.  The expected
+    bits are written out above; they are what torch produces for the reference's own expression, and what the
+    restatement below (numpy, bf16 rounding by integer arithmetic, independent of the oracle's code) gives with the
+    rounding in place."""
+    a, b = ab
+    key = np.array([(((i * a) % (2 * b + 3)) - (b + 1)) * 0.25 for i in range(128)], np.float32)  # exact in bf16
+    expected = np.array(_ALPHA_ROUNDING_KEYS[ab], np.uint16)
+    _, _, w = oracle.encode(key[None], signs, oracle.BF16)
+    got = (w[0].view(np.uint32) >> 16).astype(np.uint16)
+    assert np.array_equal(got, expected), [hex(x) for x in got]
+    # the reference's torch expression on the same key
+    _, _, rw = refforms.batch_encode(torch.from_numpy(key).to(torch.bfloat16)[None], torch.from_numpy(signs))
+    assert np.array_equal(rw.view(torch.int16).numpy()[0].astype(np.uint16), expected)
+    # independent restatement from the rotated vector on, with and without the rounding of the products
+    th, ce = oracle.mag_constants()
+    n = _bf16(np.sqrt(np.float32((key.astype(np.float64) ** 2).sum())))
+    x = _bf16(key / n) * signs
+    y = _bf16((x.astype(np.float64) @ scipy.linalg.hadamard(128)).astype(np.float32) * np.float32(1 / np.sqrt(128.0)))
+    rounded, unrounded = [], []
+    for blk in y.reshape(16, 8):
+        r = _bf16(np.sqrt(np.float32((blk.astype(np.float64) ** 2).sum())))
+        au = np.abs(_bf16(blk / r))
+        t = (th[None, :] < au[:, None]).sum(axis=1)
+        prod = (ce[t] * au).astype(np.float32)
+        for out, terms in ((rounded, _bf16(prod)), (unrounded, prod)):
+            alpha = np.float32(0)
+            for p in terms:
+                alpha = np.float32(alpha + p)
+            out.append(_bf16(np.float32(np.float32(r / max(alpha, np.float32(1e-6))) * n)))
+    rounded = (np.array(rounded, np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    unrounded = (np.array(unrounded, np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    assert np.array_equal(rounded, expected)
+    assert (unrounded != expected).sum() >= 3
 
 
 def test_encode_brute_force_nearest_sign_centroid(oracle, signs):

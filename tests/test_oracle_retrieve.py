@@ -210,6 +210,41 @@ def test_adaptive_topk_matches_reference_form(oracle, cfg):
     assert sum(1 for a, b in ks if a == b) >= len(ks) - 1
 
 
+@pytest.mark.parametrize("rate,thr", [(0.5, 0.9), (0.25, 0.75), (1.0, 0.99), (0.1, 0.6), (0.5, 0.5)])
+def test_adaptive_topk_forced_k_equals_reference_form_exactly(oracle, rate, thr):
+    """Benefits in a geometric ladder (logit of the j-th best candidate = -rate * j, unit value norms): the mass
+    reached after k candidates is known in closed form and sits far from the threshold on both sides of the answer,
+    so neither exp()'s last ulp nor the summation order can move k.  k and the whole ordered index prefix must equal
+    the reference form (adaptive_topk.py:282-311) exactly, with and without dense tokens in the mix."""
+    n, cap = 3000, 256
+    g = np.random.default_rng(int(rate * 1000) + int(thr * 100))
+    for dense_share in (0.0, 0.3):
+        ladder = (-rate * np.arange(n)).astype(np.float32)
+        perm = g.permutation(n)
+        logits = np.empty(n, np.float32)
+        logits[perm] = ladder                                   # candidate position perm[j] holds the j-th best
+        ids = g.permutation(10 ** 6)[:n].astype(np.int64)
+        vn = np.ones(n, np.float32)
+        q = math.exp(-rate)
+        cand_mass = 1.0 / (1.0 - q)                             # sum of the ladder's benefits (joint max = 0)
+        # dense tokens: two of them, each with logit -20 and a value norm that makes their mass the wanted share
+        slb = dense_share * cand_mass / (1.0 - dense_share)
+        lsl = np.full(2, -20.0, np.float32)
+        slv = np.full(2, slb / 2.0 / math.exp(-20.0), np.float32)
+        total = slb + cand_mass
+        reached = [slb + (1.0 - q ** k) / (1.0 - q) for k in range(0, cap + 1)]
+        k_true = next(k for k in range(1, cap + 1) if reached[k] >= thr * total)
+        # far from the boundary on both sides (relative margin >> fp32 round-off of a few thousand terms)
+        assert reached[k_true] > thr * total * (1 + 1e-3) and reached[k_true - 1] < thr * total * (1 - 1e-3)
+        k, idx = oracle.adaptive_topk(lsl, slv, logits, vn, ids, thr, cap)
+        k_ref, idx_ref, _ = refforms.adaptive_topk(torch.from_numpy(lsl), torch.from_numpy(slv), torch.from_numpy(logits),
+                                                   torch.from_numpy(ids), torch.from_numpy(vn), thr, cap)
+        assert k == k_ref == k_true
+        # float32 exp(-rate * j) underflows to ties far down the ladder: compare the prefix that is strictly ordered
+        strict = int(min(cap, 80.0 / rate))
+        assert np.array_equal(idx[:strict], idx_ref.numpy()[:strict]) and np.array_equal(idx[:strict], ids[perm[:strict]])
+
+
 def test_adaptive_topk_edge_cases(oracle):
     # total <= 0 -> k = 1 ; never reached -> k_out
     z = np.zeros(10, np.float32)
