@@ -429,6 +429,25 @@ def main():
         "wall_s_timed_region": round(t_wall, 4),
     }
 
+    if args.no_cpu_baseline:  # still check a few rows of the benchmarked GPU path against the oracle
+        import numpy as np
+
+        from oracle import pkv_oracle as O
+
+        O.build()
+        ly, sg = layers[0], signs.cpu().numpy()
+        step(0)
+        torch.cuda.synchronize()
+        ok = True
+        for r in (0, 1, R // 2, R - 1):
+            b, h = divmod(r, H)
+            ref = O.retrieve_row(ly["q"].view(bs, H, G, D)[b, h].float().cpu().numpy(), sg, O.BF16,
+                                 ly["codes"][b, h].cpu().numpy(), ly["nib"][b, h].cpu().numpy().reshape(N, 16, 4),
+                                 ly["w"][b, h].float().cpu().numpy(), ly["cc"][b, h].cpu().numpy(), tiers, Cn, K)
+            ok = ok and np.array_equal(out_ids.view(R, K)[r].cpu().numpy(), ref)
+        result["parity_vs_oracle_on_bench_workload"] = bool(ok)
+        result["parity_rows_checked"] = 4
+
     # ------------------------------------------------------- CPU baseline
     if not args.no_cpu_baseline:
         import numpy as np

@@ -10,7 +10,8 @@ import os
 import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-SO_PATH = os.path.join(_HERE, "libpariskv_hip.so")
+# PARISKV_HIP_SO names another build of the library (same ABI), e.g. one compiled with different flags
+SO_PATH = os.environ.get("PARISKV_HIP_SO") or os.path.join(_HERE, "libpariskv_hip.so")
 CSRC = os.path.join(_HERE, "csrc")
 
 OK, EINVAL, ENOMEM, EHIP = 0, -22, -12, -5
@@ -149,6 +150,8 @@ def lib():
                 f"Build it with `make -C {CSRC}` (or `python -c 'import __graft_entry__ as g; g.build()'`).")
         handle = C.CDLL(SO_PATH)
         for name, (res, args) in PROTOTYPES.items():
+            if os.environ.get("PARISKV_HIP_SO") and not hasattr(handle, name):
+                continue  # optional symbols: an older build named by PARISKV_HIP_SO may lack the newest entry points
             fn = getattr(handle, name)
             fn.restype = res
             fn.argtypes = args

@@ -216,7 +216,7 @@ __device__ __forceinline__ float pkv_normalize_rotate_16(const float (&x)[8], co
 
 // Mean of the G query heads of row (b, h) (polar_cache.py:1027): lane l of a wave gets dims 8(l & 15) .. +7
 // in x[], rounded to the working dtype.  The G heads are added in order; their loads are all issued before
-// the first add (8 at a time, with no branch between them, so that they are in flight together).
+// the first add (4 at a time, with no branch between them, so that they are in flight together).
 template <bool BF16>
 __device__ __forceinline__ void pkv_query_group_mean_t(const void *__restrict__ q, int b, int h, int n_kv_heads,
                                                        int group, float (&x)[8]) {
@@ -224,10 +224,11 @@ __device__ __forceinline__ void pkv_query_group_mean_t(const void *__restrict__ 
   const int s = pkv_lane() & 15;
   const int64_t base = ((int64_t)b * n_kv_heads * group + (int64_t)h * group) * 128 + 8 * s;
   float acc[8];
-  for (int g0 = 0; g0 < group; g0 += 8) {
-    pkv_u32x4 raw[8][BF16 ? 1 : 2];
+  constexpr int kHeadsInFlight = 4;
+  for (int g0 = 0; g0 < group; g0 += kHeadsInFlight) {
+    pkv_u32x4 raw[kHeadsInFlight][BF16 ? 1 : 2];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < kHeadsInFlight; ++u) {
       const int g = g0 + u < group ? g0 + u : group - 1;
       if (BF16) {
         raw[u][0] = *(const pkv_u32x4 *)((const uint16_t *)q + base + (int64_t)g * 128);
@@ -237,7 +238,7 @@ __device__ __forceinline__ void pkv_query_group_mean_t(const void *__restrict__ 
       }
     }
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < kHeadsInFlight; ++u) {
       float v[8];
       if (BF16) {
         const uint32_t ww[4] = {raw[u][0].x, raw[u][0].y, raw[u][0].z, raw[u][0].w};
@@ -267,26 +268,107 @@ __device__ __forceinline__ void pkv_query_group_mean_t(const void *__restrict__ 
   }
 }
 
-// Group mean of the G query heads of row (b, h), normalised and SRHT-rotated (polar_cache.py:1027-1031,
-// 905-922).  Called by all 64 lanes of ONE wave: 16 lanes per copy of the vector, four identical copies;
-// lane l gets dims 8(l & 15) .. +7 of the rotated unit vector in y[] and the norm of the mean as result.
-template <bool BF16>
-__device__ __forceinline__ float pkv_query_mean_rotate_t(const void *__restrict__ q, int b, int h, int n_kv_heads,
-                                                         int group, const float *__restrict__ signs, float (&y)[8]) {
-  constexpr int dtype = BF16 ? PKV_DTYPE_BF16 : PKV_DTYPE_F32;
-  const int s = pkv_lane() & 15;
-  float x[8], sg[8];
-  const float4 s0 = *(const float4 *)(signs + 8 * s), s1 = *(const float4 *)(signs + 8 * s + 4);
-  sg[0] = s0.x, sg[1] = s0.y, sg[2] = s0.z, sg[3] = s0.w, sg[4] = s1.x, sg[5] = s1.y, sg[6] = s1.z, sg[7] = s1.w;
-  pkv_query_group_mean_t<BF16>(q, b, h, n_kv_heads, group, x);
-  return pkv_normalize_rotate_16(x, sg, s, dtype, y);
+// The normalisation and rotation of pkv_normalize_rotate_16 with the 128-vector spread over the 64 lanes of ONE wave: lane l holds dims
+// l and l + 64 (x_lo, x_hi).  Every value goes through the same sequence of fp32 operations as in
+// pkv_normalize_rotate_16 (sum of squares: left to right inside each aligned block of 8 dims = 8 neighbouring lanes,
+// then the pairwise tree over the 16 blocks; the butterflies h = 1 .. 64 in that order), so the results are
+// bit-identical; what changes is the length of the dependent chain: two divisions and seven butterfly steps per
+// lane instead of eight and fifty-six.  All 64 lanes must be active.  Returns the norm; y_lo / y_hi = rotated unit
+// vector's dims l and l + 64.
+__device__ __forceinline__ float pkv_normalize_rotate_64(float x_lo, float x_hi, float sg_lo, float sg_hi, int dtype,
+                                                         float &y_lo, float &y_hi) {
+  const int lane = pkv_lane();
+  const bool first = (lane & 7) == 0;
+  const float p_lo = x_lo * x_lo, p_hi = x_hi * x_hi;
+  float r_lo = p_lo, r_hi = p_hi;
+#pragma unroll
+  for (int t = 1; t < 8; ++t) {  // after step t the lanes with (lane & 7) <= t hold p_0 + ... + p_(lane & 7), left to right
+    const float below_lo = __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(r_lo), 0x111, 0xf, 0xf, true));
+    const float below_hi = __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(r_hi), 0x111, 0xf, 0xf, true));
+    r_lo = first ? p_lo : below_lo + p_lo;
+    r_hi = first ? p_hi : below_hi + p_hi;
+  }
+  // block totals sit in the lanes with (lane & 7) == 7; tree over the block index: lane ^ 8, ^ 16, ^ 32, then the halves
+  r_lo = r_lo + pkv_lane_xor_f<8>(r_lo);
+  r_hi = r_hi + pkv_lane_xor_f<8>(r_hi);
+  r_lo = r_lo + pkv_lane_xor_f<16>(r_lo);
+  r_hi = r_hi + pkv_lane_xor_f<16>(r_hi);
+  r_lo = r_lo + pkv_lane_xor_f<32>(r_lo);
+  r_hi = r_hi + pkv_lane_xor_f<32>(r_hi);
+  const float total = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(r_lo + r_hi), 7));
+  const float n = pkv_rdt(sqrtf(total), dtype);
+  const float den = n < 1e-8f ? 1e-8f : n;
+  float t_lo = pkv_rdt(x_lo / den, dtype) * sg_lo;
+  float t_hi = pkv_rdt(x_hi / den, dtype) * sg_hi;
+#define PKV_FWHT_WAVE_STAGE(M)                         \
+  {                                                    \
+    const float o_lo = pkv_lane_xor_f<M>(t_lo);        \
+    const float o_hi = pkv_lane_xor_f<M>(t_hi);        \
+    t_lo = (lane & M) ? (o_lo - t_lo) : (t_lo + o_lo); \
+    t_hi = (lane & M) ? (o_hi - t_hi) : (t_hi + o_hi); \
+  }
+  PKV_FWHT_WAVE_STAGE(1)
+  PKV_FWHT_WAVE_STAGE(2)
+  PKV_FWHT_WAVE_STAGE(4)
+  PKV_FWHT_WAVE_STAGE(8)
+  PKV_FWHT_WAVE_STAGE(16)
+  PKV_FWHT_WAVE_STAGE(32)
+#undef PKV_FWHT_WAVE_STAGE
+  const float a = t_lo, c = t_hi;  // h = 64: the two halves of the lane
+  y_lo = pkv_rdt((a + c) * PKV_HADAMARD_SCALE, dtype);
+  y_hi = pkv_rdt((a - c) * PKV_HADAMARD_SCALE, dtype);
+  return n;
 }
 
-__device__ __forceinline__ float pkv_query_mean_rotate(const void *__restrict__ q, int dtype, int b, int h,
-                                                       int n_kv_heads, int group, const float *__restrict__ signs,
-                                                       float (&y)[8]) {
-  return dtype == PKV_DTYPE_BF16 ? pkv_query_mean_rotate_t<true>(q, b, h, n_kv_heads, group, signs, y)
-                                 : pkv_query_mean_rotate_t<false>(q, b, h, n_kv_heads, group, signs, y);
+// Group mean of the G query heads of row (b, h), dims l and l + 64 for lane l of one wave, rounded to the working
+// dtype; the heads are added in order (polar_cache.py:1027).
+template <bool BF16>
+__device__ __forceinline__ void pkv_query_group_mean_wave_t(const void *__restrict__ q, int b, int h, int n_kv_heads,
+                                                            int group, float &x_lo, float &x_hi) {
+  constexpr int dtype = BF16 ? PKV_DTYPE_BF16 : PKV_DTYPE_F32;
+  const int lane = pkv_lane();
+  const int64_t base = ((int64_t)b * n_kv_heads * group + (int64_t)h * group) * 128 + lane;
+  float a_lo = 0.f, a_hi = 0.f;
+  constexpr int kHeadsInFlight = 4;
+  for (int g0 = 0; g0 < group; g0 += kHeadsInFlight) {
+    float v_lo[kHeadsInFlight], v_hi[kHeadsInFlight];
+#pragma unroll
+    for (int u = 0; u < kHeadsInFlight; ++u) {
+      const int g = g0 + u < group ? g0 + u : group - 1;
+      if (BF16) {
+        v_lo[u] = pkv_bf16_bits_to_f32(((const uint16_t *)q)[base + (int64_t)g * 128]);
+        v_hi[u] = pkv_bf16_bits_to_f32(((const uint16_t *)q)[base + (int64_t)g * 128 + 64]);
+      } else {
+        v_lo[u] = ((const float *)q)[base + (int64_t)g * 128];
+        v_hi[u] = ((const float *)q)[base + (int64_t)g * 128 + 64];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kHeadsInFlight; ++u) {
+      const bool first = g0 + u == 0, live = g0 + u < group;
+      a_lo = first ? v_lo[u] : (live ? a_lo + v_lo[u] : a_lo);
+      a_hi = first ? v_hi[u] : (live ? a_hi + v_hi[u] : a_hi);
+    }
+  }
+  if ((group & (group - 1)) == 0) {  // power of two: multiplying by the reciprocal is the same division, exactly
+    const float inv = 1.0f / (float)group;
+    x_lo = pkv_rdt(a_lo * inv, dtype), x_hi = pkv_rdt(a_hi * inv, dtype);
+  } else {
+    x_lo = pkv_rdt(a_lo / (float)group, dtype), x_hi = pkv_rdt(a_hi / (float)group, dtype);
+  }
+}
+
+// Group mean, normalise, SRHT rotate by all 64 lanes of ONE wave: lane l gets dims l and l + 64 of the rotated unit
+// vector and the norm of the mean as result (polar_cache.py:1027-1031, 905-922).
+__device__ __forceinline__ float pkv_query_mean_rotate_wave(const void *__restrict__ q, int dtype, int b, int h,
+                                                            int n_kv_heads, int group, const float *__restrict__ signs,
+                                                            float &y_lo, float &y_hi) {
+  const int lane = pkv_lane();
+  const float sg_lo = signs[lane], sg_hi = signs[lane + 64];
+  float x_lo, x_hi;
+  if (dtype == PKV_DTYPE_BF16) pkv_query_group_mean_wave_t<true>(q, b, h, n_kv_heads, group, x_lo, x_hi);
+  else pkv_query_group_mean_wave_t<false>(q, b, h, n_kv_heads, group, x_lo, x_hi);
+  return pkv_normalize_rotate_64(x_lo, x_hi, sg_lo, sg_hi, dtype, y_lo, y_hi);
 }
 
 // ---- 4-bit rerank core (shared by the stand-alone rerank and the fused select+rerank kernels) ----

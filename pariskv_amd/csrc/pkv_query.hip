@@ -8,22 +8,15 @@
 // weight = number of tiers whose key budget is not yet exhausted at the
 // centroid's rank.
 #include "pkv_common.h"
+#include "pkv_lut.h"
 
 namespace {
 
-// Exclusive prefix of the ranked cluster sizes -> tier weight, one thread per rank.
 __device__ __forceinline__ int tier_weight_from_rank(int my_count, const PkvTiers &tiers, int *s_wave_tot) {
-  int total;
-  int prefix = pkv_block_excl_scan<256>(my_count, s_wave_tot, total);
-  int w = 0;
-#pragma unroll
-  for (int t = 0; t < PKV_MAX_TIERS; ++t)
-    if (t < tiers.n && (uint32_t)prefix < tiers.t[t]) ++w;
-  return w;
+  return pkv_tier_weight_from_rank(my_count, tiers, s_wave_tot);
 }
 
-// grid (16 subspaces, R rows), 256 threads.  The rotation runs in the first wave only (16 lanes per
-// vector, shuffles, no barriers); the 256 threads then score, rank and weigh the 256 centroids.
+// grid (16 subspaces, R rows), 256 threads.
 __global__ __launch_bounds__(256) void pkv_query_prep_lut_kernel(
     const void *__restrict__ q, int dtype, int n_kv_heads, int group, const float *__restrict__ signs,
     const int32_t *__restrict__ cc, int64_t cc_b, int64_t cc_h, PkvTiers tiers, float *__restrict__ qhat,
@@ -37,85 +30,11 @@ __global__ __launch_bounds__(256) void pkv_query_prep_lut_kernel(
   // the collision scan that follows accumulates the row's suffix histogram with atomics
   if (row_suf_to_zero && sub == 1 && tid < 128) row_suf_to_zero[(int64_t)row * 128 + tid] = 0u;
 
-  __shared__ float s_y[128];
-  __shared__ __attribute__((aligned(16))) uint32_t s_key[256];
-  __shared__ int s_id[256];
-  __shared__ int s_cc[256];
-  __shared__ int s_part[128];
-  __shared__ int s_wave_tot[4];
-
-  // cluster sizes by centroid id; issued first so that the latency overlaps the rotation
-  s_cc[tid] = cc[(int64_t)b * cc_b + (int64_t)h * cc_h + sub * 256 + tid];
-
-  if (tid < PKV_WAVE) {
-    const int s = tid & 15;
-    float y[8];
-    const float n = pkv_query_mean_rotate(q, dtype, b, h, n_kv_heads, group, signs, y);
-    if (tid < 16) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        s_y[8 * s + j] = y[j];
-        if (sub == 0) qhat[(int64_t)row * 128 + 8 * s + j] = y[j];
-      }
-      if (sub == 0 && tid == 0) qnorm[row] = n;
-    }
-  }
-  __syncthreads();
-
-  // score of centroid c = tid: sum_j (+-) qhat_sub[j], sequential j
-  {
-    float acc = 0.f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float v = s_y[8 * sub + j];
-      const float t = ((tid >> j) & 1) ? v : -v;
-      acc = (j == 0) ? t : acc + t;
-    }
-    acc = pkv_rdt(acc + 0.0f, dtype);
-    uint32_t key = pkv_ordered_u32(acc);
-    // bf16 scores occupy the top 16 bits: fold the tie rule (smaller id first) into one 32-bit key
-    if (dtype == PKV_DTYPE_BF16) key = ((key >> 16) << 8) | (uint32_t)(255 - tid);
-    s_key[tid] = key;
-  }
-  __syncthreads();
-  // rank = number of centroids ahead of this one under (score desc, id asc).  The sign codebook is
-  // antipodal (score[255-c] == -score[c] exactly), hence rank[255-c] = 255 - rank[c]: thread t counts,
-  // for centroid c = t & 127, over half (t >> 7) of the keys; the two partial counts are added.
-  {
-    const int c = tid & 127, half = tid >> 7;
-    const uint32_t mine = s_key[c];
-    int part = 0;
-    const pkv_u32x4 *k4 = (const pkv_u32x4 *)s_key + half * 32;
-    if (dtype == PKV_DTYPE_BF16) {
-#pragma unroll 8
-      for (int c4 = 0; c4 < 32; ++c4) {
-        const pkv_u32x4 k = k4[c4];
-        part += (k.x > mine) + (k.y > mine) + (k.z > mine) + (k.w > mine);
-      }
-    } else {
-#pragma unroll 8
-      for (int c4 = 0; c4 < 32; ++c4) {
-        const pkv_u32x4 k = k4[c4];
-        const int o = half * 128 + 4 * c4;
-        part += (k.x > mine || (k.x == mine && o + 0 < c)) ? 1 : 0;
-        part += (k.y > mine || (k.y == mine && o + 1 < c)) ? 1 : 0;
-        part += (k.z > mine || (k.z == mine && o + 2 < c)) ? 1 : 0;
-        part += (k.w > mine || (k.w == mine && o + 3 < c)) ? 1 : 0;
-      }
-    }
-    if (half) s_part[c] = part;
-    __syncthreads();
-    if (!half) {
-      const int rank = part + s_part[c];
-      s_id[rank] = c;
-      s_id[255 - rank] = 255 - c;
-    }
-  }
-  __syncthreads();
-  const int id = s_id[tid];
-  const int w = tier_weight_from_rank(s_cc[id], tiers, s_wave_tot);
-  lut[((int64_t)row * 16 + sub) * 256 + id] = (uint8_t)w;
-  if (sorted_ids) sorted_ids[((int64_t)row * 16 + sub) * 256 + tid] = id;
+  __shared__ PkvLutSmem sm;
+  pkv_lut_build_subspace(q, dtype, b, h, n_kv_heads, group, signs, cc + (int64_t)b * cc_b + (int64_t)h * cc_h + sub * 256,
+                         tiers, sub, sm, lut + ((int64_t)row * 16 + sub) * 256,
+                         sub == 0 ? qhat + (int64_t)row * 128 : nullptr, sub == 0 ? qnorm + row : nullptr,
+                         sorted_ids ? sorted_ids + ((int64_t)row * 16 + sub) * 256 : nullptr);
 }
 
 // Ranking supplied by the caller (reference-shaped API).  grid (16, R), 256 threads.
