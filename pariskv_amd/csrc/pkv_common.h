@@ -103,8 +103,15 @@ PKV_INTERNAL int pkv_launch_gather(const void *src_k, const void *src_v, int64_t
 typedef unsigned int pkv_u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int pkv_u32x2 __attribute__((ext_vector_type(2)));
 
-// Round to nearest even bf16 and widen again: the hardware conversion (v_cvt_pk_bf16_f32) plus a shift.
-__device__ __forceinline__ float pkv_bf16_round(float x) { return (float)(__bf16)x; }
+// Round to nearest even bf16 and widen again, in one instruction: the packed hardware conversion
+// (v_cvt_pk_bf16_f32) of the pair (0, x) leaves bf16(x) in the upper half of the register and zero in the
+// lower half, which is bf16(x) read as an fp32.
+typedef __bf16 pkv_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float pkv_f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float pkv_bf16_round(float x) {
+  const pkv_f32x2 v = {0.0f, x};
+  return __builtin_bit_cast(float, __builtin_convertvector(v, pkv_bf16x2));
+}
 
 __device__ __forceinline__ float pkv_rdt(float x, int dtype) {
   return dtype == PKV_DTYPE_BF16 ? pkv_bf16_round(x) : x;

@@ -85,6 +85,51 @@ def test_encode_append_bit_exact(ops, dtype, layout):
     assert torch.equal(cc2, cc)
 
 
+def _adversarial_bf16_keys(n, seed):
+    """bf16 keys that stress every rounding decision of the encoder: magnitudes from 2^-30 to 2^30, outlier dims,
+    exact zeros and components far below the norm, powers of two, one-hot and constant vectors, tiny norms."""
+    rng = np.random.default_rng(seed)
+    k = rng.standard_normal((n, 128)).astype(np.float32)
+    kind = np.arange(n) % 16
+    k *= np.exp2(rng.integers(-30, 31, size=(n, 1))).astype(np.float32) * (kind[:, None] < 6) + (kind[:, None] >= 6)
+    k[kind == 6] *= np.where(rng.random((int((kind == 6).sum()), 128)) < 0.05, 30.0, 1.0).astype(np.float32)   # outlier dims
+    k[kind == 7] *= (rng.random((int((kind == 7).sum()), 128)) < 0.5)                                          # half zeros
+    k[kind == 8] *= np.where(rng.random((int((kind == 8).sum()), 128)) < 0.1, 1e-30, 1.0).astype(np.float32)   # far below the norm
+    k[kind == 9] = np.exp2(rng.integers(-8, 9, size=(int((kind == 9).sum()), 128))) * rng.choice([-1.0, 1.0], size=(int((kind == 9).sum()), 128))
+    oh = np.where(kind == 10)[0]
+    k[oh] = 0.0
+    k[oh, rng.integers(0, 128, size=oh.size)] = rng.standard_normal(oh.size).astype(np.float32) + 3.0          # one-hot
+    k[kind == 11] = (rng.standard_normal((int((kind == 11).sum()), 1)) * np.ones((1, 128))).astype(np.float32)  # constant
+    k[kind == 12] *= 1e-9                                                                                      # norm below the 1e-8 clamp
+    k[kind == 13] = np.round(k[kind == 13] * 4.0) / 4.0                                                        # many exact ties and zeros
+    k[kind == 14] *= 3e-8                                                                                      # norm just above the clamp
+    return O.bf16_round(k.astype(np.float32))
+
+
+def test_encode_bf16_bit_exact_on_adversarial_keys(ops):
+    """The bf16 encoder replaces divisions by reciprocals where that provably gives the same bf16 result and falls
+    back to correctly rounded arithmetic per wave elsewhere; both routes must equal the oracle bit for bit."""
+    H, S = 4, 16384 + 5
+    signs = O.srht_signs(42)
+    keys = np.stack([_adversarial_bf16_keys(S, 700 + h) for h in range(H)]).reshape(1, H, S, 128)
+    _say(f"encode adversarial bf16 keys {keys.shape}")
+    tk = torch.from_numpy(keys).to(torch.bfloat16).to(DEV)
+    _, _, _, cb, k4, kw = ops.alloc_keymajor(1, H, S, DEV)
+    cc = torch.zeros(1, H, 16, 256, dtype=torch.int32, device=DEV)
+    ops.encode_append(tk, torch.from_numpy(signs).to(DEV), cb, k4, kw, cc)
+    torch.cuda.synchronize()
+    for h in range(H):
+        codes, nib, w = O.encode(keys[0, h], signs, O.BF16)
+        bad = np.where((cb[0, h].cpu().numpy().T != codes).any(axis=1))[0]
+        assert bad.size == 0, f"codes differ at keys {bad[:8]} (kinds {bad[:8] % 16})"
+        bad = np.where((k4[0, h].cpu().numpy().transpose(1, 0, 2) != nib).any(axis=(1, 2)))[0]
+        assert bad.size == 0, f"4-bit codes differ at keys {bad[:8]} (kinds {bad[:8] % 16})"
+        got_w = kw[0, h].float().cpu().numpy().T
+        bad = np.where((got_w.view(np.uint32) != w.astype(np.float32).view(np.uint32)).any(axis=1))[0]
+        assert bad.size == 0, f"weights differ at keys {bad[:8]} (kinds {bad[:8] % 16})"
+        assert np.array_equal(cc[0, h].cpu().numpy(), O.count_cluster_keys(codes))
+
+
 def test_encode_without_rabitq_outputs(ops):
     S = 300
     signs = O.srht_signs(42)

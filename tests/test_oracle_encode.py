@@ -190,6 +190,34 @@ def test_block_weight_rounds_the_alpha_products_before_the_sum(oracle, signs, ab
     assert (unrounded != expected).sum() >= 3
 
 
+def test_bf16_quotients_stay_clear_of_bf16_rounding_boundaries(oracle):
+    """What the GPU encoder's reciprocal path rests on: for bf16 operands the quotient x / d is never within a
+    relative 2^-18 of a bf16 rounding boundary (the midpoint of two neighbouring bf16 numbers) unless it is exactly
+    a bf16 number, so any fp32 value within 2^-21 of the quotient rounds to the same bf16 as the correctly rounded
+    fp32 quotient does.  Exhaustive over the 128 x 128 significand pairs (the exponents only scale the picture)."""
+    from fractions import Fraction
+    closest = Fraction(1)
+    for mx in range(128, 256):
+        for md in range(128, 256):
+            q = Fraction(mx, md)
+            half_ulp_den = 256 if q >= 1 else 512           # boundaries are odd multiples of 1/256 in [1, 2), of 1/512 in (1/2, 1)
+            k = (q * half_ulp_den - 1) / 2                   # q = (2k + 1) / den  <=>  k integer
+            lo, hi = Fraction(2 * int(k) + 1, half_ulp_den), Fraction(2 * int(k) + 3, half_ulp_den)
+            dist = min(abs(q - lo), abs(q - hi)) / q
+            assert dist != 0, (mx, md)
+            closest = min(closest, dist)
+    assert closest > Fraction(1, 1 << 18)
+    # the same statement as arithmetic: perturb every quotient by +-2^-21 (more than a 1-ulp reciprocal times a
+    # rounded product can be off) at several exponents and round as the kernel does
+    mx, md = np.meshgrid(np.arange(128, 256, dtype=np.float64), np.arange(128, 256, dtype=np.float64), indexing="ij")
+    for ex, ed in ((0, 0), (-20, 3), (7, -9), (-3, 30)):
+        x, d = (mx * 2.0 ** (ex - 7)).astype(np.float32), (md * 2.0 ** (ed - 7)).astype(np.float32)
+        want = oracle.bf16_round(x / d)                      # fp32 division, correctly rounded, then bf16
+        for eps in (-2.0 ** -21, 2.0 ** -21):
+            approx = ((x.astype(np.float64) / d.astype(np.float64)) * (1.0 + eps)).astype(np.float32)
+            assert np.array_equal(oracle.bf16_round(approx).view(np.uint32), want.view(np.uint32))
+
+
 def test_encode_brute_force_nearest_sign_centroid(oracle, signs):
     """Sign bit-pack == argmax over the 256 sign centroids of <V_c, y_b>."""
     keys = oracle.synth_keys(300, seed=11)
