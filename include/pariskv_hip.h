@@ -241,6 +241,22 @@ int pkv_offload_rows(const void *src_k, const void *src_v, int64_t src_stride_b,
                      int64_t src_stride_row, void *dst_k_host, void *dst_v_host, int64_t dst_len,
                      int64_t dst_row0, int64_t n_rows, int bs, int n_kv_heads, int row_bytes, void *stream);
 
+/* pkv_offload_rows through the copy engines instead of a kernel: the same
+ * move (cache_hub/polar_cache.py:457-471, :778-799, where torch issues the
+ * copy on a side stream so that it overlaps the model's kernels), as
+ * hipMemcpyAsync / hipMemcpy2DAsync commands on `stream`.  A kernel that
+ * writes to host memory holds up every other kernel's stores while it runs;
+ * the copy engines do not.  Source strides in BYTES, any values >= the
+ * extents; dst_*_host: pinned host memory [bs][h][dst_len][row_bytes].
+ * flags: PKV_OFFLOAD_ONE_COMMAND = issue one pitched copy per tensor when the
+ * source's (b, h) blocks are contiguous and evenly spaced (otherwise, and
+ * without the flag, one command per block). */
+#define PKV_OFFLOAD_ONE_COMMAND 1
+int pkv_offload_rows_dma(const void *src_k, const void *src_v, int64_t src_stride_b, int64_t src_stride_h,
+                         int64_t src_stride_row, void *dst_k_host, void *dst_v_host, int64_t dst_len,
+                         int64_t dst_row0, int64_t n_rows, int bs, int n_kv_heads, int row_bytes, int flags,
+                         void *stream);
+
 /* pkv_gather_uva with a per-row count: row (b, h) moves only its first
  * row_counts[b*h_count + h] selected rows (int64 on the device, values in
  * [0, k]); the other slots of dst are left untouched.  For the adaptive-k

@@ -100,6 +100,7 @@ PROTOTYPES = {
     "pkv_append_kv": (_i, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i, _i, _i,
                            _vp, _i64, _i64, _vp]),
     "pkv_offload_rows": (_i, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i, _i, _i, _vp]),
+    "pkv_offload_rows_dma": (_i, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i, _i, _i, _i, _vp]),
     "pkv_gather_uva_ragged": (_i, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i64, _i64, _i, _i, _i, _vp]),
     "pkv_gather_uva_packed": (_i, [_vp, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _i64, _i, _i, _i, _vp]),
     "pkv_gather_cpu": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i, _i]),

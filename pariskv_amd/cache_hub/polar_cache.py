@@ -63,7 +63,7 @@ class polar_cache(KV_Cache):
                  codebook_path: Optional[str] = None, final_topk: int = 100, dynamic_update_interval: int = 512,
                  full_attention_threshold: int = 2000, enable_offload: bool = True,
                  collision_ratio: Optional[float] = None, candidate_ratio: Optional[float] = None,
-                 host_kv_budget_bytes=None) -> None:
+                 host_kv_budget_bytes=None, offload_engine: str = "dma") -> None:
         super().__init__(layer_num, batch_size, max_length, num_key_value_heads, num_heads, head_dim, dtype,
                          layer_mapping, num_gpus, model_size)
         if head_dim != ops.HEAD_DIM:
@@ -83,6 +83,9 @@ class polar_cache(KV_Cache):
         self.current_seq_len = [0] * layer_num
         self.final_topk = final_topk
         self.enable_offload = enable_offload
+        if offload_engine not in ("dma", "kernel"):
+            raise ValueError("offload_engine must be 'dma' or 'kernel'")
+        self._offload_dma = offload_engine == "dma"
         self._collision_ratio = collision_ratio
         self._candidate_ratio = candidate_ratio
         if codebook_path is not None and not os.path.isabs(codebook_path):
@@ -117,6 +120,11 @@ class polar_cache(KV_Cache):
             self._copy_stream = torch.cuda.Stream(device=dev)
             self._copy_events = [torch.cuda.Event() for _ in range(layer_num)]
             self._offload_inflight = [False] * layer_num
+            # prefill staging: two cache-owned [bsz,H,rows,D] K/V pairs used in turn, so that layer l's rows are being
+            # copied out while layer l+1's are staged, and HBM holds two layers' worth of staging at most
+            self._prefill_stage = [None, None]
+            self._prefill_stage_event = [None, None]
+            self._prefill_stage_next = 0
             budget = host_kv_budget_bytes
             if budget is not None and budget != "auto":
                 budget = int(budget)
@@ -207,19 +215,50 @@ class polar_cache(KV_Cache):
             self._offload_inflight[layer_idx] = False
 
     def _offload_rows(self, layer_idx: int, b0: int, b1: int, src_k: torch.Tensor, src_v: torch.Tensor, cpu_row0: int):
-        """Async move of [b1-b0, H, n, D] GPU rows (any batch / head / row strides) into the pinned host zone, on the
-        copy stream (polar_cache.py:457-471, 778-799).  One kernel writes through the host store's device mapping: a
-        torch ``copy_`` into a slice of the pinned tensor is a strided device-to-host copy, which torch stages through
-        pageable memory and a blocking host loop (measured 4-7 GB/s against ~50 GB/s for the kernel)."""
+        """Async move of [b1-b0, H, n, D] GPU rows into the pinned host zone on the copy stream (polar_cache.py:457-471,
+        778-799).  Default engine: one pitched copy-engine command per tensor (the source must then be a staging
+        buffer: contiguous blocks per (b, h)); the model's kernels keep the compute units, and with them their speed,
+        while it runs.  ``offload_engine="kernel"``: one kernel that writes through the host store's device mapping
+        (any source strides; as fast alone, but it stalls the stores of every kernel that runs beside it).  A torch
+        ``copy_`` into a slice of the pinned tensor would be a strided device-to-host copy, which torch stages
+        through pageable memory and a blocking host loop (4-7 GB/s)."""
         ready = torch.cuda.Event()
         ready.record(torch.cuda.current_stream(self.device))
         self._copy_stream.wait_event(ready)
         ops.offload_rows(src_k, src_v, self.unified_keys_cpu[layer_idx][b0:b1], self.unified_values_cpu[layer_idx][b0:b1],
-                         cpu_row0, stream=self._copy_stream)
+                         cpu_row0, stream=self._copy_stream, dma=self._offload_dma, dma_flags=ops.OFFLOAD_ONE_COMMAND)
         self._copy_events[layer_idx].record(self._copy_stream)
         src_k.record_stream(self._copy_stream)
         src_v.record_stream(self._copy_stream)
         self._offload_inflight[layer_idx] = True
+        return self._copy_events[layer_idx]
+
+    def _stage_prefill_rows(self, k: torch.Tensor, v: torch.Tensor):
+        """Private contiguous copies of the [bsz,H,n,D] views k, v in one of the two staging pairs (the reference's
+        ``.contiguous()`` copies, polar_cache.py:457-458): the caller may rewrite its tensors as soon as this call
+        returns, and the copy engines get whole blocks.  Returns (slot, staged k, staged v)."""
+        slot = self._prefill_stage_next
+        self._prefill_stage_next ^= 1
+        if self._prefill_stage_event[slot] is not None:   # the copy that last read this pair must be over
+            torch.cuda.current_stream(self.device).wait_event(self._prefill_stage_event[slot])
+        need = k.shape[0] * k.shape[1] * k.shape[2] * k.shape[3]
+        pair = self._prefill_stage[slot]
+        if pair is None or pair[0].numel() < need:
+            self._prefill_stage[slot] = None
+            pair = (torch.empty(need, dtype=self.dtype, device=self.device), torch.empty(need, dtype=self.dtype, device=self.device))
+            self._prefill_stage[slot] = pair
+        sk, sv = pair[0][:need].view(k.shape), pair[1][:need].view(v.shape)
+        sk.copy_(k)
+        sv.copy_(v)
+        return slot, sk, sv
+
+    def release_prefill_staging(self) -> None:
+        """Free the prefill staging pairs (two layers' worth of retrieval-zone K/V in HBM) once prefill is over; they
+        are allocated again on demand."""
+        if self.enable_offload:
+            self._copy_stream.synchronize()
+            self._prefill_stage = [None, None]
+            self._prefill_stage_event = [None, None]
 
     def _encode(self, layer_idx: int, keys_bhsd: torch.Tensor, b0: int, b1: int, abs0: int) -> None:
         """Encode keys [b1-b0, H, n, D] (any strides) into metadata positions [abs0, abs0+n) and add to the cluster sizes."""
@@ -270,11 +309,9 @@ class polar_cache(KV_Cache):
             vg[b0:b1, :, :S0] = v[:, :, :S0].to(self.dtype)
             kg[b0:b1, :, S0:S0 + local_len] = k[:, :, r_end:].to(self.dtype)
             vg[b0:b1, :, S0:S0 + local_len] = v[:, :, r_end:].to(self.dtype)
-            stage_k, stage_v = k[:, :, S0:r_end], v[:, :, S0:r_end]  # read in place when the dtype already matches
-            if stage_k.dtype != self.dtype or stage_v.dtype != self.dtype or stage_k.stride() != stage_v.stride():
-                stage_k, stage_v = stage_k.to(self.dtype).contiguous(), stage_v.to(self.dtype).contiguous()
             self._wait_offload(layer_idx)
-            self._offload_rows(layer_idx, b0, b1, stage_k, stage_v, 0)
+            slot, stage_k, stage_v = self._stage_prefill_rows(k[:, :, S0:r_end], v[:, :, S0:r_end])
+            self._prefill_stage_event[slot] = self._offload_rows(layer_idx, b0, b1, stage_k, stage_v, 0)
             self.cpu_valid_end[layer_idx] = retrieval
             enc_src = stage_k
         else:

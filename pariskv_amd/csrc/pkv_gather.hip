@@ -292,6 +292,51 @@ extern "C" int pkv_offload_rows(const void *src_k, const void *src_v, int64_t sr
   return PKV_OK;
 }
 
+// The same move through the copy engines: hipMemcpyAsync / hipMemcpy2DAsync commands on `stream`, no shader
+// kernel, so that kernels on other streams keep the compute units and the shader write path to themselves.
+// One command per (b, h) block and tensor: a plain copy where the block's rows are contiguous in the source, a
+// pitched copy otherwise; with PKV_OFFLOAD_ONE_COMMAND and a source whose (b, h) blocks are themselves evenly
+// spaced (a staging buffer), one pitched copy per tensor whose "rows" are whole blocks.
+extern "C" int pkv_offload_rows_dma(const void *src_k, const void *src_v, int64_t src_stride_b, int64_t src_stride_h,
+                                    int64_t src_stride_row, void *dst_k_host, void *dst_v_host, int64_t dst_len,
+                                    int64_t dst_row0, int64_t n_rows, int bs, int n_kv_heads, int row_bytes, int flags,
+                                    void *stream) {
+  PKV_REQUIRE(src_k && src_v && dst_k_host && dst_v_host, "offload: null pointer");
+  PKV_REQUIRE(bs > 0 && n_kv_heads > 0 && n_rows > 0 && row_bytes > 0 && dst_row0 >= 0 && dst_row0 + n_rows <= dst_len,
+              "offload: rows [%lld, %lld) outside the host store of %lld rows", (long long)dst_row0,
+              (long long)(dst_row0 + n_rows), (long long)dst_len);
+  PKV_REQUIRE(src_stride_row >= row_bytes && src_stride_b >= 0 && src_stride_h >= 0, "offload: bad source strides");
+  hipStream_t st = (hipStream_t)stream;
+  const bool rows_contiguous = src_stride_row == row_bytes;
+  const size_t block_bytes = (size_t)n_rows * (size_t)row_bytes;
+  const size_t dst_block = (size_t)dst_len * (size_t)row_bytes;
+  const void *srcs[2] = {src_k, src_v};
+  void *dsts[2] = {dst_k_host, dst_v_host};
+  const bool blocks_even = rows_contiguous && (bs == 1 || src_stride_b == (int64_t)n_kv_heads * src_stride_h) &&
+                           src_stride_h >= (int64_t)block_bytes;
+  for (int t = 0; t < 2; ++t) {
+    char *d0 = (char *)dsts[t] + (size_t)dst_row0 * (size_t)row_bytes;
+    if ((flags & PKV_OFFLOAD_ONE_COMMAND) && blocks_even) {
+      PKV_HIP(hipMemcpy2DAsync(d0, dst_block, srcs[t], (size_t)src_stride_h, block_bytes, (size_t)bs * n_kv_heads,
+                               hipMemcpyDeviceToHost, st));
+      continue;
+    }
+    for (int b = 0; b < bs; ++b) {
+      for (int h = 0; h < n_kv_heads; ++h) {
+        const char *sp = (const char *)srcs[t] + (size_t)b * (size_t)src_stride_b + (size_t)h * (size_t)src_stride_h;
+        char *dp = d0 + ((size_t)b * n_kv_heads + h) * dst_block;
+        if (rows_contiguous) {
+          PKV_HIP(hipMemcpyAsync(dp, sp, block_bytes, hipMemcpyDeviceToHost, st));
+        } else {
+          PKV_HIP(hipMemcpy2DAsync(dp, (size_t)row_bytes, sp, (size_t)src_stride_row, (size_t)row_bytes, (size_t)n_rows,
+                                   hipMemcpyDeviceToHost, st));
+        }
+      }
+    }
+  }
+  return PKV_OK;
+}
+
 extern "C" int pkv_gather_uva_ragged(const void *src_k, const void *src_v, int64_t src_len, const int64_t *idx, int64_t k,
                                      const int64_t *row_counts, int64_t idx_offset, void *dst_k, void *dst_v,
                                      int64_t dst_len, int64_t dst_row0, int bs, int n_kv_heads, int row_bytes,

@@ -490,11 +490,15 @@ def append_kv(key_states, value_states, dst_k, dst_v, slot: int, vnorm: Optional
         _p(vnorm), vn_b, vn_h, _stream(dst_k)))
 
 
-def offload_rows(src_k, src_v, dst_k_cpu, dst_v_cpu, dst_row0: int, stream=None) -> None:
-    """dst_cpu[:, :, dst_row0:dst_row0+n] = src for K and V in one launch on ``stream`` (default: the current one).
+OFFLOAD_ONE_COMMAND = 1
+
+
+def offload_rows(src_k, src_v, dst_k_cpu, dst_v_cpu, dst_row0: int, stream=None, dma: bool = False, dma_flags: int = 0) -> None:
+    """dst_cpu[:, :, dst_row0:dst_row0+n] = src for K and V on ``stream`` (default: the current one).
     src_k/src_v: GPU [bs,H,n,D] views with any batch / head / row strides (last dim contiguous); dst_*_cpu: pinned
     CPU [bs,H,rows,D] (a batch slice of a contiguous tensor is fine).  Asynchronous
-    (cache_hub/polar_cache.py:457-471, :778-799)."""
+    (cache_hub/polar_cache.py:457-471, :778-799).  ``dma=False``: one kernel that writes through the host store's
+    device mapping; ``dma=True``: copy-engine commands, which leave the compute units to whatever runs beside."""
     bs, H, n, D = src_k.shape
     es = src_k.element_size()
     _need(src_k.is_cuda and src_v.is_cuda and src_v.shape == src_k.shape and src_v.stride() == src_k.stride() and
@@ -504,6 +508,12 @@ def offload_rows(src_k, src_v, dst_k_cpu, dst_v_cpu, dst_row0: int, stream=None)
               t.shape[3] == D and t.stride(3) == 1 and t.stride(2) == D and t.stride(1) == t.shape[2] * D and
               (bs == 1 or t.stride(0) == H * t.stride(1)), "dst: pinned CPU [bs,H,rows,D], contiguous")
     s = stream if stream is not None else torch.cuda.current_stream(src_k.device)
+    if dma:
+        _lib.check(_lib.lib().pkv_offload_rows_dma(
+            src_k.data_ptr(), src_v.data_ptr(), src_k.stride(0) * es, src_k.stride(1) * es, src_k.stride(2) * es,
+            dst_k_cpu.data_ptr(), dst_v_cpu.data_ptr(), dst_k_cpu.shape[2], dst_row0, n, bs, H, D * es, dma_flags,
+            C.c_void_p(s.cuda_stream)))
+        return
     _lib.check(_lib.lib().pkv_offload_rows(
         src_k.data_ptr(), src_v.data_ptr(), src_k.stride(0) * es, src_k.stride(1) * es, src_k.stride(2) * es,
         dst_k_cpu.data_ptr(), dst_v_cpu.data_ptr(), dst_k_cpu.shape[2], dst_row0, n, bs, H, D * es,

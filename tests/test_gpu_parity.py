@@ -1294,10 +1294,12 @@ def test_uniform_k_is_the_row_maximum(ops):
         assert torch.equal(ops.uniform_k(ak), uk)
 
 
-def test_offload_rows_equals_sliced_copy(ops):
-    """pkv_offload_rows against the sliced copy_ it replaces (reference polar_cache.py:457-471, :778-799): rows read in
+@pytest.mark.parametrize("engine", ["kernel", "dma", "dma-one-command"])
+def test_offload_rows_equals_sliced_copy(ops, engine):
+    """pkv_offload_rows / pkv_offload_rows_dma against the sliced copy_ it replaces (reference polar_cache.py:457-471, :778-799): rows read in
     place from the model's [bs,seq,h,d] layout and from a partly filled staging buffer, into a batch slice of the pinned
     store; rows outside the written window stay untouched."""
+    kw = {"kernel": {}, "dma": {"dma": True}, "dma-one-command": {"dma": True, "dma_flags": ops.OFFLOAD_ONE_COMMAND}}[engine]
     g = torch.Generator().manual_seed(3)
     bs, H, cap, D = 3, 4, 50, 128
     kc = torch.randn(bs + 1, H, cap, D, generator=g).to(torch.bfloat16).pin_memory()
@@ -1306,19 +1308,19 @@ def test_offload_rows_equals_sliced_copy(ops):
     model_k = torch.randn(bs, 40, H, D, generator=g).to(torch.bfloat16).to(DEV)    # [bs, seq, h, d]
     model_v = torch.randn(bs, 40, H, D, generator=g).to(torch.bfloat16).to(DEV)
     src_k, src_v = model_k[:, 5:33].permute(0, 2, 1, 3), model_v[:, 5:33].permute(0, 2, 1, 3)
-    ops.offload_rows(src_k, src_v, kc[1:], vc[1:], 7)
+    ops.offload_rows(src_k, src_v, kc[1:], vc[1:], 7, **kw)
     want_k[1:, :, 7:35] = src_k.cpu()
     want_v[1:, :, 7:35] = src_v.cpu()
     stage_k = torch.randn(bs, H, 16, D, generator=g).to(torch.bfloat16).to(DEV)   # staging buffer, first 9 rows valid
     stage_v = torch.randn(bs, H, 16, D, generator=g).to(torch.bfloat16).to(DEV)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
-    ops.offload_rows(stage_k[:, :, :9], stage_v[:, :, :9], kc[:bs], vc[:bs], cap - 9, stream=side)
+    ops.offload_rows(stage_k[:, :, :9], stage_v[:, :, :9], kc[:bs], vc[:bs], cap - 9, stream=side, **kw)
     want_k[:bs, :, cap - 9:] = stage_k[:, :, :9].cpu()
     want_v[:bs, :, cap - 9:] = stage_v[:, :, :9].cpu()
     torch.cuda.synchronize()
     assert torch.equal(kc, want_k) and torch.equal(vc, want_v)
     with pytest.raises(RuntimeError, match="outside the host store"):
-        ops.offload_rows(stage_k, stage_v, kc[:bs], vc[:bs], cap - 9)
+        ops.offload_rows(stage_k, stage_v, kc[:bs], vc[:bs], cap - 9, **kw)
     with pytest.raises(RuntimeError):
-        ops.offload_rows(stage_k, stage_v, kc[:bs].clone(), vc[:bs], 0)   # not pinned
+        ops.offload_rows(stage_k, stage_v, kc[:bs].clone(), vc[:bs], 0, **kw)   # not pinned

@@ -47,11 +47,14 @@ def _synth_kv(gen, bs, S, Hkv):
 
 
 # 16 rows: selected rows attended in place; "mixed": a host budget that holds one layer, the other stays in HBM
-@pytest.mark.parametrize("offload,bs,Hkv", [(True, 2, 2), (False, 2, 2), (False, 4, 4), ("mixed", 2, 2), ("mixed", 4, 4)])
+@pytest.mark.parametrize("offload,bs,Hkv", [(True, 2, 2), ("kernel", 2, 2), (False, 2, 2), (False, 4, 4), ("mixed", 2, 2), ("mixed", 4, 4)])
 def test_decode_loop_matches_oracle_and_dense_reference(offload, bs, Hkv):
     from pariskv_amd.attn_hub import polar_decode_attn
 
     print(f"polar_cache decode loop offload={offload} bs={bs} Hkv={Hkv}", flush=True)
+    extra = {}
+    if offload == "kernel":    # the host offload through the shader kernel instead of the copy engines
+        offload, extra = True, {"offload_engine": "kernel"}
     Hq, layers, S, steps = 4 * Hkv, 2, 3000, 70
     sink, local, I, topk = 4, 64, 32, 200
     G = Hq // Hkv
@@ -64,7 +67,7 @@ def test_decode_loop_matches_oracle_and_dense_reference(offload, bs, Hkv):
         assert cache.kv_placement["host_pinned_bytes"] == layer_bytes
         assert cache.unified_keys_cpu[1] is None and cache.unified_keys_gpu[1].shape[2] == S + steps + 10
     else:
-        cache = _make_cache(offload, bs, Hkv, Hq, layers, S, steps + 10, sink, local, I, topk)
+        cache = _make_cache(offload, bs, Hkv, Hq, layers, S, steps + 10, sink, local, I, topk, **extra)
         assert cache._layer_offload == [bool(offload)] * layers
     gen = torch.Generator().manual_seed(0)
     hist_k = [None] * layers
