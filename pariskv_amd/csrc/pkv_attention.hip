@@ -10,7 +10,7 @@
 // all G query heads.  Split over the key axis (flash-decoding): grid (n_splits, R);
 // every split keeps a running (max, sum, output) per query head and the partial
 // results are merged by a second small launch.
-//   bf16: one wave per split on the matrix cores (v_mfma_f32_16x16x32_bf16), see below.
+//   bf16: four waves per split on the matrix cores (v_mfma_f32_16x16x32_bf16), merged through LDS, see below.
 //   fp32: 256 threads per split, every 16 lanes own one key at a time (a wave
 //         instruction moves four whole rows), fp32 FMA and lane-exchange reductions.
 //
@@ -258,7 +258,7 @@ __global__ __launch_bounds__(kAttThreads) void pkv_attn_partial_kernel(const voi
 
 // ---- bf16 inputs: the same partial step on the matrix cores ----
 //
-// One wave per workgroup, 32 keys per step, v_mfma_f32_16x16x32_bf16 throughout.
+// Each wave: 32 keys per step, v_mfma_f32_16x16x32_bf16 throughout.
 //   scores:  S^T[key][head] = K[key][dim] . Q^T[dim][head]: A = 16 keys x 32 dims (lane (r, j) holds dims
 //            32c + 8j .. +7 of key r: one 128-bit load), B = the query heads (zero columns past `group`),
 //            4 instructions per 16 keys.  Lane (n, j) receives the scores of head n for keys 4j .. 4j+3 of the
@@ -281,22 +281,23 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return (uint32_t)pkv_f32_to_bf16_bits(lo) | ((uint32_t)pkv_f32_to_bf16_bits(hi) << 16);
 }
 
+constexpr int kMfmaWaves = 4;  // waves per workgroup: each takes a quarter of the split, merged through LDS
+
 template <bool INDEXED>
-__global__ __launch_bounds__(PKV_WAVE) void pkv_attn_partial_mfma_kernel(const void *__restrict__ q, int n_kv_heads,
-                                                                         int group, AttSegs segs, int64_t total,
-                                                                         const int32_t *__restrict__ row_keys,
-                                                                         int64_t per_split, float scale_log2e,
-                                                                         float *__restrict__ ws) {
+__global__ __launch_bounds__(kMfmaWaves * PKV_WAVE) void pkv_attn_partial_mfma_kernel(
+    const void *__restrict__ q, int n_kv_heads, int group, AttSegs segs, int64_t total,
+    const int32_t *__restrict__ row_keys, int64_t per_split, float scale_log2e, float *__restrict__ ws) {
   const int split = blockIdx.x, row = blockIdx.y;
   const int b = row / n_kv_heads, h = row % n_kv_heads;
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & (PKV_WAVE - 1), wave = threadIdx.x / PKV_WAVE;
   const int n = lane & 15, j = lane >> 4;
   if (row_keys) {
     const int64_t rk = row_keys[row];
     total = rk < total ? (rk > 0 ? rk : 1) : total;
   }
-  const int64_t j0 = (int64_t)split * per_split;
-  const int64_t j1 = (j0 + per_split < total) ? j0 + per_split : total;
+  const int64_t per_wave = per_split / kMfmaWaves;  // a multiple of the 32 keys of one step
+  const int64_t j0 = (int64_t)split * per_split + (int64_t)wave * per_wave;
+  const int64_t j1 = (j0 + per_wave < total) ? j0 + per_wave : total;  // j1 <= j0: nothing left for this wave
 
   // per segment: byte address of "concatenated key 0" for this (b, h); with indexed segments: of row 0 of the slab
   const char *kb[PKV_ATTN_MAX_SEGMENTS], *vb[PKV_ATTN_MAX_SEGMENTS];
@@ -410,15 +411,34 @@ __global__ __launch_bounds__(PKV_WAVE) void pkv_attn_partial_mfma_kernel(const v
 
   l_part += __shfl_xor(l_part, 16, PKV_WAVE);
   l_part += __shfl_xor(l_part, 32, PKV_WAVE);
-  float *part = ws + ((int64_t)row * gridDim.x + split) * group * kPartStride;
-  if (j == 0 && n < group) part[n * kPartStride] = m_run, part[n * kPartStride + 1] = l_part;
+  // merge the waves of the workgroup: every wave leaves (max, sum, output) of its keys in LDS, then the
+  // workgroup's 256 threads combine them, one (head, dim) pair at a time.  group <= 8.
+  __shared__ float s_m[kMfmaWaves][8], s_l[kMfmaWaves][8], s_o[kMfmaWaves][8][128 + 4];
+  if (j == 0 && n < group) s_m[wave][n] = m_run, s_l[wave][n] = l_part;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int head = 4 * j + i;
     if (head < group) {
-#pragma unroll
-      for (int m = 0; m < 8; ++m) part[head * kPartStride + 2 + 8 * n + m] = o[m][i];
+      *(float4 *)&s_o[wave][head][8 * n] = float4{o[0][i], o[1][i], o[2][i], o[3][i]};
+      *(float4 *)&s_o[wave][head][8 * n + 4] = float4{o[4][i], o[5][i], o[6][i], o[7][i]};
     }
+  }
+  __syncthreads();
+  float *part = ws + ((int64_t)row * gridDim.x + split) * group * kPartStride;
+  for (int e = threadIdx.x; e < group * 128; e += kMfmaWaves * PKV_WAVE) {
+    const int g = e >> 7, d = e & 127;
+    float mn = s_m[0][g];
+#pragma unroll
+    for (int w = 1; w < kMfmaWaves; ++w) mn = fmaxf(mn, s_m[w][g]);
+    float ls = 0.f, os = 0.f;
+#pragma unroll
+    for (int w = 0; w < kMfmaWaves; ++w) {
+      const float c = exp2f(s_m[w][g] - mn);
+      ls += s_l[w][g] * c;
+      os += s_o[w][g][d] * c;
+    }
+    part[g * kPartStride + 2 + d] = os;
+    if (d == 0) part[g * kPartStride] = mn, part[g * kPartStride + 1] = ls;
   }
 }
 
@@ -466,12 +486,12 @@ int pick_splits(int rows, int64_t total) {
   return (int)s;
 }
 
-// One wave per workgroup on the matrix-core path: enough waves to cover the chip several times over, at
-// least two 32-key steps each (one step each measured no faster, and the merge pays for the extra splits).
+// Matrix-core path: four waves per workgroup, one 32-key step per wave while that keeps the split count within
+// the 64 the merge kernel takes (every load of the workgroup is then in flight at once); longer key sets give
+// each wave more steps.
 int pick_splits_mfma(int rows, int64_t total) {
-  int64_t s = (4096 + rows - 1) / rows;
-  const int64_t max_by_len = (total + 63) / 64;
-  if (s > max_by_len) s = max_by_len;
+  (void)rows;
+  int64_t s = (total + kMfmaWaves * kMfmaStepKeys - 1) / (kMfmaWaves * kMfmaStepKeys);
   if (s > 64) s = 64;
   if (s < 1) s = 1;
   return (int)s;
@@ -531,7 +551,7 @@ extern "C" int pkv_decode_attention(const void *q, int dtype, int bs, int n_kv_h
     pkv_set_error("pkv_decode_attention: workspace of %zu bytes required, got %zu", need, ws_bytes);
     return PKV_ENOMEM;
   }
-  const int step = bf ? kMfmaStepKeys : kAttKeysPerIter * kAttUnroll;
+  const int step = bf ? kMfmaWaves * kMfmaStepKeys : kAttKeysPerIter * kAttUnroll;
   int64_t per_split = (total + n_splits - 1) / n_splits;
   per_split = (per_split + step - 1) / step * step;
   const float scale_log2e = scale * 1.4426950408889634f;
@@ -539,10 +559,10 @@ extern "C" int pkv_decode_attention(const void *q, int dtype, int bs, int n_kv_h
   dim3 grid((unsigned)n_splits, (unsigned)rows);
   if (bf) {
     if (indexed)
-      hipLaunchKernelGGL(pkv_attn_partial_mfma_kernel<true>, grid, dim3(PKV_WAVE), 0, s, q, n_kv_heads, group, sg, total,
+      hipLaunchKernelGGL(pkv_attn_partial_mfma_kernel<true>, grid, dim3(kMfmaWaves * PKV_WAVE), 0, s, q, n_kv_heads, group, sg, total,
                          row_keys, per_split, scale_log2e, (float *)ws);
     else
-      hipLaunchKernelGGL(pkv_attn_partial_mfma_kernel<false>, grid, dim3(PKV_WAVE), 0, s, q, n_kv_heads, group, sg, total,
+      hipLaunchKernelGGL(pkv_attn_partial_mfma_kernel<false>, grid, dim3(kMfmaWaves * PKV_WAVE), 0, s, q, n_kv_heads, group, sg, total,
                          row_keys, per_split, scale_log2e, (float *)ws);
   } else {
 #define PKV_ATT(GG, G0, GC, IDX)                                                                                  \

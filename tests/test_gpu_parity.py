@@ -800,6 +800,43 @@ def test_adaptive_topk_shapes_and_orders(ops, sl, Cn, k_out, thr, mode):
         assert max(ks) < k_out  # the threshold is reached inside the list in these cases
 
 
+def test_adaptive_topk_config4_rows_land_at_different_k(ops):
+    """BASELINE config 4's adaptive-k shape (8 rows x ceil(0.05 * 2^20) candidates, list 2048, mass 0.95, clamp
+    [256, 2048], value norms gathered from a 2^20-entry table) on scores whose mass is spread differently per row:
+    benefits decay like exp(-rank / tau_r), so the 0.95 mass is reached near 3 tau_r and every row stops at its own
+    k strictly inside the clamp.  k and the whole id list against the CPU checker."""
+    H, N, sink, sl = 8, 1 << 20, 64, 64 + 512
+    Cn, k_out, thr, k_min, k_max = int(math.ceil(N * 0.05)), 2048, 0.95, 256, 2048
+    taus = [110.0, 170.0, 240.0, 320.0, 400.0, 480.0, 560.0, 630.0]
+    g = torch.Generator().manual_seed(44)
+    scale = 1.0 / math.sqrt(128)
+    sc = torch.empty(1, H, Cn)
+    ci = torch.empty(1, H, Cn, dtype=torch.int64)
+    for h in range(H):
+        rank = torch.randperm(Cn, generator=g).float()                          # rank of candidate i in its row
+        sc[0, h] = (-(rank / taus[h]) + 0.3 * torch.rand(Cn, generator=g)) / scale
+        ci[0, h] = torch.sort(torch.randperm(N, generator=g)[:Cn]).values       # sorted positions, as the select emits them
+    sll = torch.randn(1, H, sl, generator=g) * 0.5 - 6.0                          # the dense tokens hold a small share of the mass
+    slv = torch.rand(1, H, sl, generator=g) + 0.5
+    vn = torch.rand(1, H, N + sink, generator=g) * 0.2 + 0.9
+    _say(f"adaptive-k config 4 shape: {H} rows x {Cn} candidates")
+    ak, ids, rk = ops.adaptive_topk(sll.to(DEV), slv.to(DEV), sc.to(DEV), scale, ci.to(DEV), thr, k_out,
+                                    value_norm=vn.to(DEV), vn_offset=sink, k_min=k_min, k_max=k_max, row_keys_base=sl)
+    torch.cuda.synchronize()
+    rk = rk.view(-1)
+    ks = []
+    for h in range(H):
+        cvn = vn[0, h][ci[0, h] + sink]
+        k_ref, ids_ref = O.adaptive_topk(sll[0, h].numpy(), slv[0, h].numpy(), (sc[0, h] * np.float32(scale)).numpy(),
+                                         cvn.numpy(), ci[0, h].numpy(), thr, k_out)
+        assert k_min < k_ref < k_max, (h, k_ref)
+        assert int(ak[0, h]) == k_ref and int(rk[h]) == sl + k_ref
+        assert np.array_equal(ids[0, h].cpu().numpy(), ids_ref)
+        ks.append(k_ref)
+    assert len(set(ks)) == H and ks == sorted(ks), ks
+    _say(f"adaptive k per row: {ks}")
+
+
 def test_adaptive_topk_wide_zero_mass(ops):
     """total <= 0 on the multi-workgroup path: k = 1 (adaptive_topk.py:304-306); ids still ordered by position."""
     Cn = 10000
