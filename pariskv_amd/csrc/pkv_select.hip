@@ -540,6 +540,142 @@ __device__ __forceinline__ void radix_select_regs(const uint64_t (&v)[EIN], uint
   shift_out = shift;
 }
 
+// ---- selection through 256 linear bins of the row's own score range ----
+//
+// The 8-bit radix passes above look at fixed bit fields: scores of one row share their sign and most exponent
+// bits, so the first pass separates almost nothing and three passes are the rule.  Here the bins divide
+// [row min, row max] evenly: bin(x) = min(255, floor((x - lo) * 256 / (hi - lo))), a non-decreasing function
+// of x whatever the rounding of its three operations, so every key in a higher bin is a larger key.  One
+// histogram pass finds the bin b* that holds the k-th largest key and how many of its keys are needed; the
+// exact threshold key T is then the need-th largest of that one bin, found by counting (a bin holds len / 256
+// keys on average).  Winners: bin > b*, or bin == b* and key >= T.  The bins also order the winners: those
+// of bin b occupy the output slots [off[b], off[b] + count[b]), and the slot inside the bin is again found by
+// counting, which replaces the bitonic sort (and T: the first `need` of b* by that count are its winners).
+// Rows this does not suit take the older steps: non-finite scores, a zero or subnormal range or more than
+// kLinBucketMax keys in b* the radix select; more than kLinRankMax winners in one bin the bitonic sort.  The
+// result is the same set in the same order either way.
+constexpr int kLinBucketMax = 256;
+constexpr int kLinRankMax = 128;
+
+struct LinSel {
+  float lo, scale;
+  uint32_t bstar, need;   // threshold bin, keys needed from it
+  uint32_t in_bstar;      // keys in the threshold bin
+  uint32_t max_winners;   // most winners in one bin
+  uint64_t T;             // threshold key inside bin b* (0: the whole bin wins); set by linear_threshold
+};
+
+__device__ __forceinline__ uint32_t lin_bin(uint64_t key, float lo, float scale) {
+  const float t = (pkv_from_ordered_u32((uint32_t)(key >> 32)) - lo) * scale;
+  const uint32_t b = (uint32_t)t;
+  return b > 255u ? 255u : b;
+}
+
+// Bins of the thread's keys and the threshold bin.  On return s_hist[0,256) = keys per bin, s_hist[256,512) =
+// off[b] = keys in the bins above b, s_cnt[b] = off[b] (a running output slot for the counting sort), s_bcast[6] = 0.
+// s_hist: 512 words, s_cnt: 256 words, s_bcast: 8 words.  All 1024 threads call it; false = not applicable.
+template <int EIN>
+__device__ __forceinline__ bool linear_bins(const uint64_t (&v)[EIN], uint32_t k, uint32_t *s_hist, uint32_t *s_cnt,
+                                            uint32_t *s_bcast, uint32_t (&bin)[EIN], LinSel &L) {
+  const int tid = threadIdx.x, lane = pkv_lane();
+  if (tid < 512) s_hist[tid] = 0;
+  if (tid == 0) s_bcast[0] = 0u, s_bcast[1] = 0xffffffffu, s_bcast[5] = 0u, s_bcast[6] = 0u;
+  __syncthreads();
+  uint32_t mx = 0u, mn = 0xffffffffu;
+#pragma unroll
+  for (int e = 0; e < EIN; ++e) {
+    if (v[e] != 0ull) {
+      const uint32_t hi = (uint32_t)(v[e] >> 32);
+      mx = hi > mx ? hi : mx;
+      mn = hi < mn ? hi : mn;
+    }
+  }
+#define PKV_LIN_RED(M)                              \
+  {                                                 \
+    const uint32_t a = pkv_lane_xor<M>(mx), c = pkv_lane_xor<M>(mn); \
+    mx = a > mx ? a : mx;                           \
+    mn = c < mn ? c : mn;                           \
+  }
+  PKV_LIN_RED(1) PKV_LIN_RED(2) PKV_LIN_RED(4) PKV_LIN_RED(8) PKV_LIN_RED(16) PKV_LIN_RED(32)
+#undef PKV_LIN_RED
+  if (lane == 0) {
+    atomicMax(&s_bcast[0], mx);
+    atomicMin(&s_bcast[1], mn);
+  }
+  __syncthreads();
+  mx = s_bcast[0], mn = s_bcast[1];
+  const float hi = pkv_from_ordered_u32(mx), lo = pkv_from_ordered_u32(mn);
+  const float range = hi - lo, scale = 256.0f / range;
+  const float inf = __uint_as_float(0x7f800000u);
+  // finite scores (ordered keys strictly between those of -inf and +inf), a positive finite range and scale
+  if (!(mx < 0xff800000u && mn > 0x007fffffu && range > 0.f && range < inf && scale < inf)) return false;
+#pragma unroll
+  for (int e = 0; e < EIN; ++e) {
+    bin[e] = 0;
+    if (v[e] != 0ull) {
+      bin[e] = lin_bin(v[e], lo, scale);
+      atomicAdd(&s_hist[bin[e]], 1u);
+    }
+  }
+  __syncthreads();
+  if (tid < PKV_WAVE) {  // lane l owns bins 255 - 4l .. 252 - 4l: an inclusive scan over lanes is the suffix sum over bins
+    uint32_t h[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) h[j] = s_hist[255 - 4 * tid - j];
+    const uint32_t mine = h[0] + h[1] + h[2] + h[3];
+    uint32_t above = (uint32_t)pkv_wave_incl_scan((int)mine) - mine;
+    uint32_t most = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int b = 255 - 4 * tid - j;
+      s_hist[256 + b] = above;
+      s_cnt[b] = above;
+      if (above < k) {
+        const uint32_t take = above + h[j] >= k ? k - above : h[j];
+        most = take > most ? take : most;
+        if (above + h[j] >= k) s_bcast[2] = (uint32_t)b, s_bcast[3] = take, s_bcast[4] = h[j];
+      }
+      above += h[j];
+    }
+    most = most > pkv_lane_xor<1>(most) ? most : pkv_lane_xor<1>(most);
+    most = most > pkv_lane_xor<2>(most) ? most : pkv_lane_xor<2>(most);
+    most = most > pkv_lane_xor<4>(most) ? most : pkv_lane_xor<4>(most);
+    most = most > pkv_lane_xor<8>(most) ? most : pkv_lane_xor<8>(most);
+    if ((tid & 15) == 0) atomicMax(&s_bcast[5], most);
+  }
+  __syncthreads();
+  L.lo = lo, L.scale = scale;
+  L.bstar = s_bcast[2], L.need = s_bcast[3], L.in_bstar = s_bcast[4], L.max_winners = s_bcast[5];
+  L.T = 0ull;
+  return L.in_bstar <= kLinBucketMax;
+}
+
+// Threshold key of bin b*: the need-th largest of its keys, found by counting with 16 lanes per key.
+// s_bcast[6] must be 0 (linear_bins leaves it so).  All 1024 threads call it.
+template <int EIN>
+__device__ __forceinline__ void linear_threshold(const uint64_t (&v)[EIN], const uint32_t (&bin)[EIN], uint32_t *s_bcast,
+                                                 uint64_t *s_bucket, uint64_t *s_T, LinSel &L) {
+  if (L.in_bstar == L.need) return;  // the bin is taken whole: T = 0
+#pragma unroll
+  for (int e = 0; e < EIN; ++e) {  // about one key in 256: most waves skip the atomic altogether
+    if (v[e] != 0ull && bin[e] == L.bstar) s_bucket[atomicAdd(&s_bcast[6], 1u)] = v[e];
+  }
+  __syncthreads();
+  const uint32_t n = L.in_bstar, sub = threadIdx.x & 15u;
+  for (uint32_t i = threadIdx.x >> 4; i < n; i += kTopkThreads / 16) {
+    const uint64_t key = s_bucket[i];
+    uint32_t r = 0;
+    for (uint32_t j = sub; j < n; j += 16) r += s_bucket[j] > key ? 1u : 0u;
+    r += pkv_lane_xor<1>(r);
+    r += pkv_lane_xor<2>(r);
+    r += pkv_lane_xor<4>(r);
+    r += pkv_lane_xor<8>(r);
+    if (sub == 0 && r == L.need - 1) *s_T = key;
+  }
+  __syncthreads();
+  L.T = *s_T;
+}
+
 // The same selection over keys that do not fit the registers: key_of(i), i < len, is evaluated again
 // in every pass.
 template <typename KeyFn>
@@ -594,8 +730,11 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
     int64_t k, int64_t *__restrict__ out_ids, float *__restrict__ out_vals) {
   extern __shared__ uint64_t s_keys[];
   __shared__ uint32_t s_hist[512];
+  __shared__ uint32_t s_cnt[256];
   __shared__ uint32_t s_bcast[8];
   __shared__ uint32_t s_counter;
+  __shared__ uint64_t s_bucket[kLinBucketMax];
+  __shared__ uint64_t s_T;
   const int row = blockIdx.x;
   const int tid = threadIdx.x;
   const float *xr = x + (int64_t)row * x_stride;
@@ -609,20 +748,69 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
   if (tid == 0) s_counter = 0;
   if (SORTED)
     for (int i = tid; i < (P < 1024 ? 1024 : P); i += kTopkThreads) s_keys[i] = 0ull;
-  uint64_t prefix;
-  int shift;
-  radix_select_regs<EIN>(v, (uint32_t)k, s_hist, s_bcast, prefix, shift);
+  bool win[EIN];
+  uint32_t bin[EIN];
+  LinSel L;
+  const bool lin = linear_bins<EIN>(v, (uint32_t)k, s_hist, s_cnt, s_bcast, bin, L);  // uniform over the workgroup
   int64_t *oi = out_ids + (int64_t)row * k;
   float *ov = out_vals ? out_vals + (int64_t)row * k : nullptr;
+  if (SORTED && lin && L.max_winners <= kLinRankMax) {
+    // counting sort: a key of a bin above b* takes a slot of [off[b], off[b] + count[b]) and the keys of b* go to
+    // a list of their own; then every key counts the larger keys of its own bin, which is its place inside the
+    // bin, and is written there (of b* only the first `need`)
+    const uint32_t *s_off = s_hist + 256;
+#pragma unroll
+    for (int e = 0; e < EIN; ++e) {
+      if (v[e] != 0ull) {
+        if (bin[e] > L.bstar) s_keys[atomicAdd(&s_cnt[bin[e]], 1u)] = v[e];
+        else if (bin[e] == L.bstar) s_bucket[atomicAdd(&s_bcast[6], 1u)] = v[e];
+      }
+    }
+    __syncthreads();
+    const uint32_t n_above = (uint32_t)k - L.need;
+    for (uint32_t p = tid; p < n_above; p += kTopkThreads) {
+      const uint64_t key = s_keys[p];
+      const uint32_t b = lin_bin(key, L.lo, L.scale);
+      const uint32_t start = s_off[b], cnt = s_cnt[b] - start;
+      uint32_t r = 0;
+#pragma unroll 4
+      for (uint32_t j = 0; j < cnt; ++j) r += s_keys[start + j] > key ? 1u : 0u;
+      oi[start + r] = (int64_t)(uint32_t)(~(uint32_t)key);
+      if (ov) ov[start + r] = pkv_from_ordered_u32((uint32_t)(key >> 32));
+    }
+    for (uint32_t i = kTopkThreads - 1 - tid; i < L.in_bstar; i += kTopkThreads) {  // the last threads: they have the fewest slots above
+      const uint64_t key = s_bucket[i];
+      uint32_t r = 0;
+#pragma unroll 4
+      for (uint32_t j = 0; j < L.in_bstar; ++j) r += s_bucket[j] > key ? 1u : 0u;
+      if (r < L.need) {
+        oi[n_above + r] = (int64_t)(uint32_t)(~(uint32_t)key);
+        if (ov) ov[n_above + r] = pkv_from_ordered_u32((uint32_t)(key >> 32));
+      }
+    }
+    return;
+  }
+  if (lin) {
+    linear_threshold<EIN>(v, bin, s_bcast, s_bucket, &s_T, L);
+#pragma unroll
+    for (int e = 0; e < EIN; ++e) win[e] = v[e] != 0ull && (bin[e] > L.bstar || (bin[e] == L.bstar && v[e] >= L.T));
+  } else {
+    uint64_t prefix;
+    int shift;
+    radix_select_regs<EIN>(v, (uint32_t)k, s_hist, s_bcast, prefix, shift);
+#pragma unroll
+    for (int e = 0; e < EIN; ++e) win[e] = (v[e] >> shift) >= (prefix >> shift) && v[e] != 0ull;
+  }
   if (!SORTED) {
     int mine = 0;
 #pragma unroll
-    for (int e = 0; e < EIN; ++e) mine += (v[e] >> shift) >= (prefix >> shift) && v[e] != 0ull;
+    for (int e = 0; e < EIN; ++e) mine += win[e];
     int total;
+    __syncthreads();  // the histograms have been read by everyone
     int slot = pkv_block_excl_scan<kTopkThreads>(mine, (int *)s_hist, total);  // s_hist is free again
 #pragma unroll
     for (int e = 0; e < EIN; ++e) {
-      if ((v[e] >> shift) >= (prefix >> shift) && v[e] != 0ull) {
+      if (win[e]) {
         if (slot < k) {
           oi[slot] = (int64_t)(uint32_t)(~(uint32_t)v[e]);
           if (ov) ov[slot] = pkv_from_ordered_u32((uint32_t)(v[e] >> 32));
@@ -634,9 +822,8 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
   }
 #pragma unroll
   for (int e = 0; e < EIN; ++e) {
-    const bool win = (v[e] >> shift) >= (prefix >> shift) && v[e] != 0ull;
-    const uint32_t slot = wave_take_slots(&s_counter, win);
-    if (win && slot < (uint32_t)k) s_keys[slot] = v[e];
+    const uint32_t slot = wave_take_slots(&s_counter, win[e]);
+    if (win[e] && slot < (uint32_t)k) s_keys[slot] = v[e];
   }
   __syncthreads();
 #define PKV_SORT_K(NT, E) sort_lds_keys_and_emit<NT, E>(s_keys, k, oi, ov, nullptr)

@@ -339,6 +339,46 @@ def test_topk_f32_exact(ops, rows, L, k):
     assert torch.equal(vals, tv)
 
 
+def test_topk_f32_one_workgroup_score_distributions(ops):
+    """Rows that one workgroup selects from (at most 8192 scores, k at most half of them) on score distributions
+    that steer the kernel through each of its routes: evenly spread scores (bins of the row's own range, counting
+    sort), a crowded winner bin (same bins, bitonic sort), a crowded threshold bin, a constant row, an outlier that
+    stretches the range, infinities (radix select), exact ties decided by the ids, padded rows and k = 1."""
+    rng = np.random.default_rng(2024)
+    cases = []
+    cases.append(("gaussian", rng.standard_normal((4, 4096)).astype(np.float32) * 20 + 30, 1024))
+    x = rng.standard_normal((3, 4096)).astype(np.float32)
+    x[:, 100:400] = np.float32(5.0)                                   # 300 winners in one bin
+    cases.append(("crowded winner bin", x, 1024))
+    x = rng.standard_normal((3, 4096)).astype(np.float32)
+    x[:, :2000] = np.float32(0.5) + rng.integers(0, 3, (3, 2000)).astype(np.float32) * np.float32(2.0 ** -22)
+    cases.append(("crowded threshold bin", x, 1500))
+    cases.append(("constant", np.full((2, 4096), -3.5, np.float32), 700))
+    x = rng.standard_normal((2, 4096)).astype(np.float32)
+    x[0, 17], x[1, 4000] = 1e6, -1e6
+    cases.append(("outlier", x, 1024))
+    x = (rng.standard_normal((2, 4096)) * 100).astype(np.float32)
+    x[0, 5], x[0, 77], x[1, 4095] = np.inf, -np.inf, np.inf
+    cases.append(("infinities", x, 1000))
+    cases.append(("ties by id", np.round(rng.standard_normal((3, 4096)) * 16).astype(np.float32) / 16, 1024))
+    cases.append(("negative scores", -np.abs(rng.standard_normal((2, 4096))).astype(np.float32) - 1, 1024))
+    cases.append(("padded row", rng.standard_normal((5, 3000)).astype(np.float32), 1))
+    cases.append(("padded row, k=1500", rng.standard_normal((2, 3001)).astype(np.float32), 1500))
+    cases.append(("2 keys per thread", rng.standard_normal((2, 2048)).astype(np.float32), 1024))
+    cases.append(("8 keys per thread", rng.standard_normal((2, 8192)).astype(np.float32) ** 3, 4096))
+    cases.append(("subnormal range", (rng.integers(0, 50, (2, 4096)).astype(np.float32) * np.float32(1e-45)), 512))
+    for name, x, k in cases:
+        _say(f"topk_f32 one workgroup: {name} {x.shape} k={k}")
+        rows, L = x.shape
+        ids = np.stack([rng.permutation(3 * L)[:L] for _ in range(rows)]).astype(np.int64)
+        out, vals = ops.topk_f32(torch.from_numpy(x).to(DEV), k, torch.from_numpy(ids).to(DEV), want_values=True)
+        torch.cuda.synchronize()
+        for r in range(rows):
+            ref_ids, ref_pos = O.topk_f32(x[r], ids[r], k)
+            assert np.array_equal(out[r].cpu().numpy(), ref_ids), name
+            assert np.array_equal(vals[r].cpu().numpy().view(np.uint32), x[r][ref_pos].view(np.uint32)), name
+
+
 def test_topk_f32_wide_rows_edge_cases(ops):
     """Rows wider than one workgroup sorts (more than 8192 keys): the multi-workgroup histogram / compaction
     path with a threshold bin that holds the whole row (constant scores: every key ties, ids decide), one that
