@@ -49,15 +49,16 @@ __device__ __forceinline__ int popc4(const uint32_t (&m)[4]) {
 // chunk_suf[row][c][t] = the same for chunk c alone.  theta = largest t with row_suf[t] >= k;
 // base_gt = keys above theta in earlier chunks; base_eq = (keys above theta in the row) + keys at
 // theta in earlier chunks.  Two dependent loads, no loops over bins.
-__device__ __forceinline__ void select_prologue(const uint32_t *__restrict__ row_suf,
-                                                const uint16_t *__restrict__ chunk_suf, int row, int chunk,
-                                                int n_chunks, int64_t k, uint32_t &theta, int64_t &base_gt,
+// rs_mine = row_suf[row][tid] for tid < 128, loaded by the caller as its first instruction so that the load is in
+// flight while the caller sets up whatever else it needs before the threshold.
+__device__ __forceinline__ void select_prologue(uint32_t rs_mine, const uint16_t *__restrict__ chunk_suf, int row,
+                                                int chunk, int n_chunks, int64_t k, uint32_t &theta, int64_t &base_gt,
                                                 int64_t &base_eq) {
   __shared__ uint32_t s_rs[129];
   __shared__ uint32_t s_theta, s_ngt;
   __shared__ uint32_t s_red[2][kSelThreads / PKV_WAVE];
   const int tid = threadIdx.x;
-  if (tid < 128) s_rs[tid] = row_suf[(int64_t)row * 128 + tid];
+  if (tid < 128) s_rs[tid] = rs_mine;
   if (tid == 128) {
     s_rs[128] = 0;
     s_theta = 0;
@@ -115,11 +116,12 @@ __global__ __launch_bounds__(kSelThreads) void pkv_select_kernel(const uint8_t *
   const int64_t chunk_end = (chunk_begin + chunk_keys < n_keys) ? chunk_begin + chunk_keys : n_keys;
   const pkv_u32x4 zero4 = {0u, 0u, 0u, 0u};
   int64_t i0 = chunk_begin + (int64_t)tid * kSelKeysPerThread;
+  const uint32_t rs_mine = tid < 128 ? row_suf[(int64_t)row * 128 + tid] : 0u;
   pkv_u32x4 w = i0 < chunk_end ? *(const pkv_u32x4 *)(crow + i0) : zero4;  // padded rows: always in bounds
 
   uint32_t theta;
   int64_t base_gt, base_eq;
-  select_prologue(row_suf, chunk_suf, row, chunk, gridDim.x, k, theta, base_gt, base_eq);
+  select_prologue(rs_mine, chunk_suf, row, chunk, gridDim.x, k, theta, base_gt, base_eq);
   int64_t *orow = out + (int64_t)row * k;
 
   int it = 0;
@@ -183,13 +185,14 @@ __global__ __launch_bounds__(kSelThreads) void pkv_select_rerank_kernel(
   const int64_t chunk_end = (chunk_begin + chunk_keys < n_keys) ? chunk_begin + chunk_keys : n_keys;
   const pkv_u32x4 zero4 = {0u, 0u, 0u, 0u};
   int64_t i0 = chunk_begin + (int64_t)tid * kSelKeysPerThread;
-  pkv_u32x4 w = i0 < chunk_end ? *(const pkv_u32x4 *)(crow + i0) : zero4;  // before the threshold is known
+  const uint32_t rs_mine = tid < 128 ? row_suf[(int64_t)row * 128 + tid] : 0u;  // both before the threshold is known
+  pkv_u32x4 w = i0 < chunk_end ? *(const pkv_u32x4 *)(crow + i0) : zero4;
+  const float qn = qnorm[row];
 
   pkv_build_prod_table<kSelThreads>(s_prod, qhat + (int64_t)row * 128, centers);
-  const float qn = qnorm[row];
   uint32_t theta;
   int64_t base_gt, base_eq;
-  select_prologue(row_suf, chunk_suf, row, chunk, gridDim.x, k, theta, base_gt, base_eq);
+  select_prologue(rs_mine, chunk_suf, row, chunk, gridDim.x, k, theta, base_gt, base_eq);
   int64_t *orow = out + (int64_t)row * k;
   float *srow = scores + (int64_t)row * k;
   const uint8_t *nrow = nib + (int64_t)b * ns_b + (int64_t)h * ns_h;
@@ -556,25 +559,36 @@ __device__ __forceinline__ void radix_select_regs(const uint64_t (&v)[EIN], uint
 // result is the same set in the same order either way.
 constexpr int kLinBucketMax = 256;
 constexpr int kLinRankMax = 128;
+constexpr int kCountingSortMaxP = 2048;  // largest winner list whose counting sort (a second copy in LDS) is set up
 
 struct LinSel {
-  float lo, scale;
+  float lo, scale;        // value bins: bin = floor((x - lo) * scale)
+  uint32_t lo_bits;       // bit bins: bin = (ordered bits of x - lo_bits) >> shift, piecewise logarithmic in x
+  int shift;              // < 0: value bins
   uint32_t bstar, need;   // threshold bin, keys needed from it
   uint32_t in_bstar;      // keys in the threshold bin
   uint32_t max_winners;   // most winners in one bin
   uint64_t T;             // threshold key inside bin b* (0: the whole bin wins); set by linear_threshold
 };
 
-__device__ __forceinline__ uint32_t lin_bin(uint64_t key, float lo, float scale) {
-  const float t = (pkv_from_ordered_u32((uint32_t)(key >> 32)) - lo) * scale;
-  const uint32_t b = (uint32_t)t;
+__device__ __forceinline__ uint32_t lin_bin(uint64_t key, const LinSel &L) {
+  uint32_t b;
+  if (L.shift >= 0) {
+    b = ((uint32_t)(key >> 32) - L.lo_bits) >> L.shift;
+  } else {
+    const float t = (pkv_from_ordered_u32((uint32_t)(key >> 32)) - L.lo) * L.scale;
+    b = (uint32_t)t;
+  }
   return b > 255u ? 255u : b;
 }
 
 // Bins of the thread's keys and the threshold bin.  On return s_hist[0,256) = keys per bin, s_hist[256,512) =
 // off[b] = keys in the bins above b, s_cnt[b] = off[b] (a running output slot for the counting sort), s_bcast[6] = 0.
 // s_hist: 512 words, s_cnt: 256 words, s_bcast: 8 words.  All 1024 threads call it; false = not applicable.
-template <int EIN>
+// BITS: bins of the ordered key bits instead of the values, for rows of one sign whose values span many binades
+// (e.g. the winners of a selection, about to be sorted): 256 equal steps of the bit pattern between the row's
+// smallest and largest key, i.e. equal steps of the logarithm up to the mantissa's linear pieces.
+template <int EIN, bool BITS = false>
 __device__ __forceinline__ bool linear_bins(const uint64_t (&v)[EIN], uint32_t k, uint32_t *s_hist, uint32_t *s_cnt,
                                             uint32_t *s_bcast, uint32_t (&bin)[EIN], LinSel &L) {
   const int tid = threadIdx.x, lane = pkv_lane();
@@ -604,16 +618,24 @@ __device__ __forceinline__ bool linear_bins(const uint64_t (&v)[EIN], uint32_t k
   }
   __syncthreads();
   mx = s_bcast[0], mn = s_bcast[1];
-  const float hi = pkv_from_ordered_u32(mx), lo = pkv_from_ordered_u32(mn);
-  const float range = hi - lo, scale = 256.0f / range;
-  const float inf = __uint_as_float(0x7f800000u);
-  // finite scores (ordered keys strictly between those of -inf and +inf), a positive finite range and scale
-  if (!(mx < 0xff800000u && mn > 0x007fffffu && range > 0.f && range < inf && scale < inf)) return false;
+  L.lo = 0.f, L.scale = 0.f, L.lo_bits = mn, L.shift = -1;
+  if (BITS) {
+    if (mx <= mn) return false;  // one value (or no key at all)
+    const int width = 32 - __clz((int)(mx - mn));
+    L.shift = width > 8 ? width - 8 : 0;
+  } else {
+    const float hi = pkv_from_ordered_u32(mx), lo = pkv_from_ordered_u32(mn);
+    const float range = hi - lo, scale = 256.0f / range;
+    const float inf = __uint_as_float(0x7f800000u);
+    // finite scores (ordered keys strictly between those of -inf and +inf), a positive finite range and scale
+    if (!(mx < 0xff800000u && mn > 0x007fffffu && range > 0.f && range < inf && scale < inf)) return false;
+    L.lo = lo, L.scale = scale;
+  }
 #pragma unroll
   for (int e = 0; e < EIN; ++e) {
     bin[e] = 0;
     if (v[e] != 0ull) {
-      bin[e] = lin_bin(v[e], lo, scale);
+      bin[e] = lin_bin(v[e], L);
       atomicAdd(&s_hist[bin[e]], 1u);
     }
   }
@@ -644,7 +666,6 @@ __device__ __forceinline__ bool linear_bins(const uint64_t (&v)[EIN], uint32_t k
     if ((tid & 15) == 0) atomicMax(&s_bcast[5], most);
   }
   __syncthreads();
-  L.lo = lo, L.scale = scale;
   L.bstar = s_bcast[2], L.need = s_bcast[3], L.in_bstar = s_bcast[4], L.max_winners = s_bcast[5];
   L.T = 0ull;
   return L.in_bstar <= kLinBucketMax;
@@ -674,6 +695,82 @@ __device__ __forceinline__ void linear_threshold(const uint64_t (&v)[EIN], const
   }
   __syncthreads();
   L.T = *s_T;
+}
+
+// LDS scratch of a selection / sort over one workgroup's keys.
+struct SelSmem {
+  uint32_t hist[512];
+  uint32_t cnt[256];
+  uint32_t bcast[8];
+  uint32_t counter;
+  uint64_t bucket[kLinBucketMax];
+  uint64_t T;
+};
+
+// win[e] = key e of this thread is one of the k largest of the workgroup's keys (zero keys never are).  Bins of
+// the row's own range first (BITS: of the ordered key bits), the radix select where they do not apply.
+template <int EIN, bool BITS>
+__device__ __forceinline__ void select_topk_flags(const uint64_t (&v)[EIN], uint32_t k, SelSmem &sm, bool (&win)[EIN]) {
+  uint32_t bin[EIN];
+  LinSel L;
+  if (linear_bins<EIN, BITS>(v, k, sm.hist, sm.cnt, sm.bcast, bin, L)) {
+    linear_threshold<EIN>(v, bin, sm.bcast, sm.bucket, &sm.T, L);
+#pragma unroll
+    for (int e = 0; e < EIN; ++e) win[e] = v[e] != 0ull && (bin[e] > L.bstar || (bin[e] == L.bstar && v[e] >= L.T));
+  } else {
+    uint64_t prefix;
+    int shift;
+    radix_select_regs<EIN>(v, k, sm.hist, sm.bcast, prefix, shift);
+#pragma unroll
+    for (int e = 0; e < EIN; ++e) win[e] = v[e] != 0ull && (v[e] >> shift) >= (prefix >> shift);
+  }
+}
+
+// Descending sort of the n nonzero keys held E per thread (all other entries zero) into s_out[0 .. n), through
+// s_tmp (n keys, not s_out): 256 bins of the ordered key bits between the smallest and the largest key, every key
+// placed at (keys in higher bins) + (larger keys in its own bin).  False, with nothing written, when a bin holds
+// more than kLinRankMax keys or all keys are equal: the caller then sorts by compare-exchange.
+template <int E>
+__device__ __forceinline__ bool counting_sort_desc(const uint64_t (&v)[E], uint32_t n, uint64_t *s_tmp, uint64_t *s_out,
+                                                   SelSmem &sm) {
+  uint32_t bin[E];
+  LinSel L;
+  if (!linear_bins<E, true>(v, n, sm.hist, sm.cnt, sm.bcast, bin, L) || L.max_winners > kLinRankMax) return false;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    if (v[e] != 0ull) s_tmp[atomicAdd(&sm.cnt[bin[e]], 1u)] = v[e];
+  }
+  __syncthreads();
+  const uint32_t *s_off = sm.hist + 256;
+  for (uint32_t p = threadIdx.x; p < n; p += kTopkThreads) {
+    const uint64_t key = s_tmp[p];
+    const uint32_t b = lin_bin(key, L);
+    const uint32_t start = s_off[b], cnt = sm.cnt[b] - start;
+    uint32_t r = 0;
+#pragma unroll 4
+    for (uint32_t j = 0; j < cnt; ++j) r += s_tmp[start + j] > key ? 1u : 0u;
+    s_out[start + r] = key;
+  }
+  __syncthreads();
+  return true;
+}
+
+// s_keys[0 .. P) (the n winners, any order, zero padded) sorted descending in place; s_tmp: P more keys or null.
+template <int NT, int E>
+__device__ __forceinline__ void sort_lds_keys_desc(uint64_t *s_keys, uint32_t n, uint64_t *s_tmp, SelSmem &sm) {
+  const bool active = threadIdx.x < NT;
+  uint64_t v[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) v[e] = active ? s_keys[threadIdx.x * E + e] : 0ull;
+  __syncthreads();
+  if (s_tmp && counting_sort_desc<E>(v, n, s_tmp, s_keys, sm)) return;
+  bitonic_sort_desc_regs<NT, E>(v, s_keys);
+  __syncthreads();
+  if (active) {
+#pragma unroll
+    for (int e = 0; e < E; ++e) s_keys[threadIdx.x * E + e] = v[e];
+  }
+  __syncthreads();
 }
 
 // The same selection over keys that do not fit the registers: key_of(i), i < len, is evaluated again
@@ -770,7 +867,7 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
     const uint32_t n_above = (uint32_t)k - L.need;
     for (uint32_t p = tid; p < n_above; p += kTopkThreads) {
       const uint64_t key = s_keys[p];
-      const uint32_t b = lin_bin(key, L.lo, L.scale);
+      const uint32_t b = lin_bin(key, L);
       const uint32_t start = s_off[b], cnt = s_cnt[b] - start;
       uint32_t r = 0;
 #pragma unroll 4
@@ -934,7 +1031,8 @@ __device__ __forceinline__ void wide_compact_slice(const uint64_t (&keys)[kWideE
 __device__ __forceinline__ void wide_finish_select(uint32_t k, int P, const uint32_t *__restrict__ ctl,
                                                    const uint64_t *__restrict__ list_a,
                                                    const uint64_t *__restrict__ list_b, int64_t len, uint64_t *s_keys,
-                                                   uint32_t *s_hist, uint32_t *s_bcast, uint32_t *s_counter) {
+                                                   SelSmem &sm) {
+  uint32_t *s_hist = sm.hist, *s_bcast = sm.bcast, *s_counter = &sm.counter;
   const int tid = threadIdx.x;
   uint32_t n_a = ctl[kWideBins], n_b = ctl[kWideBins + 1];
   if (n_a > k) n_a = k;  // cannot happen with a consistent histogram; keeps every index in range
@@ -951,14 +1049,17 @@ __device__ __forceinline__ void wide_finish_select(uint32_t k, int P, const uint
       const uint32_t i = (uint32_t)(tid + e * kTopkThreads);
       v[e] = i < n_b ? list_b[i] : 0ull;
     }
-    uint64_t prefix = 0;
-    int shift = 0;
-    if (need < n_b) radix_select_regs<8>(v, need, s_hist, s_bcast, prefix, shift);  // else: all of B
+    bool win[8];
+    if (need < n_b) {
+      select_topk_flags<8, true>(v, need, sm, win);  // list B shares its leading bits: bins of the remaining ones
+    } else {  // all of B
+#pragma unroll
+      for (int e = 0; e < 8; ++e) win[e] = v[e] != 0ull;
+    }
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const bool win = v[e] != 0ull && (v[e] >> shift) >= (prefix >> shift);
-      const uint32_t slot = wave_take_slots(s_counter, win);
-      if (win && slot < k) s_keys[slot] = v[e];
+      const uint32_t slot = wave_take_slots(s_counter, win[e]);
+      if (win[e] && slot < k) s_keys[slot] = v[e];
     }
   } else {
     auto key_of = [&](int64_t i) { return list_b[i]; };
@@ -995,22 +1096,26 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_wide_compact_kernel(
                          list_b + (int64_t)row * len, s_tmp);
 }
 
-// grid rows; dynamic LDS max(P,1024)*8 bytes.
+// grid rows; dynamic LDS lds_bytes_sort(P): the winners, and as many keys again for the counting sort when they fit.
 __global__ __launch_bounds__(kTopkThreads) void pkv_topk_wide_finish_kernel(
     int64_t len, int P, int64_t k, const uint32_t *__restrict__ ctl, const uint64_t *__restrict__ list_a,
     const uint64_t *__restrict__ list_b, int64_t *__restrict__ out_ids, float *__restrict__ out_vals) {
   extern __shared__ uint64_t s_keys[];
-  __shared__ uint32_t s_hist[512];
-  __shared__ uint32_t s_bcast[8];
-  __shared__ uint32_t s_counter;
+  __shared__ SelSmem sm;
+  uint64_t *s_tmp = P <= kCountingSortMaxP ? s_keys + (P < 1024 ? 1024 : P) : nullptr;
   const int row = blockIdx.x;
   wide_finish_select((uint32_t)k, P, ctl + (int64_t)row * kWideRowWords, list_a + (int64_t)row * k,
-                     list_b + (int64_t)row * len, len, s_keys, s_hist, s_bcast, &s_counter);
+                     list_b + (int64_t)row * len, len, s_keys, sm);
   int64_t *oi = out_ids + (int64_t)row * k;
   float *ov = out_vals ? out_vals + (int64_t)row * k : nullptr;
-#define PKV_SORT_K(NT, E) sort_lds_keys_and_emit<NT, E>(s_keys, k, oi, ov, nullptr)
+#define PKV_SORT_K(NT, E) sort_lds_keys_desc<NT, E>(s_keys, (uint32_t)k, s_tmp, sm)
   PKV_DISPATCH_E(P, PKV_SORT_K);
 #undef PKV_SORT_K
+  for (int64_t i = threadIdx.x; i < k; i += kTopkThreads) {
+    const uint64_t key = s_keys[i];
+    oi[i] = (int64_t)(uint32_t)(~(uint32_t)key);
+    if (ov) ov[i] = pkv_from_ordered_u32((uint32_t)(key >> 32));
+  }
 }
 
 // ------------------------------------------------------------------ adaptive-k
@@ -1200,10 +1305,13 @@ struct AdkClamp {
 __device__ __forceinline__ void adaptive_tail(uint64_t *s_keys, int P, int64_t k_out, float sl_benefit, float total,
                                               float threshold, const int64_t *__restrict__ ci, int64_t n_cand,
                                               int64_t *__restrict__ adaptive_k_row, int64_t *__restrict__ ids_row,
-                                              AdkClamp cl, int row, float *s_f, uint32_t *s_k) {
-#define PKV_SORT_K(NT, E) sort_lds_keys_and_emit<NT, E>(s_keys, 0, nullptr, nullptr, s_keys)
+                                              AdkClamp cl, int row, SelSmem &sm) {
+  uint64_t *s_tmp = P <= kCountingSortMaxP ? s_keys + (P < 1024 ? 1024 : P) : nullptr;
+#define PKV_SORT_K(NT, E) sort_lds_keys_desc<NT, E>(s_keys, (uint32_t)k_out, s_tmp, sm)
   PKV_DISPATCH_E(P, PKV_SORT_K);
 #undef PKV_SORT_K
+  float *s_f = (float *)sm.hist;
+  uint32_t *s_k = &sm.counter;
   int64_t k = 1;  // total <= 0: adaptive_topk.py:304-306
   if (total > 0.f) k = first_k_reaching(s_keys, k_out, sl_benefit, threshold * total, s_f, s_k);
   if (threadIdx.x == 0) {
@@ -1254,9 +1362,7 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adaptive_topk_kernel(
     int64_t *__restrict__ adaptive_k, int64_t *__restrict__ topk_ids, AdkClamp cl) {
   extern __shared__ uint64_t s_keys[];
   __shared__ float s_part[16];
-  __shared__ uint32_t s_hist[512];
-  __shared__ uint32_t s_bcast[8];
-  __shared__ uint32_t s_counter;
+  __shared__ SelSmem sm;
   const int row = blockIdx.x;
   const int tid = threadIdx.x;
   const AdkRow r = adk_row(row, sl_logits, sl_stride, sl_vnorm, slv_stride, cand_scores, cand_dtype, cand_vnorm,
@@ -1289,21 +1395,24 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adaptive_topk_kernel(
   const float total = sl_benefit + block_tree_sum_1024(acc, s_part);
 
   // the k_out largest (benefit, ~position) keys
-  if (tid == 0) s_counter = 0;
+  if (tid == 0) sm.counter = 0;
   for (int i = tid; i < (P < 1024 ? 1024 : P); i += kTopkThreads) s_keys[i] = 0ull;
-  uint64_t prefix = 0;
-  int shift = 0;
-  if (k_out < n_cand) radix_select_regs<EIN>(v, (uint32_t)k_out, s_hist, s_bcast, prefix, shift);
-  else __syncthreads();
+  bool win[EIN];
+  if (k_out < n_cand) {
+    select_topk_flags<EIN, true>(v, (uint32_t)k_out, sm, win);  // benefits span many binades: bins of the key bits
+  } else {
+#pragma unroll
+    for (int e = 0; e < EIN; ++e) win[e] = v[e] != 0ull;
+    __syncthreads();
+  }
 #pragma unroll
   for (int e = 0; e < EIN; ++e) {
-    const bool win = v[e] != 0ull && (v[e] >> shift) >= (prefix >> shift);
-    const uint32_t slot = wave_take_slots(&s_counter, win);
-    if (win && slot < (uint32_t)k_out) s_keys[slot] = v[e];
+    const uint32_t slot = wave_take_slots(&sm.counter, win[e]);
+    if (win[e] && slot < (uint32_t)k_out) s_keys[slot] = v[e];
   }
   __syncthreads();
   adaptive_tail(s_keys, P, k_out, sl_benefit, total, threshold, r.ci, n_cand, adaptive_k + row,
-                topk_ids + (int64_t)row * k_out, cl, row, (float *)s_hist, &s_counter);
+                topk_ids + (int64_t)row * k_out, cl, row, sm);
 }
 
 // ---- n_cand > 8192: slices of 8192 candidates, one workgroup each ----
@@ -1436,9 +1545,7 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adk_finish_kernel(
     int64_t *__restrict__ topk_ids, AdkClamp cl) {
   extern __shared__ uint64_t s_keys[];
   __shared__ float s_part[16];
-  __shared__ uint32_t s_hist[512];
-  __shared__ uint32_t s_bcast[8];
-  __shared__ uint32_t s_counter;
+  __shared__ SelSmem sm;
   const int row = blockIdx.x;
   float g, csum;
   combine_slices(ws_max + (int64_t)row * n_parts, n_parts, ws_sum + (int64_t)row * n_slices, n_slices, s_part, g, csum);
@@ -1446,9 +1553,9 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adk_finish_kernel(
                                              sl, g, s_part);
   const float total = sl_benefit + csum;
   wide_finish_select((uint32_t)k_out, P, ctl + (int64_t)row * kWideRowWords, list_a + (int64_t)row * k_out,
-                     list_b + (int64_t)row * n_cand, n_cand, s_keys, s_hist, s_bcast, &s_counter);
+                     list_b + (int64_t)row * n_cand, n_cand, s_keys, sm);
   adaptive_tail(s_keys, P, k_out, sl_benefit, total, threshold, cand_ids + (int64_t)row * n_cand, n_cand,
-                adaptive_k + row, topk_ids + (int64_t)row * k_out, cl, row, (float *)s_hist, &s_counter);
+                adaptive_k + row, topk_ids + (int64_t)row * k_out, cl, row, sm);
 }
 
 // uniform_k[r] = max over all rows of adaptive_k, row_keys[r] = base + that maximum: the dense form of the
@@ -1519,6 +1626,8 @@ __global__ __launch_bounds__(kDenseLogitThreads) void pkv_dense_logits_kernel(
 }
 
 static size_t lds_bytes(int P) { return (size_t)(P < 1024 ? 1024 : P) * 8; }
+// with room for the counting sort's second copy of the winners where the kernels use it
+static size_t lds_bytes_sort(int P) { return lds_bytes(P) * (P <= kCountingSortMaxP ? 2 : 1); }
 
 static int pow2_ceil(int64_t v) {
   int p = 1;
@@ -1702,7 +1811,7 @@ int pkv_launch_topk_f32(const float *x, int64_t x_stride, const int64_t *ids, in
     hipLaunchKernelGGL(pkv_topk_wide_compact_kernel, grid, dim3(kTopkThreads), 0, s, x, x_stride, ids, ids_stride, len, k,
                        ctl, list_a, list_b);
     PKV_LAUNCH_CHECK("pkv_topk_wide_compact_kernel");
-    hipLaunchKernelGGL(pkv_topk_wide_finish_kernel, dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes(P), s, len, P, k,
+    hipLaunchKernelGGL(pkv_topk_wide_finish_kernel, dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes_sort(P), s, len, P, k,
                        ctl, list_a, list_b, out_ids, out_vals);
     PKV_LAUNCH_CHECK("pkv_topk_wide_finish_kernel");
   }
@@ -1768,7 +1877,7 @@ extern "C" int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, cons
   if (n_cand <= kTopkMaxSort) {  // one workgroup per row, no workspace
     const int ein = pow2_ceil(n_cand) / kTopkThreads;
 #define PKV_ADK(EIN)                                                                                                  \
-  hipLaunchKernelGGL((pkv_adaptive_topk_kernel<EIN>), dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes(P), s,      \
+  hipLaunchKernelGGL((pkv_adaptive_topk_kernel<EIN>), dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes_sort(P), s,      \
                      sl_logits, sl_stride, sl_vnorm, slv_stride, sl, cand_scores, cand_dtype, cand_scale, cand_vnorm, \
                      value_norm, vn_stride, vn_offset, vn_pos_stride, cand_ids, (int)n_cand, threshold, k_out, P,     \
                      adaptive_k, topk_ids, cl)
@@ -1799,7 +1908,7 @@ extern "C" int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, cons
   PKV_LAUNCH_CHECK("pkv_adk_benefit_kernel");
   hipLaunchKernelGGL(pkv_adk_compact_kernel, grid, dim3(kTopkThreads), 0, s, ben, n_cand, k_out, ctl, list_a, list_b);
   PKV_LAUNCH_CHECK("pkv_adk_compact_kernel");
-  hipLaunchKernelGGL(pkv_adk_finish_kernel, dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes(P), s, sl_logits,
+  hipLaunchKernelGGL(pkv_adk_finish_kernel, dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes_sort(P), s, sl_logits,
                      sl_stride, sl_vnorm, slv_stride, sl, cand_ids, n_cand, n_slices, n_parts, threshold, k_out, P, smax, ssum,
                      ctl,
                      list_a, list_b, adaptive_k, topk_ids, cl);
