@@ -82,16 +82,19 @@ PKV_INTERNAL int pkv_launch_select_rerank(const uint8_t *cnt_u8, int64_t cnt_str
                                           const uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key,
                                           const float *qhat, const float *qnorm, const float *centers, int64_t *cand,
                                           float *scores, hipStream_t s, int64_t extra_off = 0,
-                                          float *extra_out = nullptr);
+                                          float *extra_out = nullptr, uint32_t *zero_ptr = nullptr,
+                                          int64_t zero_words = 0);
 PKV_INTERNAL int pkv_launch_rerank(const int64_t *cand, int bs, int n_kv_heads, int64_t n_cand, int64_t n_keys,
                                    const uint8_t *nib, int64_t ns_b, int64_t ns_h, int64_t ns_key, int64_t ns_sub,
                                    const uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key,
                                    int64_t ws_sub, const float *qhat, const float *qnorm, const float *centers,
                                    float *scores, uint16_t *v4b, hipStream_t s);
 PKV_INTERNAL size_t pkv_topk_ws_bytes_impl(int rows, int64_t len, int64_t k);
+PKV_INTERNAL int64_t pkv_topk_ctl_words(int rows, int64_t len);
 PKV_INTERNAL int pkv_launch_topk_f32(const float *x, int64_t x_stride, const int64_t *ids, int64_t ids_stride,
                                      int rows, int64_t len, int64_t k, int64_t *out_ids, float *out_vals,
-                                     void *ws, size_t ws_bytes, hipStream_t s, bool any_order = false);
+                                     void *ws, size_t ws_bytes, hipStream_t s, bool any_order = false,
+                                     bool ctl_cleared = false);
 PKV_INTERNAL int pkv_launch_gather(const void *src_k, const void *src_v, int64_t src_len, const int64_t *idx,
                                    int64_t k, int64_t idx_offset, void *dst_k, void *dst_v, int64_t dst_len,
                                    int64_t dst_row0, int rows, int row_bytes, hipStream_t s, const int64_t *row_counts = nullptr);

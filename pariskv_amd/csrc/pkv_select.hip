@@ -169,11 +169,15 @@ __global__ __launch_bounds__(kSelThreads) void pkv_select_rerank_kernel(
     const uint8_t *__restrict__ nib, int64_t ns_b, int64_t ns_h, int ns_key, const uint16_t *__restrict__ weight,
     int64_t ws_b, int64_t ws_h, int ws_key, const float *__restrict__ qhat, const float *__restrict__ qnorm,
     const float *__restrict__ centers, int64_t *__restrict__ out, float *__restrict__ scores, int extra_off,
-    float *__restrict__ extra_out) {
+    float *__restrict__ extra_out, uint32_t *__restrict__ zero_ptr, int64_t zero_words) {
   const int row = blockIdx.y;
   const int chunk = blockIdx.x;
   const int tid = threadIdx.x;
   const int b = row / n_kv_heads, h = row % n_kv_heads;
+  // words the next launch of the step wants cleared (the control blocks of a multi-workgroup top-k): spread over the launch
+  for (int64_t i = ((int64_t)row * gridDim.x + chunk) * kSelThreads + tid; i < zero_words;
+       i += (int64_t)gridDim.x * gridDim.y * kSelThreads)
+    zero_ptr[i] = 0u;
 
   __shared__ int s_scan[2][kSelThreads / PKV_WAVE];
   __shared__ float s_prod[128 * 16];
@@ -1657,7 +1661,7 @@ int pkv_launch_select_rerank(const uint8_t *cnt_u8, int64_t cnt_stride, const ui
                              int n_kv_heads, int64_t n_keys, int64_t k, const uint8_t *nib, int64_t ns_b, int64_t ns_h,
                              int64_t ns_key, const uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key,
                              const float *qhat, const float *qnorm, const float *centers, int64_t *cand, float *scores,
-                             hipStream_t s, int64_t extra_off, float *extra_out) {
+                             hipStream_t s, int64_t extra_off, float *extra_out, uint32_t *zero_ptr, int64_t zero_words) {
   PKV_REQUIRE(!extra_out || (extra_off >= 0 && extra_off % 4 == 0 && extra_off + 4 <= ns_key),
               "the extra word must lie inside the key's record (offset %lld, record %lld bytes)", (long long)extra_off,
               (long long)ns_key);
@@ -1674,7 +1678,7 @@ int pkv_launch_select_rerank(const uint8_t *cnt_u8, int64_t cnt_stride, const ui
   hipLaunchKernelGGL(pkv_select_rerank_kernel, grid, dim3(kSelThreads), 0, s, cnt_u8, cnt_stride, row_suf, chunk_suf,
                      chunk_keys,
                      n_kv_heads, n_keys, k, nib, ns_b, ns_h, (int)ns_key, weight, ws_b, ws_h, (int)ws_key, qhat, qnorm,
-                     centers, cand, scores, (int)extra_off, extra_out);
+                     centers, cand, scores, (int)extra_off, extra_out, zero_ptr, zero_ptr ? zero_words : 0);
   PKV_LAUNCH_CHECK("pkv_select_rerank_kernel");
   return PKV_OK;
 }
@@ -1752,6 +1756,9 @@ static WideWs wide_ws_layout(int rows, int64_t len, int64_t k, size_t off) {
   return w;
 }
 
+// Words at the start of pkv_topk_f32's workspace that must be zero when its first launch starts (0: none).
+int64_t pkv_topk_ctl_words(int rows, int64_t len) { return len > kTopkMaxSort ? (int64_t)rows * kWideRowWords : 0; }
+
 size_t pkv_topk_ws_bytes_impl(int rows, int64_t len, int64_t k) {
   if (rows <= 0 || len <= kTopkMaxSort || k <= 0) return 256;
   return wide_ws_layout(rows, len, k, 0).total;
@@ -1763,7 +1770,7 @@ extern "C" size_t pkv_topk_f32_ws_bytes(int rows, int64_t len, int64_t k) {
 
 int pkv_launch_topk_f32(const float *x, int64_t x_stride, const int64_t *ids, int64_t ids_stride, int rows,
                         int64_t len, int64_t k, int64_t *out_ids, float *out_vals, void *ws, size_t ws_bytes,
-                        hipStream_t s, bool any_order) {
+                        hipStream_t s, bool any_order, bool ctl_cleared) {
   PKV_REQUIRE(x && out_ids, "pkv_topk_f32: null pointer");
   PKV_REQUIRE(k > 0, "k must be positive");
   PKV_REQUIRE(k <= len, "k cannot exceed sequence length");
@@ -1803,9 +1810,11 @@ int pkv_launch_topk_f32(const float *x, int64_t x_stride, const int64_t *ids, in
     uint64_t *list_a = (uint64_t *)((char *)ws + w.list_a), *list_b = (uint64_t *)((char *)ws + w.list_b);
     const int P = pow2_ceil(k);
     const dim3 grid((unsigned)((len + kWideSlice - 1) / kWideSlice), (unsigned)rows);
-    hipLaunchKernelGGL(pkv_zero_u32_kernel, dim3((unsigned)((rows * kWideRowWords + 255) / 256)), dim3(256), 0, s, ctl,
-                       (int64_t)rows * kWideRowWords);
-    PKV_LAUNCH_CHECK("pkv_zero_u32_kernel");
+    if (!ctl_cleared) {  // an earlier launch of the caller's step may have cleared the control blocks already
+      hipLaunchKernelGGL(pkv_zero_u32_kernel, dim3((unsigned)((rows * kWideRowWords + 255) / 256)), dim3(256), 0, s, ctl,
+                         (int64_t)rows * kWideRowWords);
+      PKV_LAUNCH_CHECK("pkv_zero_u32_kernel");
+    }
     hipLaunchKernelGGL(pkv_topk_wide_hist_kernel, grid, dim3(kTopkThreads), 0, s, x, x_stride, ids, ids_stride, len, ctl);
     PKV_LAUNCH_CHECK("pkv_topk_wide_hist_kernel");
     hipLaunchKernelGGL(pkv_topk_wide_compact_kernel, grid, dim3(kTopkThreads), 0, s, x, x_stride, ids, ids_stride, len, k,
