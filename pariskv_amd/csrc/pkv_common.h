@@ -68,7 +68,8 @@ static inline int pkv_pick_chunk_keys(int rows, int64_t n_keys) {
 PKV_INTERNAL int pkv_launch_query_prep_lut(const void *q, int dtype, int bs, int n_kv_heads, int group,
                                            const float *signs, const int32_t *cc, int64_t cc_b, int64_t cc_h,
                                            const PkvTiers &tiers, float *qhat, float *qnorm, uint8_t *lut,
-                                           int64_t *sorted_ids, uint32_t *row_suf_to_zero, hipStream_t s);
+                                           int64_t *sorted_ids, uint32_t *row_suf_to_zero, hipStream_t s,
+                                           uint32_t *zero_ptr = nullptr, int64_t zero_words = 0);
 PKV_INTERNAL int pkv_launch_scan(const uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t cs_key, int64_t cs_sub,
                                  int bs, int n_kv_heads, int64_t n_keys, const uint8_t *lut, uint8_t *cnt_u8,
                                  int64_t cnt_u8_stride, int32_t *cnt_i32, uint32_t *row_suf, uint16_t *chunk_suf,
@@ -82,8 +83,7 @@ PKV_INTERNAL int pkv_launch_select_rerank(const uint8_t *cnt_u8, int64_t cnt_str
                                           const uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key,
                                           const float *qhat, const float *qnorm, const float *centers, int64_t *cand,
                                           float *scores, hipStream_t s, int64_t extra_off = 0,
-                                          float *extra_out = nullptr, uint32_t *zero_ptr = nullptr,
-                                          int64_t zero_words = 0);
+                                          float *extra_out = nullptr, uint32_t *topk_ctl = nullptr);
 PKV_INTERNAL int pkv_launch_rerank(const int64_t *cand, int bs, int n_kv_heads, int64_t n_cand, int64_t n_keys,
                                    const uint8_t *nib, int64_t ns_b, int64_t ns_h, int64_t ns_key, int64_t ns_sub,
                                    const uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key,
@@ -94,7 +94,7 @@ PKV_INTERNAL int64_t pkv_topk_ctl_words(int rows, int64_t len);
 PKV_INTERNAL int pkv_launch_topk_f32(const float *x, int64_t x_stride, const int64_t *ids, int64_t ids_stride,
                                      int rows, int64_t len, int64_t k, int64_t *out_ids, float *out_vals,
                                      void *ws, size_t ws_bytes, hipStream_t s, bool any_order = false,
-                                     bool ctl_cleared = false);
+                                     bool ctl_ready = false);
 PKV_INTERNAL int pkv_launch_gather(const void *src_k, const void *src_v, int64_t src_len, const int64_t *idx,
                                    int64_t k, int64_t idx_offset, void *dst_k, void *dst_v, int64_t dst_len,
                                    int64_t dst_row0, int rows, int row_bytes, hipStream_t s, const int64_t *row_counts = nullptr);

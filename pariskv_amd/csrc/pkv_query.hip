@@ -21,11 +21,14 @@ __global__ __launch_bounds__(256) void pkv_query_prep_lut_kernel(
     const void *__restrict__ q, int dtype, int n_kv_heads, int group, const float *__restrict__ signs,
     const int32_t *__restrict__ cc, int64_t cc_b, int64_t cc_h, PkvTiers tiers, float *__restrict__ qhat,
     float *__restrict__ qnorm, uint8_t *__restrict__ lut, int64_t *__restrict__ sorted_ids,
-    uint32_t *__restrict__ row_suf_to_zero) {
+    uint32_t *__restrict__ row_suf_to_zero, uint32_t *__restrict__ zero_ptr, int64_t zero_words) {
   const int sub = blockIdx.x;
   const int row = blockIdx.y;
   const int b = row / n_kv_heads, h = row % n_kv_heads;
   const int tid = threadIdx.x;
+  // words a later launch of the step accumulates into (the control blocks of a multi-workgroup top-k)
+  for (int64_t i = ((int64_t)row * gridDim.x + sub) * 256 + tid; i < zero_words; i += (int64_t)gridDim.x * gridDim.y * 256)
+    zero_ptr[i] = 0u;
 
   // the collision scan that follows accumulates the row's suffix histogram with atomics
   if (row_suf_to_zero && sub == 1 && tid < 128) row_suf_to_zero[(int64_t)row * 128 + tid] = 0u;
@@ -70,10 +73,10 @@ __global__ __launch_bounds__(256) void pkv_lut_from_sorted_kernel(
 int pkv_launch_query_prep_lut(const void *q, int dtype, int bs, int n_kv_heads, int group, const float *signs,
                               const int32_t *cc, int64_t cc_b, int64_t cc_h, const PkvTiers &tiers, float *qhat,
                               float *qnorm, uint8_t *lut, int64_t *sorted_ids, uint32_t *row_suf_to_zero,
-                              hipStream_t s) {
+                              hipStream_t s, uint32_t *zero_ptr, int64_t zero_words) {
   dim3 grid(16, (unsigned)(bs * n_kv_heads));
   hipLaunchKernelGGL(pkv_query_prep_lut_kernel, grid, dim3(256), 0, s, q, dtype, n_kv_heads, group, signs, cc,
-                     cc_b, cc_h, tiers, qhat, qnorm, lut, sorted_ids, row_suf_to_zero);
+                     cc_b, cc_h, tiers, qhat, qnorm, lut, sorted_ids, row_suf_to_zero, zero_ptr, zero_ptr ? zero_words : 0);
   PKV_LAUNCH_CHECK("pkv_query_prep_lut_kernel");
   return PKV_OK;
 }

@@ -134,9 +134,12 @@ static int retrieve_impl(const pkv_retrieve_args *a, void *ws, size_t ws_bytes, 
   PKV_REQUIRE(nk >= 64 && nk % 16 == 0 && wk >= 16 && wk % 8 == 0,
               "key strides of %lld / %lld bytes: nibbles need >= 64, weights >= 32, multiples of 16",
               (long long)a->nib_key_stride, (long long)a->weight_key_stride);
-  bool ctl_cleared = false;  // the select + rerank launch clears the control blocks of a multi-workgroup top-k
+  // a multi-workgroup top-k (more than 8192 candidates) wants its control blocks cleared and the rows' score
+  // ranges in them: the first launch of the step clears, the select + rerank launch leaves the ranges
+  const int64_t ctl_words = a->out_ids && a->n_cand != a->n_keys ? pkv_topk_ctl_words(rows, a->n_cand) : 0;
+  uint32_t *topk_ctl = ctl_words ? (uint32_t *)(base + w.topk) : nullptr;
   int rc = pkv_launch_query_prep_lut(a->q, a->dtype, a->bs, H, a->group, a->signs, a->cluster_counts,
-                                     (int64_t)H * 4096, 4096, t, qhat, qnorm, lut, nullptr, rowsuf, s);
+                                     (int64_t)H * 4096, 4096, t, qhat, qnorm, lut, nullptr, rowsuf, s, topk_ctl, ctl_words);
   if (rc) return rc;
   const uint8_t *codes = a->codes + a->key0 * 16;
   const uint8_t *nib = a->nib + a->key0 * nk;
@@ -154,14 +157,12 @@ static int retrieve_impl(const pkv_retrieve_args *a, void *ws, size_t ws_bytes, 
     rc = pkv_launch_select_rerank(cnt, w.cnt_stride, rowsuf, hist, w.chunk_keys, a->bs, H, a->n_keys, a->n_cand, nib,
                                   (int64_t)H * a->cap * nk, a->cap * nk, nk, weight, (int64_t)H * a->cap * wk, a->cap * wk,
                                   wk, qhat, qnorm, a->centers, cand, scores, s, a->record_word_offset,
-                                  a->record_word_offset > 0 ? (float *)(base + w.cand_extra) : nullptr,
-                                  a->out_ids ? (uint32_t *)(base + w.topk) : nullptr, pkv_topk_ctl_words(rows, a->n_cand));
-    ctl_cleared = a->out_ids != nullptr;
+                                  a->record_word_offset > 0 ? (float *)(base + w.cand_extra) : nullptr, topk_ctl);
   }
   if (rc) return rc;
   if (!a->out_ids) return PKV_OK;  // candidates only: the caller reads them out of the workspace
   rc = pkv_launch_topk_f32(scores, a->n_cand, cand, a->n_cand, rows, a->n_cand, a->k, a->out_ids, a->out_scores,
-                           (char *)ws + w.topk, w.topk_bytes, s, a->any_order != 0, ctl_cleared);
+                           (char *)ws + w.topk, w.topk_bytes, s, a->any_order != 0, topk_ctl != nullptr);
   if (rc) return rc;
   if (a->src_k) {
     PKV_REQUIRE(a->src_v && a->dst_k && a->dst_v, "pkv_retrieve: gather needs src_v, dst_k, dst_v");

@@ -16,6 +16,7 @@
 
 namespace {
 
+constexpr int kWideRangeSlots = 16;  // per row: score ranges left by a producer's workgroups for a multi-workgroup top-k, (max, ~min) each
 constexpr int kSelThreads = 256;
 constexpr int kSelKeysPerThread = 16;                                  // one 128-bit load of counts
 constexpr int kSelKeysPerIter = kSelThreads * kSelKeysPerThread;  // 4096
@@ -169,15 +170,12 @@ __global__ __launch_bounds__(kSelThreads) void pkv_select_rerank_kernel(
     const uint8_t *__restrict__ nib, int64_t ns_b, int64_t ns_h, int ns_key, const uint16_t *__restrict__ weight,
     int64_t ws_b, int64_t ws_h, int ws_key, const float *__restrict__ qhat, const float *__restrict__ qnorm,
     const float *__restrict__ centers, int64_t *__restrict__ out, float *__restrict__ scores, int extra_off,
-    float *__restrict__ extra_out, uint32_t *__restrict__ zero_ptr, int64_t zero_words) {
+    float *__restrict__ extra_out, uint32_t *__restrict__ range_slots, int64_t range_row_stride) {
   const int row = blockIdx.y;
   const int chunk = blockIdx.x;
   const int tid = threadIdx.x;
   const int b = row / n_kv_heads, h = row % n_kv_heads;
-  // words the next launch of the step wants cleared (the control blocks of a multi-workgroup top-k): spread over the launch
-  for (int64_t i = ((int64_t)row * gridDim.x + chunk) * kSelThreads + tid; i < zero_words;
-       i += (int64_t)gridDim.x * gridDim.y * kSelThreads)
-    zero_ptr[i] = 0u;
+  uint32_t smax = 0u, smin = 0xffffffffu;  // ordered bits of the largest / smallest score this thread wrote
 
   __shared__ int s_scan[2][kSelThreads / PKV_WAVE];
   __shared__ float s_prod[128 * 16];
@@ -243,12 +241,41 @@ __global__ __launch_bounds__(kSelThreads) void pkv_select_rerank_kernel(
       if (pos >= 0) {
         const int64_t key = blk0 + s_list_key[j];
         orow[pos] = key;
-        srow[pos] = pkv_rerank_keymajor(s_prod, (const pkv_u32x4 *)(nrow + key * ns_key), (const pkv_u32x4 *)(wrow + key * ws_key), qn);
+        const float sc = pkv_rerank_keymajor(s_prod, (const pkv_u32x4 *)(nrow + key * ns_key), (const pkv_u32x4 *)(wrow + key * ws_key), qn);
+        srow[pos] = sc;
+        const uint32_t o = pkv_ordered_u32(sc);
+        smax = o > smax ? o : smax;
+        smin = o < smin ? o : smin;
         // one more fp32 word of the key's record (same HBM line), passed through for the caller
         if (extra_out) extra_out[(int64_t)row * k + pos] = *(const float *)(nrow + key * ns_key + extra_off);
       }
     }
     __syncthreads();  // the list is rewritten by the next iteration
+  }
+  // this chunk's score range for a multi-workgroup top-k that follows: (max, ~min) into one of the row's 16 range
+  // slots with atomicMax from zero (one address per row would serialise the atomics of hundreds of workgroups:
+  // measured +15 us at 8 rows x 256 chunks; a slot per workgroup costs the readers 3 us of loads)
+  if (range_slots) {
+#pragma unroll
+    for (int x = 1; x < PKV_WAVE; x <<= 1) {
+      const uint32_t a = (uint32_t)__shfl_xor((int)smax, x, PKV_WAVE), c = (uint32_t)__shfl_xor((int)smin, x, PKV_WAVE);
+      smax = a > smax ? a : smax;
+      smin = c < smin ? c : smin;
+    }
+    if (pkv_lane() == 0) s_scan[0][tid / PKV_WAVE] = (int)smax, s_scan[1][tid / PKV_WAVE] = (int)smin;
+    __syncthreads();
+    if (tid == 0) {
+      for (int wv = 1; wv < kSelThreads / PKV_WAVE; ++wv) {
+        const uint32_t a = (uint32_t)s_scan[0][wv], c = (uint32_t)s_scan[1][wv];
+        smax = a > smax ? a : smax;
+        smin = c < smin ? c : smin;
+      }
+      if (smax >= smin) {
+        uint32_t *slot = range_slots + (int64_t)row * range_row_stride + 2 * (chunk % kWideRangeSlots);
+        atomicMax(&slot[0], smax);
+        atomicMax(&slot[1], ~smin);
+      }
+    }
   }
 }
 
@@ -946,7 +973,8 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
 // Keys are distinct, so the order in which the lists are filled does not reach the result.
 constexpr int kWideSlice = 8192;
 constexpr int kWideBins = 2048;
-constexpr int kWideRowWords = kWideBins + 8;  // per-row control block: histogram, |A|, |B|, padding
+constexpr int kWideCtlSlots = kWideBins + 8;
+constexpr int kWideRowWords = kWideCtlSlots + 2 * kWideRangeSlots;  // per-row control block: histogram, |A|, |B|, range, range slots
 
 struct ScoreKeys {  // key i of a row of scores with optional ids
   const float *x;
@@ -955,6 +983,52 @@ struct ScoreKeys {  // key i of a row of scores with optional ids
 };
 
 constexpr int kWideE = kWideSlice / kTopkThreads;  // keys per thread
+constexpr int kWideCtlMax = kWideBins + 2;     // largest ordered score of the row (0 = not provided)
+constexpr int kWideCtlMinInv = kWideBins + 3;  // ~(smallest ordered score): both grow under atomicMax from zero
+
+// Bin (0 .. 2047) of a key of a wide row.  With the row's score range in its control block: 2048 even steps of
+// [min, max] (non-decreasing in the score whatever the rounding, so a higher bin means a larger key), which keeps
+// the threshold bin at about len / 2048 keys for any distribution without far outliers.  Without it, or where it
+// does not apply (non-finite scores, a zero or subnormal range): bits [shift, shift + 11) of the key, which put
+// scores that share their exponent into a handful of bins.
+struct WideBinning {
+  int shift;  // >= 0: fixed bit field; < 0: value bins
+  float lo, scale;
+  __device__ __forceinline__ uint32_t operator()(uint64_t key) const {
+    if (shift >= 0) return (uint32_t)(key >> shift) & (kWideBins - 1);
+    const float t = (pkv_from_ordered_u32((uint32_t)(key >> 32)) - lo) * scale;
+    const uint32_t b = (uint32_t)t;
+    return b > (uint32_t)(kWideBins - 1) ? (uint32_t)(kWideBins - 1) : b;
+  }
+};
+
+// The same decision in every workgroup of every launch that bins the row: it depends only on the range words and
+// the n_slots range slots a producer may have filled (every wave reduces them for itself: no barrier).
+__device__ __forceinline__ WideBinning wide_binning(const uint32_t *__restrict__ ctl, int n_slots, int fallback_shift) {
+  WideBinning bn;
+  bn.shift = fallback_shift, bn.lo = 0.f, bn.scale = 0.f;
+  uint32_t mx = ctl[kWideCtlMax], mi = ctl[kWideCtlMinInv];
+  if (n_slots > 0) {
+    for (int c = pkv_lane(); c < n_slots; c += PKV_WAVE) {
+      const pkv_u32x2 sl = *(const pkv_u32x2 *)(ctl + kWideCtlSlots + 2 * c);
+      mx = sl.x > mx ? sl.x : mx;
+      mi = sl.y > mi ? sl.y : mi;
+    }
+#pragma unroll
+    for (int x = 1; x < PKV_WAVE; x <<= 1) {
+      const uint32_t a = (uint32_t)__shfl_xor((int)mx, x, PKV_WAVE), c = (uint32_t)__shfl_xor((int)mi, x, PKV_WAVE);
+      mx = a > mx ? a : mx;
+      mi = c > mi ? c : mi;
+    }
+  }
+  const uint32_t mn = ~mi;
+  const float hi = pkv_from_ordered_u32(mx), lo = pkv_from_ordered_u32(mn);
+  const float range = hi - lo, scale = (float)kWideBins / range;
+  const float inf = __uint_as_float(0x7f800000u);
+  if (mx != 0u && mx < 0xff800000u && mn > 0x007fffffu && mn <= mx && range > 0.f && range < inf && scale < inf)
+    bn.shift = -1, bn.lo = lo, bn.scale = scale;
+  return bn;
+}
 
 // The slice's keys, element e of thread t = slice*8192 + e*1024 + t; 0 beyond the row's end.  The loads are
 // unconditional (clamped index) so that all of them are in flight together.
@@ -968,16 +1042,15 @@ __device__ __forceinline__ void wide_load_keys(KeyFn key_of, int64_t len, int sl
   }
 }
 
-template <int BINSHIFT>
-__device__ __forceinline__ void wide_hist_slice(const uint64_t (&keys)[kWideE], int64_t len, int slice, uint32_t *s_bins,
-                                                uint32_t *__restrict__ g_hist) {
+__device__ __forceinline__ void wide_hist_slice(const WideBinning &bn, const uint64_t (&keys)[kWideE], int64_t len,
+                                                int slice, uint32_t *s_bins, uint32_t *__restrict__ g_hist) {
   const int tid = threadIdx.x;
   for (int b = tid; b < kWideBins; b += kTopkThreads) s_bins[b] = 0;
   __syncthreads();
 #pragma unroll
   for (int e = 0; e < kWideE; ++e) {
     const int64_t i = (int64_t)slice * kWideSlice + e * kTopkThreads + tid;
-    wave_hist_add(s_bins, (uint32_t)(keys[e] >> BINSHIFT) & (kWideBins - 1), i < len, 1);
+    wave_hist_add(s_bins, bn(keys[e]), i < len, 1);
   }
   __syncthreads();
   for (int b = tid; b < kWideBins; b += kTopkThreads) {
@@ -988,10 +1061,10 @@ __device__ __forceinline__ void wide_hist_slice(const uint64_t (&keys)[kWideE], 
 
 // s_tmp: 24 words.  ctl: the row's control block (histogram complete at launch).  Every workgroup
 // reserves its share of both lists with one atomic each.
-template <int BINSHIFT>
-__device__ __forceinline__ void wide_compact_slice(const uint64_t (&keys)[kWideE], int64_t len, int slice, uint32_t k,
-                                                   uint32_t *__restrict__ ctl, uint64_t *__restrict__ list_a,
-                                                   uint64_t *__restrict__ list_b, uint32_t *s_tmp) {
+__device__ __forceinline__ void wide_compact_slice(const WideBinning &bn, const uint64_t (&keys)[kWideE], int64_t len,
+                                                   int slice, uint32_t k, uint32_t *__restrict__ ctl,
+                                                   uint64_t *__restrict__ list_a, uint64_t *__restrict__ list_b,
+                                                   uint32_t *s_tmp) {
   const int tid = threadIdx.x;
   // thread t owns bins 2047 - 2t and 2046 - 2t: an exclusive scan over threads counts the keys in higher bins
   const uint32_t h0 = ctl[kWideBins - 1 - 2 * tid], h1 = ctl[kWideBins - 2 - 2 * tid];
@@ -1007,7 +1080,7 @@ __device__ __forceinline__ void wide_compact_slice(const uint64_t (&keys)[kWideE
 #pragma unroll
   for (int e = 0; e < kWideE; ++e) {
     const int64_t i = (int64_t)slice * kWideSlice + e * kTopkThreads + tid;
-    const uint32_t bin = (uint32_t)(keys[e] >> BINSHIFT) & (kWideBins - 1);
+    const uint32_t bin = bn(keys[e]);
     const bool a = i < len && bin > bstar, b = i < len && bin == bstar;
     in_a |= (uint32_t)a << e, in_b |= (uint32_t)b << e;
     n_a += a, n_b += b;
@@ -1075,28 +1148,72 @@ __device__ __forceinline__ void wide_finish_select(uint32_t k, int P, const uint
   __syncthreads();
 }
 
+// Largest and smallest ordered score of a workgroup's values into the row's control block (both words grow from
+// zero under atomicMax: the minimum is kept complemented).  s_red: 32 words.  All threads of the workgroup.
+__device__ __forceinline__ void wide_range_atomics(uint32_t mx, uint32_t mn, uint32_t *__restrict__ rctl, uint32_t *s_red) {
+#pragma unroll
+  for (int x = 1; x < PKV_WAVE; x <<= 1) {
+    const uint32_t a = (uint32_t)__shfl_xor((int)mx, x, PKV_WAVE), c = (uint32_t)__shfl_xor((int)mn, x, PKV_WAVE);
+    mx = a > mx ? a : mx;
+    mn = c < mn ? c : mn;
+  }
+  const int wave = threadIdx.x / PKV_WAVE, n_waves = (blockDim.x + PKV_WAVE - 1) / PKV_WAVE;
+  if (pkv_lane() == 0) s_red[wave] = mx, s_red[16 + wave] = mn;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < n_waves; ++w) {
+      mx = s_red[w] > mx ? s_red[w] : mx;
+      mn = s_red[16 + w] < mn ? s_red[16 + w] : mn;
+    }
+    if (mx >= mn) {  // at least one value
+      atomicMax(&rctl[kWideCtlMax], mx);
+      atomicMax(&rctl[kWideCtlMinInv], ~mn);
+    }
+  }
+}
+
+// grid (slices, rows).  ctl zero at launch.  The rows' score ranges for the launches that follow.
+__global__ __launch_bounds__(kTopkThreads) void pkv_topk_wide_range_kernel(const float *__restrict__ x, int64_t x_stride,
+                                                                           int64_t len, uint32_t *__restrict__ ctl) {
+  __shared__ uint32_t s_red[32];
+  const int row = blockIdx.y;
+  const float *xr = x + (int64_t)row * x_stride;
+  uint32_t mx = 0u, mn = 0xffffffffu;
+#pragma unroll
+  for (int e = 0; e < kWideE; ++e) {
+    const int64_t i = (int64_t)blockIdx.x * kWideSlice + e * kTopkThreads + threadIdx.x;
+    const uint32_t o = pkv_ordered_u32(xr[i < len ? i : len - 1]);
+    mx = o > mx ? o : mx;
+    mn = o < mn ? o : mn;
+  }
+  wide_range_atomics(mx, mn, ctl + (int64_t)row * kWideRowWords, s_red);
+}
+
 // grid (slices, rows).  ctl: u32 [rows][kWideRowWords], zero at launch.
 __global__ __launch_bounds__(kTopkThreads) void pkv_topk_wide_hist_kernel(const float *__restrict__ x, int64_t x_stride,
                                                                           const int64_t *__restrict__ ids,
                                                                           int64_t ids_stride, int64_t len,
-                                                                          uint32_t *__restrict__ ctl) {
+                                                                          uint32_t *__restrict__ ctl, int n_range_slots) {
   __shared__ uint32_t s_bins[kWideBins];
   const int row = blockIdx.y;
   uint64_t keys[kWideE];
   wide_load_keys(ScoreKeys{x + (int64_t)row * x_stride, ids ? ids + (int64_t)row * ids_stride : nullptr}, len, blockIdx.x,
                  keys);
-  wide_hist_slice<53>(keys, len, blockIdx.x, s_bins, ctl + (int64_t)row * kWideRowWords);
+  wide_hist_slice(wide_binning(ctl + (int64_t)row * kWideRowWords, n_range_slots, 53), keys, len, blockIdx.x, s_bins,
+                  ctl + (int64_t)row * kWideRowWords);
 }
 
 __global__ __launch_bounds__(kTopkThreads) void pkv_topk_wide_compact_kernel(
     const float *__restrict__ x, int64_t x_stride, const int64_t *__restrict__ ids, int64_t ids_stride, int64_t len,
-    int64_t k, uint32_t *__restrict__ ctl, uint64_t *__restrict__ list_a, uint64_t *__restrict__ list_b) {
+    int64_t k, uint32_t *__restrict__ ctl, uint64_t *__restrict__ list_a, uint64_t *__restrict__ list_b,
+    int n_range_slots) {
   __shared__ uint32_t s_tmp[24];
   const int row = blockIdx.y;
   uint64_t keys[kWideE];
   wide_load_keys(ScoreKeys{x + (int64_t)row * x_stride, ids ? ids + (int64_t)row * ids_stride : nullptr}, len, blockIdx.x,
                  keys);
-  wide_compact_slice<53>(keys, len, blockIdx.x, (uint32_t)k, ctl + (int64_t)row * kWideRowWords, list_a + (int64_t)row * k,
+  wide_compact_slice(wide_binning(ctl + (int64_t)row * kWideRowWords, n_range_slots, 53), keys, len, blockIdx.x, (uint32_t)k,
+                     ctl + (int64_t)row * kWideRowWords, list_a + (int64_t)row * k,
                          list_b + (int64_t)row * len, s_tmp);
 }
 
@@ -1523,7 +1640,7 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adk_benefit_kernel(
   }
   const float ssum = block_tree_sum_1024(acc, s_part);
   if (tid == 0) ws_sum[(int64_t)row * n_slices + slice] = ssum;
-  wide_hist_slice<52>(keys, n_cand, slice, s_bins, ctl + (int64_t)row * kWideRowWords);
+  wide_hist_slice(WideBinning{52, 0.f, 0.f}, keys, n_cand, slice, s_bins, ctl + (int64_t)row * kWideRowWords);
 }
 
 __global__ __launch_bounds__(kTopkThreads) void pkv_adk_compact_kernel(const float *__restrict__ ws_ben, int64_t n_cand,
@@ -1534,7 +1651,7 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adk_compact_kernel(const flo
   const int row = blockIdx.y;
   uint64_t keys[kWideE];
   wide_load_keys(BenefitKeys{ws_ben + (int64_t)row * n_cand}, n_cand, blockIdx.x, keys);
-  wide_compact_slice<52>(keys, n_cand, blockIdx.x, (uint32_t)k_out,
+  wide_compact_slice(WideBinning{52, 0.f, 0.f}, keys, n_cand, blockIdx.x, (uint32_t)k_out,
                          ctl + (int64_t)row * kWideRowWords, list_a + (int64_t)row * k_out,
                          list_b + (int64_t)row * n_cand, s_tmp);
 }
@@ -1661,7 +1778,7 @@ int pkv_launch_select_rerank(const uint8_t *cnt_u8, int64_t cnt_stride, const ui
                              int n_kv_heads, int64_t n_keys, int64_t k, const uint8_t *nib, int64_t ns_b, int64_t ns_h,
                              int64_t ns_key, const uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key,
                              const float *qhat, const float *qnorm, const float *centers, int64_t *cand, float *scores,
-                             hipStream_t s, int64_t extra_off, float *extra_out, uint32_t *zero_ptr, int64_t zero_words) {
+                             hipStream_t s, int64_t extra_off, float *extra_out, uint32_t *topk_ctl) {
   PKV_REQUIRE(!extra_out || (extra_off >= 0 && extra_off % 4 == 0 && extra_off + 4 <= ns_key),
               "the extra word must lie inside the key's record (offset %lld, record %lld bytes)", (long long)extra_off,
               (long long)ns_key);
@@ -1678,7 +1795,8 @@ int pkv_launch_select_rerank(const uint8_t *cnt_u8, int64_t cnt_stride, const ui
   hipLaunchKernelGGL(pkv_select_rerank_kernel, grid, dim3(kSelThreads), 0, s, cnt_u8, cnt_stride, row_suf, chunk_suf,
                      chunk_keys,
                      n_kv_heads, n_keys, k, nib, ns_b, ns_h, (int)ns_key, weight, ws_b, ws_h, (int)ws_key, qhat, qnorm,
-                     centers, cand, scores, (int)extra_off, extra_out, zero_ptr, zero_ptr ? zero_words : 0);
+                     centers, cand, scores, (int)extra_off, extra_out,
+                     topk_ctl ? topk_ctl + kWideCtlSlots : nullptr, (int64_t)kWideRowWords);
   PKV_LAUNCH_CHECK("pkv_select_rerank_kernel");
   return PKV_OK;
 }
@@ -1770,7 +1888,7 @@ extern "C" size_t pkv_topk_f32_ws_bytes(int rows, int64_t len, int64_t k) {
 
 int pkv_launch_topk_f32(const float *x, int64_t x_stride, const int64_t *ids, int64_t ids_stride, int rows,
                         int64_t len, int64_t k, int64_t *out_ids, float *out_vals, void *ws, size_t ws_bytes,
-                        hipStream_t s, bool any_order, bool ctl_cleared) {
+                        hipStream_t s, bool any_order, bool ctl_ready) {
   PKV_REQUIRE(x && out_ids, "pkv_topk_f32: null pointer");
   PKV_REQUIRE(k > 0, "k must be positive");
   PKV_REQUIRE(k <= len, "k cannot exceed sequence length");
@@ -1810,15 +1928,19 @@ int pkv_launch_topk_f32(const float *x, int64_t x_stride, const int64_t *ids, in
     uint64_t *list_a = (uint64_t *)((char *)ws + w.list_a), *list_b = (uint64_t *)((char *)ws + w.list_b);
     const int P = pow2_ceil(k);
     const dim3 grid((unsigned)((len + kWideSlice - 1) / kWideSlice), (unsigned)rows);
-    if (!ctl_cleared) {  // an earlier launch of the caller's step may have cleared the control blocks already
+    if (!ctl_ready) {  // else: earlier launches of the caller's step cleared the control blocks and left the rows' score ranges
       hipLaunchKernelGGL(pkv_zero_u32_kernel, dim3((unsigned)((rows * kWideRowWords + 255) / 256)), dim3(256), 0, s, ctl,
                          (int64_t)rows * kWideRowWords);
       PKV_LAUNCH_CHECK("pkv_zero_u32_kernel");
+      hipLaunchKernelGGL(pkv_topk_wide_range_kernel, grid, dim3(kTopkThreads), 0, s, x, x_stride, len, ctl);
+      PKV_LAUNCH_CHECK("pkv_topk_wide_range_kernel");
     }
-    hipLaunchKernelGGL(pkv_topk_wide_hist_kernel, grid, dim3(kTopkThreads), 0, s, x, x_stride, ids, ids_stride, len, ctl);
+    const int n_range_slots = ctl_ready ? kWideRangeSlots : 0;  // a producer's per-workgroup score ranges
+    hipLaunchKernelGGL(pkv_topk_wide_hist_kernel, grid, dim3(kTopkThreads), 0, s, x, x_stride, ids, ids_stride, len, ctl,
+                       n_range_slots);
     PKV_LAUNCH_CHECK("pkv_topk_wide_hist_kernel");
     hipLaunchKernelGGL(pkv_topk_wide_compact_kernel, grid, dim3(kTopkThreads), 0, s, x, x_stride, ids, ids_stride, len, k,
-                       ctl, list_a, list_b);
+                       ctl, list_a, list_b, n_range_slots);
     PKV_LAUNCH_CHECK("pkv_topk_wide_compact_kernel");
     hipLaunchKernelGGL(pkv_topk_wide_finish_kernel, dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes_sort(P), s, len, P, k,
                        ctl, list_a, list_b, out_ids, out_vals);

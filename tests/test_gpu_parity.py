@@ -396,6 +396,13 @@ def test_topk_f32_wide_rows_edge_cases(ops):
     y[0, 5], y[0, 77], y[1, 20000] = np.inf, -np.inf, np.inf
     y[:, 100:4000] = -np.abs(y[:, 100:4000])
     cases.append(("signs and infinities", y, 3000))
+    # scores that share their exponent: bins of fixed key bits would put the whole row into a few bins; the bins of
+    # the row's own range keep the threshold bin small
+    cases.append(("one binade", (rng.standard_normal((3, 52429)) * 2 + 100).astype(np.float32), 2048))
+    cases.append(("narrow range", (rng.standard_normal((2, 20000)) * 1e-3 + 1.5).astype(np.float32), 1000))
+    z = (rng.standard_normal((2, 30000)) * 5).astype(np.float32)
+    z[0, 123] = 1e30                                   # an outlier stretches the range: everything else in one bin
+    cases.append(("outlier", z, 512))
     for name, x, k in cases:
         _say(f"topk_f32 wide: {name} {x.shape} k={k}")
         rows, L = x.shape
