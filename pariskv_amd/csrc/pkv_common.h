@@ -83,7 +83,8 @@ PKV_INTERNAL int pkv_launch_select_rerank(const uint8_t *cnt_u8, int64_t cnt_str
                                           const uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key,
                                           const float *qhat, const float *qnorm, const float *centers, int64_t *cand,
                                           float *scores, hipStream_t s, int64_t extra_off = 0,
-                                          float *extra_out = nullptr, uint32_t *topk_ctl = nullptr);
+                                          float *extra_out = nullptr, uint32_t *range_slots = nullptr,
+                                          int64_t range_row_stride = 0);
 PKV_INTERNAL int pkv_launch_rerank(const int64_t *cand, int bs, int n_kv_heads, int64_t n_cand, int64_t n_keys,
                                    const uint8_t *nib, int64_t ns_b, int64_t ns_h, int64_t ns_key, int64_t ns_sub,
                                    const uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key,
@@ -91,6 +92,7 @@ PKV_INTERNAL int pkv_launch_rerank(const int64_t *cand, int bs, int n_kv_heads, 
                                    float *scores, uint16_t *v4b, hipStream_t s);
 PKV_INTERNAL size_t pkv_topk_ws_bytes_impl(int rows, int64_t len, int64_t k);
 PKV_INTERNAL int64_t pkv_topk_ctl_words(int rows, int64_t len);
+PKV_INTERNAL uint32_t *pkv_topk_range_slots(uint32_t *ctl, int64_t len, int64_t *row_stride);
 PKV_INTERNAL int pkv_launch_topk_f32(const float *x, int64_t x_stride, const int64_t *ids, int64_t ids_stride,
                                      int rows, int64_t len, int64_t k, int64_t *out_ids, float *out_vals,
                                      void *ws, size_t ws_bytes, hipStream_t s, bool any_order = false,

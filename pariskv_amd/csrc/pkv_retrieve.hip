@@ -41,7 +41,10 @@ WsLayout layout(int rows, int64_t n_keys, int64_t n_cand, int64_t k) {
   w.cand = take((size_t)rows * (size_t)n_cand * sizeof(int64_t));
   w.scores = take((size_t)rows * (size_t)n_cand * sizeof(float));
   w.cand_extra = take((size_t)rows * (size_t)n_cand * sizeof(float));  // record word passed through per candidate
-  w.topk_bytes = pkv_topk_ws_bytes_impl(rows, n_cand, k);  // lists of the multi-workgroup top-k (wide rows only)
+  // the top-k's control area (range slots; for wide rows the control blocks and lists of the multi-workgroup form)
+  w.topk_bytes = pkv_topk_ws_bytes_impl(rows, n_cand, k);
+  const size_t ctl_bytes = pkv_align_up((size_t)pkv_topk_ctl_words(rows, n_cand) * 4, 256);
+  if (w.topk_bytes < ctl_bytes) w.topk_bytes = ctl_bytes;
   w.topk = take(w.topk_bytes);
   w.total = off;
   return w;
@@ -80,6 +83,8 @@ extern "C" int pkv_retrieve_ws_view(void *ws, int rows, int64_t n_keys, int64_t 
     *ptr = base + w.cand, *bytes = (size_t)rows * (size_t)n_cand * 8;
   } else if (!strcmp(name, "scores")) {
     *ptr = base + w.scores, *bytes = (size_t)rows * (size_t)n_cand * 4;
+  } else if (!strcmp(name, "topk_control")) {
+    *ptr = base + w.topk, *bytes = w.topk_bytes;
   } else if (!strcmp(name, "cand_record_word")) {
     *ptr = base + w.cand_extra, *bytes = (size_t)rows * (size_t)n_cand * 4;
   } else {
@@ -134,10 +139,13 @@ static int retrieve_impl(const pkv_retrieve_args *a, void *ws, size_t ws_bytes, 
   PKV_REQUIRE(nk >= 64 && nk % 16 == 0 && wk >= 16 && wk % 8 == 0,
               "key strides of %lld / %lld bytes: nibbles need >= 64, weights >= 32, multiples of 16",
               (long long)a->nib_key_stride, (long long)a->weight_key_stride);
-  // a multi-workgroup top-k (more than 8192 candidates) wants its control blocks cleared and the rows' score
-  // ranges in them: the first launch of the step clears, the select + rerank launch leaves the ranges
+  // the top-k takes the rows' score ranges from its control area (and a multi-workgroup top-k, more than 8192
+  // candidates, wants its control blocks cleared): the first launch of the step clears, the select + rerank launch
+  // leaves the ranges
   const int64_t ctl_words = a->out_ids && a->n_cand != a->n_keys ? pkv_topk_ctl_words(rows, a->n_cand) : 0;
   uint32_t *topk_ctl = ctl_words ? (uint32_t *)(base + w.topk) : nullptr;
+  int64_t range_stride = 0;
+  uint32_t *range_slots = topk_ctl ? pkv_topk_range_slots(topk_ctl, a->n_cand, &range_stride) : nullptr;
   int rc = pkv_launch_query_prep_lut(a->q, a->dtype, a->bs, H, a->group, a->signs, a->cluster_counts,
                                      (int64_t)H * 4096, 4096, t, qhat, qnorm, lut, nullptr, rowsuf, s, topk_ctl, ctl_words);
   if (rc) return rc;
@@ -157,7 +165,8 @@ static int retrieve_impl(const pkv_retrieve_args *a, void *ws, size_t ws_bytes, 
     rc = pkv_launch_select_rerank(cnt, w.cnt_stride, rowsuf, hist, w.chunk_keys, a->bs, H, a->n_keys, a->n_cand, nib,
                                   (int64_t)H * a->cap * nk, a->cap * nk, nk, weight, (int64_t)H * a->cap * wk, a->cap * wk,
                                   wk, qhat, qnorm, a->centers, cand, scores, s, a->record_word_offset,
-                                  a->record_word_offset > 0 ? (float *)(base + w.cand_extra) : nullptr, topk_ctl);
+                                  a->record_word_offset > 0 ? (float *)(base + w.cand_extra) : nullptr,
+                                  range_slots, range_stride);
   }
   if (rc) return rc;
   if (!a->out_ids) return PKV_OK;  // candidates only: the caller reads them out of the workspace

@@ -690,10 +690,15 @@ __device__ __forceinline__ bool linear_bins(const uint64_t (&v)[EIN], uint32_t k
       }
       above += h[j];
     }
-    most = most > pkv_lane_xor<1>(most) ? most : pkv_lane_xor<1>(most);
-    most = most > pkv_lane_xor<2>(most) ? most : pkv_lane_xor<2>(most);
-    most = most > pkv_lane_xor<4>(most) ? most : pkv_lane_xor<4>(most);
-    most = most > pkv_lane_xor<8>(most) ? most : pkv_lane_xor<8>(most);
+    // every lane exchange is evaluated once, by all lanes: inside a conditional expression the compiler may run it
+    // under a partial execution mask, and a lane-crossing read of an inactive lane returns nothing
+#define PKV_MAX_XOR(M)                               \
+  {                                                  \
+    const uint32_t o = pkv_lane_xor<M>(most);        \
+    most = o > most ? o : most;                      \
+  }
+    PKV_MAX_XOR(1) PKV_MAX_XOR(2) PKV_MAX_XOR(4) PKV_MAX_XOR(8)
+#undef PKV_MAX_XOR
     if ((tid & 15) == 0) atomicMax(&s_bcast[5], most);
   }
   __syncthreads();
@@ -1778,7 +1783,8 @@ int pkv_launch_select_rerank(const uint8_t *cnt_u8, int64_t cnt_stride, const ui
                              int n_kv_heads, int64_t n_keys, int64_t k, const uint8_t *nib, int64_t ns_b, int64_t ns_h,
                              int64_t ns_key, const uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key,
                              const float *qhat, const float *qnorm, const float *centers, int64_t *cand, float *scores,
-                             hipStream_t s, int64_t extra_off, float *extra_out, uint32_t *topk_ctl) {
+                             hipStream_t s, int64_t extra_off, float *extra_out, uint32_t *range_slots,
+                             int64_t range_row_stride) {
   PKV_REQUIRE(!extra_out || (extra_off >= 0 && extra_off % 4 == 0 && extra_off + 4 <= ns_key),
               "the extra word must lie inside the key's record (offset %lld, record %lld bytes)", (long long)extra_off,
               (long long)ns_key);
@@ -1796,7 +1802,7 @@ int pkv_launch_select_rerank(const uint8_t *cnt_u8, int64_t cnt_stride, const ui
                      chunk_keys,
                      n_kv_heads, n_keys, k, nib, ns_b, ns_h, (int)ns_key, weight, ws_b, ws_h, (int)ws_key, qhat, qnorm,
                      centers, cand, scores, (int)extra_off, extra_out,
-                     topk_ctl ? topk_ctl + kWideCtlSlots : nullptr, (int64_t)kWideRowWords);
+                     range_slots, range_row_stride);
   PKV_LAUNCH_CHECK("pkv_select_rerank_kernel");
   return PKV_OK;
 }
@@ -1875,7 +1881,15 @@ static WideWs wide_ws_layout(int rows, int64_t len, int64_t k, size_t off) {
 }
 
 // Words at the start of pkv_topk_f32's workspace that must be zero when its first launch starts (0: none).
+// (Handing the range to the one-workgroup kernel as well was measured: its min/max pass is cheaper than the
+// producer's extra epilogue, +0.6 us on the step at 32 rows x 4096 candidates.)
 int64_t pkv_topk_ctl_words(int rows, int64_t len) { return len > kTopkMaxSort ? (int64_t)rows * kWideRowWords : 0; }
+// Where a producer's workgroups leave their (max, ~min) in that area, and the distance between rows in words.
+uint32_t *pkv_topk_range_slots(uint32_t *ctl, int64_t len, int64_t *row_stride) {
+  (void)len;
+  *row_stride = (int64_t)kWideRowWords;
+  return ctl + kWideCtlSlots;
+}
 
 size_t pkv_topk_ws_bytes_impl(int rows, int64_t len, int64_t k) {
   if (rows <= 0 || len <= kTopkMaxSort || k <= 0) return 256;
