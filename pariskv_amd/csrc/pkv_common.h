@@ -418,6 +418,14 @@ __device__ __forceinline__ float pkv_block_dot(const float *__restrict__ s_prod,
 // The four 16-byte groups are walked by a rolled loop that rotates the data registers, so that only one
 // group's 32 table reads are in flight at a time (fully unrolled, the scheduler hoists all 128 reads and
 // the kernel needs ~170 registers).
+// LDS byte address base + 4 * (nibble of `word` at bit `shift`): a bit-field extract and a shift-and-add.  Written
+// out because the compiler turns the same expression into shift, mask and add (three instructions, 128 times per key).
+__device__ __forceinline__ uint32_t pkv_nibble_lds_addr(uint32_t word, int shift, uint32_t base) {
+  uint32_t a;
+  asm("v_bfe_u32 %0, %1, %2, 4\n\tv_lshl_add_u32 %0, %0, 2, %3" : "=&v"(a) : "v"(word), "s"(shift), "s"(base));
+  return a;
+}
+
 __device__ __forceinline__ float pkv_rerank_keymajor(const float *__restrict__ s_prod, const pkv_u32x4 *__restrict__ np,
                                                      const pkv_u32x4 *__restrict__ wp, float qnorm) {
   pkv_u32x4 n0 = np[0], n1 = np[1], n2 = np[2], n3 = np[3];
@@ -428,12 +436,13 @@ __device__ __forceinline__ float pkv_rerank_keymajor(const float *__restrict__ s
   for (int u = 0; u < 4; ++u) {
     const uint32_t words[4] = {n0.x, n0.y, n0.z, n0.w};
     const uint32_t wpair[2] = {w0.x, w0.y};
+    const uint32_t group_base = (uint32_t)(uintptr_t)(lp + 512 * u);  // LDS byte address of this group's 32 table rows
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       float t = 0.f;
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float prod = lp[(32 * u + 8 * i + j) * 16 + ((words[i] >> (4 * j)) & 15u)];
+        const float prod = ((pkv_lds_cfloat_ptr)(uintptr_t)pkv_nibble_lds_addr(words[i], 4 * j, group_base))[(8 * i + j) * 16];
         t = (j == 0) ? prod : t + prod;
       }
       const uint32_t wb = (i & 1) ? (wpair[i >> 1] >> 16) : (wpair[i >> 1] & 0xffffu);
