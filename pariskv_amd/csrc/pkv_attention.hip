@@ -450,6 +450,13 @@ __global__ void pkv_attn_merge_kernel(const float *__restrict__ ws, int n_splits
   const int g = tid >> 7, d = tid & 127;
   __shared__ float s_w[8][64];   // weight of split s for head g, already divided by the total
   const float *rowp = ws + (int64_t)row * n_splits * G * kPartStride;
+  // the first 16 splits' partial outputs are requested before the weights are known: one memory round trip
+  // instead of two for the usual case (a few thousand keys)
+  constexpr int kEarly = 16;
+  const float *po = rowp + (int64_t)g * kPartStride + 2 + d;
+  float early[kEarly];
+#pragma unroll
+  for (int s = 0; s < kEarly; ++s) early[s] = s < n_splits ? po[(int64_t)s * G * kPartStride] : 0.f;
   if (d < PKV_WAVE) {  // one wave per head: lane = split
     const bool live = d < n_splits;
     const float *p = rowp + ((int64_t)(live ? d : 0) * G + g) * kPartStride;
@@ -465,9 +472,10 @@ __global__ void pkv_attn_merge_kernel(const float *__restrict__ ws, int n_splits
   }
   __syncthreads();
   float os = 0.f;
-  const float *po = rowp + (int64_t)g * kPartStride + 2 + d;
+#pragma unroll
+  for (int s = 0; s < kEarly; ++s) os += early[s] * (s < n_splits ? s_w[g][s] : 0.f);
 #pragma unroll 8
-  for (int s = 0; s < n_splits; ++s) os += po[(int64_t)s * G * kPartStride] * s_w[g][s];
+  for (int s = kEarly; s < n_splits; ++s) os += po[(int64_t)s * G * kPartStride] * s_w[g][s];
   const int64_t oi = ((int64_t)row * G + g) * 128 + d;
   if (BF16)
     ((uint16_t *)out)[oi] = pkv_f32_to_bf16_bits(os);
