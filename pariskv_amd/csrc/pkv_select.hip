@@ -619,14 +619,20 @@ __device__ __forceinline__ uint32_t lin_bin(uint64_t key, const LinSel &L) {
 // BITS: bins of the ordered key bits instead of the values, for rows of one sign whose values span many binades
 // (e.g. the winners of a selection, about to be sorted): 256 equal steps of the bit pattern between the row's
 // smallest and largest key, i.e. equal steps of the logarithm up to the mantissa's linear pieces.
+// range: null, or the largest and the smallest ordered score of the nonzero keys (range[0] < range[1]: no key at
+// all) where the caller knows them already, which saves the reduction that finds them.
 template <int EIN, bool BITS = false>
 __device__ __forceinline__ bool linear_bins(const uint64_t (&v)[EIN], uint32_t k, uint32_t *s_hist, uint32_t *s_cnt,
-                                            uint32_t *s_bcast, uint32_t (&bin)[EIN], LinSel &L) {
+                                            uint32_t *s_bcast, uint32_t (&bin)[EIN], LinSel &L,
+                                            const uint32_t *range = nullptr) {
   const int tid = threadIdx.x, lane = pkv_lane();
   if (tid < 512) s_hist[tid] = 0;
   if (tid == 0) s_bcast[0] = 0u, s_bcast[1] = 0xffffffffu, s_bcast[5] = 0u, s_bcast[6] = 0u;
   __syncthreads();
   uint32_t mx = 0u, mn = 0xffffffffu;
+  if (range) {
+    mx = range[0], mn = range[1];
+  } else {
 #pragma unroll
   for (int e = 0; e < EIN; ++e) {
     if (v[e] != 0ull) {
@@ -649,6 +655,7 @@ __device__ __forceinline__ bool linear_bins(const uint64_t (&v)[EIN], uint32_t k
   }
   __syncthreads();
   mx = s_bcast[0], mn = s_bcast[1];
+  }
   L.lo = 0.f, L.scale = 0.f, L.lo_bits = mn, L.shift = -1;
   if (BITS) {
     if (mx <= mn) return false;  // one value (or no key at all)
@@ -791,6 +798,64 @@ __device__ __forceinline__ bool counting_sort_desc(const uint64_t (&v)[E], uint3
   return true;
 }
 
+// emit(key, rank) for every key of s_bucket[0 .. n), n <= kLinBucketMax <= 256: rank = number of larger keys, counted
+// by 4 lanes per key, the workgroup's last threads first (the callers' other loops keep the first ones busier).
+// All 1024 threads call it.
+template <typename Emit>
+__device__ __forceinline__ void rank_bucket_desc(const uint64_t *s_bucket, uint32_t n, Emit emit) {
+  const uint32_t i = (kTopkThreads - 1 - threadIdx.x) >> 2, sub = threadIdx.x & 3u;
+  const uint64_t key = s_bucket[i < n ? i : 0];
+  uint32_t r = 0;
+#pragma unroll 4
+  for (uint32_t j = sub; j < n; j += 4) r += s_bucket[j] > key ? 1u : 0u;
+  r += pkv_lane_xor<1>(r);
+  r += pkv_lane_xor<2>(r);
+  if (sub == 0 && i < n) emit(key, r);
+}
+
+// Selection and sort in one binning: the k largest of the nonzero keys held E per thread (there are at least k),
+// sorted descending, into s_out[0 .. k), through s_tmp (k keys, not s_out).  Bins as in counting_sort_desc, over all
+// the keys: those of the bins above the threshold bin b* are placed as there, those of b* are ranked among themselves
+// and the first `need` follow.  False, with s_out untouched, when b* holds more than kLinBucketMax keys, a bin more
+// than kLinRankMax winners, or all keys are equal: the caller then selects and sorts in two steps.  range: as for
+// linear_bins.
+template <int E>
+__device__ __forceinline__ bool select_sort_desc(const uint64_t (&v)[E], uint32_t k, uint64_t *s_tmp, uint64_t *s_out,
+                                                 SelSmem &sm, const uint32_t *range = nullptr) {
+  uint32_t bin[E];
+  LinSel L;
+  if (!linear_bins<E, true>(v, k, sm.hist, sm.cnt, sm.bcast, bin, L, range) || L.max_winners > kLinRankMax) return false;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    if (v[e] != 0ull) {
+      if (bin[e] > L.bstar) s_tmp[atomicAdd(&sm.cnt[bin[e]], 1u)] = v[e];
+      else if (bin[e] == L.bstar) sm.bucket[atomicAdd(&sm.bcast[6], 1u)] = v[e];
+    }
+  }
+  __syncthreads();
+  const uint32_t *s_off = sm.hist + 256;
+  const uint32_t n_above = k - L.need;
+  // The lower a slot, the fewer keys its bin holds: the slots are handed out in pairs (p, n_above - 1 - p), so that
+  // a wave takes crowded and sparse bins in turn.
+  const uint32_t half = (n_above + 1) / 2;
+  for (uint32_t q = threadIdx.x; q < 2 * half; q += kTopkThreads) {
+    const uint32_t p = q < half ? q : n_above - 1 - (q - half);
+    if (q >= half && p < half) continue;  // the middle slot of an odd count is the first half's
+    const uint64_t key = s_tmp[p];
+    const uint32_t b = lin_bin(key, L);
+    const uint32_t start = s_off[b], cnt = sm.cnt[b] - start;
+    uint32_t r = 0;
+#pragma unroll 4
+    for (uint32_t j = 0; j < cnt; ++j) r += s_tmp[start + j] > key ? 1u : 0u;
+    s_out[start + r] = key;
+  }
+  rank_bucket_desc(sm.bucket, L.in_bstar, [&](uint64_t key, uint32_t r) {
+    if (r < L.need) s_out[n_above + r] = key;
+  });
+  __syncthreads();
+  return true;
+}
+
 // s_keys[0 .. P) (the n winners, any order, zero padded) sorted descending in place; s_tmp: P more keys or null.
 template <int NT, int E>
 __device__ __forceinline__ void sort_lds_keys_desc(uint64_t *s_keys, uint32_t n, uint64_t *s_tmp, SelSmem &sm) {
@@ -911,16 +976,12 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
       oi[start + r] = (int64_t)(uint32_t)(~(uint32_t)key);
       if (ov) ov[start + r] = pkv_from_ordered_u32((uint32_t)(key >> 32));
     }
-    for (uint32_t i = kTopkThreads - 1 - tid; i < L.in_bstar; i += kTopkThreads) {  // the last threads: they have the fewest slots above
-      const uint64_t key = s_bucket[i];
-      uint32_t r = 0;
-#pragma unroll 4
-      for (uint32_t j = 0; j < L.in_bstar; ++j) r += s_bucket[j] > key ? 1u : 0u;
+    rank_bucket_desc(s_bucket, L.in_bstar, [&](uint64_t key, uint32_t r) {
       if (r < L.need) {
         oi[n_above + r] = (int64_t)(uint32_t)(~(uint32_t)key);
         if (ov) ov[n_above + r] = pkv_from_ordered_u32((uint32_t)(key >> 32));
       }
-    }
+    });
     return;
   }
   if (lin) {
@@ -1153,6 +1214,54 @@ __device__ __forceinline__ void wide_finish_select(uint32_t k, int P, const uint
   __syncthreads();
 }
 
+// The same with the sort: the k winners sorted descending into s_keys[0 .. k) (zero padded up to max(P, 1024)) by
+// one binning of list A and list B together; EA = max(P, 1024) / 1024 keys of list A per thread, s_tmp: k more keys.
+// Both lists are requested before their lengths are known (clamped indices: one memory round trip, the unused
+// entries are dropped afterwards).  False, with s_keys undefined, where that does not apply: wide_finish_select
+// and a sort then do the same work in two steps.
+template <int EA>
+__device__ __forceinline__ bool wide_finish_select_sort(uint32_t k, int P, const uint32_t *__restrict__ ctl,
+                                                        const uint64_t *__restrict__ list_a,
+                                                        const uint64_t *__restrict__ list_b, int64_t len,
+                                                        uint64_t *s_keys, uint64_t *s_tmp, SelSmem &sm) {
+  const int tid = threadIdx.x;
+  uint64_t v[EA + 8];
+#pragma unroll
+  for (int e = 0; e < EA; ++e) {
+    const uint32_t i = (uint32_t)(tid + e * kTopkThreads);
+    v[e] = list_a[i < k ? i : k - 1];
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int64_t i = tid + e * kTopkThreads;
+    v[EA + e] = list_b[i < len ? i : len - 1];
+  }
+  const uint32_t n_a = ctl[kWideBins], n_b = ctl[kWideBins + 1];
+  if (n_a > k || n_b > (uint32_t)kWideSlice || (int64_t)n_b > len || n_a + n_b < k) return false;
+#pragma unroll
+  for (int e = 0; e < EA; ++e) v[e] = (uint32_t)(tid + e * kTopkThreads) < n_a ? v[e] : 0ull;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[EA + e] = (uint32_t)(tid + e * kTopkThreads) < n_b ? v[EA + e] : 0ull;
+  for (int i = tid; i < (P < 1024 ? 1024 : P); i += kTopkThreads) s_keys[i] = 0ull;
+  return select_sort_desc<EA + 8>(v, k, s_tmp, s_keys, sm);
+}
+
+// Either way: true = s_keys is sorted already.  s_tmp: null when the second copy of the list is not set up.
+__device__ __forceinline__ bool wide_finish_keys(uint32_t k, int P, const uint32_t *__restrict__ ctl,
+                                                 const uint64_t *__restrict__ list_a,
+                                                 const uint64_t *__restrict__ list_b, int64_t len, uint64_t *s_keys,
+                                                 uint64_t *s_tmp, SelSmem &sm) {
+  bool sorted = false;
+  if (s_tmp) {
+    sorted = P <= 1024 ? wide_finish_select_sort<1>(k, P, ctl, list_a, list_b, len, s_keys, s_tmp, sm)
+                       : wide_finish_select_sort<2>(k, P, ctl, list_a, list_b, len, s_keys, s_tmp, sm);
+    if (sorted) return true;
+    __syncthreads();
+  }
+  wide_finish_select(k, P, ctl, list_a, list_b, len, s_keys, sm);
+  return false;
+}
+
 // Largest and smallest ordered score of a workgroup's values into the row's control block (both words grow from
 // zero under atomicMax: the minimum is kept complemented).  s_red: 32 words.  All threads of the workgroup.
 __device__ __forceinline__ void wide_range_atomics(uint32_t mx, uint32_t mn, uint32_t *__restrict__ rctl, uint32_t *s_red) {
@@ -1230,13 +1339,15 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_wide_finish_kernel(
   __shared__ SelSmem sm;
   uint64_t *s_tmp = P <= kCountingSortMaxP ? s_keys + (P < 1024 ? 1024 : P) : nullptr;
   const int row = blockIdx.x;
-  wide_finish_select((uint32_t)k, P, ctl + (int64_t)row * kWideRowWords, list_a + (int64_t)row * k,
-                     list_b + (int64_t)row * len, len, s_keys, sm);
+  const bool sorted = wide_finish_keys((uint32_t)k, P, ctl + (int64_t)row * kWideRowWords, list_a + (int64_t)row * k,
+                                       list_b + (int64_t)row * len, len, s_keys, s_tmp, sm);
   int64_t *oi = out_ids + (int64_t)row * k;
   float *ov = out_vals ? out_vals + (int64_t)row * k : nullptr;
+  if (!sorted) {
 #define PKV_SORT_K(NT, E) sort_lds_keys_desc<NT, E>(s_keys, (uint32_t)k, s_tmp, sm)
-  PKV_DISPATCH_E(P, PKV_SORT_K);
+    PKV_DISPATCH_E(P, PKV_SORT_K);
 #undef PKV_SORT_K
+  }
   for (int64_t i = threadIdx.x; i < k; i += kTopkThreads) {
     const uint64_t key = s_keys[i];
     oi[i] = (int64_t)(uint32_t)(~(uint32_t)key);
@@ -1301,6 +1412,43 @@ __device__ __forceinline__ float block_max_1024(float v, float *s_part) {
   return r;
 }
 
+// Two sums, each in the order of block_tree_sum_1024, and the largest / smallest of two unsigned words, all in one
+// pass (two barriers).  s_red: 64 words.  Every thread returns the same values.
+struct AdkReduced {
+  float sum_a, sum_b;
+  uint32_t mx, mn;
+};
+__device__ __forceinline__ AdkReduced block_reduce_adk_1024(float a, float b, uint32_t mx, uint32_t mn, uint32_t *s_red) {
+#pragma unroll
+  for (int m = 1; m < PKV_WAVE; m <<= 1) {
+    const float oa = __shfl_xor(a, m, PKV_WAVE), ob = __shfl_xor(b, m, PKV_WAVE);
+    const uint32_t ox = (uint32_t)__shfl_xor((int)mx, m, PKV_WAVE), on = (uint32_t)__shfl_xor((int)mn, m, PKV_WAVE);
+    a = a + oa, b = b + ob;
+    mx = ox > mx ? ox : mx, mn = on < mn ? on : mn;
+  }
+  __syncthreads();
+  if (pkv_lane() == 0) {
+    const int w = threadIdx.x / PKV_WAVE;
+    s_red[w] = __float_as_uint(a), s_red[16 + w] = __float_as_uint(b), s_red[32 + w] = mx, s_red[48 + w] = mn;
+  }
+  __syncthreads();
+  float wa[16], wb[16];
+  AdkReduced r;
+  r.mx = 0u, r.mn = 0xffffffffu;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    wa[i] = __uint_as_float(s_red[i]), wb[i] = __uint_as_float(s_red[16 + i]);
+    r.mx = s_red[32 + i] > r.mx ? s_red[32 + i] : r.mx;
+    r.mn = s_red[48 + i] < r.mn ? s_red[48 + i] : r.mn;
+  }
+#pragma unroll
+  for (int h = 1; h < 16; h <<= 1)
+#pragma unroll
+    for (int i = 0; i < 16; i += 2 * h) wa[i] = wa[i] + wa[i + h], wb[i] = wb[i] + wb[i + h];
+  r.sum_a = wa[0], r.sum_b = wb[0];
+  return r;
+}
+
 __device__ __forceinline__ float cand_logit(const void *__restrict__ scores, int dtype, float scale, int64_t i) {
   const float x = (dtype == PKV_DTYPE_BF16) ? pkv_bf16_bits_to_f32(((const uint16_t *)scores)[i])
                                             : ((const float *)scores)[i];
@@ -1351,12 +1499,15 @@ __device__ __forceinline__ float wave_running_sum(float val, float carry) {
 // target is never reached).  prefix is the cumulative sum of the reference (adaptive_topk.py:300-303) in
 // a fixed two-level order: blocks of 64 consecutive benefits are summed left to right, the block totals
 // are summed left to right, prefix_i = (total of the earlier blocks) + (running sum inside the block).
-// All 1024 threads call it; k_out <= 8192.  s_f: 256 floats, s_k: one word.
+// Benefits are not negative, so the prefixes never decrease: the first block whose last prefix reaches the
+// target holds the answer.  Every wave runs the short second level for itself (no barrier for its result);
+// the wave that owns that block finds the element.  All 1024 threads call it; k_out <= 8192.
+// s_f: 128 floats, s_k: one word.
 __device__ __forceinline__ int64_t first_k_reaching(const uint64_t *s_keys, int64_t k_out, float sl_benefit, float tgt,
                                                     float *s_f, uint32_t *s_k) {
   const int lane = pkv_lane(), wave = threadIdx.x / PKV_WAVE;
   const int n_blocks = (int)((k_out + PKV_WAVE - 1) / PKV_WAVE);  // <= 128; wave w owns blocks w, w+16, ...
-  float *s_tot = s_f, *s_before = s_f + 128;
+  float *s_tot = s_f;
   float run[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
@@ -1370,56 +1521,59 @@ __device__ __forceinline__ int64_t first_k_reaching(const uint64_t *s_keys, int6
   }
   if (threadIdx.x == 0) *s_k = (uint32_t)k_out;
   __syncthreads();
-  if (wave == 0) {
-    float carry = 0.f;
-    for (int base = 0; base < n_blocks; base += PKV_WAVE) {
-      const int c = base + lane;
-      const float incl = wave_running_sum(c < n_blocks ? s_tot[c] : 0.f, carry);
-      const float before =
-          __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(carry), __float_as_int(incl), 0x138, 0xf, 0xf, false));
-      if (c < n_blocks) s_before[c] = before;
-      carry = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(incl), PKV_WAVE - 1));
+  // second level: lane l of pass p holds block 64p + l; the chain of adds needs as many steps as there are blocks
+  int cstar = -1;
+  float before_star = 0.f, carry = 0.f;
+  for (int base = 0; base < n_blocks && cstar < 0; base += PKV_WAVE) {
+    const int c = base + lane, live = n_blocks - base < PKV_WAVE ? n_blocks - base : PKV_WAVE;
+    const float val = c < n_blocks ? s_tot[c] : 0.f;
+    float acc = val;
+    for (int st = 0; st < live; ++st) {
+      const float below =
+          __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(carry), __float_as_int(acc), 0x138, 0xf, 0xf, false));
+      acc = below + val;
     }
+    const float before =
+        __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(carry), __float_as_int(acc), 0x138, 0xf, 0xf, false));
+    const uint64_t hit = __ballot(c < n_blocks && sl_benefit + acc >= tgt);
+    if (hit) {
+      const int l = __ffsll((long long)hit) - 1;
+      cstar = base + l;
+      before_star = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(before), l));
+    }
+    carry = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(acc), live - 1));
   }
-  __syncthreads();
+  if (cstar >= 0 && (cstar & 15) == wave) {
+    float mine = run[0];
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int c = wave + 16 * j;
-    if (c < n_blocks) {
-      const int64_t i = (int64_t)c * PKV_WAVE + lane;
-      const uint64_t hit = __ballot(i < k_out && sl_benefit + (s_before[c] + run[j]) >= tgt);
-      if (hit && lane == 0) atomicMin(s_k, (uint32_t)(c * PKV_WAVE + __ffsll((long long)hit)));
-    }
+    for (int j = 1; j < 8; ++j) mine = (cstar >> 4) == j ? run[j] : mine;
+    const int64_t i = (int64_t)cstar * PKV_WAVE + lane;
+    const uint64_t hit = __ballot(i < k_out && sl_benefit + (before_star + mine) >= tgt);
+    if (lane == 0 && hit) *s_k = (uint32_t)(cstar * PKV_WAVE + __ffsll((long long)hit));
   }
   __syncthreads();
   return (int64_t)*s_k;
 }
 
-// Joint maximum of the partial maxima and sum of the per-slice sums of a row, the sums in slice order
-// starting from the first.  All 1024 threads call it (one barrier); s_out: 2 floats.
-__device__ __forceinline__ void combine_slices(const float *__restrict__ pmax, int n_parts,
-                                               const float *__restrict__ ssum, int n_slices, float *s_out, float &g,
-                                               float &csum) {
+// Sum of the per-slice sums of a row in slice order, starting from the first.  `first` is ssum[lane] (0 beyond
+// n_slices) as loaded by the caller's first wave ahead of time.  All 1024 threads call it (one barrier); s_out: 1 float.
+__device__ __forceinline__ float combine_slices(const float *__restrict__ ssum, int n_slices, float first, float *s_out) {
   if (threadIdx.x < PKV_WAVE) {
     const int lane = pkv_lane();
-    float m = -__uint_as_float(0x7f800000u), carry = 0.f;
-    for (int i = lane; i < n_parts; i += PKV_WAVE) m = fmaxf(m, pmax[i]);
+    float carry = 0.f;
     for (int base = 0; base < n_slices; base += PKV_WAVE) {
       const int i = base + lane;
-      const float acc = wave_running_sum(i < n_slices ? ssum[i] : 0.f, carry);
+      const float acc = wave_running_sum(base == 0 ? first : (i < n_slices ? ssum[i] : 0.f), carry);
       carry = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(acc), PKV_WAVE - 1));
     }
-#pragma unroll
-    for (int x = 1; x < PKV_WAVE; x <<= 1) m = fmaxf(m, __shfl_xor(m, x, PKV_WAVE));
-    if (lane == 0) s_out[0] = m, s_out[1] = carry;
+    if (lane == 0) s_out[0] = carry;
   }
   __syncthreads();
-  g = s_out[0];
-  csum = s_out[1];
+  return s_out[0];
 }
 
-// Shared tail: s_keys[0 .. P) holds the k_out winners (zero padded, any order).  Sorts them, finds k,
-// writes adaptive_k[row] and the candidate ids in benefit order.
+// Shared tail: s_keys[0 .. P) holds the k_out winners (zero padded; sorted descending already, or in any order).
+// Sorts them where they are not, finds k, writes adaptive_k[row] and the candidate ids in benefit order.
 // What the caller does with k right after the kernel, folded into it: the clamp to [k_min, k_max] (off when
 // k_max <= 0) and the per-row key count row_keys[row] = row_keys_base + k that the attention kernel reads.
 struct AdkClamp {
@@ -1431,13 +1585,26 @@ struct AdkClamp {
 __device__ __forceinline__ void adaptive_tail(uint64_t *s_keys, int P, int64_t k_out, float sl_benefit, float total,
                                               float threshold, const int64_t *__restrict__ ci, int64_t n_cand,
                                               int64_t *__restrict__ adaptive_k_row, int64_t *__restrict__ ids_row,
-                                              AdkClamp cl, int row, SelSmem &sm) {
-  uint64_t *s_tmp = P <= kCountingSortMaxP ? s_keys + (P < 1024 ? 1024 : P) : nullptr;
+                                              AdkClamp cl, int row, SelSmem &sm, bool sorted) {
+  if (!sorted) {
+    uint64_t *s_tmp = P <= kCountingSortMaxP ? s_keys + (P < 1024 ? 1024 : P) : nullptr;
 #define PKV_SORT_K(NT, E) sort_lds_keys_desc<NT, E>(s_keys, (uint32_t)k_out, s_tmp, sm)
-  PKV_DISPATCH_E(P, PKV_SORT_K);
+    PKV_DISPATCH_E(P, PKV_SORT_K);
 #undef PKV_SORT_K
+  }
   float *s_f = (float *)sm.hist;
   uint32_t *s_k = &sm.counter;
+  // the winners' ids do not depend on k: they are requested now and stored after the search for k
+  int64_t id[kTopkMaxSort / kTopkThreads];
+#pragma unroll
+  for (int e = 0; e < kTopkMaxSort / kTopkThreads; ++e) {
+    const int64_t i = threadIdx.x + e * kTopkThreads;
+    id[e] = 0;
+    if (i < k_out) {
+      const uint32_t pos = ~(uint32_t)s_keys[i];
+      if (pos < (uint64_t)n_cand) id[e] = ci[pos];
+    }
+  }
   int64_t k = 1;  // total <= 0: adaptive_topk.py:304-306
   if (total > 0.f) k = first_k_reaching(s_keys, k_out, sl_benefit, threshold * total, s_f, s_k);
   if (threadIdx.x == 0) {
@@ -1445,9 +1612,10 @@ __device__ __forceinline__ void adaptive_tail(uint64_t *s_keys, int P, int64_t k
     *adaptive_k_row = k;
     if (cl.row_keys) cl.row_keys[row] = (int32_t)(cl.row_keys_base + k);
   }
-  for (int64_t i = threadIdx.x; i < k_out; i += kTopkThreads) {
-    const uint32_t pos = ~(uint32_t)s_keys[i];
-    ids_row[i] = (pos < (uint64_t)n_cand) ? ci[pos] : 0;
+#pragma unroll
+  for (int e = 0; e < kTopkMaxSort / kTopkThreads; ++e) {
+    const int64_t i = threadIdx.x + e * kTopkThreads;
+    if (i < k_out) ids_row[i] = id[e];
   }
 }
 
@@ -1488,6 +1656,7 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adaptive_topk_kernel(
     int64_t *__restrict__ adaptive_k, int64_t *__restrict__ topk_ids, AdkClamp cl) {
   extern __shared__ uint64_t s_keys[];
   __shared__ float s_part[16];
+  __shared__ uint32_t s_red[64];
   __shared__ SelSmem sm;
   const int row = blockIdx.x;
   const int tid = threadIdx.x;
@@ -1503,47 +1672,90 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adaptive_topk_kernel(
     logit[e] = i < n_cand ? lg : -__uint_as_float(0x7f800000u);
     vnorm[e] = i < n_cand ? vv : 0.f;
   }
+  // the first 2048 dense tokens stay in registers for the maximum and for their benefits
+  constexpr int kDenseRegs = 2;
+  float dl[kDenseRegs], dv[kDenseRegs];
+#pragma unroll
+  for (int e = 0; e < kDenseRegs; ++e) {
+    const int64_t i = tid + e * kTopkThreads;
+    dl[e] = -__uint_as_float(0x7f800000u), dv[e] = 0.f;
+    if (i < sl) dl[e] = r.sll[i], dv[e] = r.slv[i];
+  }
   float m = -__uint_as_float(0x7f800000u);
-  for (int64_t i = tid; i < sl; i += kTopkThreads) m = fmaxf(m, r.sll[i]);
+  for (int64_t i = tid + kDenseRegs * kTopkThreads; i < sl; i += kTopkThreads) m = fmaxf(m, r.sll[i]);
+#pragma unroll
+  for (int e = 0; e < kDenseRegs; ++e) m = fmaxf(m, dl[e]);
 #pragma unroll
   for (int e = 0; e < EIN; ++e) m = fmaxf(m, logit[e]);
   const float g = block_max_1024(m, s_part);  // joint max (adaptive_topk.py:282-286)
-  const float sl_benefit = dense_benefit_sum(r.sll, r.slv, sl, g, s_part);
+  // benefits of the first slice of dense tokens (a lane adds its elements in increasing i, as dense_benefit_sum
+  // does) and of the candidates; both sums and the range of the candidates' keys in one reduction
+  float dacc = 0.f;
+#pragma unroll
+  for (int e = 0; e < kWideSlice / kTopkThreads; ++e) {
+    const int64_t i = tid + e * kTopkThreads;
+    if (i < sl) {
+      const float x = e < kDenseRegs ? dl[e < kDenseRegs ? e : 0] : r.sll[i];
+      const float w = e < kDenseRegs ? dv[e < kDenseRegs ? e : 0] : r.slv[i];
+      dacc = dacc + pkv_expf(x - g) * w;
+    }
+  }
   uint64_t v[EIN];
   float acc = 0.f;
+  uint32_t kmax = 0u, kmin = 0xffffffffu;
 #pragma unroll
   for (int e = 0; e < EIN; ++e) {
     const int i = tid + e * kTopkThreads;
     const float b = i < n_cand ? pkv_expf(logit[e] - g) * vnorm[e] : 0.f;
     acc = acc + b;
-    v[e] = i < n_cand ? (((uint64_t)pkv_ordered_u32(b) << 32) | (uint64_t)(~(uint32_t)i)) : 0ull;
+    const uint32_t ob = pkv_ordered_u32(b);
+    v[e] = i < n_cand ? (((uint64_t)ob << 32) | (uint64_t)(~(uint32_t)i)) : 0ull;
+    if (i < n_cand) kmax = ob > kmax ? ob : kmax, kmin = ob < kmin ? ob : kmin;
   }
-  const float total = sl_benefit + block_tree_sum_1024(acc, s_part);
-
-  // the k_out largest (benefit, ~position) keys
-  if (tid == 0) sm.counter = 0;
-  for (int i = tid; i < (P < 1024 ? 1024 : P); i += kTopkThreads) s_keys[i] = 0ull;
-  bool win[EIN];
-  if (k_out < n_cand) {
-    select_topk_flags<EIN, true>(v, (uint32_t)k_out, sm, win);  // benefits span many binades: bins of the key bits
-  } else {
+  const AdkReduced red = block_reduce_adk_1024(dacc, acc, kmax, kmin, s_red);
+  float sl_benefit = red.sum_a;
+  for (int64_t s0 = kWideSlice; s0 < sl; s0 += kWideSlice) {  // further slices of dense tokens, added in slice order
+    float a2 = 0.f;
 #pragma unroll
-    for (int e = 0; e < EIN; ++e) win[e] = v[e] != 0ull;
+    for (int e = 0; e < kWideSlice / kTopkThreads; ++e) {
+      const int64_t i = s0 + e * kTopkThreads + tid;
+      if (i < sl) a2 = a2 + pkv_expf(r.sll[i] - g) * r.slv[i];
+    }
+    sl_benefit = add_slice_sum(sl_benefit, false, a2, s_part);
+  }
+  const float total = sl_benefit + red.sum_b;
+  const uint32_t key_range[2] = {red.mx, red.mn};
+
+  // the k_out largest (benefit, ~position) keys, sorted: in one binning where that applies (benefits span many
+  // binades: bins of the key bits), else selected first and sorted afterwards
+  if (tid == 0) sm.counter = 0;
+  const int Pz = P < 1024 ? 1024 : P;
+  for (int i = tid; i < Pz; i += kTopkThreads) s_keys[i] = 0ull;
+  const bool sorted = P <= kCountingSortMaxP &&
+                      select_sort_desc<EIN>(v, (uint32_t)k_out, s_keys + Pz, s_keys, sm, key_range);  // k_out <= n_cand
+  if (!sorted) {
+    bool win[EIN];
+    if (k_out < n_cand) {
+      select_topk_flags<EIN, true>(v, (uint32_t)k_out, sm, win);
+    } else {
+#pragma unroll
+      for (int e = 0; e < EIN; ++e) win[e] = v[e] != 0ull;
+      __syncthreads();
+    }
+#pragma unroll
+    for (int e = 0; e < EIN; ++e) {
+      const uint32_t slot = wave_take_slots(&sm.counter, win[e]);
+      if (win[e] && slot < (uint32_t)k_out) s_keys[slot] = v[e];
+    }
     __syncthreads();
   }
-#pragma unroll
-  for (int e = 0; e < EIN; ++e) {
-    const uint32_t slot = wave_take_slots(&sm.counter, win[e]);
-    if (win[e] && slot < (uint32_t)k_out) s_keys[slot] = v[e];
-  }
-  __syncthreads();
   adaptive_tail(s_keys, P, k_out, sl_benefit, total, threshold, r.ci, n_cand, adaptive_k + row,
-                topk_ids + (int64_t)row * k_out, cl, row, sm);
+                topk_ids + (int64_t)row * k_out, cl, row, sm, sorted);
 }
 
 // ---- n_cand > 8192: slices of 8192 candidates, one workgroup each ----
 // Workspace per row: ben f32 [n_cand]; gathered norms f32 [n_cand]; partial maxima f32 [n_cand/2048];
-// slice sums f32 [n_slices];
+// slice sums f32 [n_slices], then the sum over the dense tokens;
 // control block u32 [kWideRowWords]; list A u64 [k_out]; list B u64 [n_cand].
 
 struct BenefitKeys {  // key i = (benefit, ~position)
@@ -1607,15 +1819,17 @@ __global__ __launch_bounds__(kAdkPartThreads) void pkv_adk_max_gather_kernel(
   }
 }
 
-// grid (slices, rows) x 1024: benefits of the slice into ws_ben, their sum (lane order, then the 1024-lane tree)
-// into ws_sum, and their top key bits into the row histogram.
+// grid (slices + 1, rows) x 1024: benefits of the slice into ws_ben, their sum (lane order, then the 1024-lane tree)
+// into ws_sum, and their top key bits into the row histogram; one more workgroup per row sums the benefits of the
+// dense tokens meanwhile.
 __global__ __launch_bounds__(kTopkThreads) void pkv_adk_benefit_kernel(
-    const void *__restrict__ cand_scores, int cand_dtype, float cand_scale, const float *__restrict__ cand_vnorm,
-    int64_t n_cand, const float *__restrict__ ws_max, int n_parts, float *__restrict__ ws_ben,
-    float *__restrict__ ws_sum, uint32_t *__restrict__ ctl) {
+    const float *__restrict__ sl_logits, int64_t sl_stride, const float *__restrict__ sl_vnorm, int64_t slv_stride,
+    int64_t sl, const void *__restrict__ cand_scores, int cand_dtype, float cand_scale,
+    const float *__restrict__ cand_vnorm, int64_t n_cand, const float *__restrict__ ws_max, int n_parts,
+    float *__restrict__ ws_ben, float *__restrict__ ws_sum, uint32_t *__restrict__ ctl) {
   __shared__ float s_part[16];
   __shared__ uint32_t s_bins[kWideBins];
-  const int row = blockIdx.y, slice = blockIdx.x, tid = threadIdx.x, n_slices = gridDim.x;
+  const int row = blockIdx.y, slice = blockIdx.x, tid = threadIdx.x, n_slices = gridDim.x - 1;
   const char *cs = (const char *)cand_scores + (int64_t)row * n_cand * (cand_dtype == PKV_DTYPE_BF16 ? 2 : 4);
   const float *cv = cand_vnorm + (int64_t)row * n_cand;  // the caller's, or the ones gathered by the first launch
   float *ben = ws_ben + (int64_t)row * n_cand;
@@ -1623,6 +1837,12 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adk_benefit_kernel(
   for (int w = tid & (PKV_WAVE - 1); w < n_parts; w += PKV_WAVE) g = fmaxf(g, ws_max[(int64_t)row * n_parts + w]);
 #pragma unroll
   for (int x = 1; x < PKV_WAVE; x <<= 1) g = fmaxf(g, __shfl_xor(g, x, PKV_WAVE));
+  if (slice == n_slices) {  // the row's last workgroup: the dense tokens' benefit, kept after the slice sums
+    const float d = dense_benefit_sum(sl_logits + (int64_t)row * sl_stride, sl_vnorm + (int64_t)row * slv_stride, sl, g,
+                                      s_part);
+    if (tid == 0) ws_sum[(int64_t)row * (n_slices + 1) + n_slices] = d;
+    return;
+  }
   float lg[kWideE], vv[kWideE];
 #pragma unroll
   for (int e = 0; e < kWideE; ++e) {
@@ -1644,7 +1864,7 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adk_benefit_kernel(
     }
   }
   const float ssum = block_tree_sum_1024(acc, s_part);
-  if (tid == 0) ws_sum[(int64_t)row * n_slices + slice] = ssum;
+  if (tid == 0) ws_sum[(int64_t)row * (n_slices + 1) + slice] = ssum;
   wide_hist_slice(WideBinning{52, 0.f, 0.f}, keys, n_cand, slice, s_bins, ctl + (int64_t)row * kWideRowWords);
 }
 
@@ -1661,27 +1881,27 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_adk_compact_kernel(const flo
                          list_b + (int64_t)row * n_cand, s_tmp);
 }
 
-// grid rows; dynamic LDS max(P,1024)*8 bytes.
+// grid rows; dynamic LDS: lds_bytes_sort(P).
 __global__ __launch_bounds__(kTopkThreads) void pkv_adk_finish_kernel(
-    const float *__restrict__ sl_logits, int64_t sl_stride, const float *__restrict__ sl_vnorm, int64_t slv_stride,
-    int64_t sl, const int64_t *__restrict__ cand_ids, int64_t n_cand, int n_slices, int n_parts, float threshold,
-    int64_t k_out, int P,
-    const float *__restrict__ ws_max, const float *__restrict__ ws_sum, const uint32_t *__restrict__ ctl,
-    const uint64_t *__restrict__ list_a, const uint64_t *__restrict__ list_b, int64_t *__restrict__ adaptive_k,
-    int64_t *__restrict__ topk_ids, AdkClamp cl) {
+    const int64_t *__restrict__ cand_ids, int64_t n_cand, int n_slices, float threshold, int64_t k_out, int P,
+    const float *__restrict__ ws_sum, const uint32_t *__restrict__ ctl, const uint64_t *__restrict__ list_a,
+    const uint64_t *__restrict__ list_b, int64_t *__restrict__ adaptive_k, int64_t *__restrict__ topk_ids, AdkClamp cl) {
   extern __shared__ uint64_t s_keys[];
   __shared__ float s_part[16];
   __shared__ SelSmem sm;
   const int row = blockIdx.x;
-  float g, csum;
-  combine_slices(ws_max + (int64_t)row * n_parts, n_parts, ws_sum + (int64_t)row * n_slices, n_slices, s_part, g, csum);
-  const float sl_benefit = dense_benefit_sum(sl_logits + (int64_t)row * sl_stride, sl_vnorm + (int64_t)row * slv_stride,
-                                             sl, g, s_part);
-  const float total = sl_benefit + csum;
-  wide_finish_select((uint32_t)k_out, P, ctl + (int64_t)row * kWideRowWords, list_a + (int64_t)row * k_out,
-                     list_b + (int64_t)row * n_cand, n_cand, s_keys, sm);
+  // the sums left by the benefit launch are requested now and added up after the selection
+  const float *ss = ws_sum + (int64_t)row * (n_slices + 1);
+  const int lane = pkv_lane();
+  const float first = lane < n_slices ? ss[lane] : 0.f;
+  const float sl_benefit = ss[n_slices];
+  uint64_t *s_tmp = P <= kCountingSortMaxP ? s_keys + (P < 1024 ? 1024 : P) : nullptr;
+  const bool sorted = wide_finish_keys((uint32_t)k_out, P, ctl + (int64_t)row * kWideRowWords,
+                                       list_a + (int64_t)row * k_out, list_b + (int64_t)row * n_cand, n_cand, s_keys,
+                                       s_tmp, sm);
+  const float total = sl_benefit + combine_slices(ss, n_slices, first, s_part);
   adaptive_tail(s_keys, P, k_out, sl_benefit, total, threshold, cand_ids + (int64_t)row * n_cand, n_cand,
-                adaptive_k + row, topk_ids + (int64_t)row * k_out, cl, row, sm);
+                adaptive_k + row, topk_ids + (int64_t)row * k_out, cl, row, sm, sorted);
 }
 
 // uniform_k[r] = max over all rows of adaptive_k, row_keys[r] = base + that maximum: the dense form of the
@@ -1986,7 +2206,7 @@ static AdkWs adk_ws_layout(int rows, int64_t n_cand, int64_t k_out) {
   w.smax = off;
   off = pkv_align_up(off + (size_t)rows * (size_t)((n_cand + kAdkPart - 1) / kAdkPart) * sizeof(float), 256);
   w.ssum = off;
-  off = pkv_align_up(off + (size_t)rows * n_slices * sizeof(float), 256);
+  off = pkv_align_up(off + (size_t)rows * (n_slices + 1) * sizeof(float), 256);  // slice sums, then the dense tokens' sum
   w.wide = wide_ws_layout(rows, n_cand, k_out, off);
   w.total = w.wide.total;
   return w;
@@ -2048,15 +2268,14 @@ extern "C" int pkv_adaptive_topk(const float *sl_logits, int64_t sl_stride, cons
                      sl_logits, sl_stride, sl, cand_scores, cand_dtype, cand_scale, cand_vnorm ? nullptr : value_norm,
                      vn_stride, vn_offset, vn_pos_stride, cand_ids, n_cand, smax, gathered, ctl);
   PKV_LAUNCH_CHECK("pkv_adk_max_gather_kernel");
-  hipLaunchKernelGGL(pkv_adk_benefit_kernel, grid, dim3(kTopkThreads), 0, s, cand_scores, cand_dtype, cand_scale,
+  hipLaunchKernelGGL(pkv_adk_benefit_kernel, dim3((unsigned)n_slices + 1, (unsigned)rows), dim3(kTopkThreads), 0, s,
+                     sl_logits, sl_stride, sl_vnorm, slv_stride, sl, cand_scores, cand_dtype, cand_scale,
                      cand_vnorm ? cand_vnorm : gathered, n_cand, smax, n_parts, ben, ssum, ctl);
   PKV_LAUNCH_CHECK("pkv_adk_benefit_kernel");
   hipLaunchKernelGGL(pkv_adk_compact_kernel, grid, dim3(kTopkThreads), 0, s, ben, n_cand, k_out, ctl, list_a, list_b);
   PKV_LAUNCH_CHECK("pkv_adk_compact_kernel");
-  hipLaunchKernelGGL(pkv_adk_finish_kernel, dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes_sort(P), s, sl_logits,
-                     sl_stride, sl_vnorm, slv_stride, sl, cand_ids, n_cand, n_slices, n_parts, threshold, k_out, P, smax, ssum,
-                     ctl,
-                     list_a, list_b, adaptive_k, topk_ids, cl);
+  hipLaunchKernelGGL(pkv_adk_finish_kernel, dim3((unsigned)rows), dim3(kTopkThreads), lds_bytes_sort(P), s, cand_ids,
+                     n_cand, n_slices, threshold, k_out, P, ssum, ctl, list_a, list_b, adaptive_k, topk_ids, cl);
   PKV_LAUNCH_CHECK("pkv_adk_finish_kernel");
   return PKV_OK;
 }
