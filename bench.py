@@ -103,10 +103,11 @@ def main():
     ap.add_argument("--candidates", type=int, default=4096)
     ap.add_argument("--topk", type=int, default=1024)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["scan", "copy", "adaptive", "decode-loop", "model-decode"], default=None,
-                    help="profiling aid: launch only the collision scan, the calibration copy, or the adaptive-k stage "
+    ap.add_argument("--only", choices=["scan", "copy", "adaptive", "topk", "decode-loop", "model-decode"], default=None,
+                    help="profiling aid: launch only the collision scan, the calibration copy, the adaptive-k stage "
                          "(--candidates scores per row, dense prefix 1600, value norms gathered from a --context table, "
-                         "list length --topk) --steps times; decode-loop: the polar_cache class itself, --layers layers, "
+                         "list length --topk) or the exact top-k (--topk of --candidates N(30,20) scores per row) "
+                         "--steps times; decode-loop: the polar_cache class itself, --layers layers, "
                          "--context prompt tokens, --steps generated tokens (append + retrieval + gather + attention per "
                          "layer, index refresh and host offload every 1024 tokens); model-decode: the same loop inside a "
                          "random-initialised Qwen3-8B-shaped decoder (config 5: --layers 36 --batch 8 --context 65536 "
@@ -221,6 +222,17 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"only": "adaptive", "launches": args.warmup + args.steps, "rows": R, "candidates": Cn,
                           "list": K, "adaptive_k_row0": int(ak.flatten()[0])}))
+        return
+
+    if args.only == "topk":
+        g = torch.Generator(device=dev).manual_seed(0)
+        scores = torch.randn(R, Cn, generator=g, device=dev) * 20 + 30
+        for _ in range(args.warmup + args.steps):
+            ids = ops.topk_f32(scores, K)
+        torch.cuda.synchronize()
+        print(json.dumps({"only": "topk", "launches": args.warmup + args.steps, "rows": R, "scores_per_row": Cn, "k": K,
+                          "values_equal_torch_topk": bool(torch.equal(torch.gather(scores, 1, ids),
+                                                                      torch.topk(scores, K, dim=-1).values))}))
         return
 
     # ---------------------------------------------------------------- inputs

@@ -1262,9 +1262,11 @@ __device__ __forceinline__ bool wide_finish_keys(uint32_t k, int P, const uint32
   return false;
 }
 
-// Largest and smallest ordered score of a workgroup's values into the row's control block (both words grow from
-// zero under atomicMax: the minimum is kept complemented).  s_red: 32 words.  All threads of the workgroup.
-__device__ __forceinline__ void wide_range_atomics(uint32_t mx, uint32_t mn, uint32_t *__restrict__ rctl, uint32_t *s_red) {
+// Largest and smallest ordered score of a workgroup's values into the row's control block.  slot < 0: the range
+// words (both grow from zero under atomicMax: the minimum is kept complemented; ctl zero at launch); slot >= 0: that
+// range slot, written plainly, no matter what it held.  s_red: 32 words.  All threads of the workgroup.
+__device__ __forceinline__ void wide_range_out(uint32_t mx, uint32_t mn, uint32_t *__restrict__ rctl, int slot,
+                                               uint32_t *s_red) {
 #pragma unroll
   for (int x = 1; x < PKV_WAVE; x <<= 1) {
     const uint32_t a = (uint32_t)__shfl_xor((int)mx, x, PKV_WAVE), c = (uint32_t)__shfl_xor((int)mn, x, PKV_WAVE);
@@ -1279,19 +1281,27 @@ __device__ __forceinline__ void wide_range_atomics(uint32_t mx, uint32_t mn, uin
       mx = s_red[w] > mx ? s_red[w] : mx;
       mn = s_red[16 + w] < mn ? s_red[16 + w] : mn;
     }
-    if (mx >= mn) {  // at least one value
+    const bool any = mx >= mn;  // at least one value
+    if (slot >= 0) {
+      rctl[kWideCtlSlots + 2 * slot] = any ? mx : 0u;
+      rctl[kWideCtlSlots + 2 * slot + 1] = any ? ~mn : 0u;
+    } else if (any) {
       atomicMax(&rctl[kWideCtlMax], mx);
       atomicMax(&rctl[kWideCtlMinInv], ~mn);
     }
   }
 }
 
-// grid (slices, rows).  ctl zero at launch.  The rows' score ranges for the launches that follow.
+// grid (slices, rows).  The rows' score ranges for the launches that follow.  own_slots = 0: ctl zero at launch, the
+// ranges go to the range words.  own_slots = 1 (at most kWideRangeSlots slices): nothing is assumed about ctl; every
+// slice fills its own range slot and the row's first slice clears the rest of the control block.
 __global__ __launch_bounds__(kTopkThreads) void pkv_topk_wide_range_kernel(const float *__restrict__ x, int64_t x_stride,
-                                                                           int64_t len, uint32_t *__restrict__ ctl) {
+                                                                           int64_t len, uint32_t *__restrict__ ctl,
+                                                                           int own_slots) {
   __shared__ uint32_t s_red[32];
   const int row = blockIdx.y;
   const float *xr = x + (int64_t)row * x_stride;
+  uint32_t *rctl = ctl + (int64_t)row * kWideRowWords;
   uint32_t mx = 0u, mn = 0xffffffffu;
 #pragma unroll
   for (int e = 0; e < kWideE; ++e) {
@@ -1300,7 +1310,11 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_wide_range_kernel(const
     mx = o > mx ? o : mx;
     mn = o < mn ? o : mn;
   }
-  wide_range_atomics(mx, mn, ctl + (int64_t)row * kWideRowWords, s_red);
+  if (own_slots && blockIdx.x == 0) {
+    for (int i = threadIdx.x; i < kWideRowWords; i += kTopkThreads)
+      if (i < kWideCtlSlots || i >= kWideCtlSlots + 2 * (int)gridDim.x) rctl[i] = 0u;
+  }
+  wide_range_out(mx, mn, rctl, own_slots ? (int)blockIdx.x : -1, s_red);
 }
 
 // grid (slices, rows).  ctl: u32 [rows][kWideRowWords], zero at launch.
@@ -2162,14 +2176,20 @@ int pkv_launch_topk_f32(const float *x, int64_t x_stride, const int64_t *ids, in
     uint64_t *list_a = (uint64_t *)((char *)ws + w.list_a), *list_b = (uint64_t *)((char *)ws + w.list_b);
     const int P = pow2_ceil(k);
     const dim3 grid((unsigned)((len + kWideSlice - 1) / kWideSlice), (unsigned)rows);
+    // a row of at most kWideRangeSlots slices: every slice leaves its range in a slot of its own and the first one
+    // clears the control block, which saves the clearing launch
+    const bool own_slots = !ctl_ready && grid.x <= (unsigned)kWideRangeSlots;
     if (!ctl_ready) {  // else: earlier launches of the caller's step cleared the control blocks and left the rows' score ranges
-      hipLaunchKernelGGL(pkv_zero_u32_kernel, dim3((unsigned)((rows * kWideRowWords + 255) / 256)), dim3(256), 0, s, ctl,
-                         (int64_t)rows * kWideRowWords);
-      PKV_LAUNCH_CHECK("pkv_zero_u32_kernel");
-      hipLaunchKernelGGL(pkv_topk_wide_range_kernel, grid, dim3(kTopkThreads), 0, s, x, x_stride, len, ctl);
+      if (!own_slots) {
+        hipLaunchKernelGGL(pkv_zero_u32_kernel, dim3((unsigned)((rows * kWideRowWords + 255) / 256)), dim3(256), 0, s,
+                           ctl, (int64_t)rows * kWideRowWords);
+        PKV_LAUNCH_CHECK("pkv_zero_u32_kernel");
+      }
+      hipLaunchKernelGGL(pkv_topk_wide_range_kernel, grid, dim3(kTopkThreads), 0, s, x, x_stride, len, ctl,
+                         own_slots ? 1 : 0);
       PKV_LAUNCH_CHECK("pkv_topk_wide_range_kernel");
     }
-    const int n_range_slots = ctl_ready ? kWideRangeSlots : 0;  // a producer's per-workgroup score ranges
+    const int n_range_slots = (ctl_ready || own_slots) ? kWideRangeSlots : 0;  // per-workgroup score ranges
     hipLaunchKernelGGL(pkv_topk_wide_hist_kernel, grid, dim3(kTopkThreads), 0, s, x, x_stride, ids, ids_stride, len, ctl,
                        n_range_slots);
     PKV_LAUNCH_CHECK("pkv_topk_wide_hist_kernel");

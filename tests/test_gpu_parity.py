@@ -403,6 +403,9 @@ def test_topk_f32_wide_rows_edge_cases(ops):
     z = (rng.standard_normal((2, 30000)) * 5).astype(np.float32)
     z[0, 123] = 1e30                                   # an outlier stretches the range: everything else in one bin
     cases.append(("outlier", z, 512))
+    # more slices than a row has range slots of its own: the control block is cleared by a launch and the slices'
+    # ranges meet in two atomic words
+    cases.append(("eighteen slices", rng.standard_normal((2, 140000)).astype(np.float32), 1500))
     for name, x, k in cases:
         _say(f"topk_f32 wide: {name} {x.shape} k={k}")
         rows, L = x.shape
