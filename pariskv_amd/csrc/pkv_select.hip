@@ -919,9 +919,9 @@ __device__ __forceinline__ void collect_winners_streamed(KeyFn key_of, int64_t l
 }
 
 // len <= 8192 and k well below len: select the k winners exactly, then sort only those.
-// SORTED = false leaves the sort out: the winners come out in the order of their positions in the row
-// (a fixed function of the inputs), for callers that use them as a set (gather + attention).  A thread then
-// owns EIN consecutive positions, so that one exclusive scan over the threads gives every winner its slot.
+// SORTED = false leaves the sort out: the winners come out in a fixed order of their positions in the row (by the
+// wave that loaded them, then by element index, then by lane: a function of the inputs only), for callers that use
+// them as a set (gather + attention).
 template <int EIN, bool SORTED>
 __global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
     const float *__restrict__ x, int64_t x_stride, const int64_t *__restrict__ ids, int64_t ids_stride, int len, int P,
@@ -940,7 +940,7 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
   uint64_t v[EIN];
 #pragma unroll
   for (int e = 0; e < EIN; ++e) {
-    const int i = SORTED ? tid + e * kTopkThreads : tid * EIN + e;
+    const int i = tid + e * kTopkThreads;
     v[e] = i < len ? make_key(xr, ir, i) : 0ull;
   }
   if (tid == 0) s_counter = 0;
@@ -996,21 +996,31 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
     for (int e = 0; e < EIN; ++e) win[e] = (v[e] >> shift) >= (prefix >> shift) && v[e] != 0ull;
   }
   if (!SORTED) {
-    int mine = 0;
-#pragma unroll
-    for (int e = 0; e < EIN; ++e) mine += win[e];
-    int total;
-    __syncthreads();  // the histograms have been read by everyone
-    int slot = pkv_block_excl_scan<kTopkThreads>(mine, (int *)s_hist, total);  // s_hist is free again
+    // slot of a winner = winners of the lower waves + winners of its own wave at lower e + those at its e in lower
+    // lanes: a fixed function of the inputs, found with one ballot per e and one exchange of the 16 wave totals
+    uint64_t ballot[EIN];
+    uint32_t wave_total = 0;
 #pragma unroll
     for (int e = 0; e < EIN; ++e) {
-      if (win[e]) {
-        if (slot < k) {
-          oi[slot] = (int64_t)(uint32_t)(~(uint32_t)v[e]);
-          if (ov) ov[slot] = pkv_from_ordered_u32((uint32_t)(v[e] >> 32));
-        }
-        ++slot;
+      ballot[e] = __ballot(win[e]);
+      wave_total += (uint32_t)__popcll(ballot[e]);
+    }
+    __syncthreads();  // the histograms have been read by everyone: s_hist is free again
+    const int wave = tid / PKV_WAVE;
+    if (pkv_lane() == 0) s_hist[wave] = wave_total;
+    __syncthreads();
+    uint32_t slot = 0;
+#pragma unroll
+    for (int w = 0; w < kTopkThreads / PKV_WAVE; ++w) slot += w < wave ? s_hist[w] : 0u;
+    const uint64_t below = ((uint64_t)1 << pkv_lane()) - 1;
+#pragma unroll
+    for (int e = 0; e < EIN; ++e) {
+      const uint32_t mine = slot + (uint32_t)__popcll(ballot[e] & below);
+      if (win[e] && mine < (uint32_t)k) {
+        oi[mine] = (int64_t)(uint32_t)(~(uint32_t)v[e]);
+        if (ov) ov[mine] = pkv_from_ordered_u32((uint32_t)(v[e] >> 32));
       }
+      slot += (uint32_t)__popcll(ballot[e]);
     }
     return;
   }
