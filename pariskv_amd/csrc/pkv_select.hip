@@ -180,7 +180,6 @@ __global__ __launch_bounds__(kSelThreads) void pkv_select_rerank_kernel(
   __shared__ int s_scan[2][kSelThreads / PKV_WAVE];
   __shared__ float s_prod[128 * 16];
   __shared__ uint16_t s_list_key[kSelKeysPerIter];  // offset of the key inside the iteration's 4096-key block
-  __shared__ int32_t s_list_pos[kSelKeysPerIter];   // output position, -1 = dropped tie
 
   const uint8_t *crow = cnt + (int64_t)row * cnt_stride;
   const int64_t chunk_begin = (int64_t)chunk * chunk_keys;
@@ -210,35 +209,34 @@ __global__ __launch_bounds__(kSelThreads) void pkv_select_rerank_kernel(
     int total;
     const int excl = pkv_block_excl_scan<kSelThreads>(packed, s_scan[it & 1], total);
     const int n_gt_it = total & 0xffff, n_sel_it = n_gt_it + (total >> 16);
-    int64_t pg = base_gt + (excl & 0xffff);
-    int64_t pe = base_eq + (excl >> 16);
-    int lg = excl & 0xffff;            // slot in this iteration's LDS list: strictly-above keys first,
-    int le = n_gt_it + (excl >> 16);   // then the keys at the threshold
+    // slot in this iteration's LDS list: strictly-above keys first, then the keys at the threshold.  The output
+    // position of slot j follows from j alone: pos_gt0 + j for the former, pos_eq0 + j for the latter; ties whose
+    // position would reach k are dropped, and they are the list's last slots.
+    int lg = excl & 0xffff;
+    int le = n_gt_it + (excl >> 16);
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
       uint32_t g = gt[d], e = eq[d];
       while (g) {
         const int bit = __ffs((int)g) - 1;
         g &= g - 1;
-        s_list_key[lg] = (uint16_t)(tid * kSelKeysPerThread + 4 * d + (bit >> 3));
-        s_list_pos[lg] = pg < k ? (int32_t)pg : -1;
-        ++lg, ++pg;
+        s_list_key[lg++] = (uint16_t)(tid * kSelKeysPerThread + 4 * d + (bit >> 3));
       }
       while (e) {
         const int bit = __ffs((int)e) - 1;
         e &= e - 1;
-        s_list_key[le] = (uint16_t)(tid * kSelKeysPerThread + 4 * d + (bit >> 3));
-        s_list_pos[le] = pe < k ? (int32_t)pe : -1;
-        ++le, ++pe;
+        s_list_key[le++] = (uint16_t)(tid * kSelKeysPerThread + 4 * d + (bit >> 3));
       }
     }
+    const int64_t pos_gt0 = base_gt, pos_eq0 = base_eq - n_gt_it, eq_room = k - base_eq;
+    const int n_use = eq_room >= (total >> 16) ? n_sel_it : n_gt_it + (int)(eq_room > 0 ? eq_room : 0);
     base_gt += n_gt_it;
     base_eq += total >> 16;
     __syncthreads();
 #pragma unroll 1
-    for (int j = tid; j < n_sel_it; j += kSelThreads) {
-      const int32_t pos = s_list_pos[j];
-      if (pos >= 0) {
+    for (int j = tid; j < n_use; j += kSelThreads) {
+      const int64_t pos = j < n_gt_it ? pos_gt0 + j : pos_eq0 + j;
+      {
         const int64_t key = blk0 + s_list_key[j];
         orow[pos] = key;
         const float sc = pkv_rerank_keymajor(s_prod, (const pkv_u32x4 *)(nrow + key * ns_key), (const pkv_u32x4 *)(wrow + key * ws_key), qn);
