@@ -572,20 +572,22 @@ __device__ __forceinline__ void radix_select_regs(const uint64_t (&v)[EIN], uint
   shift_out = shift;
 }
 
-// ---- selection through 256 linear bins of the row's own score range ----
+// ---- selection through kLinBins linear bins of the row's own score range ----
 //
 // The 8-bit radix passes above look at fixed bit fields: scores of one row share their sign and most exponent
 // bits, so the first pass separates almost nothing and three passes are the rule.  Here the bins divide
-// [row min, row max] evenly: bin(x) = min(255, floor((x - lo) * 256 / (hi - lo))), a non-decreasing function
+// [row min, row max] evenly: bin(x) = min(kLinBins - 1, floor((x - lo) * kLinBins / (hi - lo))), a non-decreasing function
 // of x whatever the rounding of its three operations, so every key in a higher bin is a larger key.  One
 // histogram pass finds the bin b* that holds the k-th largest key and how many of its keys are needed; the
-// exact threshold key T is then the need-th largest of that one bin, found by counting (a bin holds len / 256
+// exact threshold key T is then the need-th largest of that one bin, found by counting (a bin holds len / kLinBins
 // keys on average).  Winners: bin > b*, or bin == b* and key >= T.  The bins also order the winners: those
 // of bin b occupy the output slots [off[b], off[b] + count[b]), and the slot inside the bin is again found by
 // counting, which replaces the bitonic sort (and T: the first `need` of b* by that count are its winners).
 // Rows this does not suit take the older steps: non-finite scores, a zero or subnormal range or more than
 // kLinBucketMax keys in b* the radix select; more than kLinRankMax winners in one bin the bitonic sort.  The
 // result is the same set in the same order either way.
+constexpr int kLinBins = 512;   // a multiple of 64: wave 0 owns kLinBins / 64 bins per lane
+constexpr int kLinBinBits = 9;
 constexpr int kLinBucketMax = 256;
 constexpr int kLinRankMax = 128;
 constexpr int kCountingSortMaxP = 2048;  // largest winner list whose counting sort (a second copy in LDS) is set up
@@ -608,14 +610,14 @@ __device__ __forceinline__ uint32_t lin_bin(uint64_t key, const LinSel &L) {
     const float t = (pkv_from_ordered_u32((uint32_t)(key >> 32)) - L.lo) * L.scale;
     b = (uint32_t)t;
   }
-  return b > 255u ? 255u : b;
+  return b > (uint32_t)(kLinBins - 1) ? (uint32_t)(kLinBins - 1) : b;
 }
 
-// Bins of the thread's keys and the threshold bin.  On return s_hist[0,256) = keys per bin, s_hist[256,512) =
+// Bins of the thread's keys and the threshold bin.  On return s_hist[0,kLinBins) = keys per bin, s_hist[kLinBins,2*kLinBins) =
 // off[b] = keys in the bins above b, s_cnt[b] = off[b] (a running output slot for the counting sort), s_bcast[6] = 0.
-// s_hist: 512 words, s_cnt: 256 words, s_bcast: 8 words.  All 1024 threads call it; false = not applicable.
+// s_hist: 2*kLinBins words, s_cnt: kLinBins words, s_bcast: 8 words.  All 1024 threads call it; false = not applicable.
 // BITS: bins of the ordered key bits instead of the values, for rows of one sign whose values span many binades
-// (e.g. the winners of a selection, about to be sorted): 256 equal steps of the bit pattern between the row's
+// (e.g. the winners of a selection, about to be sorted): kLinBins equal steps of the bit pattern between the row's
 // smallest and largest key, i.e. equal steps of the logarithm up to the mantissa's linear pieces.
 // range: null, or the largest and the smallest ordered score of the nonzero keys (range[0] < range[1]: no key at
 // all) where the caller knows them already, which saves the reduction that finds them.
@@ -624,7 +626,7 @@ __device__ __forceinline__ bool linear_bins(const uint64_t (&v)[EIN], uint32_t k
                                             uint32_t *s_bcast, uint32_t (&bin)[EIN], LinSel &L,
                                             const uint32_t *range = nullptr) {
   const int tid = threadIdx.x, lane = pkv_lane();
-  if (tid < 512) s_hist[tid] = 0;
+  for (int i = tid; i < 2 * kLinBins; i += kTopkThreads) s_hist[i] = 0;
   if (tid == 0) s_bcast[0] = 0u, s_bcast[1] = 0xffffffffu, s_bcast[5] = 0u, s_bcast[6] = 0u;
   __syncthreads();
   uint32_t mx = 0u, mn = 0xffffffffu;
@@ -658,10 +660,10 @@ __device__ __forceinline__ bool linear_bins(const uint64_t (&v)[EIN], uint32_t k
   if (BITS) {
     if (mx <= mn) return false;  // one value (or no key at all)
     const int width = 32 - __clz((int)(mx - mn));
-    L.shift = width > 8 ? width - 8 : 0;
+    L.shift = width > kLinBinBits ? width - kLinBinBits : 0;
   } else {
     const float hi = pkv_from_ordered_u32(mx), lo = pkv_from_ordered_u32(mn);
-    const float range = hi - lo, scale = 256.0f / range;
+    const float range = hi - lo, scale = (float)kLinBins / range;
     const float inf = __uint_as_float(0x7f800000u);
     // finite scores (ordered keys strictly between those of -inf and +inf), a positive finite range and scale
     if (!(mx < 0xff800000u && mn > 0x007fffffu && range > 0.f && range < inf && scale < inf)) return false;
@@ -676,17 +678,21 @@ __device__ __forceinline__ bool linear_bins(const uint64_t (&v)[EIN], uint32_t k
     }
   }
   __syncthreads();
-  if (tid < PKV_WAVE) {  // lane l owns bins 255 - 4l .. 252 - 4l: an inclusive scan over lanes is the suffix sum over bins
-    uint32_t h[4];
+  if (tid < PKV_WAVE) {  // lane l owns the kPer bins below kLinBins - kPer * l: an inclusive scan over lanes is the suffix sum over bins
+    constexpr int kPer = kLinBins / PKV_WAVE;
+    uint32_t h[kPer];
+    uint32_t mine = 0;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) h[j] = s_hist[255 - 4 * tid - j];
-    const uint32_t mine = h[0] + h[1] + h[2] + h[3];
+    for (int j = 0; j < kPer; ++j) {
+      h[j] = s_hist[kLinBins - 1 - kPer * tid - j];
+      mine += h[j];
+    }
     uint32_t above = (uint32_t)pkv_wave_incl_scan((int)mine) - mine;
     uint32_t most = 0;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int b = 255 - 4 * tid - j;
-      s_hist[256 + b] = above;
+    for (int j = 0; j < kPer; ++j) {
+      const int b = kLinBins - 1 - kPer * tid - j;
+      s_hist[kLinBins + b] = above;
       s_cnt[b] = above;
       if (above < k) {
         const uint32_t take = above + h[j] >= k ? k - above : h[j];
@@ -719,7 +725,7 @@ __device__ __forceinline__ void linear_threshold(const uint64_t (&v)[EIN], const
                                                  uint64_t *s_bucket, uint64_t *s_T, LinSel &L) {
   if (L.in_bstar == L.need) return;  // the bin is taken whole: T = 0
 #pragma unroll
-  for (int e = 0; e < EIN; ++e) {  // about one key in 256: most waves skip the atomic altogether
+  for (int e = 0; e < EIN; ++e) {  // about one key in kLinBins: most waves skip the atomic altogether
     if (v[e] != 0ull && bin[e] == L.bstar) s_bucket[atomicAdd(&s_bcast[6], 1u)] = v[e];
   }
   __syncthreads();
@@ -740,8 +746,8 @@ __device__ __forceinline__ void linear_threshold(const uint64_t (&v)[EIN], const
 
 // LDS scratch of a selection / sort over one workgroup's keys.
 struct SelSmem {
-  uint32_t hist[512];
-  uint32_t cnt[256];
+  uint32_t hist[2 * kLinBins];
+  uint32_t cnt[kLinBins];
   uint32_t bcast[8];
   uint32_t counter;
   uint64_t bucket[kLinBucketMax];
@@ -768,7 +774,7 @@ __device__ __forceinline__ void select_topk_flags(const uint64_t (&v)[EIN], uint
 }
 
 // Descending sort of the n nonzero keys held E per thread (all other entries zero) into s_out[0 .. n), through
-// s_tmp (n keys, not s_out): 256 bins of the ordered key bits between the smallest and the largest key, every key
+// s_tmp (n keys, not s_out): kLinBins bins of the ordered key bits between the smallest and the largest key, every key
 // placed at (keys in higher bins) + (larger keys in its own bin).  False, with nothing written, when a bin holds
 // more than kLinRankMax keys or all keys are equal: the caller then sorts by compare-exchange.
 template <int E>
@@ -782,7 +788,7 @@ __device__ __forceinline__ bool counting_sort_desc(const uint64_t (&v)[E], uint3
     if (v[e] != 0ull) s_tmp[atomicAdd(&sm.cnt[bin[e]], 1u)] = v[e];
   }
   __syncthreads();
-  const uint32_t *s_off = sm.hist + 256;
+  const uint32_t *s_off = sm.hist + kLinBins;
   for (uint32_t p = threadIdx.x; p < n; p += kTopkThreads) {
     const uint64_t key = s_tmp[p];
     const uint32_t b = lin_bin(key, L);
@@ -831,7 +837,7 @@ __device__ __forceinline__ bool select_sort_desc(const uint64_t (&v)[E], uint32_
     }
   }
   __syncthreads();
-  const uint32_t *s_off = sm.hist + 256;
+  const uint32_t *s_off = sm.hist + kLinBins;
   const uint32_t n_above = k - L.need;
   // The lower a slot, the fewer keys its bin holds: the slots are handed out in pairs (p, n_above - 1 - p), so that
   // a wave takes crowded and sparse bins in turn.
@@ -925,8 +931,8 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
     const float *__restrict__ x, int64_t x_stride, const int64_t *__restrict__ ids, int64_t ids_stride, int len, int P,
     int64_t k, int64_t *__restrict__ out_ids, float *__restrict__ out_vals) {
   extern __shared__ uint64_t s_keys[];
-  __shared__ uint32_t s_hist[512];
-  __shared__ uint32_t s_cnt[256];
+  __shared__ uint32_t s_hist[2 * kLinBins];
+  __shared__ uint32_t s_cnt[kLinBins];
   __shared__ uint32_t s_bcast[8];
   __shared__ uint32_t s_counter;
   __shared__ uint64_t s_bucket[kLinBucketMax];
@@ -954,7 +960,7 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
     // counting sort: a key of a bin above b* takes a slot of [off[b], off[b] + count[b]) and the keys of b* go to
     // a list of their own; then every key counts the larger keys of its own bin, which is its place inside the
     // bin, and is written there (of b* only the first `need`)
-    const uint32_t *s_off = s_hist + 256;
+    const uint32_t *s_off = s_hist + kLinBins;
 #pragma unroll
     for (int e = 0; e < EIN; ++e) {
       if (v[e] != 0ull) {
