@@ -365,6 +365,26 @@ def main():
     step_with_attention(0)
     us_step_attn = timed(step_with_attention, args.steps)
 
+    # the same on-GPU stages recorded once into a HIP graph and replayed (a caller that captures its decode step;
+    # reported beside the metric): the launches then follow each other without the host in between
+    us_gpu_graph = None
+    try:
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            for i in range(L):
+                step(i, False)
+            graph = torch.cuda.CUDAGraph()
+            torch.cuda.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(args.steps):
+                    step(i, False)
+        torch.cuda.synchronize()
+        graph.replay()
+        us_gpu_graph = timed(lambda i: graph.replay(), 4) / args.steps
+        del graph
+    except Exception as exc:  # a build of torch without graph capture: the figure is left out
+        print(f"bench.py: graph replay not measured ({exc})", file=sys.stderr)
+
     # dominant kernel: the collision scan, timed by its own begin/end timestamps
     kus = C.c_float()
     scan_us = []
@@ -419,6 +439,7 @@ def main():
                    "rows": R, "keys_per_row": N, "candidates": Cn, "topk": K, "collision_ratio": 0.2},
         "stages_us": {"full_retrieval_with_uva_gather": round(us_step, 2), "on_gpu_stages": round(us_gpu, 2),
                       "on_gpu_stages_ids_in_any_order": round(us_gpu_any, 2),
+                      "on_gpu_stages_replayed_from_a_hip_graph": None if us_gpu_graph is None else round(us_gpu_graph, 2),
                       "uva_gather_alone": round(us_gather, 2),
                       "decode_attention_over_gathered_set": round(us_attn, 2),
                       "full_step_plus_attention_one_host_call": round(us_step_attn, 2)},
