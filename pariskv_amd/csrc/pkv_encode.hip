@@ -180,9 +180,11 @@ __device__ __forceinline__ float enc_min_abs8(const float (&v)[8]) {
 // word), sgw[] = the SRHT sign bits in the same packing.  Returns true when this lane's key needs enc_key_exact
 // (norm or radius outside [1e-8, 2^60], or a component below 2^-40 in magnitude, zero included); o is then
 // unspecified.  sm1/sm2/sm8 = the sign bit where the lane's block index has bit 0/1/3 set.  s_mag[p - 0x3C00] =
-// {magnitude code, magnitude centre} for the bf16 pattern p of |u|.
+// {magnitude code, magnitude centre} for the bf16 pattern p of |u|; s_spread[c] = bit j of the sign code c moved to
+// bit 4j + 3.
 __device__ __forceinline__ bool enc_key_fast(const uint32_t (&w)[4], const uint32_t (&sgw)[4], uint32_t sm1,
-                                             uint32_t sm2, uint32_t sm8, bool rerank, const uint2 *s_mag, EncOut &o) {
+                                             uint32_t sm2, uint32_t sm8, bool rerank, const uint2 *s_mag,
+                                             const uint32_t *s_spread, EncOut &o) {
   float x[8];  // components times their SRHT sign: the sign commutes with the division and its rounding
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
@@ -190,9 +192,12 @@ __device__ __forceinline__ bool enc_key_fast(const uint32_t (&w)[4], const uint3
     x[2 * p] = __uint_as_float(v << 16);
     x[2 * p + 1] = __uint_as_float(v & 0xffff0000u);
   }
+  // the square of a bf16 value of magnitude in [2^-40, 2^60] is exact in fp32 (16 significant bits, a normal
+  // number), so a fused multiply-add rounds once, to the same bits as the product and the sum rounded in turn; a key
+  // with a component outside that range is handed to enc_key_exact whatever is computed here
   float acc = x[0] * x[0];
 #pragma unroll
-  for (int j = 1; j < 8; ++j) acc = acc + x[j] * x[j];
+  for (int j = 1; j < 8; ++j) acc = __builtin_fmaf(x[j], x[j], acc);
   acc = enc_dpp<0xB1>(acc) + acc;   // lane ^ 1
   acc = enc_dpp<0x4E>(acc) + acc;   // lane ^ 2
   acc = enc_sum_xor4(acc);
@@ -232,9 +237,9 @@ __device__ __forceinline__ bool enc_key_fast(const uint32_t (&w)[4], const uint3
   o.code = ~sneg & 0xffu;
   if (!rerank) return bad;
 
-  float r2 = y[0] * y[0];
+  float r2 = y[0] * y[0];  // y: bf16 values, magnitudes checked above: exact squares again
 #pragma unroll
-  for (int j = 1; j < 8; ++j) r2 = r2 + y[j] * y[j];
+  for (int j = 1; j < 8; ++j) r2 = __builtin_fmaf(y[j], y[j], r2);
   const float r = enc_sqrt_bf16(r2);
   bad |= !(r >= 1e-8f) || r > 0x1p60f;
   const float r_inv = __builtin_amdgcn_rcpf(r);
@@ -247,7 +252,7 @@ __device__ __forceinline__ bool enc_key_fast(const uint32_t (&w)[4], const uint3
     const uint32_t byte_off = __builtin_amdgcn_ubfe(__float_as_uint(cl), 13, kMagTableBits + 3);  // 8 * (pattern - 0x3C00)
     e[j] = *(const uint2 *)((const char *)s_mag + byte_off);
   }
-  uint32_t mags = 0, negs = 0;
+  uint32_t mags = 0;
   float alpha = 0.f;
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
@@ -255,10 +260,8 @@ __device__ __forceinline__ bool enc_key_fast(const uint32_t (&w)[4], const uint3
     const float p = pkv_bf16_round(__uint_as_float(e[j].y) * au[j]);
     alpha = (j == 0) ? p : alpha + p;
   }
-#pragma unroll
-  for (int j = 7; j >= 0; --j) negs = __builtin_amdgcn_alignbit(negs, __float_as_uint(y[j]), 28);  // bit 3 of nibble j = sign of y[j]
   if (alpha < 1e-6f) alpha = 1e-6f;
-  o.packed = (mags & 0x77777777u) | (~negs & 0x88888888u);
+  o.packed = (mags & 0x77777777u) | s_spread[o.code];  // bit 3 of nibble j = bit j of the sign code
   // (r / alpha) * n: both forms are within 2^-22 of the exact value, at most 6 ulp apart; the reciprocal form
   // decides the bf16 rounding unless it lies within 8 ulp of a rounding boundary
   float wt = (r * __builtin_amdgcn_rcpf(alpha)) * n;
@@ -283,7 +286,14 @@ __global__ __launch_bounds__(kEncThreads) __attribute__((amdgpu_waves_per_eu(6, 
   __shared__ uint32_t s_hist[16 * 256];
   __shared__ uint2 s_mag[BF16 ? (1 << kMagTableBits) : 1];
   __shared__ float s_centers[8];  // magnitude centres, looked up by code (an LDS read instead of a load from constant memory)
+  __shared__ uint32_t s_spread[BF16 ? 256 : 1];
   if (tid < 8) s_centers[tid] = c_centers[tid];
+  if (BF16) {
+    uint32_t sp = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) sp |= ((uint32_t)(tid >> j) & 1u) << (4 * j + 3);
+    s_spread[tid] = sp;  // kEncThreads == 256: one entry per thread
+  }
   if (BF16) {
     for (int i = tid; i < (1 << kMagTableBits); i += kEncThreads) {
       const float v = __uint_as_float(kMagTableLo + ((uint32_t)i << 16));
@@ -342,7 +352,7 @@ __global__ __launch_bounds__(kEncThreads) __attribute__((amdgpu_waves_per_eu(6, 
     float x[8];
     if (BF16) {
       const uint32_t w[4] = {cur[0].x, cur[0].y, cur[0].z, cur[0].w};
-      exact = __builtin_amdgcn_ballot_w64(enc_key_fast(w, sgw, sm1, sm2, sm8, rerank, s_mag, o)) != 0;
+      exact = __builtin_amdgcn_ballot_w64(enc_key_fast(w, sgw, sm1, sm2, sm8, rerank, s_mag, s_spread, o)) != 0;
       if (exact) {
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
