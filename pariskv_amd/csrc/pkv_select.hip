@@ -988,6 +988,45 @@ __global__ __launch_bounds__(kTopkThreads) void pkv_topk_select_sort_kernel(
     });
     return;
   }
+  if (!SORTED && lin) {
+    // any order, without the threshold key: the keys of the bins above b* all win and take the first k - need slots
+    // (slot = winners of the lower waves + winners of the own wave at lower e + those at the same e in lower lanes:
+    // one ballot per e and one exchange of the 16 wave totals); the keys of b* are ranked among themselves and the
+    // first `need` follow.  A fixed function of the inputs.
+    uint64_t ballot[EIN];
+    uint32_t wave_total = 0;
+#pragma unroll
+    for (int e = 0; e < EIN; ++e) {
+      const bool nz = v[e] != 0ull;
+      if (nz && bin[e] == L.bstar) s_bucket[atomicAdd(&s_bcast[6], 1u)] = v[e];
+      ballot[e] = __ballot(nz && bin[e] > L.bstar);
+      wave_total += (uint32_t)__popcll(ballot[e]);
+    }
+    const int wave = tid / PKV_WAVE;
+    if (pkv_lane() == 0) s_hist[wave] = wave_total;  // the histograms have been read by everyone
+    __syncthreads();
+    uint32_t slot = 0;
+#pragma unroll
+    for (int w = 0; w < kTopkThreads / PKV_WAVE; ++w) slot += w < wave ? s_hist[w] : 0u;
+    const uint64_t below = ((uint64_t)1 << pkv_lane()) - 1;
+    const uint32_t n_above = (uint32_t)k - L.need;
+#pragma unroll
+    for (int e = 0; e < EIN; ++e) {
+      const uint32_t mine = slot + (uint32_t)__popcll(ballot[e] & below);
+      if (((ballot[e] >> pkv_lane()) & 1ull) && mine < n_above) {
+        oi[mine] = (int64_t)(uint32_t)(~(uint32_t)v[e]);
+        if (ov) ov[mine] = pkv_from_ordered_u32((uint32_t)(v[e] >> 32));
+      }
+      slot += (uint32_t)__popcll(ballot[e]);
+    }
+    rank_bucket_desc(s_bucket, L.in_bstar, [&](uint64_t key, uint32_t r) {
+      if (r < L.need) {
+        oi[n_above + r] = (int64_t)(uint32_t)(~(uint32_t)key);
+        if (ov) ov[n_above + r] = pkv_from_ordered_u32((uint32_t)(key >> 32));
+      }
+    });
+    return;
+  }
   if (lin) {
     linear_threshold<EIN>(v, bin, s_bcast, s_bucket, &s_T, L);
 #pragma unroll
