@@ -53,12 +53,14 @@ __global__ __launch_bounds__(256) void pkv_add_rmsnorm_kernel(const uint16_t *__
   const int row = blockIdx.x, tid = threadIdx.x;
   const int n_vec = width / 8;
   float v[8][8];
+  pkv_u32x4 wts[8];  // the weights do not depend on the sum: requested with the inputs, not after the reduction
   float ss = 0.f;
 #pragma unroll
   for (int r = 0; r < 8; ++r) {
     const int vec = tid + r * 256;
     if (vec < n_vec) {
       const pkv_u32x4 a = *(const pkv_u32x4 *)(x + (int64_t)row * width + vec * 8);
+      wts[r] = *(const pkv_u32x4 *)(weight + vec * 8);
       pkv_u32x4 b = {0u, 0u, 0u, 0u};
       if (residual) b = *(const pkv_u32x4 *)(residual + (int64_t)row * width + vec * 8);
       const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
@@ -83,8 +85,7 @@ __global__ __launch_bounds__(256) void pkv_add_rmsnorm_kernel(const uint16_t *__
   for (int r = 0; r < 8; ++r) {
     const int vec = tid + r * 256;
     if (vec < n_vec) {
-      const pkv_u32x4 w4 = *(const pkv_u32x4 *)(weight + vec * 8);
-      const uint32_t ww[4] = {w4.x, w4.y, w4.z, w4.w};
+      const uint32_t ww[4] = {wts[r].x, wts[r].y, wts[r].z, wts[r].w};
       uint32_t ow[4];
 #pragma unroll
       for (int p = 0; p < 4; ++p) {
