@@ -390,6 +390,11 @@ def test_topk_f32_wide_rows_edge_cases(ops):
     x = rng.standard_normal((3, L)).astype(np.float32)
     x[:, : L // 2] = np.float32(0.75) + rng.integers(0, 4, (3, L // 2)).astype(np.float32) * np.float32(2.0 ** -20)
     cases.append(("crowded threshold bin", x, 9000 // 2))
+    # the same with a list short enough for the one-binning selection + sort of the finish kernel, which must hand a
+    # threshold bin this crowded (15 000 keys in four values) to the two-step path
+    x2 = rng.standard_normal((3, L)).astype(np.float32)
+    x2[:, : L // 2] = np.float32(2.5) + rng.integers(0, 4, (3, L // 2)).astype(np.float32) * np.float32(2.0 ** -20)
+    cases.append(("crowded threshold bin, short list", x2, 1500))
     cases.append(("k=8192", rng.standard_normal((2, 70000)).astype(np.float32), 8192))
     cases.append(("len=8193", rng.standard_normal((5, 8193)).astype(np.float32), 100))
     y = (rng.standard_normal((2, 20001)) * 1e3).astype(np.float32)
