@@ -490,7 +490,19 @@ typedef struct pkv_retrieve_args {
    * it arrives with the candidate's HBM line instead of through a second scattered read
    * (cache_hub/polar_cache_adaptivek_varlen.py:1741-1753 gathers value_norm_gpu at cand_idx + sink). */
   int64_t record_word_offset;
+  /* How the stages before the top-k are launched; the results are the same.
+   * PKV_PLAN_AUTO (0): query prep, collision scan and select + rerank as ONE launch whose workgroups hand the
+   *   row's vote table and histogram to each other, where the shape allows it (chunks of at most 8192 keys,
+   *   at most 256 chunks per row) and `stream` is not being captured into a graph; otherwise as below.
+   * PKV_PLAN_SEPARATE (1): always as three launches (the reference's structure: collision kernel,
+   *   top-k kernel, rerank kernel, cache_hub/polar_cache.py:1207-1298). */
+  int launch_plan;
+  /* nonzero: the per-key vote counts need not be left in the workspace segment "cnt_u8" (the one-launch plan then
+   * keeps them on chip). */
+  int skip_vote_counts;
 } pkv_retrieve_args;
+#define PKV_PLAN_AUTO 0
+#define PKV_PLAN_SEPARATE 1
 
 size_t pkv_retrieve_ws_bytes(int rows, int64_t n_keys, int64_t n_cand, int64_t k);
 int pkv_retrieve(const pkv_retrieve_args *args, void *ws, size_t ws_bytes, void *stream);

@@ -50,8 +50,11 @@ class RetrieveArgs(C.Structure):
         ("src_len", _i64), ("idx_offset", _i64),
         ("dst_k", _vp), ("dst_v", _vp), ("dst_len", _i64), ("dst_row0", _i64),
         ("row_bytes", _i), ("any_order", _i), ("nib_key_stride", _i64), ("weight_key_stride", _i64),
-        ("record_word_offset", _i64),
+        ("record_word_offset", _i64), ("launch_plan", _i), ("skip_vote_counts", _i),
     ]
+
+
+PLAN_AUTO, PLAN_SEPARATE = 0, 1  # pkv_retrieve_args.launch_plan
 
 
 class AdaptiveArgs(C.Structure):

@@ -383,6 +383,67 @@ __device__ __forceinline__ float pkv_query_mean_rotate_wave(const void *__restri
   return pkv_normalize_rotate_64(x_lo, x_hi, sg_lo, sg_hi, dtype, y_lo, y_hi);
 }
 
+// ---- hand-overs between workgroups inside one launch ----
+// The chip's eight dies have an L2 each and a launch's workgroups are dealt out over all of them, so plain stores
+// of one workgroup (held in its die's write-back L2) and plain loads of another (served from its own die's L2 or the
+// compute unit's L1) do not meet inside a launch.  Accesses that carry the agent-scope bit (sc1: what the compiler
+// emits for relaxed atomic loads and stores at agent scope) do: such a store is written through to memory before it
+// is acknowledged, such a load misses the L1 and is not served from a stale L2 line.  The protocol built on them:
+// a producer writes its data with pkv_st_agent_*, every wave waits for its stores' acknowledgements
+// (pkv_wait_vmem) before a workgroup barrier, then ONE lane publishes a flag with pkv_st_agent_u64; a consumer polls
+// the flag with pkv_ld_agent_u64 and reads the data with pkv_ld_agent_* afterwards.  No cache write-back or
+// invalidate instruction is involved.
+__device__ __forceinline__ void pkv_wait_vmem() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void pkv_st_agent_u16(void *p, uint32_t v) {
+  asm volatile("global_store_short %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void pkv_st_agent_u32(void *p, uint32_t v) {
+  asm volatile("global_store_dword %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void pkv_st_agent_u64(void *p, uint64_t v) {
+  asm volatile("global_store_dwordx2 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void pkv_st_agent_x4(void *p, pkv_u32x4 v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+}
+// Loads: the request and the wait for its data are ONE asm statement, so the compiler never sees the destination
+// register before the data is in it (it may otherwise move or merge the register between a bare load and a later wait).
+__device__ __forceinline__ uint32_t pkv_ld_agent_u32(const void *p) {
+  uint32_t v;
+  asm volatile("global_load_dword %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
+__device__ __forceinline__ uint64_t pkv_ld_agent_u64(const void *p) {
+  uint64_t v;
+  asm volatile("global_load_dwordx2 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
+__device__ __forceinline__ pkv_u32x4 pkv_ld_agent_x4(const void *p) {
+  pkv_u32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
+// two half-words, both requests in flight together
+__device__ __forceinline__ void pkv_ld_agent_u16_pair(const void *p0, const void *p1, uint32_t &a, uint32_t &b) {
+  asm volatile("global_load_ushort %0, %2, off sc1\n\tglobal_load_ushort %1, %3, off sc1\n\ts_waitcnt vmcnt(0)"
+               : "=&v"(a), "=&v"(b)
+               : "v"(p0), "v"(p1)
+               : "memory");
+}
+
+// Wait (lanes [0, n) of the calling wave, n <= 64, one flag each) until flags[lane] == epoch for all of them, for at
+// most `ticks` of the 100 MHz wall clock.  All 64 lanes of the wave call it; returns false if it gave up.
+__device__ __forceinline__ bool pkv_wait_flags(const uint64_t *flags, int n, uint64_t epoch, uint64_t ticks) {
+  const int lane = pkv_lane();
+  const uint64_t t0 = __builtin_amdgcn_s_memrealtime();
+  while (true) {
+    const uint64_t f = lane < n ? pkv_ld_agent_u64(flags + lane) : epoch;
+    if (__ballot(f != epoch) == 0ull) return true;
+    __builtin_amdgcn_s_sleep(2);
+    if (__builtin_amdgcn_s_memrealtime() - t0 > ticks) return false;
+  }
+}
+
 // ---- 4-bit rerank core (shared by the stand-alone rerank and the fused select+rerank kernels) ----
 // s_prod[d][v] = qhat[d] * value(v) for the 16 possible 4-bit codes v (bit 3 = sign, set = positive;
 // bits 0-2 = magnitude centre): the product of the reference's expression is looked up instead of

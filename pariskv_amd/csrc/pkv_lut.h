@@ -31,6 +31,14 @@ __device__ __forceinline__ int pkv_tier_weight_from_rank(int my_count, const Pkv
   return w;
 }
 
+// Votes of one subspace from the rotated query in sm.y (all 128 dims, written and made visible by the caller:
+// a barrier lies between that write and this call).  Called by all 256 threads of a workgroup; contains barriers.
+//   cc_sub      cluster sizes of this (row, subspace): 256 ints in global memory
+//   lut_out     256 bytes (global or LDS): votes per centroid id
+//   sorted_out  int64[256] or null: centroid ids in ranked order
+__device__ __forceinline__ void pkv_lut_rank_subspace(int dtype, const int32_t *__restrict__ cc_sub, const PkvTiers &tiers,
+                                                      int sub, PkvLutSmem &sm, uint8_t *lut_out, int64_t *sorted_out);
+
 // Called by all 256 threads of a workgroup (contains barriers; `sm` may be reused after the call once the
 // caller has passed a barrier).  The rotation runs in the first wave only (two dims per lane, lane exchanges, no
 // barriers); the 256 threads then score, rank and weigh the 256 centroids.
@@ -45,7 +53,7 @@ __device__ __forceinline__ void pkv_lut_build_subspace(const void *__restrict__ 
                                                        int64_t *sorted_out) {
   const int tid = threadIdx.x;
   // cluster sizes by centroid id; issued first so that the latency overlaps the rotation
-  sm.cc[tid] = cc_sub[tid];
+  const int my_cc = cc_sub[tid];
 
   if (tid < PKV_WAVE) {
     float y_lo, y_hi;
@@ -54,7 +62,15 @@ __device__ __forceinline__ void pkv_lut_build_subspace(const void *__restrict__ 
     if (qhat_out) qhat_out[tid] = y_lo, qhat_out[tid + 64] = y_hi;
     if (qnorm_out && tid == 0) *qnorm_out = n;
   }
+  sm.cc[tid] = my_cc;
   __syncthreads();
+  pkv_lut_rank_subspace(dtype, nullptr, tiers, sub, sm, lut_out, sorted_out);
+}
+
+__device__ __forceinline__ void pkv_lut_rank_subspace(int dtype, const int32_t *__restrict__ cc_sub, const PkvTiers &tiers,
+                                                      int sub, PkvLutSmem &sm, uint8_t *lut_out, int64_t *sorted_out) {
+  const int tid = threadIdx.x;
+  if (cc_sub) sm.cc[tid] = cc_sub[tid];  // read again only after the barriers below
 
   // score of centroid c = tid: sum_j (+-) qhat_sub[j], sequential j
   {

@@ -11,11 +11,22 @@
 #include <mutex>
 
 PKV_INTERNAL int pkv_launch_identity_fill(int64_t *out, int64_t len, int64_t k, int rows, hipStream_t s);
+PKV_INTERNAL size_t pkv_fused_sync_bytes(int rows, int64_t n_chunks);
+PKV_INTERNAL bool pkv_fused_usable(int rows, int64_t n_keys, int chunk_keys, hipStream_t s);
+PKV_INTERNAL int pkv_launch_fused_retrieve(const void *q, int dtype, int bs, int n_kv_heads, int group, const float *signs,
+                              const int32_t *cc, int64_t cc_b, int64_t cc_h, const PkvTiers &tiers, float *qhat,
+                              float *qnorm, uint8_t *lut, const uint8_t *codes, int64_t cs_b, int64_t cs_h,
+                              int64_t n_keys, int chunk_keys, uint8_t *cnt_u8, int64_t cnt_stride, uint32_t *row_suf,
+                              uint16_t *chunk_suf, void *sync_area, uint32_t *zero_ptr, int64_t zero_row_words,
+                              int64_t zero_row_stride, int64_t k, const uint8_t *nib, int64_t ns_b, int64_t ns_h,
+                              int64_t ns_key, const uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key,
+                              const float *centers, int64_t *cand, float *scores, int64_t extra_off, float *extra_out,
+                              uint32_t *range_slots, int64_t range_row_stride, hipStream_t s);
 
 namespace {
 
 struct WsLayout {
-  size_t qhat, qnorm, lut, cnt, hist, rowsuf, cand, scores, cand_extra, topk, topk_bytes, total;
+  size_t qhat, qnorm, lut, cnt, hist, rowsuf, cand, scores, cand_extra, topk, topk_bytes, sync, sync_bytes, total;
   int64_t cnt_stride;
   int chunk_keys;
   int64_t n_chunks;
@@ -46,6 +57,9 @@ WsLayout layout(int rows, int64_t n_keys, int64_t n_cand, int64_t k) {
   const size_t ctl_bytes = pkv_align_up((size_t)pkv_topk_ctl_words(rows, n_cand) * 4, 256);
   if (w.topk_bytes < ctl_bytes) w.topk_bytes = ctl_bytes;
   w.topk = take(w.topk_bytes);
+  // flags and status word of the one-launch form of the first three stages
+  w.sync_bytes = pkv_fused_sync_bytes(rows, w.n_chunks);
+  w.sync = take(w.sync_bytes);
   w.total = off;
   return w;
 }
@@ -85,6 +99,9 @@ extern "C" int pkv_retrieve_ws_view(void *ws, int rows, int64_t n_keys, int64_t 
     *ptr = base + w.scores, *bytes = (size_t)rows * (size_t)n_cand * 4;
   } else if (!strcmp(name, "topk_control")) {
     *ptr = base + w.topk, *bytes = w.topk_bytes;
+  } else if (!strcmp(name, "handover_status")) {
+    // one word at the end of the hand-over area: workgroups of one-launch retrievals that gave up a wait (0 = none)
+    *ptr = base + w.sync + w.sync_bytes - 256, *bytes = 4;
   } else if (!strcmp(name, "cand_record_word")) {
     *ptr = base + w.cand_extra, *bytes = (size_t)rows * (size_t)n_cand * 4;
   } else {
@@ -146,27 +163,41 @@ static int retrieve_impl(const pkv_retrieve_args *a, void *ws, size_t ws_bytes, 
   uint32_t *topk_ctl = ctl_words ? (uint32_t *)(base + w.topk) : nullptr;
   int64_t range_stride = 0;
   uint32_t *range_slots = topk_ctl ? pkv_topk_range_slots(topk_ctl, a->n_cand, &range_stride) : nullptr;
-  int rc = pkv_launch_query_prep_lut(a->q, a->dtype, a->bs, H, a->group, a->signs, a->cluster_counts,
-                                     (int64_t)H * 4096, 4096, t, qhat, qnorm, lut, nullptr, rowsuf, s, topk_ctl, ctl_words);
-  if (rc) return rc;
   const uint8_t *codes = a->codes + a->key0 * 16;
   const uint8_t *nib = a->nib + a->key0 * nk;
   const uint16_t *weight = a->weight + a->key0 * wk;
-  if (a->n_cand == a->n_keys) {
-    rc = pkv_launch_identity_fill(cand, a->n_keys, a->n_cand, rows, s);
-    if (rc) return rc;
-    rc = pkv_launch_rerank(cand, a->bs, H, a->n_cand, a->n_keys, nib, (int64_t)H * a->cap * nk, a->cap * nk, nk, 4,
-                           weight, (int64_t)H * a->cap * wk, a->cap * wk, wk, 1, qhat, qnorm, a->centers, scores,
-                           nullptr, s);
+  int rc;
+  if (a->n_cand != a->n_keys && a->launch_plan != PKV_PLAN_SEPARATE && pkv_fused_usable(rows, a->n_keys, w.chunk_keys, s)) {
+    // query prep, scan and select + rerank as one launch
+    rc = pkv_launch_fused_retrieve(a->q, a->dtype, a->bs, H, a->group, a->signs, a->cluster_counts, (int64_t)H * 4096, 4096,
+                                   t, qhat, qnorm, lut, codes, (int64_t)H * a->cap * 16, a->cap * 16, a->n_keys,
+                                   w.chunk_keys, a->skip_vote_counts ? nullptr : cnt, w.cnt_stride, rowsuf, hist,
+                                   base + w.sync, topk_ctl, topk_ctl ? ctl_words / rows : 0, topk_ctl ? ctl_words / rows : 0,
+                                   a->n_cand, nib, (int64_t)H * a->cap * nk, a->cap * nk, nk, weight,
+                                   (int64_t)H * a->cap * wk, a->cap * wk, wk, a->centers, cand, scores,
+                                   a->record_word_offset,
+                                   a->record_word_offset > 0 ? (float *)(base + w.cand_extra) : nullptr, range_slots,
+                                   range_stride, s);
   } else {
-    rc = pkv_launch_scan(codes, (int64_t)H * a->cap * 16, a->cap * 16, 16, 1, a->bs, H, a->n_keys, lut, cnt,
-                         w.cnt_stride, nullptr, rowsuf, hist, w.chunk_keys, s);
+    rc = pkv_launch_query_prep_lut(a->q, a->dtype, a->bs, H, a->group, a->signs, a->cluster_counts,
+                                   (int64_t)H * 4096, 4096, t, qhat, qnorm, lut, nullptr, rowsuf, s, topk_ctl, ctl_words);
     if (rc) return rc;
-    rc = pkv_launch_select_rerank(cnt, w.cnt_stride, rowsuf, hist, w.chunk_keys, a->bs, H, a->n_keys, a->n_cand, nib,
-                                  (int64_t)H * a->cap * nk, a->cap * nk, nk, weight, (int64_t)H * a->cap * wk, a->cap * wk,
-                                  wk, qhat, qnorm, a->centers, cand, scores, s, a->record_word_offset,
-                                  a->record_word_offset > 0 ? (float *)(base + w.cand_extra) : nullptr,
-                                  range_slots, range_stride);
+    if (a->n_cand == a->n_keys) {
+      rc = pkv_launch_identity_fill(cand, a->n_keys, a->n_cand, rows, s);
+      if (rc) return rc;
+      rc = pkv_launch_rerank(cand, a->bs, H, a->n_cand, a->n_keys, nib, (int64_t)H * a->cap * nk, a->cap * nk, nk, 4,
+                             weight, (int64_t)H * a->cap * wk, a->cap * wk, wk, 1, qhat, qnorm, a->centers, scores,
+                             nullptr, s);
+    } else {
+      rc = pkv_launch_scan(codes, (int64_t)H * a->cap * 16, a->cap * 16, 16, 1, a->bs, H, a->n_keys, lut, cnt,
+                           w.cnt_stride, nullptr, rowsuf, hist, w.chunk_keys, s);
+      if (rc) return rc;
+      rc = pkv_launch_select_rerank(cnt, w.cnt_stride, rowsuf, hist, w.chunk_keys, a->bs, H, a->n_keys, a->n_cand, nib,
+                                    (int64_t)H * a->cap * nk, a->cap * nk, nk, weight, (int64_t)H * a->cap * wk, a->cap * wk,
+                                    wk, qhat, qnorm, a->centers, cand, scores, s, a->record_word_offset,
+                                    a->record_word_offset > 0 ? (float *)(base + w.cand_extra) : nullptr,
+                                    range_slots, range_stride);
+    }
   }
   if (rc) return rc;
   if (!a->out_ids) return PKV_OK;  // candidates only: the caller reads them out of the workspace

@@ -784,7 +784,7 @@ def _retrieve_args(bs, H, group, cap, queries, signs, centers, cluster_counts, c
 
 
 def retrieve_noalloc(queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, k,
-                     out_ids, out_scores=None, gather=None, any_order=False):
+                     out_ids, out_scores=None, gather=None, any_order=False, launch_plan=0):
     """One layer's retrieval through ``pkv_retrieve_noalloc``: the call of :meth:`RetrievePlan.run` for callers that may
     not allocate device memory.  The workspace is a fixed array inside the library (one per GPU, shared by every call
     on that GPU: overlapping calls race), so no plan is needed; ``out_ids`` int64 [bs,H,k] (and the optional
@@ -798,6 +798,7 @@ def retrieve_noalloc(queries, signs, centers, cluster_counts, codes_km, nib_km, 
                                  out_scores.numel() == bs * H * k), "out_scores: contiguous float32 [bs,H,k]")
     a = _retrieve_args(bs, H, group, cap, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys,
                        tier_counts, n_cand, k, out_ids, out_scores, gather, False, any_order)
+    a.launch_plan = int(launch_plan)
     _lib.check(_lib.lib().pkv_retrieve_noalloc(C.byref(a), _stream(codes_km)))
     return out_ids
 
@@ -813,6 +814,11 @@ class RetrievePlan:
         # the layout depends on (n_keys, n_cand); size for the worst case of each segment
         self.ws = torch.empty(int(nbytes) + (1 << 16), dtype=torch.uint8, device=device)
         self.max = (max_keys, max_cand, max_k)
+        # pkv_retrieve_args.launch_plan / skip_vote_counts of every argument block this plan fills: 0 = the stages
+        # before the top-k as one launch where the shape allows it, 1 = always as three launches; skip_vote_counts
+        # = the u8 vote counts need not reach the workspace (callers that never look at the "cnt_u8" view)
+        self.launch_plan = _lib.PLAN_AUTO
+        self.skip_vote_counts = False
 
     def run_candidates(self, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts,
                        n_cand):
@@ -831,9 +837,11 @@ class RetrievePlan:
         _need(need > 0, "need 0 < k <= n_cand <= n_keys")
         if need > self.ws.numel():
             self.ws = torch.empty(int(need), dtype=torch.uint8, device=self.device)
-        return _retrieve_args(self.bs, self.H, self.group, self.cap, queries, signs, centers, cluster_counts, codes_km,
-                              nib_km, w_km, key0, n_keys, tier_counts, n_cand, k, out_ids, out_scores, gather,
-                              candidates_only, any_order, record_word_offset)
+        a = _retrieve_args(self.bs, self.H, self.group, self.cap, queries, signs, centers, cluster_counts, codes_km,
+                           nib_km, w_km, key0, n_keys, tier_counts, n_cand, k, out_ids, out_scores, gather,
+                           candidates_only, any_order, record_word_offset)
+        a.launch_plan, a.skip_vote_counts = int(self.launch_plan), int(bool(self.skip_vote_counts))
+        return a
 
     def run(self, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts, n_cand, k,
             out_ids=None, out_scores=None, gather=None, candidates_only=False, attention=None, any_order=False):
