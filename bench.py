@@ -92,6 +92,250 @@ def model_decode(torch, dev, L, bs, S, T, K, warmup, offload, host_budget):
             "decode_tokens_per_s": round(bs * n_tok / dt, 1), "us_per_layer": round(dt * 1e6 / n_tok / L, 1)}
 
 
+def decode_loop(torch, dev, L, bs, S, T, K, adaptive=False, offload=True, k_range=(256, 2048), threshold=0.95,
+                key_drift=0.0, H=8, G=4, D=128):
+    """The cache class itself in a loop, no model around it: L layers, S prompt tokens of synthetic K/V (keys ~ N(0,1)
+    with four outlier channels, optionally a mean of norm 2 turning by ``key_drift`` degrees per 1K tokens), T decode
+    tokens (append + retrieval + gather + attention per layer; index refresh and host offload every 1024 tokens).
+    Returns (figures, cache, queries of the last step)."""
+    from pariskv_amd.attn_hub import polar_decode_attn
+    if adaptive:
+        from pariskv_amd.cache_hub.polar_cache_adaptivek_varlen import polar_cache
+    else:
+        from pariskv_amd.cache_hub.polar_cache import polar_cache
+
+    extra = {}
+    if adaptive:  # the class takes its caps from the environment, like the reference
+        os.environ["ADAPTIVE_TOPK_MIN_K"], os.environ["ADAPTIVE_TOPK_MAX_K"] = (str(v) for v in k_range)
+        extra["adaptive_topk_threshold"] = threshold
+    cache = polar_cache(valid_start=[0] * bs, layer_num=L, batch_size=bs, max_length=S + T + 8, num_key_value_heads=H,
+                        num_heads=H * G, head_dim=D, dtype=torch.bfloat16, layer_mapping={i: dev for i in range(L)},
+                        max_new_length=T + 8, sink_size=64, local_size=512, core=1, nprobe=1, cache_unit_size=1,
+                        cache_cluster_num=1, num_gpus=1, model_size=8, final_topk=K, dynamic_update_interval=1024,
+                        full_attention_threshold=2000, enable_offload=offload, **extra)
+    g = torch.Generator(device=dev).manual_seed(0)
+    t0 = time.perf_counter()
+    for l in range(L):
+        k = torch.randn(bs, S, H, D, generator=g, device=dev, dtype=torch.bfloat16)
+        k[..., [7, 31, 64, 101]] *= 10.0
+        if key_drift:  # key mean of norm 2 turning in the plane of dims (0, 1)
+            ang = torch.arange(S, device=dev, dtype=torch.float32) * (key_drift * math.pi / 180.0 / 1000.0)
+            k[..., 0] += (2.0 * torch.cos(ang)).to(torch.bfloat16)[None, :, None]
+            k[..., 1] += (2.0 * torch.sin(ang)).to(torch.bfloat16)[None, :, None]
+        v = torch.randn(bs, S, H, D, generator=g, device=dev, dtype=torch.bfloat16)
+        cache.prefill_update_kv_cache(None, k, v, l, 0)
+        kmean = k[:, -1024:].float().mean(dim=1)  # [bs, H, D]
+        del k, v
+    torch.cuda.synchronize()
+    t_prefill = time.perf_counter() - t0
+    k1 = torch.randn(T, bs, 1, H, D, generator=g, device=dev, dtype=torch.bfloat16)
+    v1 = torch.randn(T, bs, 1, H, D, generator=g, device=dev, dtype=torch.bfloat16)
+    # queries = mean of the recent keys of the head + N(0, 0.5), one per query head
+    q = (kmean.repeat_interleave(G, dim=1) + 0.5 * torch.randn(bs, H * G, D, generator=g, device=dev)
+         ).to(torch.bfloat16).view(bs, 1, H * G, D)
+    torch.cuda.synchronize()
+    tok_us, issue = [], []
+    for t in range(T):
+        a = time.perf_counter()
+        for l in range(L):
+            cache.decode_update_kv_cache(k1[t], v1[t], l)
+            polar_decode_attn(q, None, None, l, cache)
+        b = time.perf_counter()
+        torch.cuda.synchronize()
+        tok_us.append((time.perf_counter() - a) * 1e6)
+        issue.append((b - a) * 1e6)
+    skip = min(8, T // 2)
+    body = sorted(tok_us[skip:])
+    res = {"cache": "adaptive-k" if adaptive else "fixed-k", "key_drift_deg_per_1k": key_drift, "offload": bool(offload),
+           "layers": L, "batch": bs, "prompt": S, "generated": T, "final_topk": K, "prefill_s": round(t_prefill, 2),
+           "us_per_layer_step_median": round(body[len(body) // 2] / L, 1),
+           "us_per_layer_step_mean": round(sum(tok_us[skip:]) / len(tok_us[skip:]) / L, 1),
+           "us_per_layer_step_worst_token": round(body[-1] / L, 1),
+           "host_issue_us_per_layer_step": round(sorted(issue[skip:])[len(issue[skip:]) // 2] / L, 1),
+           "index_refreshes": T // 1024}
+    if adaptive:
+        ak = cache.last_adaptive_k.flatten().tolist()
+        res["adaptive"] = {"k_range": list(k_range), "threshold": threshold, "k_of_last_step": [min(ak), max(ak)]}
+    return res, cache, q
+
+
+def build_index_layers(torch, ops, dev, bs, H, G, N, L, signs, seed0=0, D=128):
+    """L layers of synthetic keys (~N(0,1), four outlier channels x10, independent seed per sequence and layer) encoded
+    on the GPU into the key-major index, with one query per query head = key mean + N(0, 0.5).  Returns the list of
+    layers and the bf16 keys / values of layer 0 (for the callers that keep full-precision K/V)."""
+    layers, k0, v0 = [], None, None
+    for l in range(L):
+        codes_km, nib_km, w_km, cb, k4, kw = ops.alloc_keymajor(bs, H, N, dev)
+        cc = torch.zeros(bs, H, 16, 256, dtype=torch.int32, device=dev)
+        q = torch.empty(bs, 1, H * G, D, dtype=torch.bfloat16, device=dev)
+        if l == 0:
+            k0 = torch.empty(bs, H, N, D, dtype=torch.bfloat16, device=dev)
+            v0 = torch.empty(bs, H, N, D, dtype=torch.bfloat16, device=dev)
+        for b in range(bs):
+            g = torch.Generator(device=dev).manual_seed(seed0 + 1000 * l + b)
+            keys = torch.randn(1, H, N, D, generator=g, device=dev, dtype=torch.float32)
+            keys[..., [7, 31, 64, 101]] *= 10.0
+            kb = keys.to(torch.bfloat16)
+            qq = keys.mean(dim=2, keepdim=True) + 0.5 * torch.randn(1, H, G, D, generator=g, device=dev)
+            q[b, 0] = qq.view(H * G, D).to(torch.bfloat16)
+            ops.encode_append(kb, signs, cb[b:b + 1], k4[b:b + 1], kw[b:b + 1], cc[b:b + 1])
+            if l == 0:
+                k0[b].copy_(kb[0])
+                v0[b].copy_(torch.randn(H, N, D, generator=g, device=dev).to(torch.bfloat16))
+            del keys, kb
+        layers.append(dict(codes=codes_km, nib=nib_km, w=w_km, cc=cc, q=q))
+    return layers, k0, v0
+
+
+def timed_us(torch, fn, n):
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for i in range(n):
+        fn(i)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1000.0 / n  # us per call
+
+
+def oracle_rows_equal(torch, O, layer, signs, out_ids, rows, bs, H, G, N, tiers, Cn, K, D=128):
+    """out_ids [bs,H,K] of one layer against O.retrieve_row on the GPU-encoded index, for the given rows."""
+    import numpy as np
+
+    sg = signs.cpu().numpy()
+    ok = True
+    for r in rows:
+        b, h = divmod(r, H)
+        ref = O.retrieve_row(layer["q"].view(bs, H, G, D)[b, h].float().cpu().numpy(), sg, O.BF16,
+                             layer["codes"][b, h].cpu().numpy(), layer["nib"][b, h][:, :64].cpu().numpy().reshape(N, 16, 4),
+                             layer["w"][b, h].float().cpu().numpy(), layer["cc"][b, h].cpu().numpy(), tiers, Cn, K)
+        ok = ok and bool(np.array_equal(out_ids.view(bs * H, K)[r].cpu().numpy(), ref))
+    return ok
+
+
+def cfg2_leg(torch, ops, _lib, dev, steps, warmup):
+    """BASELINE config 2: batch 1, 32 q / 8 KV heads, 32K keys per head, 2048 candidates, top-512, K/V in HBM: the
+    retrieval with the gather of the selected rows out of HBM, as one host call per step."""
+    from oracle import pkv_oracle as O
+
+    bs, H, G, N, Cn, K, L = 1, 8, 4, 32768, 2048, 512, 8
+    R = bs * H
+    signs, centers = ops.srht_signs(dev), ops.mag_centers(dev)
+    tiers = [int(math.ceil(N * 0.2 * r)) for r in TIER_RATIOS]
+    layers, kd, vd = build_index_layers(torch, ops, dev, bs, H, G, N, L, signs, seed0=20000)
+    dst_k = torch.empty(bs, H, K, 128, dtype=torch.bfloat16, device=dev)
+    dst_v = torch.empty_like(dst_k)
+    out_ids = torch.empty(bs, H, K, dtype=torch.int64, device=dev)
+    plan = ops.RetrievePlan(bs, H, G, N, dev, N, Cn, K)
+    plan.skip_vote_counts = True
+    gather = dict(src_k=kd, src_v=vd, from_host=False, dst_k=dst_k, dst_v=dst_v)
+
+    def step(i, with_gather=True):
+        ly = layers[i % L]
+        plan.run(ly["q"], signs, centers, ly["cc"], ly["codes"], ly["nib"], ly["w"], 0, N, tiers, Cn, K, out_ids=out_ids,
+                 gather=gather if with_gather else None)
+
+    for i in range(warmup):
+        step(i)
+    us_full = timed_us(torch, step, steps)
+    us_nogather = timed_us(torch, lambda i: step(i, False), steps)
+    plan.launch_plan = _lib.PLAN_ONE_LAUNCH
+    step(0)
+    us_full_one = timed_us(torch, step, steps)
+    plan.launch_plan = _lib.PLAN_SEPARATE
+    step(0)
+    torch.cuda.synchronize()
+    idx = out_ids.unsqueeze(-1).expand(-1, -1, -1, 128)
+    gather_ok = bool(torch.equal(dst_k, torch.gather(kd, 2, idx)) and torch.equal(dst_v, torch.gather(vd, 2, idx)))
+    O.build()
+    parity = oracle_rows_equal(torch, O, layers[0], signs, out_ids, (0, 3, 5, 7), bs, H, G, N, tiers, Cn, K)
+    a_hbm = R * (16 * N + 96 * Cn + 8 * K + 512 * K + 512 * K)  # codes + records + ids + rows read + rows written
+    return {"workload": f"BASELINE config 2: batch {bs} x {H} KV heads (GQA {G}), {N} keys/head, collision -> {Cn} "
+                        f"candidates, 4-bit rerank -> top-{K}, K/V in HBM (gather of the selected rows out of HBM "
+                        f"included), {L} rotating layers",
+            "rows": R, "on_gpu_stages_us": round(us_full, 2), "on_gpu_stages_without_the_gather_us": round(us_nogather, 2),
+            "on_gpu_stages_one_launch_plan_us": round(us_full_one, 2),
+            "algorithmic_bytes_hbm_per_step": a_hbm,
+            "hbm_fraction_on_gpu_stages": round(a_hbm / (us_full * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+            "parity_vs_oracle_rows_checked": 4, "parity_vs_oracle": bool(parity), "gathered_rows_equal_torch_gather": gather_ok}
+
+
+def cfg4_leg(torch, ops, _lib, dev):
+    """BASELINE config 4: batch 1, 32 q / 8 KV heads, 2^20 keys per head whose mean turns by 0.5 degrees per 1K tokens,
+    adaptive-k (k in [256, 2048] by benefit mass 0.95): the layer step through the adaptive cache class (one host call
+    = pkv_adaptive_decode_step: candidates, dense logits, adaptive k, ragged UVA gather, attention), and beside it the
+    fixed-k retrieval of the same index (query prep, scan, select + rerank, top-2048 of the 52429 candidates) as the
+    on-GPU figure."""
+    import numpy as np
+
+    from oracle import pkv_oracle as O
+
+    bs, H, G, S, L, T = 1, 8, 4, 1 << 20, 2, 40
+    res, cache, q = decode_loop(torch, dev, L, bs, S, T, 100, adaptive=True, offload=True, k_range=(256, 2048),
+                                threshold=0.95, key_drift=0.5)
+    torch.cuda.synchronize()
+    l = L - 1
+    n_keys, n_cand, _, tiers = cache.retrieval_shape(l)
+    sink = cache.sink_size
+    # the step's own outputs for this layer are still in place (it ran last): k per row and the ids in benefit order
+    ak = cache.last_adaptive_k.cpu().numpy()
+    cap_k, k_min, _ = cache._caps(n_cand)
+    ids_gpu = cache._topk_ids[:bs * H * cap_k].view(bs * H, cap_k).cpu().numpy()
+    z = cache._zones[l]
+    sl_end = z.gpu_prefix_rows
+    O.build()
+    signs = O.srht_signs(42)
+    scale = 1.0 / math.sqrt(128)
+    ok = True
+    for r in (0, 2, 5, 7):
+        b, h = divmod(r, H)
+        zone = slice(sink, sink + n_keys)
+        qrow = q[b, 0, h * G:(h + 1) * G].float().cpu().numpy()
+        qh, qn = O.query_prep(qrow, signs, O.BF16)
+        lut = O.tier_lut(O.rank_centroids(qh, O.BF16), cache.cluster_key_counts_gpu[l][b, h].cpu().numpy(), tiers)
+        cand_ref, _ = O.select_candidates(O.collision_count(cache._codes_km[l][b, h][zone].cpu().numpy(), lut), n_cand)
+        sc = O.rerank(cand_ref, cache._nib_km[l][b, h][zone][:, :64].cpu().numpy().reshape(-1, 16, 4),
+                      cache._w_km[l][b, h][zone].float().cpu().numpy(), qh, qn)
+        vn = cache.value_norm_gpu[l][b, h].cpu().numpy()[cand_ref + sink]
+        sl_logits = O.dense_logits(qrow, cache.unified_keys_gpu[l][b, h, :sl_end].float().cpu().numpy(), scale, O.BF16)
+        k_ref, ids_ref = O.adaptive_topk(sl_logits, cache._sl_vnorm_cache[l][b, h, :sl_end].cpu().numpy(),
+                                         sc * np.float32(scale), vn, cand_ref, 0.95, cap_k)
+        k_ref = min(max(k_ref, k_min), cap_k)
+        ok = ok and int(ak[b, h]) == k_ref and bool(np.array_equal(ids_gpu[r, :k_ref], ids_ref[:k_ref]))
+    # the fixed-k retrieval over the same index: on-GPU stages only, one host call per step
+    K = 2048
+    plan = ops.RetrievePlan(bs, H, G, cache._codes_km[0].shape[2], dev, n_keys, n_cand, K)
+    plan.skip_vote_counts = True
+    out_ids = torch.empty(bs, H, K, dtype=torch.int64, device=dev)
+
+    def step(i):
+        ll = i % L
+        plan.run(q, cache._srht_signs, cache._mag_centers, cache.cluster_key_counts_gpu[ll], cache._codes_km[ll],
+                 cache._nib_km[ll], cache._w_km[ll], sink, n_keys, tiers, n_cand, K, out_ids=out_ids)
+
+    for i in range(4):
+        step(i)
+    us_gpu = timed_us(torch, step, 24)
+    plan.launch_plan = _lib.PLAN_ONE_LAUNCH
+    step(0)
+    us_gpu_one = timed_us(torch, step, 24)
+    R = bs * H
+    a_hbm = R * (16 * n_keys + 96 * n_cand + 8 * K)
+    k_sum = int(ak.sum())
+    return {"workload": f"BASELINE config 4: batch {bs} x {H} KV heads (GQA {G}), {S} prompt tokens per head, key mean "
+                        f"turning 0.5 degrees per 1K tokens, {n_keys} indexed keys, {n_cand} candidates, adaptive k in "
+                        f"[256, 2048] at mass 0.95, K/V in pinned host memory, {L} layers",
+            "rows": R, "adaptive_layer_step": res,
+            "pcie_bytes_last_step": k_sum * 512, "k_of_last_step_sum_over_rows": k_sum,
+            "fixed_k_retrieval_on_gpu_stages_us": round(us_gpu, 2),
+            "fixed_k_retrieval_one_launch_plan_us": round(us_gpu_one, 2),
+            "fixed_k_retrieval": f"query prep, scan, select + rerank, top-{K} of {n_cand} candidates; no gather",
+            "algorithmic_bytes_hbm_per_step": a_hbm,
+            "hbm_fraction_on_gpu_stages": round(a_hbm / (us_gpu * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+            "parity_vs_oracle_rows_checked": 4, "parity_vs_oracle": bool(ok),
+            "parity_checked": "adaptive k and the first k ids of the last step, layer " + str(l)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -117,6 +361,8 @@ def main():
                     help="model-decode / the default run's cfg5 leg: pinned host memory the cache may use for offloaded "
                          "K/V; layers beyond it keep their K/V in HBM (0: no limit, every layer offloads)")
     ap.add_argument("--no-cfg5", action="store_true", help="default run: leave out the config-5 decode leg")
+    ap.add_argument("--no-cfg2", action="store_true", help="default run: leave out the config-2 leg (32K keys, K/V in HBM)")
+    ap.add_argument("--no-cfg4", action="store_true", help="default run: leave out the config-4 leg (1M keys, adaptive k)")
     ap.add_argument("--adaptive", action="store_true", help="decode-loop: the adaptive-k cache class (config 4's mode)")
     ap.add_argument("--adaptive-k-range", type=int, nargs=2, default=[256, 2048], metavar=("MIN", "MAX"),
                     help="decode-loop --adaptive: clamp of k (config 4: 256 2048; the reference's built-in caps: 100 800)")
@@ -147,67 +393,9 @@ def main():
         return
 
     if args.only == "decode-loop":
-        from pariskv_amd.attn_hub import polar_decode_attn
-        if args.adaptive:
-            from pariskv_amd.cache_hub.polar_cache_adaptivek_varlen import polar_cache
-        else:
-            from pariskv_amd.cache_hub.polar_cache import polar_cache
-
-        S, T = N, args.steps
-        extra = {}
-        if args.adaptive:  # the class takes its caps from the environment, like the reference
-            os.environ["ADAPTIVE_TOPK_MIN_K"], os.environ["ADAPTIVE_TOPK_MAX_K"] = (str(v) for v in args.adaptive_k_range)
-            extra["adaptive_topk_threshold"] = args.adaptive_threshold
-        cache = polar_cache(valid_start=[0] * bs, layer_num=L, batch_size=bs, max_length=S + T + 8, num_key_value_heads=H,
-                            num_heads=H * G, head_dim=D, dtype=torch.bfloat16, layer_mapping={i: dev for i in range(L)},
-                            max_new_length=T + 8, sink_size=64, local_size=512, core=1, nprobe=1, cache_unit_size=1,
-                            cache_cluster_num=1, num_gpus=1, model_size=8, final_topk=K, dynamic_update_interval=1024,
-                            full_attention_threshold=2000, enable_offload=not args.no_offload, **extra)
-        g = torch.Generator(device=dev).manual_seed(0)
-        t0 = time.perf_counter()
-        for l in range(L):
-            k = torch.randn(bs, S, H, D, generator=g, device=dev, dtype=torch.bfloat16)
-            k[..., [7, 31, 64, 101]] *= 10.0
-            if args.key_drift:  # key mean of norm 2 turning in the plane of dims (0, 1)
-                ang = torch.arange(S, device=dev, dtype=torch.float32) * (args.key_drift * math.pi / 180.0 / 1000.0)
-                k[..., 0] += (2.0 * torch.cos(ang)).to(torch.bfloat16)[None, :, None]
-                k[..., 1] += (2.0 * torch.sin(ang)).to(torch.bfloat16)[None, :, None]
-            v = torch.randn(bs, S, H, D, generator=g, device=dev, dtype=torch.bfloat16)
-            cache.prefill_update_kv_cache(None, k, v, l, 0)
-            kmean = k[:, -1024:].float().mean(dim=1)  # [bs, H, D]
-            del k, v
-        torch.cuda.synchronize()
-        t_prefill = time.perf_counter() - t0
-        k1 = torch.randn(T, bs, 1, H, D, generator=g, device=dev, dtype=torch.bfloat16)
-        v1 = torch.randn(T, bs, 1, H, D, generator=g, device=dev, dtype=torch.bfloat16)
-        # queries = mean of the recent keys of the head + N(0, 0.5), one per query head
-        q = (kmean.repeat_interleave(G, dim=1) + 0.5 * torch.randn(bs, H * G, D, generator=g, device=dev)
-             ).to(torch.bfloat16).view(bs, 1, H * G, D)
-        torch.cuda.synchronize()
-        tok_us, issue = [], []
-        for t in range(T):
-            a = time.perf_counter()
-            for l in range(L):
-                cache.decode_update_kv_cache(k1[t], v1[t], l)
-                polar_decode_attn(q, None, None, l, cache)
-            b = time.perf_counter()
-            torch.cuda.synchronize()
-            tok_us.append((time.perf_counter() - a) * 1e6)
-            issue.append((b - a) * 1e6)
-        body = sorted(tok_us[8:])
-        if args.adaptive:
-            ak = cache.last_adaptive_k.flatten().tolist()
-            adaptive_info = {"k_range": args.adaptive_k_range, "threshold": args.adaptive_threshold,
-                             "k_of_last_step": [min(ak), max(ak)]}
-        print(json.dumps({"only": "decode-loop", "cache": "adaptive-k" if args.adaptive else "fixed-k",
-                          **({"adaptive": adaptive_info} if args.adaptive else {}), "key_drift_deg_per_1k": args.key_drift,
-                          "offload": not args.no_offload, "layers": L, "batch": bs, "prompt": S,
-                          "generated": T, "final_topk": K, "prefill_s": round(t_prefill, 2),
-                          "us_per_layer_step_median": round(body[len(body) // 2] / L, 1),
-                          "us_per_layer_step_mean": round(sum(tok_us[8:]) / len(tok_us[8:]) / L, 1),
-                          "us_per_layer_step_worst_token": round(body[-1] / L, 1),
-                          "host_issue_us_per_layer_step": round(sorted(issue[8:])[len(issue[8:]) // 2] / L, 1),
-                          "index_refreshes": T // 1024}))
+        res, _, _ = decode_loop(torch, dev, L, bs, N, args.steps, K, adaptive=args.adaptive, offload=not args.no_offload,
+                                k_range=args.adaptive_k_range, threshold=args.adaptive_threshold, key_drift=args.key_drift)
+        print(json.dumps({"only": "decode-loop", **res}))
         return
 
     if args.only == "adaptive":
@@ -263,6 +451,7 @@ def main():
     dst_v = torch.empty_like(dst_k)
     out_ids = torch.empty(bs, H, K, dtype=torch.int64, device=dev)
     plan = ops.RetrievePlan(bs, H, G, N, dev, N, Cn, K)
+    plan.skip_vote_counts = True  # nothing here looks at the per-key vote counts
     gather = dict(src_k=kcpu, src_v=vcpu, from_host=True, dst_k=dst_k, dst_v=dst_v)
     torch.cuda.synchronize()
 
@@ -324,6 +513,12 @@ def main():
     us_step = timed(step, args.steps)                       # full retrieval incl. UVA gather  (the metric)
     t_wall = time.perf_counter() - t_wall0
     us_gpu = timed(lambda i: step(i, False), args.steps)    # on-GPU stages only
+    plan.launch_plan = _lib.PLAN_ONE_LAUNCH                 # the same with query prep, scan, select + rerank as one launch
+    step(0, False)
+    us_gpu_one = timed(lambda i: step(i, False), args.steps)
+    one_launch_status = int(plan.view("handover_status", N, Cn, K, torch.int32)[0])
+    plan.launch_plan = _lib.PLAN_SEPARATE
+    step(0, False)
 
     def step_any_order(i):  # what polar_cache.compute asks for: the same k ids as a set, final sort left out
         ly = layers[i % L]
@@ -417,8 +612,11 @@ def main():
     read_only(0)
     read_gbps = code_bytes / (timed(read_only, args.steps) * 1e-6) / 1e9
 
-    a_hbm = R * (16 * N + 96 * Cn + 8 * K + 512 * K)  # algorithmic HBM bytes of the whole on-GPU pipeline
+    a_hbm = R * (16 * N + 96 * Cn + 8 * K + 512 * K)  # algorithmic HBM bytes of the whole pipeline, gathered rows written included
+    a_hbm_timed = R * (16 * N + 96 * Cn + 8 * K)      # ... of the launches `on_gpu_stages` times (no gather: no rows written)
     a_pcie = R * 512 * K
+    default_shape = (bs, N, Cn, K) == (4, 131072, 4096, 1024)
+    shape_name = "BASELINE config 3" if default_shape else "config 3's pipeline at another shape"
 
     result = {
         "metric": "retrieval us/layer/decode-step at 128K ctx; achieved HBM GB/s vs peak",
@@ -433,26 +631,31 @@ def main():
         "vs_baseline": None,
         "dtype": "u8 votes / f32 rerank (bf16 keys)",
         "data": "synthetic",
-        "config": {"workload": f"BASELINE config 3: batch {bs} x {H} KV heads (GQA {G}), head_dim {D}, {N} keys/head, "
+        "config": {"workload": f"{shape_name}: batch {bs} x {H} KV heads (GQA {G}), head_dim {D}, {N} keys/head, "
                                f"collision -> {Cn} candidates, 4-bit rerank -> top-{K}, KV in pinned host memory "
                                f"(UVA gather), {L} rotating layers",
                    "rows": R, "keys_per_row": N, "candidates": Cn, "topk": K, "collision_ratio": 0.2},
         "stages_us": {"full_retrieval_with_uva_gather": round(us_step, 2), "on_gpu_stages": round(us_gpu, 2),
+                      "on_gpu_stages_one_launch_plan": round(us_gpu_one, 2),
                       "on_gpu_stages_ids_in_any_order": round(us_gpu_any, 2),
                       "on_gpu_stages_replayed_from_a_hip_graph": None if us_gpu_graph is None else round(us_gpu_graph, 2),
                       "uva_gather_alone": round(us_gather, 2),
                       "decode_attention_over_gathered_set": round(us_attn, 2),
                       "full_step_plus_attention_one_host_call": round(us_step_attn, 2)},
         "hbm_fraction_on_gpu_stages": round(a_hbm / (us_gpu * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
-        "algorithmic_bytes": {"hbm_per_step": a_hbm, "pcie_per_step": a_pcie},
+        "hbm_fraction_on_gpu_stages_counting_only_bytes_the_timed_launches_move": round(
+            a_hbm_timed / (us_gpu * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+        "algorithmic_bytes": {"hbm_per_step": a_hbm, "hbm_per_step_without_the_gathered_rows": a_hbm_timed,
+                              "pcie_per_step": a_pcie},
         "streaming_read_GBps_same_arrays": round(read_gbps, 1),
         "pcie_GBps_gather": round(a_pcie / (us_gather * 1e-6) / 1e9, 2),
         "pcie_GBps_plain_memcpy_same_bytes": round(a_pcie / (us_memcpy * 1e-6) / 1e9, 2),
         "roofline": {"kernel": SCAN_KERNEL, "bound": "hbm", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": SCAN_TRAFFIC_BYTES,
-                     "traffic_source": "constant from " + SCAN_TRAFFIC_SOURCE + " (rocprofv3 --pmc FETCH_SIZE / "
-                                       "WRITE_SIZE of this command), not measured in this run",
+                     "traffic": SCAN_TRAFFIC_BYTES if default_shape else None,
+                     "traffic_source": ("constant from " + SCAN_TRAFFIC_SOURCE + " (rocprofv3 --pmc FETCH_SIZE / "
+                                        "WRITE_SIZE of this command), not measured in this run") if default_shape
+                                       else "not measured at this shape",
                      "bytes_per_launch": scan_bytes, "bytes_per_key": 16,
                      "avg_launch_us": round(scan_avg_us, 2),
                      "avg_launch_us_source": "begin/end timestamps of each dispatch (hipExtLaunchKernelGGL events); "
@@ -460,6 +663,7 @@ def main():
                      "GBps_counting_the_1B_vote_count_written": round(
                          scan_bytes_with_counts / (scan_avg_us * 1e-6) / 1e9, 1)},
         "wall_s_timed_region": round(t_wall, 4),
+        "one_launch_plan_handover_status": one_launch_status,
     }
 
     if args.no_cpu_baseline:  # still check a few rows of the benchmarked GPU path against the oracle
@@ -559,25 +763,46 @@ def main():
                                   "torch_cpu_one_thread": {"value": round(t_one * 1e6, 1), "threads": 1,
                                                            "repetitions": n_one},
                                   "torch_cpu_sample": f"the same {R} rows as batched torch ops on the reference's "
-                                                      f"subspace-major tensors (oracle/torch_baseline.py), host gather "
-                                                      f"included, median; final ids overlap with the C oracle's: "
-                                                      f"{overlap:.4f}"}
+                                                      f"subspace-major tensors, in the form of the reference's torch "
+                                                      f"fallback code (oracle/torch_baseline.py; a timing yardstick, "
+                                                      f"not a parity target: its ties and bf16 matmul are torch's), "
+                                                      f"host gather included, median; final ids overlap with the C "
+                                                      f"oracle's: {overlap:.4f}"}
         result["parity_vs_oracle_on_bench_workload"] = bool(parity)
 
-    # ------------------------------------- config 5: end-to-end decode tokens/s
-    if not args.no_cfg5:
-        del layers, luts, kcpu, vcpu, dst_k, dst_v, cnt_ws, hist_ws, plan, gather
-        if not args.no_cpu_baseline:
-            del host, tb
-        import gc
+    # ------------------- the other configs' shapes (objects beside the headline; a failure costs only its own object)
+    del layers, luts, kcpu, vcpu, dst_k, dst_v, cnt_ws, hist_ws, plan, gather
+    if not args.no_cpu_baseline:
+        del host, tb
+    import gc
 
+    gc.collect()
+    torch.cuda.empty_cache()
+
+    def leg(name, fn):
+        try:
+            result[name] = fn()
+        except Exception as e:  # e.g. an allocation the box cannot satisfy
+            result[name] = {"error": f"{type(e).__name__}: {e}"[:400]}
         gc.collect()
         torch.cuda.empty_cache()
-        try:
-            result["cfg5"] = model_decode(torch, dev, 36, 8, 65536, 256, 100, 8, True, int(args.host_kv_budget_gib * 2**30)
-                                          if args.host_kv_budget_gib > 0 else None)
-        except Exception as e:  # an allocation the box cannot satisfy must not cost the record its headline line
-            result["cfg5"] = {"error": f"{type(e).__name__}: {e}"[:400]}
+
+    if not args.no_cfg2:
+        leg("cfg2", lambda: cfg2_leg(torch, ops, _lib, dev, args.steps, args.warmup))
+    if not args.no_cfg4:
+        leg("cfg4", lambda: cfg4_leg(torch, ops, _lib, dev))
+    # config 5: end-to-end decode tokens/s
+    if not args.no_cfg5:
+        def cfg5():
+            r = model_decode(torch, dev, 36, 8, 65536, 256, 100, 8, True, int(args.host_kv_budget_gib * 2**30)
+                             if args.host_kv_budget_gib > 0 else None)
+            pl = r["placement"]
+            r["headline"] = (f"decode_tokens_per_s with {pl['host_layers']} of 36 layers' K/V offloaded to pinned host "
+                             f"memory and {pl['hbm_layers']} resident in HBM (the box pins at most ~65 GiB; the "
+                             f"reference's enable_offload would put all 36 on the host)")
+            return r
+
+        leg("cfg5", cfg5)
     print(json.dumps(result))
 
 

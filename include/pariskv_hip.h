@@ -491,18 +491,23 @@ typedef struct pkv_retrieve_args {
    * (cache_hub/polar_cache_adaptivek_varlen.py:1741-1753 gathers value_norm_gpu at cand_idx + sink). */
   int64_t record_word_offset;
   /* How the stages before the top-k are launched; the results are the same.
-   * PKV_PLAN_AUTO (0): query prep, collision scan and select + rerank as ONE launch whose workgroups hand the
-   *   row's vote table and histogram to each other, where the shape allows it (chunks of at most 8192 keys,
-   *   at most 256 chunks per row) and `stream` is not being captured into a graph; otherwise as below.
-   * PKV_PLAN_SEPARATE (1): always as three launches (the reference's structure: collision kernel,
-   *   top-k kernel, rerank kernel, cache_hub/polar_cache.py:1207-1298). */
+   * PKV_PLAN_SEPARATE (0, default): three launches (the reference's structure: collision kernel, top-k kernel,
+   *   rerank kernel, cache_hub/polar_cache.py:1207-1298).
+   * PKV_PLAN_ONE_LAUNCH (1): query prep, collision scan and select + rerank as ONE launch whose workgroups hand
+   *   the row's vote table and histogram to each other through agent-scope stores, flags and bounded waits.
+   *   Taken where the shape allows it (chunks of at most 8192 keys, at most 1024 workgroups, i.e. a grid that is
+   *   resident as a whole) and `stream` is not being captured into a graph; otherwise the call proceeds as
+   *   PKV_PLAN_SEPARATE.  Measured on MI355X it is within +-1 us of the three launches at 32 rows x 128K keys
+   *   and 8 rows x 32K keys, up to 4 % faster at 8 rows x 1M keys: a hand-over between workgroups costs about
+   *   what a launch boundary costs.  A workgroup that gives up a wait (2 s) counts itself in the workspace
+   *   segment "handover_status" (0 after a good launch) and the results of that call are undefined. */
   int launch_plan;
   /* nonzero: the per-key vote counts need not be left in the workspace segment "cnt_u8" (the one-launch plan then
    * keeps them on chip). */
   int skip_vote_counts;
 } pkv_retrieve_args;
-#define PKV_PLAN_AUTO 0
-#define PKV_PLAN_SEPARATE 1
+#define PKV_PLAN_SEPARATE 0
+#define PKV_PLAN_ONE_LAUNCH 1
 
 size_t pkv_retrieve_ws_bytes(int rows, int64_t n_keys, int64_t n_cand, int64_t k);
 int pkv_retrieve(const pkv_retrieve_args *args, void *ws, size_t ws_bytes, void *stream);

@@ -54,7 +54,7 @@ class RetrieveArgs(C.Structure):
     ]
 
 
-PLAN_AUTO, PLAN_SEPARATE = 0, 1  # pkv_retrieve_args.launch_plan
+PLAN_SEPARATE, PLAN_ONE_LAUNCH = 0, 1  # pkv_retrieve_args.launch_plan
 
 
 class AdaptiveArgs(C.Structure):

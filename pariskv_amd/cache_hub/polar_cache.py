@@ -175,6 +175,7 @@ class polar_cache(KV_Cache):
         max_keys = max(1, cap - sink_size)
         max_cand = max(1, math.ceil(max_keys * 0.5))
         self._plan = ops.RetrievePlan(bs, H, self.group_size, cap, dev, max_keys, max_cand, max(1, min(final_topk, max_cand)))
+        self._plan.skip_vote_counts = True  # the cache never looks at the per-key vote counts of a step
         self._attn_k = self._attn_v = None  # no-offload mode with few rows: staging buffer of the selected rows
         self._bound = [None] * layer_num  # per layer: (n_keys, ops.BoundStep, topk, out_ids, index of the local segment)
         self._out_ids = torch.empty((bs, H, max(1, final_topk)), dtype=torch.int64, device=dev)

@@ -167,7 +167,7 @@ static int retrieve_impl(const pkv_retrieve_args *a, void *ws, size_t ws_bytes, 
   const uint8_t *nib = a->nib + a->key0 * nk;
   const uint16_t *weight = a->weight + a->key0 * wk;
   int rc;
-  if (a->n_cand != a->n_keys && a->launch_plan != PKV_PLAN_SEPARATE && pkv_fused_usable(rows, a->n_keys, w.chunk_keys, s)) {
+  if (a->n_cand != a->n_keys && a->launch_plan == PKV_PLAN_ONE_LAUNCH && pkv_fused_usable(rows, a->n_keys, w.chunk_keys, s)) {
     // query prep, scan and select + rerank as one launch
     rc = pkv_launch_fused_retrieve(a->q, a->dtype, a->bs, H, a->group, a->signs, a->cluster_counts, (int64_t)H * 4096, 4096,
                                    t, qhat, qnorm, lut, codes, (int64_t)H * a->cap * 16, a->cap * 16, a->n_keys,

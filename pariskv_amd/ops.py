@@ -815,9 +815,9 @@ class RetrievePlan:
         self.ws = torch.empty(int(nbytes) + (1 << 16), dtype=torch.uint8, device=device)
         self.max = (max_keys, max_cand, max_k)
         # pkv_retrieve_args.launch_plan / skip_vote_counts of every argument block this plan fills: 0 = the stages
-        # before the top-k as one launch where the shape allows it, 1 = always as three launches; skip_vote_counts
-        # = the u8 vote counts need not reach the workspace (callers that never look at the "cnt_u8" view)
-        self.launch_plan = _lib.PLAN_AUTO
+        # before the top-k as three launches, 1 = as one launch where the shape allows it; skip_vote_counts = the
+        # u8 vote counts need not reach the workspace (callers that never look at the "cnt_u8" view)
+        self.launch_plan = _lib.PLAN_SEPARATE
         self.skip_vote_counts = False
 
     def run_candidates(self, queries, signs, centers, cluster_counts, codes_km, nib_km, w_km, key0, n_keys, tier_counts,

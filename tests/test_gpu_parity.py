@@ -629,6 +629,50 @@ def test_retrieve_fused_matches_oracle(ops, request, wl_name):
         assert np.array_equal(out[b, h].cpu().numpy(), whole)
 
 
+@pytest.mark.parametrize("wl_name", ["wl_cfg1", "wl_cfg2", "wl_small_bf16"])
+def test_one_launch_plan_equals_three_launches(ops, request, wl_name):
+    """pkv_retrieve_args.launch_plan = PKV_PLAN_ONE_LAUNCH (query prep, scan and select + rerank as one launch whose
+    workgroups hand the vote table and the histogram over) against the three launches: every intermediate and every
+    output bit for bit, and against the oracle; with the flag area full of garbage before the first launch, three
+    launches back to back on one workspace, no workgroup giving up a wait."""
+    from pariskv_amd import _lib
+
+    w = request.getfixturevalue(wl_name)
+    _say(f"one-launch plan {w.name}: R={w.R} N={w.N} C={w.C} K={w.K}")
+    d = W.to_device(w, DEV, torch)
+    args = (d["queries"], d["signs"], d["centers"], d["cluster_counts"], d["codes_km"], d["nib_km"], d["w_km"], 0, w.N, w.tiers,
+            w.C, w.K)
+    names = (("qhat", torch.float32), ("qnorm", torch.float32), ("lut", torch.uint8), ("chunk_suffix_hist", torch.int16),
+             ("row_suffix_hist", torch.int32), ("cand", torch.int64), ("scores", torch.float32))
+    cnt_stride = (w.N + 15) // 16 * 16
+    plan = ops.RetrievePlan(w.bs, w.H, w.G, w.N, DEV, w.N, w.C, w.K)
+    ref_sc = torch.empty(w.bs, w.H, w.K, dtype=torch.float32, device=DEV)
+    ref_ids = plan.run(*args, out_scores=ref_sc).clone()
+    ref = {n: plan.view(n, w.N, w.C, w.K, dt).clone() for n, dt in names}
+    ref_cnt = plan.view("cnt_u8", w.N, w.C, w.K, torch.uint8).view(w.R, cnt_stride)[:, :w.N].clone()
+    plan.launch_plan = _lib.PLAN_ONE_LAUNCH
+    plan.ws.fill_(0xA5)
+    for rep in range(3):
+        plan.skip_vote_counts = rep == 2
+        if rep == 2:
+            plan.view("cnt_u8", w.N, w.C, w.K, torch.uint8).zero_()
+        sc = torch.empty_like(ref_sc)
+        ids = plan.run(*args, out_scores=sc)
+        torch.cuda.synchronize()
+        assert int(plan.view("handover_status", w.N, w.C, w.K, torch.int32)[0]) == 0
+        assert torch.equal(ids, ref_ids) and torch.equal(sc, ref_sc)
+        for n, dt in names:
+            assert torch.equal(plan.view(n, w.N, w.C, w.K, dt), ref[n]), f"{n} differs in launch {rep}"
+        cnt = plan.view("cnt_u8", w.N, w.C, w.K, torch.uint8).view(w.R, cnt_stride)[:, :w.N]
+        if rep == 2:
+            assert not bool(cnt.any())  # the counts stayed on chip
+        else:
+            assert torch.equal(cnt, ref_cnt)
+    for r in range(w.R):
+        b, h = divmod(r, w.H)
+        assert np.array_equal(ids[b, h].cpu().numpy(), W.oracle_stages(w, r)["final"])
+
+
 def test_retrieve_subrange_and_candidates_equal_keys(ops, wl_small_bf16):
     """Retrieval zone = [key0, key0+n) of a larger capacity; and C == N (identity candidates)."""
     w = wl_small_bf16
@@ -690,30 +734,53 @@ def test_retrieve_argument_errors(ops, wl_small_bf16):
 
 @pytest.mark.parametrize("N,R,C,K", [(131072, 32, 4096, 1024)])
 def test_full_size_properties(ops, N, R, C, K):
-    """BASELINE config 3 shape on GPU-generated inputs: size-independent properties plus a
-    sampled-row comparison with the oracle (GPU-encoded index copied back to the host)."""
+    """BASELINE config 3 at full size on GPU-generated inputs (batch 4, an independent seed per sequence, K/V in
+    pinned host memory): size-independent properties of the whole step, the UVA gather of all 32 x 1024 selected rows
+    bit for bit against torch.gather on the pinned tensors, and 8 rows spread over the four sequences against the
+    oracle (GPU-encoded index copied back to the host; the encode of those rows against the oracle's too).  Both
+    launch plans."""
+    from pariskv_amd import _lib
+
     _say(f"full-size N={N} R={R} C={C} K={K}")
     bs, H, G = 4, 8, 4
-    g = torch.Generator(device=DEV).manual_seed(0)
-    keys = torch.randn(bs, H, N, 128, generator=g, device=DEV, dtype=torch.float32)
-    keys[..., [7, 31, 64, 101]] *= 10
-    keys = keys.to(torch.bfloat16)
-    q = (keys.float().mean(dim=2, keepdim=True) + 0.5 * torch.randn(bs, H, G, 128, generator=g, device=DEV)).to(torch.bfloat16)
-    q = q.view(bs, 1, H * G, 128).contiguous()
     signs = ops.srht_signs(DEV)
     codes_km, nib_km, w_km, cb, k4, kw = ops.alloc_keymajor(bs, H, N, DEV)
     cc = torch.zeros(bs, H, 16, 256, dtype=torch.int32, device=DEV)
-    ops.encode_append(keys, signs, cb, k4, kw, cc)
+    q = torch.empty(bs, 1, H * G, 128, dtype=torch.bfloat16, device=DEV)
+    keys = torch.empty(bs, H, N, 128, dtype=torch.bfloat16, device=DEV)
+    kcpu = torch.empty(bs, H, N, 128, dtype=torch.bfloat16, pin_memory=True)
+    vcpu = torch.empty(bs, H, N, 128, dtype=torch.bfloat16, pin_memory=True)
+    for b in range(bs):
+        g = torch.Generator(device=DEV).manual_seed(1000 * 3 + b)  # one seed per sequence
+        kf = torch.randn(1, H, N, 128, generator=g, device=DEV, dtype=torch.float32)
+        kf[..., [7, 31, 64, 101]] *= 10
+        keys[b] = kf[0].to(torch.bfloat16)
+        q[b, 0] = (kf.mean(dim=2, keepdim=True) + 0.5 * torch.randn(1, H, G, 128, generator=g, device=DEV)).view(H * G, 128).to(torch.bfloat16)
+        ops.encode_append(keys[b:b + 1], signs, cb[b:b + 1], k4[b:b + 1], kw[b:b + 1], cc[b:b + 1])
+        kcpu[b].copy_(keys[b])
+        vcpu[b].copy_(torch.randn(H, N, 128, generator=g, device=DEV).to(torch.bfloat16))
+        del kf
     assert int(cc.sum()) == R * N * 16 and bool((cc.sum(dim=-1) == N).all())  # every key lands in one cluster per subspace
     tiers = O.tier_counts(N, 0.2)
     plan = ops.RetrievePlan(bs, H, G, N, DEV, N, C, K)
     sc = torch.empty(bs, H, K, device=DEV)
-    out1 = plan.run(q, signs, ops.mag_centers(DEV), cc, codes_km, nib_km, w_km, 0, N, tiers, C, K, out_scores=sc).clone()
+    dk = torch.zeros(bs, H, K, 128, dtype=torch.bfloat16, device=DEV)
+    dv = torch.zeros_like(dk)
+    gather = dict(src_k=kcpu, src_v=vcpu, from_host=True, dst_k=dk, dst_v=dv)
+    out1 = plan.run(q, signs, ops.mag_centers(DEV), cc, codes_km, nib_km, w_km, 0, N, tiers, C, K, out_scores=sc, gather=gather).clone()
     cand = plan.view("cand", N, C, K, torch.int64).view(R, C).clone()
     cnt = plan.view("cnt_u8", N, C, K, torch.uint8).view(R, N).clone()
     out2 = plan.run(q, signs, ops.mag_centers(DEV), cc, codes_km, nib_km, w_km, 0, N, tiers, C, K)
+    plan.launch_plan = _lib.PLAN_ONE_LAUNCH
+    out3 = plan.run(q, signs, ops.mag_centers(DEV), cc, codes_km, nib_km, w_km, 0, N, tiers, C, K).clone()
+    out4 = plan.run(q, signs, ops.mag_centers(DEV), cc, codes_km, nib_km, w_km, 0, N, tiers, C, K)
     torch.cuda.synchronize()
-    assert torch.equal(out1, out2)                                   # deterministic / idempotent
+    assert int(plan.view("handover_status", N, C, K, torch.int32)[0]) == 0
+    assert torch.equal(out1, out2) and torch.equal(out1, out3) and torch.equal(out1, out4)  # deterministic, both plans
+    assert torch.equal(plan.view("cand", N, C, K, torch.int64).view(R, C), cand)
+    # the gather of every selected row out of pinned host memory
+    idx = out1.cpu().unsqueeze(-1).expand(-1, -1, -1, 128)
+    assert torch.equal(dk.cpu(), torch.gather(kcpu, 2, idx)) and torch.equal(dv.cpu(), torch.gather(vcpu, 2, idx))
     assert bool((sc[..., :-1] >= sc[..., 1:]).all())                 # descending scores
     assert bool((out1 >= 0).all()) and bool((out1 < N).all())
     srt = out1.sort(dim=-1).values
@@ -727,15 +794,17 @@ def test_full_size_properties(ops, N, R, C, K):
     assert bool((cand_cnt.min(dim=1).values >= rest_max).all())
     # final ids are a subset of the candidates
     assert bool(torch.isin(out1.view(R, K), cand).all())
-    # sampled rows against the oracle, using the GPU-encoded index
-    for r in (0, 13, 31):
+    # rows of every sequence against the oracle, using the GPU-encoded index
+    sg = signs.cpu().numpy()
+    for r in (0, 5, 10, 13, 19, 22, 28, 31):
         b, h = divmod(r, H)
-        ref = O.retrieve_row(q.view(bs, H, G, 128)[b, h].float().cpu().numpy(), signs.cpu().numpy(), O.BF16,
+        ref = O.retrieve_row(q.view(bs, H, G, 128)[b, h].float().cpu().numpy(), sg, O.BF16,
                              codes_km[b, h].cpu().numpy(), nib_km[b, h].cpu().numpy().reshape(N, 16, 4),
                              w_km[b, h].float().cpu().numpy(), cc[b, h].cpu().numpy(), tiers, C, K)
-        assert np.array_equal(out1[b, h].cpu().numpy(), ref)
-        # and the GPU encode of that row equals the oracle's encode
-        codes, nib, wt = O.encode(keys[b, h].float().cpu().numpy(), signs.cpu().numpy(), O.BF16)
+        assert np.array_equal(out1[b, h].cpu().numpy(), ref), f"row {r}"
+    for r in (0, 13, 31):  # and the GPU encode of these rows equals the oracle's encode
+        b, h = divmod(r, H)
+        codes, nib, wt = O.encode(keys[b, h].float().cpu().numpy(), sg, O.BF16)
         assert np.array_equal(codes_km[b, h].cpu().numpy(), codes)
         assert np.array_equal(nib_km[b, h].cpu().numpy().reshape(N, 16, 4), nib)
         assert np.array_equal(w_km[b, h].float().cpu().numpy(), wt)
