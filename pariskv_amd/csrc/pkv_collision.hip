@@ -36,12 +36,19 @@ __device__ __forceinline__ void load_lut(uint32_t *s_lut, const uint8_t *__restr
 }
 
 // Key-major codes ([key][16] bytes, 16-byte aligned).  grid (n_chunks, R).
+// sub_blocks = 1: workgroup c scans keys [c * chunk_keys, +chunk_keys) and leaves one suffix histogram.
+// sub_blocks = S > 1: the chunk is S pieces of chunk_keys / S keys spread over the row, workgroup c scans pieces
+// c, c + n_chunks, c + 2 n_chunks, ... (numbered in key order) and leaves one suffix histogram per piece, in the
+// bin-major table chunk_suf[row][bin][chunk][piece of the chunk] (S = 4): the candidate select that follows works on the same pieces, so that where candidates
+// bunch along the row (keys whose mean drifts) every workgroup gets a share of the crowded and of the sparse parts.
 __global__ __launch_bounds__(kScanThreads) void pkv_scan_keymajor_kernel(
     const uint8_t *__restrict__ codes, int64_t cs_b, int64_t cs_h, int n_kv_heads, int64_t n_keys,
     const uint8_t *__restrict__ lut, uint8_t *__restrict__ cnt_u8, int64_t cnt_u8_stride,
-    int32_t *__restrict__ cnt_i32, uint32_t *__restrict__ row_suf, uint16_t *__restrict__ chunk_suf, int chunk_keys) {
+    int32_t *__restrict__ cnt_i32, uint32_t *__restrict__ row_suf, uint16_t *__restrict__ chunk_suf, int chunk_keys,
+    int sub_blocks) {
   const int row = blockIdx.y;
   const int chunk = blockIdx.x;
+  const int n_chunks = gridDim.x;
   const int b = row / n_kv_heads, h = row % n_kv_heads;
   const int tid = threadIdx.x;
 
@@ -54,41 +61,74 @@ __global__ __launch_bounds__(kScanThreads) void pkv_scan_keymajor_kernel(
   const int copy = tid & (kHistCopies - 1);
 
   const pkv_u32x4 *base = (const pkv_u32x4 *)(codes + (int64_t)b * cs_b + (int64_t)h * cs_h);
-  const int64_t k0 = (int64_t)chunk * chunk_keys;
-  const int64_t k1 = (k0 + chunk_keys < n_keys) ? k0 + chunk_keys : n_keys;
   uint8_t *out8 = cnt_u8 ? cnt_u8 + (int64_t)row * cnt_u8_stride : nullptr;
   int32_t *out32 = cnt_i32 ? cnt_i32 + (int64_t)row * n_keys : nullptr;
+  const int piece_keys = chunk_keys / sub_blocks;
+  uint64_t piece_bins = 0;  // sub_blocks == 4: this thread's bin of the four pieces' suffix histograms, 16 bits each
+  uint32_t bin_total = 0;
 
-  for (int64_t i0 = k0 + tid; i0 < k1; i0 += 4 * kScanThreads) {
-    pkv_u32x4 v[4];
+  for (int j = 0; j < sub_blocks; ++j) {
+    const int64_t piece = (int64_t)chunk + (int64_t)j * n_chunks;
+    const int64_t k0 = piece * piece_keys < n_keys ? piece * piece_keys : n_keys;
+    const int64_t k1 = (k0 + piece_keys < n_keys) ? k0 + piece_keys : n_keys;
+    for (int64_t i0 = k0 + tid; i0 < k1; i0 += 4 * kScanThreads) {
+      pkv_u32x4 v[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int64_t i = i0 + u * kScanThreads;
-      v[u] = (i < k1) ? __builtin_nontemporal_load(base + i) : pkv_u32x4{0u, 0u, 0u, 0u};
+      for (int u = 0; u < 4; ++u) {
+        const int64_t i = i0 + u * kScanThreads;
+        v[u] = (i < k1) ? __builtin_nontemporal_load(base + i) : pkv_u32x4{0u, 0u, 0u, 0u};
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t i = i0 + u * kScanThreads;
+        if (i < k1) {
+          const int c = lut_sum16(l8, v[u]);
+          if (out8) out8[i] = (uint8_t)c;
+          if (out32) out32[i] = c;
+          if (chunk_suf) atomicAdd(&s_hist[c * kHistCopies + copy], 1u);
+        }
+      }
     }
+    if (chunk_suf) {
+      __syncthreads();
+      uint32_t sum = 0;
+      if (tid < 128) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int64_t i = i0 + u * kScanThreads;
-      if (i < k1) {
-        const int c = lut_sum16(l8, v[u]);
-        if (out8) out8[i] = (uint8_t)c;
-        if (out32) out32[i] = c;
-        if (chunk_suf) atomicAdd(&s_hist[c * kHistCopies + copy], 1u);
+        for (int c = 0; c < kHistCopies; ++c) sum += s_hist[tid * kHistCopies + c];
+      }
+      __syncthreads();
+      if (tid < 128) s_hist[tid] = sum;  // compacted histogram in the first 128 words
+      __syncthreads();
+      if (sub_blocks == 1) {
+        pkv_store_suffix_hist(s_hist, &s_hist[128], row_suf + (int64_t)row * 128,
+                              chunk_suf + ((int64_t)row * n_chunks + chunk) * 128);
+      } else {
+        // suffix sums of this piece; thread t owns bin 127 - t and keeps its pieces' values until the last one
+        int incl = 0;
+        if (tid < 128) {
+          incl = pkv_wave_incl_scan((int)s_hist[127 - tid]);
+          if (tid == PKV_WAVE - 1) s_hist[128] = (uint32_t)incl;
+        }
+        __syncthreads();
+        if (tid < 128) {
+          if (tid >= PKV_WAVE) incl += (int)s_hist[128];
+          piece_bins |= (uint64_t)(uint32_t)incl << (16 * j);
+          bin_total += (uint32_t)incl;
+        }
+      }
+      if (j + 1 < sub_blocks) {  // the next piece starts from an empty histogram
+        __syncthreads();
+        for (int i = tid; i < 128 * kHistCopies; i += kScanThreads) s_hist[i] = 0;
+        __syncthreads();
       }
     }
   }
-  if (chunk_suf) {
-    __syncthreads();
-    uint32_t sum = 0;
-    if (tid < 128) {
-#pragma unroll
-      for (int c = 0; c < kHistCopies; ++c) sum += s_hist[tid * kHistCopies + c];
-    }
-    __syncthreads();
-    if (tid < 128) s_hist[tid] = sum;  // compacted histogram in the first 128 words
-    __syncthreads();
-    pkv_store_suffix_hist(s_hist, &s_hist[128], row_suf + (int64_t)row * 128,
-                          chunk_suf + ((int64_t)row * gridDim.x + chunk) * 128);
+  // several pieces: the bin-major table [row][bin][chunk][piece of the chunk] takes the chunk's four values of a bin
+  // as one 8-byte store, and the row totals one addition per bin
+  if (chunk_suf && sub_blocks > 1 && tid < 128) {
+    uint16_t *dst = chunk_suf + ((int64_t)row * 128 + (127 - tid)) * n_chunks * sub_blocks + (int64_t)chunk * sub_blocks;
+    *(uint64_t *)dst = piece_bins;
+    if (bin_total) atomicAdd(&row_suf[(int64_t)row * 128 + 127 - tid], bin_total);
   }
 }
 
@@ -166,7 +206,7 @@ __global__ __launch_bounds__(kScanThreads) void pkv_scan_i32_codes_kernel(const 
 static int launch_scan_impl(const uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t cs_key, int64_t cs_sub, int bs,
                             int n_kv_heads, int64_t n_keys, const uint8_t *lut, uint8_t *cnt_u8,
                             int64_t cnt_u8_stride, int32_t *cnt_i32, uint32_t *row_suf, uint16_t *chunk_suf,
-                            int chunk_keys, hipStream_t s, hipEvent_t ev_start, hipEvent_t ev_stop) {
+                            int chunk_keys, hipStream_t s, hipEvent_t ev_start, hipEvent_t ev_stop, int sub_blocks = 1) {
   PKV_REQUIRE(chunk_keys >= 2048 && chunk_keys % 2048 == 0 && chunk_keys <= 32768,
               "chunk_keys must be a multiple of 2048 in [2048,32768], got %d", chunk_keys);
   const int64_t n_chunks = (n_keys + chunk_keys - 1) / chunk_keys;
@@ -174,10 +214,13 @@ static int launch_scan_impl(const uint8_t *codes, int64_t cs_b, int64_t cs_h, in
   PKV_REQUIRE(pkv_aligned(lut, 4), "lut must be 4-byte aligned");
   dim3 grid((unsigned)n_chunks, (unsigned)(bs * n_kv_heads));
   const bool keymajor = cs_sub == 1 && cs_key == 16 && pkv_aligned(codes, 16) && cs_b % 16 == 0 && cs_h % 16 == 0;
+  PKV_REQUIRE((sub_blocks == 1 || (sub_blocks == 4 && keymajor && chunk_suf)) && chunk_keys % (sub_blocks * 1024) == 0,
+              "a chunk of %d keys cannot be scanned as %d strided pieces", chunk_keys, sub_blocks);
   if (keymajor) {
     // the ext launch ties the two events to this dispatch's own begin/end timestamps
     hipExtLaunchKernelGGL(pkv_scan_keymajor_kernel, grid, dim3(kScanThreads), 0, s, ev_start, ev_stop, 0, codes, cs_b,
-                          cs_h, n_kv_heads, n_keys, lut, cnt_u8, cnt_u8_stride, cnt_i32, row_suf, chunk_suf, chunk_keys);
+                          cs_h, n_kv_heads, n_keys, lut, cnt_u8, cnt_u8_stride, cnt_i32, row_suf, chunk_suf, chunk_keys,
+                          sub_blocks);
     PKV_LAUNCH_CHECK("pkv_scan_keymajor_kernel");
   } else {
     hipExtLaunchKernelGGL(pkv_scan_strided_kernel, grid, dim3(kScanThreads), 0, s, ev_start, ev_stop, 0, codes, cs_b,
@@ -190,9 +233,9 @@ static int launch_scan_impl(const uint8_t *codes, int64_t cs_b, int64_t cs_h, in
 
 int pkv_launch_scan(const uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t cs_key, int64_t cs_sub, int bs,
                     int n_kv_heads, int64_t n_keys, const uint8_t *lut, uint8_t *cnt_u8, int64_t cnt_u8_stride,
-                    int32_t *cnt_i32, uint32_t *row_suf, uint16_t *chunk_suf, int chunk_keys, hipStream_t s) {
+                    int32_t *cnt_i32, uint32_t *row_suf, uint16_t *chunk_suf, int chunk_keys, hipStream_t s, int sub_blocks) {
   return launch_scan_impl(codes, cs_b, cs_h, cs_key, cs_sub, bs, n_kv_heads, n_keys, lut, cnt_u8, cnt_u8_stride, cnt_i32,
-                          row_suf, chunk_suf, chunk_keys, s, nullptr, nullptr);
+                          row_suf, chunk_suf, chunk_keys, s, nullptr, nullptr, sub_blocks);
 }
 
 int pkv_launch_scan_i32_codes(const int32_t *codebook, int rows, int64_t n_keys, const uint8_t *lut, int32_t *cnt,

@@ -73,7 +73,13 @@ PKV_INTERNAL int pkv_launch_query_prep_lut(const void *q, int dtype, int bs, int
 PKV_INTERNAL int pkv_launch_scan(const uint8_t *codes, int64_t cs_b, int64_t cs_h, int64_t cs_key, int64_t cs_sub,
                                  int bs, int n_kv_heads, int64_t n_keys, const uint8_t *lut, uint8_t *cnt_u8,
                                  int64_t cnt_u8_stride, int32_t *cnt_i32, uint32_t *row_suf, uint16_t *chunk_suf,
-                                 int chunk_keys, hipStream_t s);
+                                 int chunk_keys, hipStream_t s, int sub_blocks = 1);
+// Pieces per chunk for the scan -> select + rerank pair of a retrieval: chunks of 8192 keys and more are cut into four
+// pieces spread over the row (where the row's piece tables stay within what the select keeps in LDS), smaller
+// chunks stay whole.
+static inline int pkv_pick_sub_blocks(int chunk_keys, int64_t n_chunks) {
+  return (chunk_keys >= 8192 && n_chunks * 4 <= 512) ? 4 : 1;
+}
 PKV_INTERNAL int pkv_launch_select(const uint8_t *cnt_u8, int64_t cnt_stride, const uint32_t *row_suf,
                                    const uint16_t *chunk_suf, int chunk_keys, int rows, int64_t n_keys, int64_t k,
                                    int64_t *out, hipStream_t s);
@@ -84,7 +90,7 @@ PKV_INTERNAL int pkv_launch_select_rerank(const uint8_t *cnt_u8, int64_t cnt_str
                                           const float *qhat, const float *qnorm, const float *centers, int64_t *cand,
                                           float *scores, hipStream_t s, int64_t extra_off = 0,
                                           float *extra_out = nullptr, uint32_t *range_slots = nullptr,
-                                          int64_t range_row_stride = 0);
+                                          int64_t range_row_stride = 0, int sub_blocks = 1);
 PKV_INTERNAL int pkv_launch_rerank(const int64_t *cand, int bs, int n_kv_heads, int64_t n_cand, int64_t n_keys,
                                    const uint8_t *nib, int64_t ns_b, int64_t ns_h, int64_t ns_key, int64_t ns_sub,
                                    const uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key,
@@ -518,11 +524,12 @@ __device__ __forceinline__ float pkv_rerank_keymajor(const float *__restrict__ s
 }
 
 // Turn a 128-bin histogram in LDS (s_hist) into its suffix sums suf[t] = sum_{t' >= t} hist[t'],
-// store them as the chunk's uint16 suffix histogram and add them to the row's uint32 suffix totals
-// (row_suf may be null).
+// store them as the chunk's uint16 suffix histogram (bin t at chunk_suf[t * bin_stride]) and add them to the
+// row's uint32 suffix totals (row_suf may be null).
 // Called by all threads of a workgroup with >= 128 threads; contains barriers.  s_w0: one LDS word.
 __device__ __forceinline__ void pkv_store_suffix_hist(const uint32_t *s_hist, uint32_t *s_w0,
-                                                      uint32_t *__restrict__ row_suf, uint16_t *__restrict__ chunk_suf) {
+                                                      uint32_t *__restrict__ row_suf, uint16_t *__restrict__ chunk_suf,
+                                                      int64_t bin_stride = 1) {
   const int tid = threadIdx.x;
   int incl = 0;
   if (tid < 128) {  // thread t owns bin 127 - t: an inclusive scan over t is the suffix sum over bins
@@ -532,7 +539,7 @@ __device__ __forceinline__ void pkv_store_suffix_hist(const uint32_t *s_hist, ui
   __syncthreads();
   if (tid < 128) {
     if (tid >= PKV_WAVE) incl += (int)*s_w0;
-    chunk_suf[127 - tid] = (uint16_t)incl;
+    chunk_suf[(int64_t)(127 - tid) * bin_stride] = (uint16_t)incl;  // bin_stride > 1: a bin-major table shared with other chunks
     if (row_suf && incl) atomicAdd(&row_suf[127 - tid], (uint32_t)incl);
   }
 }

@@ -30,6 +30,7 @@ struct WsLayout {
   int64_t cnt_stride;
   int chunk_keys;
   int64_t n_chunks;
+  int sub_blocks;  // pieces per chunk of the scan -> select + rerank pair (one suffix histogram each)
 };
 
 WsLayout layout(int rows, int64_t n_keys, int64_t n_cand, int64_t k) {
@@ -47,7 +48,8 @@ WsLayout layout(int rows, int64_t n_keys, int64_t n_cand, int64_t k) {
   w.qnorm = take((size_t)rows * sizeof(float));
   w.lut = take((size_t)rows * 4096);
   w.cnt = take((size_t)rows * (size_t)w.cnt_stride);
-  w.hist = take((size_t)rows * (size_t)w.n_chunks * 128 * sizeof(uint16_t));
+  w.sub_blocks = pkv_pick_sub_blocks(w.chunk_keys, w.n_chunks);
+  w.hist = take((size_t)rows * (size_t)w.n_chunks * w.sub_blocks * 128 * sizeof(uint16_t));
   w.rowsuf = take((size_t)rows * 128 * sizeof(uint32_t));
   w.cand = take((size_t)rows * (size_t)n_cand * sizeof(int64_t));
   w.scores = take((size_t)rows * (size_t)n_cand * sizeof(float));
@@ -90,7 +92,7 @@ extern "C" int pkv_retrieve_ws_view(void *ws, int rows, int64_t n_keys, int64_t 
   } else if (!strcmp(name, "cnt_u8")) {
     *ptr = base + w.cnt, *bytes = (size_t)rows * (size_t)w.cnt_stride;
   } else if (!strcmp(name, "chunk_suffix_hist")) {
-    *ptr = base + w.hist, *bytes = (size_t)rows * (size_t)w.n_chunks * 256;
+    *ptr = base + w.hist, *bytes = (size_t)rows * (size_t)w.n_chunks * w.sub_blocks * 256;
   } else if (!strcmp(name, "row_suffix_hist")) {
     *ptr = base + w.rowsuf, *bytes = (size_t)rows * 512;
   } else if (!strcmp(name, "cand")) {
@@ -190,13 +192,13 @@ static int retrieve_impl(const pkv_retrieve_args *a, void *ws, size_t ws_bytes, 
                              nullptr, s);
     } else {
       rc = pkv_launch_scan(codes, (int64_t)H * a->cap * 16, a->cap * 16, 16, 1, a->bs, H, a->n_keys, lut, cnt,
-                           w.cnt_stride, nullptr, rowsuf, hist, w.chunk_keys, s);
+                           w.cnt_stride, nullptr, rowsuf, hist, w.chunk_keys, s, w.sub_blocks);
       if (rc) return rc;
       rc = pkv_launch_select_rerank(cnt, w.cnt_stride, rowsuf, hist, w.chunk_keys, a->bs, H, a->n_keys, a->n_cand, nib,
                                     (int64_t)H * a->cap * nk, a->cap * nk, nk, weight, (int64_t)H * a->cap * wk, a->cap * wk,
                                     wk, qhat, qnorm, a->centers, cand, scores, s, a->record_word_offset,
                                     a->record_word_offset > 0 ? (float *)(base + w.cand_extra) : nullptr,
-                                    range_slots, range_stride);
+                                    range_slots, range_stride, w.sub_blocks);
     }
   }
   if (rc) return rc;

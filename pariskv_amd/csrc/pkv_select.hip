@@ -196,6 +196,177 @@ __global__ __launch_bounds__(kSelThreads) void pkv_select_rerank_kernel(
   }
 }
 
+// The same for chunks that the collision scan cut into S strided pieces (S even): workgroup c owns pieces
+// c, c + n_chunks, ... of piece_keys keys each (pieces numbered in key order), piece_suf holds one suffix histogram per
+// piece as a bin-major table [row][bin][chunk][piece of the chunk], and the output positions follow from the prefixes
+// over the pieces in key order.  Where the candidates bunch along the row (keys whose
+// mean drifts: bands of the zone hold a multiple of the average) a workgroup that owned one contiguous chunk would
+// score up to twice the average number of candidates and the launch would last as long as that workgroup; pieces a
+// quarter of the row apart average the bands out (8 rows x 1M keys, mean turning 2 degrees per 1K keys: most
+// candidates of one workgroup 851 -> 496 for an average of 410).  The candidate list and every score are the same as
+// with whole chunks: positions depend on the keys alone.
+// Two pieces per pass (threads [0,128) and [128,256) when piece_keys = 2048): the block scan ranks both at once.
+constexpr int kSelMaxPieces = 512;
+
+__global__ __launch_bounds__(kSelThreads) void pkv_select_rerank_pieces_kernel(
+    const uint8_t *__restrict__ cnt, int64_t cnt_stride, const uint32_t *__restrict__ row_suf,
+    const uint16_t *__restrict__ piece_suf, int piece_keys, int pieces_per_chunk, int n_kv_heads, int64_t n_keys, int64_t k,
+    const uint8_t *__restrict__ nib, int64_t ns_b, int64_t ns_h, int ns_key, const uint16_t *__restrict__ weight,
+    int64_t ws_b, int64_t ws_h, int ws_key, const float *__restrict__ qhat, const float *__restrict__ qnorm,
+    const float *__restrict__ centers, int64_t *__restrict__ out, float *__restrict__ scores, int extra_off,
+    float *__restrict__ extra_out, uint32_t *__restrict__ range_slots, int64_t range_row_stride) {
+  const int row = blockIdx.y;
+  const int chunk = blockIdx.x;
+  const int n_chunks = gridDim.x;
+  const int n_pieces = n_chunks * pieces_per_chunk;
+  const int tid = threadIdx.x;
+  const int b = row / n_kv_heads, h = row % n_kv_heads;
+  uint32_t smax = 0u, smin = 0xffffffffu;
+
+  __shared__ int s_scan[2][kSelThreads / PKV_WAVE];
+  __shared__ float s_prod[128 * 16];
+  __shared__ uint16_t s_list_key[kSelKeysPerIter];  // offset of the key inside the pass's two pieces (second piece: + piece_keys)
+  __shared__ uint32_t s_pg[kSelMaxPieces + 1], s_pe[kSelMaxPieces + 1];  // keys above / at the threshold in the pieces before
+  __shared__ uint32_t s_rs[129];
+  __shared__ uint32_t s_theta, s_ngt;
+
+  const uint8_t *crow = cnt + (int64_t)row * cnt_stride;
+  const pkv_u32x4 zero4 = {0u, 0u, 0u, 0u};
+  const uint32_t rs_mine = tid < 128 ? row_suf[(int64_t)row * 128 + tid] : 0u;
+  // thread t of a pass: half hh = t / (threads per piece), 16 keys at offset (t % threads per piece) * 16 of its piece
+  const int tpp = piece_keys / kSelKeysPerThread;  // threads per piece; 2 * tpp <= 256
+  const int hh = tid / tpp, tl = tid % tpp;
+  const int n_pass = pieces_per_chunk / 2;
+  // counts of the first pass, requested before the threshold is known
+  auto piece_of = [&](int pass, int half) { return chunk + (pass + half * n_pass) * n_chunks; };  // halves half a chunk's pieces apart
+  auto load_counts = [&](int pass) {
+    if (hh >= 2) return zero4;
+    const int64_t j0 = (int64_t)piece_of(pass, hh) * piece_keys + (int64_t)tl * kSelKeysPerThread;
+    return j0 < n_keys ? *(const pkv_u32x4 *)(crow + j0) : zero4;
+  };
+  pkv_u32x4 w = load_counts(0);
+  const float qn = qnorm[row];
+  pkv_build_prod_table<kSelThreads>(s_prod, qhat + (int64_t)row * 128, centers);
+
+  // threshold, then the two columns it names for every piece of the row and their prefixes
+  if (tid < 128) s_rs[tid] = rs_mine;
+  if (tid == 128) s_rs[128] = 0, s_theta = 0, s_ngt = 0;
+  __syncthreads();
+  if (tid < 128 && (int64_t)s_rs[tid] >= k && (int64_t)s_rs[tid + 1] < k) s_theta = (uint32_t)tid, s_ngt = s_rs[tid + 1];
+  __syncthreads();
+  const uint32_t theta = s_theta;
+  const int64_t n_gt_row = s_ngt;
+  {
+    // bin-major table [bin][chunk][piece of the chunk]: entries 2t and 2t + 1 of a bin are one 32-bit word; they are
+    // put into key order (piece = chunk + j * n_chunks) through LDS before the prefix sums
+    const uint32_t *cs = (const uint32_t *)(piece_suf + (int64_t)row * n_pieces * 128);
+    if (2 * tid < n_pieces) {
+      const uint32_t ge2 = cs[((int64_t)theta * n_pieces) / 2 + tid];
+      const uint32_t g2 = theta < 127 ? cs[((int64_t)(theta + 1) * n_pieces) / 2 + tid] : 0u;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int idx = 2 * tid + u, c = idx / pieces_per_chunk, jj = idx % pieces_per_chunk;
+        const uint32_t gv = u ? g2 >> 16 : g2 & 0xffffu, gev = u ? ge2 >> 16 : ge2 & 0xffffu;
+        s_pg[c + jj * n_chunks] = gv;
+        s_pe[c + jj * n_chunks] = gev - gv;
+      }
+    }
+    __syncthreads();
+    uint32_t g[2] = {0u, 0u}, e[2] = {0u, 0u};
+    if (2 * tid < n_pieces) g[0] = s_pg[2 * tid], g[1] = s_pg[2 * tid + 1], e[0] = s_pe[2 * tid], e[1] = s_pe[2 * tid + 1];
+    int tot_g, tot_e;
+    const uint32_t xg = (uint32_t)pkv_block_excl_scan<kSelThreads>((int)(g[0] + g[1]), s_scan[0], tot_g);
+    const uint32_t xe = (uint32_t)pkv_block_excl_scan<kSelThreads>((int)(e[0] + e[1]), s_scan[1], tot_e);
+    s_pg[2 * tid] = xg, s_pg[2 * tid + 1] = xg + g[0];
+    s_pe[2 * tid] = xe, s_pe[2 * tid + 1] = xe + e[0];
+    if (tid == 0) s_pg[kSelMaxPieces] = (uint32_t)tot_g, s_pe[kSelMaxPieces] = (uint32_t)tot_e;  // entry n_pieces when that is the maximum
+  }
+  __syncthreads();
+  int64_t *orow = out + (int64_t)row * k;
+  float *srow = scores + (int64_t)row * k;
+  const uint8_t *nrow = nib + (int64_t)b * ns_b + (int64_t)h * ns_h;
+  const uint16_t *wrow = weight + (int64_t)b * ws_b + (int64_t)h * ws_h;
+
+  for (int pass = 0; pass < n_pass; ++pass) {
+    const int p0 = piece_of(pass, 0), p1 = piece_of(pass, 1);
+    const int64_t j0 = (int64_t)(hh ? p1 : p0) * piece_keys + (int64_t)tl * kSelKeysPerThread;
+    const int64_t piece_end = ((int64_t)(hh ? p1 : p0) + 1) * piece_keys < n_keys ? ((int64_t)(hh ? p1 : p0) + 1) * piece_keys : n_keys;
+    uint32_t gt[4], eq[4];
+    count_masks16(w, theta, hh < 2 ? piece_end - j0 : 0, gt, eq);
+    if (pass + 1 < n_pass) w = load_counts(pass + 1);
+    const int packed = popc4(gt) | (popc4(eq) << 16);
+    int total;
+    const int excl = pkv_block_excl_scan<kSelThreads>(packed, s_scan[pass & 1], total);
+    // the piece tables already hold what the scan would tell: keys above / at the threshold in each of the two pieces
+    const int n_g0 = (int)(s_pg[p0 + 1] - s_pg[p0]), n_g1 = (int)(s_pg[p1 + 1] - s_pg[p1]);
+    const int n_e0 = (int)(s_pe[p0 + 1] - s_pe[p0]);
+    const int64_t room0 = k - n_gt_row - (int64_t)s_pe[p0], room1 = k - n_gt_row - (int64_t)s_pe[p1];
+    const int u_e0 = (int)(room0 <= 0 ? 0 : (room0 < n_e0 ? room0 : n_e0));                  // keys at the threshold that find room
+    const int n_e1 = (int)(s_pe[p1 + 1] - s_pe[p1]);
+    const int u_e1 = (int)(room1 <= 0 ? 0 : (room1 < n_e1 ? room1 : n_e1));
+    const int n_g = n_g0 + n_g1;
+    // list of the pass: [above, piece 0][above, piece 1][at, piece 0, first u_e0][at, piece 1, first u_e1]
+    int lg = excl & 0xffff;                                              // ranks both halves in thread order = this layout
+    int re = (excl >> 16) - (hh ? n_e0 : 0);                             // rank among the keys at the threshold of the own piece
+    const int e_used = hh ? u_e1 : u_e0, e_base = n_g + (hh ? u_e0 : 0);
+    const uint32_t off0 = (uint32_t)(hh * piece_keys + tl * kSelKeysPerThread);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      uint32_t g = gt[d], e = eq[d];
+      while (g) {
+        const int bit = __ffs((int)g) - 1;
+        g &= g - 1;
+        s_list_key[lg++] = (uint16_t)(off0 + 4 * d + (bit >> 3));
+      }
+      while (e) {
+        const int bit = __ffs((int)e) - 1;
+        e &= e - 1;
+        if (re < e_used) s_list_key[e_base + re] = (uint16_t)(off0 + 4 * d + (bit >> 3));
+        ++re;
+      }
+    }
+    const int n_use = n_g + u_e0 + u_e1;
+    const int64_t pg0 = s_pg[p0], pg1 = s_pg[p1], pe0 = n_gt_row + s_pe[p0], pe1 = n_gt_row + s_pe[p1];
+    __syncthreads();
+#pragma unroll 1
+    for (int j = tid; j < n_use; j += kSelThreads) {
+      const int64_t pos = j < n_g0 ? pg0 + j : (j < n_g ? pg1 + (j - n_g0) : (j < n_g + u_e0 ? pe0 + (j - n_g) : pe1 + (j - n_g - u_e0)));
+      const uint32_t off = s_list_key[j];
+      const int64_t key = (off < (uint32_t)piece_keys ? (int64_t)p0 * piece_keys : (int64_t)(p1 - 1) * piece_keys) + off;
+      orow[pos] = key;
+      const float sc = pkv_rerank_keymajor(s_prod, (const pkv_u32x4 *)(nrow + key * ns_key), (const pkv_u32x4 *)(wrow + key * ws_key), qn);
+      srow[pos] = sc;
+      const uint32_t o = pkv_ordered_u32(sc);
+      smax = o > smax ? o : smax;
+      smin = o < smin ? o : smin;
+      if (extra_out) extra_out[(int64_t)row * k + pos] = *(const float *)(nrow + key * ns_key + extra_off);
+    }
+    __syncthreads();  // the list is rewritten by the next pass
+  }
+  if (range_slots) {
+#pragma unroll
+    for (int x = 1; x < PKV_WAVE; x <<= 1) {
+      const uint32_t a = (uint32_t)__shfl_xor((int)smax, x, PKV_WAVE), c = (uint32_t)__shfl_xor((int)smin, x, PKV_WAVE);
+      smax = a > smax ? a : smax;
+      smin = c < smin ? c : smin;
+    }
+    if (pkv_lane() == 0) s_scan[0][tid / PKV_WAVE] = (int)smax, s_scan[1][tid / PKV_WAVE] = (int)smin;
+    __syncthreads();
+    if (tid == 0) {
+      for (int wv = 1; wv < kSelThreads / PKV_WAVE; ++wv) {
+        const uint32_t a = (uint32_t)s_scan[0][wv], c = (uint32_t)s_scan[1][wv];
+        smax = a > smax ? a : smax;
+        smin = c < smin ? c : smin;
+      }
+      if (smax >= smin) {
+        uint32_t *slot = range_slots + (int64_t)row * range_row_stride + 2 * (chunk % kWideRangeSlots);
+        atomicMax(&slot[0], smax);
+        atomicMax(&slot[1], ~smin);
+      }
+    }
+  }
+}
+
 // out[row][i] = i (i < len) else 0: the reference's `length <= k` branch
 // (radix_topk.cu:154-159).
 __global__ void pkv_identity_fill_kernel(int64_t *__restrict__ out, int64_t len, int64_t k, int rows) {
@@ -1990,7 +2161,7 @@ int pkv_launch_select_rerank(const uint8_t *cnt_u8, int64_t cnt_stride, const ui
                              int64_t ns_key, const uint16_t *weight, int64_t ws_b, int64_t ws_h, int64_t ws_key,
                              const float *qhat, const float *qnorm, const float *centers, int64_t *cand, float *scores,
                              hipStream_t s, int64_t extra_off, float *extra_out, uint32_t *range_slots,
-                             int64_t range_row_stride) {
+                             int64_t range_row_stride, int sub_blocks) {
   PKV_REQUIRE(!extra_out || (extra_off >= 0 && extra_off % 4 == 0 && extra_off + 4 <= ns_key),
               "the extra word must lie inside the key's record (offset %lld, record %lld bytes)", (long long)extra_off,
               (long long)ns_key);
@@ -2004,6 +2175,19 @@ int pkv_launch_select_rerank(const uint8_t *cnt_u8, int64_t cnt_stride, const ui
               "key-major nibbles / weights must be 16-byte aligned, 64 bytes / 16 weights per key");
   const int64_t n_chunks = (n_keys + chunk_keys - 1) / chunk_keys;
   dim3 grid((unsigned)n_chunks, (unsigned)(bs * n_kv_heads));
+  if (sub_blocks > 1) {
+    const int piece_keys = chunk_keys / sub_blocks;
+    PKV_REQUIRE(sub_blocks % 2 == 0 && chunk_keys % sub_blocks == 0 && piece_keys % 16 == 0 && 2 * piece_keys <= kSelKeysPerIter &&
+                    n_chunks * sub_blocks <= kSelMaxPieces,
+                "select + rerank: %d pieces of a %d-key chunk, %lld chunks per row not supported", sub_blocks, chunk_keys,
+                (long long)n_chunks);
+    hipLaunchKernelGGL(pkv_select_rerank_pieces_kernel, grid, dim3(kSelThreads), 0, s, cnt_u8, cnt_stride, row_suf, chunk_suf,
+                       piece_keys, sub_blocks, n_kv_heads, n_keys, k, nib, ns_b, ns_h, (int)ns_key, weight, ws_b, ws_h,
+                       (int)ws_key, qhat, qnorm, centers, cand, scores, (int)extra_off, extra_out, range_slots,
+                       range_row_stride);
+    PKV_LAUNCH_CHECK("pkv_select_rerank_pieces_kernel");
+    return PKV_OK;
+  }
   hipLaunchKernelGGL(pkv_select_rerank_kernel, grid, dim3(kSelThreads), 0, s, cnt_u8, cnt_stride, row_suf, chunk_suf,
                      chunk_keys,
                      n_kv_heads, n_keys, k, nib, ns_b, ns_h, (int)ns_key, weight, ws_b, ws_h, (int)ws_key, qhat, qnorm,

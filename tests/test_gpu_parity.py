@@ -673,6 +673,57 @@ def test_one_launch_plan_equals_three_launches(ops, request, wl_name):
         assert np.array_equal(ids[b, h].cpu().numpy(), W.oracle_stages(w, r)["final"])
 
 
+def test_retrieve_large_rows_strided_pieces(ops):
+    """Rows long enough for 8192-key chunks (8 rows x 600 000 keys): the collision scan and the select + rerank then
+    work on four pieces per chunk spread over the row.  Keys with a drifting mean (candidates bunch in bands) and a
+    ragged last chunk; candidate list, scores and final ids of three rows against the oracle, all rows against the
+    one-launch plan (whole chunks)."""
+    from pariskv_amd import _lib
+
+    bs, H, G, N, C, K = 1, 8, 4, 600_000, 30_000, 512
+    _say(f"strided pieces: N={N} C={C} K={K}")
+    assert ops.pick_chunk_keys(bs * H, N) == 8192
+    g = torch.Generator(device=DEV).manual_seed(11)
+    keys = torch.randn(bs, H, N, 128, generator=g, device=DEV)
+    keys[..., [7, 31, 64, 101]] *= 10.0
+    ang = torch.arange(N, device=DEV, dtype=torch.float32) * (5.0 / 1000.0) * (math.pi / 180.0)
+    keys[..., 0] += 2.0 * torch.cos(ang)
+    keys[..., 1] += 2.0 * torch.sin(ang)
+    keys = keys.to(torch.bfloat16)
+    q = (keys[:, :, -2048:].float().mean(dim=2, keepdim=True) + 0.5 * torch.randn(bs, H, G, 128, generator=g, device=DEV))
+    q = q.to(torch.bfloat16).view(bs, 1, H * G, 128).contiguous()
+    signs, centers = ops.srht_signs(DEV), ops.mag_centers(DEV)
+    codes_km, nib_km, w_km, cb, k4, kw = ops.alloc_keymajor(bs, H, N, DEV)
+    cc = torch.zeros(bs, H, 16, 256, dtype=torch.int32, device=DEV)
+    ops.encode_append(keys, signs, cb, k4, kw, cc)
+    tiers = O.tier_counts(N, 0.2)
+    plan = ops.RetrievePlan(bs, H, G, N, DEV, N, C, K)
+    args = (q, signs, centers, cc, codes_km, nib_km, w_km, 0, N, tiers, C, K)
+    sc = torch.empty(bs, H, K, device=DEV)
+    ids = plan.run(*args, out_scores=sc).clone()
+    cand = plan.view("cand", N, C, K, torch.int64).view(H, C).clone()
+    csc = plan.view("scores", N, C, K, torch.float32).view(H, C).clone()
+    per_chunk = torch.bincount(cand[0] // 8192, minlength=(N + 8191) // 8192)
+    assert int(per_chunk.max()) > 1.5 * C / per_chunk.numel()  # the data does bunch
+    plan.launch_plan = _lib.PLAN_ONE_LAUNCH
+    ids1 = plan.run(*args)
+    torch.cuda.synchronize()
+    assert int(plan.view("handover_status", N, C, K, torch.int32)[0]) == 0
+    assert torch.equal(ids, ids1)
+    assert torch.equal(plan.view("cand", N, C, K, torch.int64).view(H, C), cand)
+    assert torch.equal(plan.view("scores", N, C, K, torch.float32).view(H, C), csc)
+    sg = signs.cpu().numpy()
+    for r in (0, 4, 7):
+        qh, qn = O.query_prep(q.view(bs, H, G, 128)[0, r].float().cpu().numpy(), sg, O.BF16)
+        lut = O.tier_lut(O.rank_centroids(qh, O.BF16), cc[0, r].cpu().numpy(), tiers)
+        cand_ref, _ = O.select_candidates(O.collision_count(codes_km[0, r].cpu().numpy(), lut), C)
+        assert np.array_equal(cand[r].cpu().numpy(), cand_ref), f"candidate list of row {r}"
+        sc_ref = O.rerank(cand_ref, nib_km[0, r].cpu().numpy().reshape(N, 16, 4), w_km[0, r].float().cpu().numpy(), qh, qn)
+        np.testing.assert_allclose(csc[r].cpu().numpy(), sc_ref, rtol=1e-5, atol=1e-5 * np.abs(sc_ref).max())
+        final, _ = O.topk_f32(sc_ref, cand_ref, K)
+        assert np.array_equal(ids[0, r].cpu().numpy(), final), f"final ids of row {r}"
+
+
 def test_retrieve_subrange_and_candidates_equal_keys(ops, wl_small_bf16):
     """Retrieval zone = [key0, key0+n) of a larger capacity; and C == N (identity candidates)."""
     w = wl_small_bf16
