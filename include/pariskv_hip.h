@@ -519,7 +519,11 @@ int pkv_retrieve(const pkv_retrieve_args *args, void *ws, size_t ws_bytes, void 
  * GPU, held until the process ends.  The call allocates and frees nothing.
  * No counterpart in the reference (its kernels allocate their outputs and
  * temporaries with torch::zeros on every call).
- *   - The GPU of `stream` must be the calling thread's current device.
+ *   - The GPU of `stream` must be the calling thread's current device (checked: PKV_EINVAL otherwise).
+ *   - The first use of the array on a GPU looks its address up (hipGetSymbolAddress), which may make the HIP
+ *     runtime load the library's code object there, and that allocates.  pkv_retrieve_noalloc_prepare() does the
+ *     look-up for the current device ahead of time: call it once per GPU during set-up (before a graph capture,
+ *     before the serving loop); afterwards pkv_retrieve_noalloc only reads the cached address.
  *   - Shapes whose workspace (pkv_retrieve_ws_bytes) exceeds the array are
  *     rejected with PKV_ENOMEM and a message naming both sizes;
  *     pkv_retrieve_noalloc_max_bytes() returns the array's size.
@@ -531,6 +535,7 @@ int pkv_retrieve(const pkv_retrieve_args *args, void *ws, size_t ws_bytes, void 
  *     two threads) race on it: serialise them, or use pkv_retrieve. */
 #define PKV_NOALLOC_SCRATCH_BYTES (32u << 20)
 size_t pkv_retrieve_noalloc_max_bytes(void);
+int pkv_retrieve_noalloc_prepare(void);
 int pkv_retrieve_noalloc(const pkv_retrieve_args *args, void *stream);
 
 /* The whole decode step of one layer from one host call: pkv_retrieve (with its

@@ -123,6 +123,7 @@ PROTOTYPES = {
     "pkv_retrieve_ws_bytes": (_sz, [_i, _i64, _i64, _i64]),
     "pkv_retrieve": (_i, [C.POINTER(RetrieveArgs), _vp, _sz, _vp]),
     "pkv_retrieve_noalloc_max_bytes": (_sz, []),
+    "pkv_retrieve_noalloc_prepare": (_i, []),
     "pkv_retrieve_noalloc": (_i, [C.POINTER(RetrieveArgs), _vp]),
     "pkv_decode_step": (_i, [C.POINTER(RetrieveArgs), _vp, _sz, C.POINTER(AttnArgs), _vp]),
     "pkv_adaptive_decode_step": (_i, [C.POINTER(RetrieveArgs), _vp, _sz, C.POINTER(AdaptiveArgs), C.POINTER(AttnArgs), _vp]),

@@ -43,7 +43,8 @@ def adaptive_topk_cuda(query_avg: torch.Tensor, sink_local_keys: torch.Tensor, s
     assert 0.0 < threshold <= 1.0, f"threshold must be in (0, 1], got {threshold}"
     assert topk_cap > 0, f"topk_cap must be > 0, got {topk_cap}"
     assert attn_scale > 0, f"attn_scale must be > 0, got {attn_scale}"
-    # exact logits of the dense tokens: a [sl,128] x [128] product per head, left to the BLAS as in the reference (:383-386)
-    sl_logits = torch.einsum("bhd,bhkd->bhk", query_avg, sink_local_keys).to(torch.float32) * attn_scale
-    return ops.adaptive_topk(sl_logits.contiguous(), sl_vnorm, cand_scores, float(attn_scale), cand_indices, float(threshold),
+    # logits of the dense tokens (reference :383-386: einsum + cast + scale, four launches): one launch of
+    # pkv_dense_logits; a [bs,H,D] mean query is a query group of one head
+    sl_logits = ops.dense_logits(query_avg, sink_local_keys, sl_len, float(attn_scale))
+    return ops.adaptive_topk(sl_logits, sl_vnorm, cand_scores, float(attn_scale), cand_indices, float(threshold),
                              int(K_out), cand_vnorm=cand_vnorm)

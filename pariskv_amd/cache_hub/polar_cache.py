@@ -330,6 +330,8 @@ class polar_cache(KV_Cache):
     def decode_update_kv_cache(self, key_states, value_states, layer_idx):
         """Append one token ([bs,1,Hkv,D]); refresh the index when this layer's update buffer fills (:827-881)."""
         z = self._zones[layer_idx]
+        if self.enable_offload and (self._prefill_stage[0] is not None or self._prefill_stage[1] is not None):
+            self.release_prefill_staging()  # prefill is over: its staging pairs (two layers of K/V) go back to the allocator
         slot = z.append_slot()
         if key_states.dtype != self.dtype or value_states.dtype != self.dtype:
             key_states, value_states = key_states.to(self.dtype), value_states.to(self.dtype)

@@ -258,6 +258,11 @@ int scratch_for_current_device(void **out) {
 
 extern "C" size_t pkv_retrieve_noalloc_max_bytes(void) { return (size_t)PKV_NOALLOC_SCRATCH_BYTES; }
 
+extern "C" int pkv_retrieve_noalloc_prepare(void) {
+  void *ws = nullptr;
+  return scratch_for_current_device(&ws);
+}
+
 extern "C" int pkv_retrieve_noalloc(const pkv_retrieve_args *a, void *stream) {
   PKV_REQUIRE(a != nullptr, "pkv_retrieve_noalloc: null args");
   PKV_REQUIRE(a->out_ids != nullptr,
@@ -274,6 +279,16 @@ extern "C" int pkv_retrieve_noalloc(const pkv_retrieve_args *a, void *stream) {
                   need, (size_t)PKV_NOALLOC_SCRATCH_BYTES, rows, (long long)a->n_keys, (long long)a->n_cand,
                   (long long)a->k);
     return PKV_ENOMEM;
+  }
+  // the scratch array is the current device's: a stream of another GPU would be handed the wrong copy's address
+  int cur = -1;
+  hipDevice_t sdev = -1;
+  PKV_HIP(hipGetDevice(&cur));
+  if (stream != nullptr && hipStreamGetDevice((hipStream_t)stream, &sdev) == hipSuccess) {
+    PKV_REQUIRE((int)sdev == cur, "pkv_retrieve_noalloc: the stream belongs to device %d, the calling thread's current device is %d",
+                (int)sdev, cur);
+  } else {
+    (void)hipGetLastError();
   }
   void *ws = nullptr;
   const int rc = scratch_for_current_device(&ws);

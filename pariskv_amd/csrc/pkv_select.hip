@@ -36,8 +36,16 @@ __global__ __launch_bounds__(kSelThreads) void pkv_select_kernel(const uint8_t *
   const int64_t chunk_end = (chunk_begin + chunk_keys < n_keys) ? chunk_begin + chunk_keys : n_keys;
   const pkv_u32x4 zero4 = {0u, 0u, 0u, 0u};
   int64_t i0 = chunk_begin + (int64_t)tid * kSelKeysPerThread;
-  const uint32_t rs_mine = tid < 128 ? row_suf[(int64_t)row * 128 + tid] : 0u;
   pkv_u32x4 w = i0 < chunk_end ? *(const pkv_u32x4 *)(crow + i0) : zero4;  // padded rows: always in bounds
+  uint32_t rs_mine = 0u;
+  if (tid < 128) {
+    if (row_suf) {
+      rs_mine = row_suf[(int64_t)row * 128 + tid];
+    } else {  // no row totals kept: add the chunks' suffix histograms up (a producer without atomics, nothing to clear)
+      const uint16_t *cs = chunk_suf + (int64_t)row * gridDim.x * 128 + tid;
+      for (int c = 0; c < (int)gridDim.x; ++c) rs_mine += cs[(int64_t)c * 128];
+    }
+  }
 
   uint32_t theta;
   int64_t base_gt, base_eq;
@@ -395,7 +403,7 @@ __global__ __launch_bounds__(256) void pkv_counts_to_u8_kernel(const int32_t *__
     atomicAdd(&s_hist[v], 1u);
   }
   __syncthreads();
-  pkv_store_suffix_hist(s_hist, &s_w0, row_suf + (int64_t)row * 128,
+  pkv_store_suffix_hist(s_hist, &s_w0, row_suf ? row_suf + (int64_t)row * 128 : nullptr,
                         chunk_suf + ((int64_t)row * gridDim.x + chunk) * 128);
 }
 
@@ -717,7 +725,11 @@ __device__ __forceinline__ bool linear_bins(const uint64_t (&v)[EIN], uint32_t k
                                             const uint32_t *range = nullptr) {
   const int tid = threadIdx.x, lane = pkv_lane();
   for (int i = tid; i < 2 * kLinBins; i += kTopkThreads) s_hist[i] = 0;
-  if (tid == 0) s_bcast[0] = 0u, s_bcast[1] = 0xffffffffu, s_bcast[5] = 0u, s_bcast[6] = 0u;
+  // [2..4]: threshold bin, keys needed from it, keys in it.  They are set below only if some bin reaches k; a row
+  // with fewer than k keys leaves "keys in the threshold bin" at its all-ones start and the caller falls back.
+  if (tid == 0)
+    s_bcast[0] = 0u, s_bcast[1] = 0xffffffffu, s_bcast[2] = 0u, s_bcast[3] = 0u, s_bcast[4] = 0xffffffffu, s_bcast[5] = 0u,
+    s_bcast[6] = 0u;
   __syncthreads();
   uint32_t mx = 0u, mn = 0xffffffffu;
   if (range) {
@@ -2245,13 +2257,13 @@ extern "C" int pkv_bucket_topk(const int32_t *x, int64_t x_stride, int rows, int
   uint16_t *hist = (uint16_t *)((char *)ws + oh);
   uint32_t *row_suf = (uint32_t *)((char *)ws + orow);
   const int64_t n_chunks = (len + ck - 1) / ck;
-  hipLaunchKernelGGL(pkv_zero_u32_kernel, dim3((unsigned)((rows * 128 + 255) / 256)), dim3(256), 0, s, row_suf,
-                     (int64_t)rows * 128);
-  PKV_LAUNCH_CHECK("pkv_zero_u32_kernel");
+  // two launches: counts -> clamped bytes + chunk suffix histograms, then the select, which adds the chunks'
+  // histograms up for the row totals itself (no atomics, so nothing has to be cleared first)
+  (void)row_suf;
   hipLaunchKernelGGL(pkv_counts_to_u8_kernel, dim3((unsigned)n_chunks, (unsigned)rows), dim3(256), 0, s, x, x_stride,
-                     len, cnt, cs, row_suf, hist, ck);
+                     len, cnt, cs, (uint32_t *)nullptr, hist, ck);
   PKV_LAUNCH_CHECK("pkv_counts_to_u8_kernel");
-  return pkv_launch_select(cnt, cs, row_suf, hist, ck, rows, len, k, out, s);
+  return pkv_launch_select(cnt, cs, nullptr, hist, ck, rows, len, k, out, s);
 }
 
 // Wide rows (len > 8192): control blocks, list A [rows][k], list B [rows][len].

@@ -50,6 +50,7 @@ def test_noalloc_equals_retrieve_on_two_calls_in_a_row():
 
     print("no-alloc: cfg2-sized call, then a smaller ragged one", flush=True)
     assert _lib.lib().pkv_retrieve_noalloc_max_bytes() == 32 << 20
+    assert _lib.lib().pkv_retrieve_noalloc_prepare() == 0  # the address look-up a caller does during set-up
     big = W.cfg2()                                                                    # 8 rows x 32768 keys, C 2048, K 512
     small = W.make_workload("small", 2, 2, 4, 5000 + 37, 333, 100, O.BF16, 0.5, seed0=5)  # 4 rows, ragged length
     db, ds = W.to_device(big, DEV, torch), W.to_device(small, DEV, torch)
