@@ -505,12 +505,28 @@ typedef struct pkv_retrieve_args {
   /* nonzero: the per-key vote counts need not be left in the workspace segment "cnt_u8" (the one-launch plan then
    * keeps them on chip). */
   int skip_vote_counts;
+  /* nonzero: the workspace already holds this step's rotated query, its norm and the vote table, written by
+   * pkv_qk_norm_rope_table for the queries `q` points to with these cluster counts and tier counts, and the words
+   * the query-prep launch clears for the later stages are cleared: that launch is left out (PKV_PLAN_SEPARATE only). */
+  int table_ready;
 } pkv_retrieve_args;
 #define PKV_PLAN_SEPARATE 0
 #define PKV_PLAN_ONE_LAUNCH 1
 
 size_t pkv_retrieve_ws_bytes(int rows, int64_t n_keys, int64_t n_cand, int64_t k);
 int pkv_retrieve(const pkv_retrieve_args *args, void *ws, size_t ws_bytes, void *stream);
+
+/* pkv_qk_norm_rope with the query side of the layer's retrieval in the same launch: besides q_out / k_out (as
+ * pkv_qk_norm_rope writes them) the launch leaves in `ws` what the query-prep launch of pkv_retrieve(args, ws) would
+ * compute from q_out - group mean, SRHT rotation, centroid ranking, vote table (cache_hub/polar_cache.py:1027-1031,
+ * 905-922, 1216-1222) - so that the retrieval that follows, called with args->table_ready = 1 and args->q = q_out,
+ * starts at the collision scan.  In the reference's decode step the two sit in different modules (model_hub/qwen.py:
+ * 327-498 and cache_hub/polar_cache.py:1126-1162) with the cache update between them; nothing between them touches
+ * the queries, the cluster sizes or the tier counts unless the update refreshes the index, after which the caller
+ * must not set table_ready.  bf16 only; args->q is not read; n_q_heads = args->n_kv_heads * args->group. */
+int pkv_qk_norm_rope_table(const void *qkv, int64_t stride_b, int n_q_heads, const void *q_weight, const void *k_weight,
+                           float eps, const void *cos_row, const void *sin_row, void *q_out, void *k_out,
+                           const pkv_retrieve_args *args, void *ws, size_t ws_bytes, void *stream);
 
 /* pkv_retrieve for callers that cannot allocate device memory (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc): the

@@ -50,7 +50,7 @@ class RetrieveArgs(C.Structure):
         ("src_len", _i64), ("idx_offset", _i64),
         ("dst_k", _vp), ("dst_v", _vp), ("dst_len", _i64), ("dst_row0", _i64),
         ("row_bytes", _i), ("any_order", _i), ("nib_key_stride", _i64), ("weight_key_stride", _i64),
-        ("record_word_offset", _i64), ("launch_plan", _i), ("skip_vote_counts", _i),
+        ("record_word_offset", _i64), ("launch_plan", _i), ("skip_vote_counts", _i), ("table_ready", _i),
     ]
 
 
@@ -122,6 +122,7 @@ PROTOTYPES = {
     "pkv_silu_mul": (_i, [_vp, _i64, _i, _i, _vp, _vp]),
     "pkv_retrieve_ws_bytes": (_sz, [_i, _i64, _i64, _i64]),
     "pkv_retrieve": (_i, [C.POINTER(RetrieveArgs), _vp, _sz, _vp]),
+    "pkv_qk_norm_rope_table": (_i, [_vp, _i64, _i, _vp, _vp, C.c_float, _vp, _vp, _vp, _vp, C.POINTER(RetrieveArgs), _vp, _sz, _vp]),
     "pkv_retrieve_noalloc_max_bytes": (_sz, []),
     "pkv_retrieve_noalloc_prepare": (_i, []),
     "pkv_retrieve_noalloc": (_i, [C.POINTER(RetrieveArgs), _vp]),

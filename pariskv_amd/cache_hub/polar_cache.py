@@ -426,6 +426,25 @@ class polar_cache(KV_Cache):
         tiers = [int(math.ceil(n_keys * coll_ratio * r)) for r in ops.TIER_RATIOS]  # :1221-1222
         return n_keys, n_cand, k, tiers
 
+    def query_table_target(self, layer_idx):
+        """The bound step whose retrieval the next ``compute`` of this layer will launch, for callers that build the
+        retrieval's vote table in the launch that produces the queries (``ops.qk_norm_rope(table_for=...)``, called
+        before ``decode_update_kv_cache``); None where that launch would not use it: no step bound yet for the
+        current index, the coming token refreshes the index (cluster sizes and tier counts change), or the step
+        will take the dense branch."""
+        z = self._zones[layer_idx]
+        step = self._bound_step_of(layer_idx)
+        if step is None or self.dtype != torch.bfloat16:
+            return None
+        n_keys = self.cpu_valid_end[layer_idx] if self._layer_offload[layer_idx] else z.encoded
+        if step[0] != n_keys or z.next_append_refreshes():
+            return None
+        min_total = max(self.FULL_ATTENTION_THRESHOLD, self.sink_size + self.local_size + self.final_topk * 2)
+        return step[1] if z.seq_len + 1 >= min_total and n_keys > 0 else None
+
+    def _bound_step_of(self, layer_idx):
+        return self._bound[layer_idx]
+
     def compute(self, queries, layer_idx):
         """Decode attention for one token: [bs,1,Hq,D] -> [bs,1,Hq,D] (:1002-1107)."""
         z = self._zones[layer_idx]

@@ -155,6 +155,9 @@ class polar_cache(_polar_cache_base):
         global_k = int(adaptive_k.max().item())
         return adaptive_k, self._pack_indices(topk_ids, adaptive_k, topk_cap), global_k
 
+    def _bound_step_of(self, layer_idx):
+        return self._adaptive_bound[layer_idx]
+
     def compute(self, queries, layer_idx):
         """Decode attention for one token: [bs,1,Hq,D] -> [bs,1,Hq,D] (reference :1391-1677)."""
         z = self._zones[layer_idx]

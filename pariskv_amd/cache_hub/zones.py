@@ -82,6 +82,10 @@ class LayerZones:
         self.buffered = 0
         return r
 
+    def next_append_refreshes(self) -> bool:
+        """Whether the next ``appended()`` will return a Refresh (the token that fills the update buffer)."""
+        return self.seq_len >= self.steady and self.buffered + 1 >= self.interval
+
     # ---------------------------------------------------------------- regions
     @property
     def retrieval_start(self) -> int:

@@ -5,11 +5,46 @@
 // flashinfer.rmsnorm on [tokens*heads, head_dim]) and :434-498 (rotary embedding, rotate-half form) -
 // two norm launches and about sixteen element-wise torch launches per layer and token there.
 #include "pkv_common.h"
+#include "pkv_lut.h"
 
 namespace {
 
-// One wave per head; lane l holds dims l and l + 64 (the rotate-half pair).  head index in [0, Hq + Hkv):
-// query heads first.  fp32 arithmetic, one rounding to bf16 at the end.
+// RMSNorm + rotary embedding of one head held by one wave: lane l holds dims l and l + 64 (the rotate-half pair) in
+// x1 / x2 and gets the same dims of the result.  fp32 arithmetic; the caller rounds to bf16.
+__device__ __forceinline__ void qk_norm_rope_head(float x1, float x2, const uint16_t *__restrict__ w, float eps, float c,
+                                                  float s, float &y1, float &y2) {
+  const int lane = pkv_lane();
+  float ss = x1 * x1 + x2 * x2;
+#pragma unroll
+  for (int m = 1; m < PKV_WAVE; m <<= 1) ss += __shfl_xor(ss, m, PKV_WAVE);
+  const float inv = 1.0f / sqrtf(ss * (1.0f / 128.0f) + eps);
+  if (w) {
+    x1 = x1 * inv * pkv_bf16_bits_to_f32(w[lane]);
+    x2 = x2 * inv * pkv_bf16_bits_to_f32(w[lane + 64]);
+  }
+  y1 = x1 * c - x2 * s, y2 = x2 * c + x1 * s;
+}
+
+// One wave per head.  head index in [0, Hq + Hkv): query heads first.
+__device__ __forceinline__ void qk_norm_rope_task(int task, const uint16_t *__restrict__ qkv, int64_t stride_b, int n_q_heads,
+                                                  int n_kv_heads, const uint16_t *__restrict__ q_weight,
+                                                  const uint16_t *__restrict__ k_weight, float eps,
+                                                  const uint16_t *__restrict__ cos_row, const uint16_t *__restrict__ sin_row,
+                                                  uint16_t *__restrict__ q_out, uint16_t *__restrict__ k_out) {
+  const int lane = pkv_lane();
+  const int heads = n_q_heads + n_kv_heads;
+  const int b = task / heads, head = task % heads;
+  const bool is_q = head < n_q_heads;
+  const uint16_t *src = qkv + (int64_t)b * stride_b + (int64_t)head * 128;  // q heads, then k heads, contiguous in qkv
+  float y1, y2;
+  qk_norm_rope_head(pkv_bf16_bits_to_f32(src[lane]), pkv_bf16_bits_to_f32(src[lane + 64]), is_q ? q_weight : k_weight, eps,
+                    pkv_bf16_bits_to_f32(cos_row[lane]), pkv_bf16_bits_to_f32(sin_row[lane]), y1, y2);
+  uint16_t *dst = is_q ? q_out + ((int64_t)b * n_q_heads + head) * 128
+                       : k_out + ((int64_t)b * n_kv_heads + (head - n_q_heads)) * 128;
+  dst[lane] = pkv_f32_to_bf16_bits(y1);
+  dst[lane + 64] = pkv_f32_to_bf16_bits(y2);
+}
+
 __global__ __launch_bounds__(256) void pkv_qk_norm_rope_kernel(const uint16_t *__restrict__ qkv, int64_t stride_b, int n_q_heads,
                                                                int n_kv_heads, const uint16_t *__restrict__ q_weight,
                                                                const uint16_t *__restrict__ k_weight, float eps,
@@ -19,27 +54,78 @@ __global__ __launch_bounds__(256) void pkv_qk_norm_rope_kernel(const uint16_t *_
                                                                int n_tasks) {
   const int task = blockIdx.x * 4 + threadIdx.x / PKV_WAVE;
   if (task >= n_tasks) return;
-  const int lane = pkv_lane();
-  const int heads = n_q_heads + n_kv_heads;
-  const int b = task / heads, head = task % heads;
-  const bool is_q = head < n_q_heads;
-  const uint16_t *src = qkv + (int64_t)b * stride_b + (int64_t)head * 128;  // q heads, then k heads, contiguous in qkv
-  const uint16_t *w = is_q ? q_weight : k_weight;
-  float x1 = pkv_bf16_bits_to_f32(src[lane]), x2 = pkv_bf16_bits_to_f32(src[lane + 64]);
-  float ss = x1 * x1 + x2 * x2;
-#pragma unroll
-  for (int m = 1; m < PKV_WAVE; m <<= 1) ss += __shfl_xor(ss, m, PKV_WAVE);
-  const float inv = 1.0f / sqrtf(ss * (1.0f / 128.0f) + eps);
-  if (w) {
-    x1 = x1 * inv * pkv_bf16_bits_to_f32(w[lane]);
-    x2 = x2 * inv * pkv_bf16_bits_to_f32(w[lane + 64]);
+  qk_norm_rope_task(task, qkv, stride_b, n_q_heads, n_kv_heads, q_weight, k_weight, eps, cos_row, sin_row, q_out, k_out);
+}
+
+// The same launch with the retrieval's query side riding along: workgroups [0, n_rope_blocks) are the norm + rotary
+// embedding above; the 16 * rows workgroups after them build one subspace's slice of a (batch, kv-head) row's vote
+// table each, from the same raw qkv: the wave that rotates the row's query normalises and rotates the group's query
+// heads itself (the arithmetic of qk_norm_rope_head, rounded to bf16 as q_out is), so nothing waits for q_out.
+// What pkv_query_prep_lut_kernel would write for those queries lands in the same workspace segments, and the words
+// that launch clears for the later stages are cleared here.
+__global__ __launch_bounds__(256) void pkv_qk_norm_rope_table_kernel(
+    const uint16_t *__restrict__ qkv, int64_t stride_b, int n_q_heads, int n_kv_heads, const uint16_t *__restrict__ q_weight,
+    const uint16_t *__restrict__ k_weight, float eps, const uint16_t *__restrict__ cos_row, const uint16_t *__restrict__ sin_row,
+    uint16_t *__restrict__ q_out, uint16_t *__restrict__ k_out, int n_tasks, int n_rope_blocks, int bs,
+    const float *__restrict__ signs, const int32_t *__restrict__ cc, PkvTiers tiers, float *__restrict__ qhat,
+    float *__restrict__ qnorm, uint8_t *__restrict__ lut, uint32_t *__restrict__ row_suf, uint32_t *__restrict__ zero_ptr,
+    int64_t zero_words) {
+  const int tid = threadIdx.x;
+  if ((int)blockIdx.x < n_rope_blocks) {
+    const int task = blockIdx.x * 4 + tid / PKV_WAVE;
+    if (task < n_tasks)
+      qk_norm_rope_task(task, qkv, stride_b, n_q_heads, n_kv_heads, q_weight, k_weight, eps, cos_row, sin_row, q_out, k_out);
+    return;
   }
+  const int t = blockIdx.x - n_rope_blocks, n_table = 16 * bs * n_kv_heads;
+  const int sub = t % 16, row = t / 16;
+  const int b = row / n_kv_heads, h = row % n_kv_heads, group = n_q_heads / n_kv_heads;
+  for (int64_t i = (int64_t)t * 256 + tid; i < zero_words; i += (int64_t)n_table * 256) zero_ptr[i] = 0u;
+  if (sub == 1 && tid < 128) row_suf[(int64_t)row * 128 + tid] = 0u;
+
+  __shared__ PkvLutSmem sm;
+  __shared__ float s_head[4][128];  // the group's heads after norm + rotary embedding (bf16 values), four at a time
+  const int my_cc = cc[((int64_t)row * 16 + sub) * 256 + tid];
+  const int lane = pkv_lane(), wave = tid / PKV_WAVE;
   const float c = pkv_bf16_bits_to_f32(cos_row[lane]), s = pkv_bf16_bits_to_f32(sin_row[lane]);
-  const float y1 = x1 * c - x2 * s, y2 = x2 * c + x1 * s;
-  uint16_t *dst = is_q ? q_out + ((int64_t)b * n_q_heads + head) * 128
-                       : k_out + ((int64_t)b * n_kv_heads + (head - n_q_heads)) * 128;
-  dst[lane] = pkv_f32_to_bf16_bits(y1);
-  dst[lane + 64] = pkv_f32_to_bf16_bits(y2);
+  // the group mean of pkv_query_group_mean_wave_t over heads that are normalised and rotated on the way: the four
+  // waves take a head each, the first wave adds them up in head order
+  float a_lo = 0.f, a_hi = 0.f;
+  for (int g0 = 0; g0 < group; g0 += 4) {
+    if (g0 + wave < group) {
+      const uint16_t *src = qkv + (int64_t)b * stride_b + (int64_t)(h * group + g0 + wave) * 128;
+      float y1, y2;
+      qk_norm_rope_head(pkv_bf16_bits_to_f32(src[lane]), pkv_bf16_bits_to_f32(src[lane + 64]), q_weight, eps, c, s, y1, y2);
+      s_head[wave][lane] = pkv_bf16_round(y1), s_head[wave][lane + 64] = pkv_bf16_round(y2);
+    }
+    __syncthreads();
+    if (tid < PKV_WAVE) {
+      for (int u = 0; u < 4 && g0 + u < group; ++u) {
+        a_lo = g0 + u == 0 ? s_head[u][lane] : a_lo + s_head[u][lane];
+        a_hi = g0 + u == 0 ? s_head[u][lane + 64] : a_hi + s_head[u][lane + 64];
+      }
+    }
+    if (g0 + 4 < group) __syncthreads();
+  }
+  if (tid < PKV_WAVE) {
+    float x_lo, x_hi;
+    if ((group & (group - 1)) == 0) {
+      const float inv = 1.0f / (float)group;
+      x_lo = pkv_bf16_round(a_lo * inv), x_hi = pkv_bf16_round(a_hi * inv);
+    } else {
+      x_lo = pkv_bf16_round(a_lo / (float)group), x_hi = pkv_bf16_round(a_hi / (float)group);
+    }
+    float y_lo, y_hi;
+    const float n = pkv_normalize_rotate_64(x_lo, x_hi, signs[lane], signs[lane + 64], PKV_DTYPE_BF16, y_lo, y_hi);
+    sm.y[tid] = y_lo, sm.y[tid + 64] = y_hi;
+    if (sub == 0) {
+      qhat[(int64_t)row * 128 + tid] = y_lo, qhat[(int64_t)row * 128 + tid + 64] = y_hi;
+      if (tid == 0) qnorm[row] = n;
+    }
+  }
+  sm.cc[tid] = my_cc;
+  __syncthreads();
+  pkv_lut_rank_subspace(PKV_DTYPE_BF16, nullptr, tiers, sub, sm, lut + ((int64_t)row * 16 + sub) * 256, nullptr);
 }
 
 // out_sum = x + residual (residual may be NULL), out_norm = RMSNorm(out_sum) * weight.  One workgroup of 256
@@ -136,6 +222,29 @@ extern "C" int pkv_qk_norm_rope(const void *qkv, int64_t stride_b, int bs, int n
                      (const uint16_t *)k_weight, eps, (const uint16_t *)cos_row, (const uint16_t *)sin_row,
                      (uint16_t *)q_out, (uint16_t *)k_out, n_tasks);
   PKV_LAUNCH_CHECK("pkv_qk_norm_rope_kernel");
+  return PKV_OK;
+}
+
+// Launcher of the norm + rotary embedding with the retrieval's query side in the same launch (pkv_retrieve.hip lays the
+// workspace out and checks the retrieval's arguments).
+int pkv_launch_qk_norm_rope_table(const void *qkv, int64_t stride_b, int bs, int n_q_heads, int n_kv_heads,
+                                  const void *q_weight, const void *k_weight, float eps, const void *cos_row,
+                                  const void *sin_row, void *q_out, void *k_out, const float *signs, const int32_t *cc,
+                                  const PkvTiers &tiers, float *qhat, float *qnorm, uint8_t *lut, uint32_t *row_suf,
+                                  uint32_t *zero_ptr, int64_t zero_words, hipStream_t s) {
+  PKV_REQUIRE(qkv && cos_row && sin_row && q_out && k_out, "pkv_qk_norm_rope_table: null pointer");
+  PKV_REQUIRE(bs > 0 && n_q_heads > 0 && n_kv_heads > 0 && n_q_heads % n_kv_heads == 0 &&
+                  (int64_t)bs * (n_q_heads + n_kv_heads) < (1 << 24) && stride_b >= (int64_t)(n_q_heads + n_kv_heads) * 128,
+              "pkv_qk_norm_rope_table: bad shape bs=%d heads=%d+%d stride=%lld", bs, n_q_heads, n_kv_heads, (long long)stride_b);
+  PKV_REQUIRE((q_weight == nullptr) == (k_weight == nullptr), "q and k norm weights go together");
+  const int n_tasks = bs * (n_q_heads + n_kv_heads);
+  const int n_rope_blocks = (n_tasks + 3) / 4;
+  hipLaunchKernelGGL(pkv_qk_norm_rope_table_kernel, dim3((unsigned)(n_rope_blocks + 16 * bs * n_kv_heads)), dim3(256), 0, s,
+                     (const uint16_t *)qkv, stride_b, n_q_heads, n_kv_heads, (const uint16_t *)q_weight,
+                     (const uint16_t *)k_weight, eps, (const uint16_t *)cos_row, (const uint16_t *)sin_row, (uint16_t *)q_out,
+                     (uint16_t *)k_out, n_tasks, n_rope_blocks, bs, signs, cc, tiers, qhat, qnorm, lut, row_suf, zero_ptr,
+                     zero_ptr ? zero_words : 0);
+  PKV_LAUNCH_CHECK("pkv_qk_norm_rope_table_kernel");
   return PKV_OK;
 }
 

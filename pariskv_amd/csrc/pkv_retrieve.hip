@@ -11,6 +11,11 @@
 #include <mutex>
 
 PKV_INTERNAL int pkv_launch_identity_fill(int64_t *out, int64_t len, int64_t k, int rows, hipStream_t s);
+PKV_INTERNAL int pkv_launch_qk_norm_rope_table(const void *qkv, int64_t stride_b, int bs, int n_q_heads, int n_kv_heads,
+                                  const void *q_weight, const void *k_weight, float eps, const void *cos_row,
+                                  const void *sin_row, void *q_out, void *k_out, const float *signs, const int32_t *cc,
+                                  const PkvTiers &tiers, float *qhat, float *qnorm, uint8_t *lut, uint32_t *row_suf,
+                                  uint32_t *zero_ptr, int64_t zero_words, hipStream_t s);
 PKV_INTERNAL size_t pkv_fused_sync_bytes(int rows, int64_t n_chunks);
 PKV_INTERNAL bool pkv_fused_usable(int rows, int64_t n_keys, int chunk_keys, hipStream_t s);
 PKV_INTERNAL int pkv_launch_fused_retrieve(const void *q, int dtype, int bs, int n_kv_heads, int group, const float *signs,
@@ -181,8 +186,12 @@ static int retrieve_impl(const pkv_retrieve_args *a, void *ws, size_t ws_bytes, 
                                    a->record_word_offset > 0 ? (float *)(base + w.cand_extra) : nullptr, range_slots,
                                    range_stride, s);
   } else {
-    rc = pkv_launch_query_prep_lut(a->q, a->dtype, a->bs, H, a->group, a->signs, a->cluster_counts,
-                                   (int64_t)H * 4096, 4096, t, qhat, qnorm, lut, nullptr, rowsuf, s, topk_ctl, ctl_words);
+    // table_ready: pkv_qk_norm_rope_table already left the rotated query, its norm and the vote table of these
+    // queries in the workspace and cleared what this launch would clear
+    rc = a->table_ready ? PKV_OK
+                        : pkv_launch_query_prep_lut(a->q, a->dtype, a->bs, H, a->group, a->signs, a->cluster_counts,
+                                                    (int64_t)H * 4096, 4096, t, qhat, qnorm, lut, nullptr, rowsuf, s, topk_ctl,
+                                                    ctl_words);
     if (rc) return rc;
     if (a->n_cand == a->n_keys) {
       rc = pkv_launch_identity_fill(cand, a->n_keys, a->n_cand, rows, s);
@@ -221,6 +230,35 @@ static int retrieve_impl(const pkv_retrieve_args *a, void *ws, size_t ws_bytes, 
                            a->dst_row0, rows, a->row_bytes, s);
   }
   return rc;
+}
+
+extern "C" int pkv_qk_norm_rope_table(const void *qkv, int64_t stride_b, int n_q_heads, const void *q_weight,
+                                      const void *k_weight, float eps, const void *cos_row, const void *sin_row, void *q_out,
+                                      void *k_out, const pkv_retrieve_args *a, void *ws, size_t ws_bytes, void *stream) {
+  PKV_REQUIRE(a != nullptr, "pkv_qk_norm_rope_table: null retrieval arguments");
+  PKV_REQUIRE(a->dtype == PKV_DTYPE_BF16 && a->bs > 0 && a->n_kv_heads > 0 && a->group > 0 &&
+                  n_q_heads == a->n_kv_heads * a->group,
+              "pkv_qk_norm_rope_table: bf16 queries of %d x %d heads expected, got %d query heads", a->n_kv_heads, a->group,
+              n_q_heads);
+  PKV_REQUIRE(a->signs && a->cluster_counts && a->n_tiers >= 1 && a->n_tiers <= PKV_MAX_TIERS,
+              "pkv_qk_norm_rope_table: the retrieval's signs / cluster counts / tiers are missing");
+  const int rows = a->bs * a->n_kv_heads;
+  PKV_REQUIRE(shape_ok(rows, a->n_keys, a->n_cand, a->k), "pkv_qk_norm_rope_table: bad retrieval shape");
+  const WsLayout w = layout(rows, a->n_keys, a->n_cand, a->k);
+  if (!ws || ws_bytes < w.total || !pkv_aligned(ws, 256)) {
+    pkv_set_error("pkv_qk_norm_rope_table: workspace of %zu bytes (256-aligned) required, got %zu", w.total, ws_bytes);
+    return PKV_ENOMEM;
+  }
+  char *base = (char *)ws;
+  PkvTiers t;
+  memset(&t, 0, sizeof t);
+  t.n = a->n_tiers;
+  for (int i = 0; i < a->n_tiers; ++i) t.t[i] = a->tier_counts[i];
+  const int64_t ctl_words = a->out_ids && a->n_cand != a->n_keys ? pkv_topk_ctl_words(rows, a->n_cand) : 0;
+  return pkv_launch_qk_norm_rope_table(qkv, stride_b, a->bs, n_q_heads, a->n_kv_heads, q_weight, k_weight, eps, cos_row,
+                                       sin_row, q_out, k_out, a->signs, a->cluster_counts, t, (float *)(base + w.qhat),
+                                       (float *)(base + w.qnorm), (uint8_t *)(base + w.lut), (uint32_t *)(base + w.rowsuf),
+                                       ctl_words ? (uint32_t *)(base + w.topk) : nullptr, ctl_words, (hipStream_t)stream);
 }
 
 extern "C" int pkv_retrieve(const pkv_retrieve_args *a, void *ws, size_t ws_bytes, void *stream) {

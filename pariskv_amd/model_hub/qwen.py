@@ -169,8 +169,11 @@ class QwenModel:
         bsz, seq_len, _ = normed.shape
         qkv = F.linear(normed, layer.wqkv)
         pos = self._position
+        # where this layer's step will retrieve, its vote table is built by the same launch that finishes the queries
+        target = self.kv_cache.query_table_target(layer_idx) if hasattr(self.kv_cache, "query_table_target") else None
         q, k = ops.qk_norm_rope(qkv, self.num_heads, self.num_key_value_heads, layer.q_norm_weight, layer.k_norm_weight,
-                                layer.q_norm_variance_epsilon or 0.0, self.cos_cache[pos], self.sin_cache[pos])
+                                layer.q_norm_variance_epsilon or 0.0, self.cos_cache[pos], self.sin_cache[pos],
+                                table_for=target)
         v = qkv[..., (self.num_heads + self.num_key_value_heads) * self.head_dim:].reshape(bsz, -1, self.num_key_value_heads,
                                                                                              self.head_dim)
         k, v = self.kv_cache.decode_update_kv_cache(k, v, layer_idx)

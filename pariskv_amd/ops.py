@@ -606,10 +606,13 @@ class DecodeAttention:
 
 
 def qk_norm_rope(qkv: torch.Tensor, n_q_heads: int, n_kv_heads: int, q_weight, k_weight, eps: float,
-                 cos_row: torch.Tensor, sin_row: torch.Tensor):
+                 cos_row: torch.Tensor, sin_row: torch.Tensor, table_for=None):
     """Per-head RMSNorm of q and k plus rotary embedding for one decode token per sequence, one launch
     (model_hub/qwen.py:327-340, 410-431, 434-498).  qkv bf16 [bs,1,(Hq+2Hkv)*128] (last dim contiguous); cos_row /
-    sin_row bf16 [64] of the token's position.  Returns (q [bs,1,Hq,128], k [bs,1,Hkv,128])."""
+    sin_row bf16 [64] of the token's position.  Returns (q [bs,1,Hq,128], k [bs,1,Hkv,128]).
+    ``table_for``: a :class:`BoundStep` / :class:`BoundAdaptiveStep` whose retrieval will run on the returned q next:
+    the same launch then also leaves the retrieval's rotated query and vote table in that step's workspace
+    (pkv_qk_norm_rope_table) and the step's next launch skips its query-prep kernel."""
     bs = qkv.shape[0]
     _need(qkv.is_cuda and qkv.dtype == torch.bfloat16 and qkv.stride(-1) == 1 and qkv.numel() == bs * qkv.shape[-1] and
           qkv.shape[-1] >= (n_q_heads + 2 * n_kv_heads) * HEAD_DIM, "qkv: bf16 [bs,1,(Hq+2Hkv)*128]")
@@ -620,6 +623,12 @@ def qk_norm_rope(qkv: torch.Tensor, n_q_heads: int, n_kv_heads: int, q_weight, k
               "norm weights: bf16 [128]")
     q = torch.empty(bs, 1, n_q_heads, HEAD_DIM, dtype=torch.bfloat16, device=qkv.device)
     k = torch.empty(bs, 1, n_kv_heads, HEAD_DIM, dtype=torch.bfloat16, device=qkv.device)
+    if table_for is not None:
+        _lib.check(_lib.lib().pkv_qk_norm_rope_table(_p(qkv), qkv.stride(0), n_q_heads, _p(q_weight), _p(k_weight), float(eps),
+                                                     _p(cos_row), _p(sin_row), _p(q), _p(k), table_for._ra, table_for._ws,
+                                                     table_for._ws_bytes, _stream(qkv)))
+        table_for.a.table_ready = 1   # consumed (and reset) by the step's next launch
+        return q, k
     _lib.check(_lib.lib().pkv_qk_norm_rope(_p(qkv), qkv.stride(0), bs, n_q_heads, n_kv_heads, _p(q_weight), _p(k_weight),
                                            float(eps), _p(cos_row), _p(sin_row), _p(q), _p(k), _stream(qkv)))
     return q, k
@@ -717,6 +726,7 @@ class BoundStep:
         out = torch.empty_like(q)
         self.a.q, self.aa.out = q.data_ptr(), out.data_ptr()
         rc = self._fn(self._ra, self._ws, self._ws_bytes, self._raa, torch.cuda.current_stream(q.device).cuda_stream)
+        self.a.table_ready = 0  # a table left by qk_norm_rope(table_for=self) serves one launch
         if rc != 0:
             _lib.check(rc)
         return out
@@ -743,6 +753,7 @@ class BoundAdaptiveStep:
         self.a.q, self.aa.out = q.data_ptr(), out.data_ptr()
         rc = self._fn(self._ra, self._ws, self._ws_bytes, self._rad, self._raa,
                       torch.cuda.current_stream(q.device).cuda_stream)
+        self.a.table_ready = 0  # a table left by qk_norm_rope(table_for=self) serves one launch
         if rc != 0:
             _lib.check(rc)
         return out

@@ -687,6 +687,57 @@ def test_qk_norm_rope_matches_torch_ops():
         ops.qk_norm_rope(qkv, Hq, Hkv, qw, None, eps, cos, sin)
 
 
+def test_qk_norm_rope_with_the_vote_table_in_the_same_launch():
+    """pkv_qk_norm_rope_table: q / k bit for bit as pkv_qk_norm_rope writes them, and in the bound step's workspace the
+    rotated query, its norm and the vote table exactly as the query-prep launch computes them from that q; the
+    decode step launched with table_ready then returns the attention output and the ids of the ordinary step.  Run
+    through the cache class (offload and no-offload) on its own bound step, as the model glue does."""
+    from pariskv_amd import ops
+    from pariskv_amd.cache_hub.polar_cache import polar_cache
+
+    bs, Hq, Hkv, D, S = 2, 8, 2, 128, 3000
+    g = torch.Generator(device=DEV).manual_seed(9)
+    for offload in (True, False):
+        cache = _make_cache(offload, bs, Hkv, Hq, 1, S, 64, 4, 64, 16, 100)
+        k, v = _synth_kv(torch.Generator().manual_seed(1), bs, S, Hkv)
+        cache.prefill_update_kv_cache(None, k.to(DEV), v.to(DEV), 0, 0)
+        width = (Hq + 2 * Hkv) * D
+        qw = (1 + 0.1 * torch.randn(D, generator=g, device=DEV)).to(torch.bfloat16)
+        kw = (1 + 0.1 * torch.randn(D, generator=g, device=DEV)).to(torch.bfloat16)
+        ang = torch.rand(D // 2, generator=g, device=DEV) * 6.28
+        cos, sin = ang.cos().to(torch.bfloat16), ang.sin().to(torch.bfloat16)
+        assert cache.query_table_target(0) is None           # nothing bound before the first retrieval
+        used = 0
+        for step in range(20):                                # crosses an index refresh (interval 16)
+            qkv = torch.randn(bs, 1, width, generator=g, device=DEV).to(torch.bfloat16)
+            target = cache.query_table_target(0)
+            q0, k0 = ops.qk_norm_rope(qkv, Hq, Hkv, qw, kw, 1e-6, cos, sin)
+            q1, k1 = ops.qk_norm_rope(qkv, Hq, Hkv, qw, kw, 1e-6, cos, sin, table_for=target)
+            assert torch.equal(q0, q1) and torch.equal(k0, k1)
+            vv = qkv[..., (Hq + Hkv) * D:].reshape(bs, 1, Hkv, D)
+            if target is not None:
+                used += 1
+                n_keys, n_cand, topk, tiers = cache.retrieval_shape(0)
+                plan = cache._plan
+                tab = {n: plan.view(n, n_keys, n_cand, topk, dt).clone() for n, dt in
+                       (("qhat", torch.float32), ("qnorm", torch.float32), ("lut", torch.uint8))}
+                assert not bool(plan.view("row_suffix_hist", n_keys, n_cand, topk, torch.int32).any())
+                qhat, qnorm, lut, _ = ops.query_prep_lut(q1, Hkv, cache._srht_signs, cache.cluster_key_counts_gpu[0], tiers)
+                assert torch.equal(tab["qhat"].view(-1), qhat.reshape(-1)) and torch.equal(tab["qnorm"].view(-1), qnorm.reshape(-1))
+                assert torch.equal(tab["lut"].view(-1), lut.reshape(-1))
+            cache.decode_update_kv_cache(k1, vv, 0)
+            assert target is None or target.a.table_ready == 1
+            out1 = cache.compute(q1, 0)
+            ids1 = cache.last_topk_indices.clone() if getattr(cache, "last_topk_indices", None) is not None else None
+            assert target is None or target.a.table_ready == 0
+            out0 = cache.compute(q0, 0)                       # the same step again, its own query-prep launch this time
+            torch.cuda.synchronize()
+            assert torch.equal(out0, out1), f"step {step}: attention output differs with the table from the q/k launch"
+            if ids1 is not None:
+                assert torch.equal(ids1, cache.last_topk_indices)
+        assert used >= 15, used
+
+
 def test_add_rmsnorm_and_silu_mul_match_torch_ops():
     """The two fused element-wise kernels of the decode glue against the torch op sequences they replace (bf16 add then
     F.rms_norm; F.silu then multiply), element for element up to one bf16 rounding."""

@@ -28,7 +28,9 @@ def simulate(sink, local, interval, offload, prefill, steps):
     for step in range(steps):
         tok = prefill + step
         gpu[z.append_slot()] = tok
+        predicted = z.next_append_refreshes()
         r = z.appended()
+        assert predicted == (r is not None)
         if r is not None:
             moved = [gpu[r.gpu_row0 + i] for i in range(r.n_new)]
             assert r.encode_abs0 == sink + len(encoded)
