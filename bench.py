@@ -12,8 +12,12 @@ Steps rotate over LAYERS distinct layer indexes (448 MiB each) so that no
 layer's codes are still in the 256 MB last-level cache when it is scanned again,
 as in a real decode step, which walks all layers of the model.
 
-Prints ONE JSON line: metric/value/unit, the per-stage times (`stages_us`), the roofline of the dominant
-kernel (collision scan, timed by its own dispatch timestamps) and the single-thread CPU baseline.
+Prints ONE JSON line: metric/value/unit, the per-stage times (`stages_us`, with both launch plans of the on-GPU
+stages), the roofline of the dominant kernel (collision scan, timed by its own dispatch timestamps), the
+single-thread CPU baseline, and three more objects measured the same way on their own data: `cfg2` and `cfg4`
+(the retrieval at BASELINE configs 2 and 4, each with its algorithmic bytes, HBM fraction and oracle check) and `cfg5`
+(decode tokens/s of the model loop).  `--no-cfg2 / --no-cfg4 / --no-cfg5 / --no-cpu-baseline` leave legs out; `--only
+scan | copy | decode-loop | model-decode` runs one leg alone (for profiling).
 """
 import argparse
 import ctypes as C

@@ -614,7 +614,12 @@ int pkv_adaptive_decode_step(const pkv_retrieve_args *retrieve, void *ws, size_t
 
 /* Names and device pointers of the intermediates inside a pkv_retrieve
  * workspace (for tests and profiling): qhat, qnorm, lut, cnt_u8,
- * chunk_suffix_hist, row_suffix_hist, cand, scores, cand_record_word.  Returns PKV_EINVAL for an unknown name. */
+ * chunk_suffix_hist, row_suffix_hist, cand, scores, cand_record_word, handover_status.  Returns PKV_EINVAL for an
+ * unknown name.  chunk_suffix_hist holds uint16 counts of the keys of a chunk with at least `bin` votes:
+ * [row][chunk][128 bins] for rows scanned one chunk per workgroup, and [row][128 bins][chunk][4 pieces] where the
+ * chunk size (the smallest power of two from 2048 that keeps a launch within 1024 workgroups) is 8192 keys or more and
+ * a row has at most 128 chunks: a workgroup then scans four pieces of chunk_keys / 4 keys that lie n_chunks pieces
+ * apart, and piece p of the row, in key order, is entry [p % n_chunks][p / n_chunks]. */
 int pkv_retrieve_ws_view(void *ws, int rows, int64_t n_keys, int64_t n_cand, int64_t k,
                          const char *name, void **ptr, size_t *bytes);
 
