@@ -340,6 +340,33 @@ def cfg4_leg(torch, ops, _lib, dev):
             "parity_checked": "adaptive k and the first k ids of the last step, layer " + str(l)}
 
 
+def encoder_leg(torch, ops, dev, shapes=((8, 8, 65536), (1, 8, 131072)), reps=10):
+    """The index build of a prefill or refresh (`pkv_encode_append`: bf16 keys -> codes, 4-bit records, weights,
+    cluster sizes) on synthetic keys, per shape (batch, kv heads, keys per head): microseconds per 2^20 key-heads and
+    the rate over the 368 bytes a key-head must move (256 read, 112 written)."""
+    signs = ops.srht_signs(dev)
+    out = []
+    for bs, H, N in shapes:
+        g = torch.Generator(device=dev).manual_seed(5)
+        keys = torch.randn(bs, H, N, 128, generator=g, device=dev)
+        keys[..., [7, 31, 64, 101]] *= 10.0
+        kb = keys.to(torch.bfloat16)
+        del keys
+        _, _, _, cb, k4, kw = ops.alloc_keymajor(bs, H, N, dev)
+        cc = torch.zeros(bs, H, 16, 256, dtype=torch.int32, device=dev)
+        for _ in range(max(3, (48 << 20) // (bs * H * N))):  # ~6 ms of the same launch first: the shader clock settles
+            ops.encode_append(kb, signs, cb, k4, kw, cc)
+        us = timed_us(torch, lambda i: ops.encode_append(kb, signs, cb, k4, kw, cc), reps)
+        kh = bs * H * N
+        out.append({"batch": bs, "kv_heads": H, "keys_per_head": N, "us_per_launch": round(us, 1),
+                    "us_per_2^20_key_heads": round(us / kh * 2**20, 1),
+                    "GBps_over_368B_per_key_head": round(kh * 368 / us / 1e3, 1),
+                    "hbm_fraction": round(kh * 368 / us / 1e3 / HBM_PEAK_GBPS, 4)})
+        del kb, cb, k4, kw, cc
+    return {"kernel": "pkv_encode_kernel<bf16>", "bound": "between vector issue (about 225 instructions per key and 16-lane group) and the memory system",
+            "shapes": out}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -351,7 +378,8 @@ def main():
     ap.add_argument("--candidates", type=int, default=4096)
     ap.add_argument("--topk", type=int, default=1024)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["scan", "copy", "adaptive", "topk", "decode-loop", "model-decode"], default=None,
+    ap.add_argument("--only", choices=["scan", "copy", "adaptive", "topk", "decode-loop", "model-decode", "encode"],
+                    default=None,
                     help="profiling aid: launch only the collision scan, the calibration copy, the adaptive-k stage "
                          "(--candidates scores per row, dense prefix 1600, value norms gathered from a --context table, "
                          "list length --topk) or the exact top-k (--topk of --candidates N(30,20) scores per row) "
@@ -359,7 +387,8 @@ def main():
                          "--context prompt tokens, --steps generated tokens (append + retrieval + gather + attention per "
                          "layer, index refresh and host offload every 1024 tokens); model-decode: the same loop inside a "
                          "random-initialised Qwen3-8B-shaped decoder (config 5: --layers 36 --batch 8 --context 65536 "
-                         "--topk 100 --steps 256), end-to-end decode tokens/s")
+                         "--topk 100 --steps 256), end-to-end decode tokens/s; encode: the index build "
+                         "(pkv_encode_append) at two shapes")
     ap.add_argument("--no-offload", action="store_true", help="decode-loop: keep K/V in HBM (config 2's mode)")
     ap.add_argument("--host-kv-budget-gib", type=float, default=56.0,
                     help="model-decode / the default run's cfg5 leg: pinned host memory the cache may use for offloaded "
@@ -394,6 +423,10 @@ def main():
         print(json.dumps({"only": "model-decode",
                           **model_decode(torch, dev, L, bs, N, args.steps, K, args.warmup, not args.no_offload,
                                          None if args.host_kv_budget_gib <= 0 else int(args.host_kv_budget_gib * 2**30))}))
+        return
+
+    if args.only == "encode":
+        print(json.dumps({"only": "encode", **encoder_leg(torch, ops, dev, reps=max(4, args.steps // 4))}))
         return
 
     if args.only == "decode-loop":
@@ -791,6 +824,7 @@ def main():
         gc.collect()
         torch.cuda.empty_cache()
 
+    leg("encoder", lambda: encoder_leg(torch, ops, dev))
     if not args.no_cfg2:
         leg("cfg2", lambda: cfg2_leg(torch, ops, _lib, dev, args.steps, args.warmup))
     if not args.no_cfg4:

@@ -150,13 +150,16 @@ __device__ __forceinline__ float pkv_from_ordered_u32(uint32_t k) {
 
 __device__ __forceinline__ int pkv_lane() { return (int)(threadIdx.x & (PKV_WAVE - 1)); }
 
-// Value of lane (lane ^ M).  M = 1, 2, 4, 8 are data-parallel-primitive moves inside a row of 16 lanes
+// Value of lane (lane ^ M).  M = 1, 2, 3, 4, 7, 8, 15 are data-parallel-primitive moves inside a row of 16 lanes
 // (no trip through the LDS crossbar); 16 and 32 use the generic lane permute.
 template <int M>
 __device__ __forceinline__ uint32_t pkv_lane_xor(uint32_t v) {
   const int x = (int)v;
   if (M == 1) return (uint32_t)__builtin_amdgcn_mov_dpp(x, 0xB1, 0xf, 0xf, false);   // quad_perm [1,0,3,2]
   if (M == 2) return (uint32_t)__builtin_amdgcn_mov_dpp(x, 0x4E, 0xf, 0xf, false);   // quad_perm [2,3,0,1]
+  if (M == 3) return (uint32_t)__builtin_amdgcn_mov_dpp(x, 0x1B, 0xf, 0xf, false);   // quad_perm [3,2,1,0]
+  if (M == 7) return (uint32_t)__builtin_amdgcn_mov_dpp(x, 0x141, 0xf, 0xf, false);  // row_half_mirror
+  if (M == 15) return (uint32_t)__builtin_amdgcn_mov_dpp(x, 0x140, 0xf, 0xf, false); // row_mirror
   if (M == 4) {
     int r = __builtin_amdgcn_update_dpp(x, x, 0x104, 0xf, 0x5, false);  // banks 0,2 read lane + 4 (row_shl:4)
     r = __builtin_amdgcn_update_dpp(r, x, 0x114, 0xf, 0xa, false);      // banks 1,3 read lane - 4 (row_shr:4)
@@ -186,12 +189,15 @@ __device__ __forceinline__ int pkv_wave_incl_scan(int v) {
   return v;
 }
 
-// Normalise and SRHT-rotate one 128-vector spread over 16 lanes: lane s (= lane id & 15) holds
+// Normalise and SRHT-rotate one 128-vector spread over 16 lanes: the lane of block s holds
 // dims 8s..8s+7 in x[] (and the matching SRHT signs in sg[]).  On return y[] holds the rotated unit
 // vector's dims 8s..8s+7 and the norm is returned (both rounded to `dtype` where the reference's
 // tensors are).  Operation order: sum of squares sequential inside the 8 dims, then a pairwise tree
-// over the 16 lanes; natural-order Walsh-Hadamard butterflies h = 1..64 (three in-lane stages, four
+// over the 16 blocks; natural-order Walsh-Hadamard butterflies h = 1..64 (three in-lane stages, four
 // lane-xor stages); then * 1/sqrt(128).  All 16 lanes of the group must be active.
+// M4 / M8: the lane distance (xor) to the block s ^ 4 / s ^ 8; blocks s ^ 1 and s ^ 2 sit at lane ^ 1 and lane ^ 2.
+// The natural placement (block s in lane s) has M4 = 4, M8 = 8.
+template <int M4 = 4, int M8 = 8>
 __device__ __forceinline__ float pkv_normalize_rotate_16(const float (&x)[8], const float (&sg)[8], int s, int dtype,
                                                          float (&y)[8]) {
   float acc = x[0] * x[0];
@@ -199,8 +205,8 @@ __device__ __forceinline__ float pkv_normalize_rotate_16(const float (&x)[8], co
   for (int j = 1; j < 8; ++j) acc = acc + x[j] * x[j];
   acc = acc + pkv_lane_xor_f<1>(acc);
   acc = acc + pkv_lane_xor_f<2>(acc);
-  acc = acc + pkv_lane_xor_f<4>(acc);
-  acc = acc + pkv_lane_xor_f<8>(acc);
+  acc = acc + pkv_lane_xor_f<M4>(acc);
+  acc = acc + pkv_lane_xor_f<M8>(acc);
   const float n = pkv_rdt(sqrtf(acc), dtype);
   const float den = n < 1e-8f ? 1e-8f : n;
   float t[8];
@@ -217,15 +223,15 @@ __device__ __forceinline__ float pkv_normalize_rotate_16(const float (&x)[8], co
       }
     }
   }
-#define PKV_FWHT_LANE_STAGE(M)                              \
+#define PKV_FWHT_LANE_STAGE(BIT, M)                         \
   _Pragma("unroll") for (int j = 0; j < 8; ++j) {           \
     const float o = pkv_lane_xor_f<M>(t[j]);                \
-    t[j] = (s & M) ? (o - t[j]) : (t[j] + o);               \
+    t[j] = (s & BIT) ? (o - t[j]) : (t[j] + o);             \
   }
-  PKV_FWHT_LANE_STAGE(1)
-  PKV_FWHT_LANE_STAGE(2)
-  PKV_FWHT_LANE_STAGE(4)
-  PKV_FWHT_LANE_STAGE(8)
+  PKV_FWHT_LANE_STAGE(1, 1)
+  PKV_FWHT_LANE_STAGE(2, 2)
+  PKV_FWHT_LANE_STAGE(4, M4)
+  PKV_FWHT_LANE_STAGE(8, M8)
 #undef PKV_FWHT_LANE_STAGE
 #pragma unroll
   for (int j = 0; j < 8; ++j) y[j] = pkv_rdt(t[j] * PKV_HADAMARD_SCALE, dtype);

@@ -5,34 +5,50 @@
 // three permute copies and [.,S,16,8] intermediates) and :980-996
 // (_count_cluster_keys: bincount per batch element).
 //
-// One key is handled by 16 lanes, lane s owning the 8 dims of block s, so four
+// One key is handled by 16 lanes, each owning the 8 dims of one block, so four
 // keys share a wave64.  The 128-point Walsh-Hadamard transform is three in-lane
-// butterfly stages plus four cross-lane stages (lane xor 1,2,4,8); everything
+// butterfly stages plus four cross-lane stages (block xor 1,2,4,8); everything
 // after the rotation is lane-local.  256 B read + 112 B written per key.
+//
+// Block s (bits s3 s2 s1 s0) sits in lane s0*1 ^ s1*2 ^ s2*7 ^ s3*15 of its
+// row of 16, so that the partner of every cross-lane stage is one
+// data-parallel-primitive move away (quad_perm [1,0,3,2], [2,3,0,1],
+// row_half_mirror, row_mirror) and the move folds into the arithmetic
+// instruction that uses it.
 //
 // The order of every floating-point operation is fixed (and contraction into
 // FMA is disabled at build time) because the integer outputs must be
 // reproducible bit for bit:
 //   sum of squares: sequential inside a block, then a pairwise tree over blocks.
 //
-// The kernel is bound by vector-instruction issue, not by HBM.  fp32 keys take
-// enc_key_exact (correctly rounded divisions and roots, about 700 instructions
-// per lane and key); bf16 keys take enc_key_fast (about 300), which reaches the
-// same bits through reciprocals, a table for the magnitude code and centre, and
-// lane-crossing adds folded into one instruction, and hands a wave over to
-// enc_key_exact when one of its keys is outside the range where that is proven.
+// The kernel sits between vector-instruction issue and the memory system (about
+// 3.4 TB/s of mixed traffic: 256 B read, 16 + 96 B written in pieces, 64 B of
+// histogram atomics per key): forty more instructions per key cost 5 - 10 %, a
+// quarter fewer gained 5 %.  fp32 keys take enc_key_exact (correctly
+// rounded divisions and roots, about 700 instructions per lane and key); bf16
+// keys take enc_key_fast (about 225), which reaches the same bits through
+// reciprocals, a table for the magnitude code and its term of the weight, and
+// lane-crossing butterflies of one instruction per value, and hands a wave
+// over to enc_key_exact when one of its keys is outside the range where that
+// is proven.
 #include "pkv_common.h"
 
 namespace {
 
+// 256 threads with four workgroups per CU (LDS: 16 KB histogram + 16 KB table each) and 512 threads with three measure
+// the same; eight waves per SIMD need 64 registers and run a third slower.
 constexpr int kEncThreads = 256;
-constexpr int kEncKeysPerIter = kEncThreads / 16;  // 16
-constexpr int kEncKeysPerWg = 256;
+constexpr int kEncWavesPerSimd = 4;
+constexpr int kEncKeysPerIter = kEncThreads / 16;
+constexpr int kEncKeysPerWg = 16 * kEncKeysPerIter;
+constexpr int kEncAhead = 2;  // iterations whose keys a wave has in flight (1, 2 and 3 measure the same)
 
-__constant__ float c_thresholds[7] = {0.08447265625f, 0.169921875f, 0.2578125f, 0.349609375f,
-                                      0.44921875f,    0.55859375f,  0.69140625f};
-__constant__ float c_centers[8] = {0.0419921875f, 0.126953125f, 0.212890625f, 0.302734375f,
-                                   0.396484375f,  0.5f,         0.6171875f,   0.76171875f};
+#define PKV_ENC_THRESHOLDS 0.08447265625f, 0.169921875f, 0.2578125f, 0.349609375f, 0.44921875f, 0.55859375f, 0.69140625f
+#define PKV_ENC_CENTERS 0.0419921875f, 0.126953125f, 0.212890625f, 0.302734375f, 0.396484375f, 0.5f, 0.6171875f, 0.76171875f
+__constant__ float c_thresholds[7] = {PKV_ENC_THRESHOLDS};
+__constant__ float c_centers[8] = {PKV_ENC_CENTERS};
+constexpr float kEncThresholds[7] = {PKV_ENC_THRESHOLDS};
+constexpr float kEncCenters[8] = {PKV_ENC_CENTERS};
 
 // Adds a workgroup's 16 x 256 histogram to a row's cluster sizes.  Two neighbouring counters travel in one 64-bit
 // atomic where the row is 8-byte aligned (a counter would have to pass 2^32 to carry into its neighbour; they
@@ -59,12 +75,16 @@ struct EncOut {
 
 // One key's block, every operation in the reference's order with correctly rounded division and square root.
 // BF16 = the rounding chain of the reference's bf16 tensors (compile-time, so that no rounding point branches).
+// Block owned by lane l of a row of 16 (the inverse of l = s0*1 ^ s1*2 ^ s2*7 ^ s3*15).
+__device__ __forceinline__ int enc_block_of_lane(int l) { return l ^ ((l & 4) ? 3 : 0) ^ ((l & 8) ? 4 : 0); }
+constexpr int kEncLaneXor4 = 7, kEncLaneXor8 = 15;  // lane distance to the blocks s ^ 4 and s ^ 8
+
 template <bool BF16>
 __device__ __forceinline__ void enc_key_exact(const float (&x)[8], const float (&sg)[8], int s, bool rerank,
                                               const float *s_centers, EncOut &o) {
   constexpr int dtype = BF16 ? PKV_DTYPE_BF16 : PKV_DTYPE_F32;
   float y[8];
-  const float n = pkv_normalize_rotate_16(x, sg, s, dtype, y);
+  const float n = pkv_normalize_rotate_16<kEncLaneXor4, kEncLaneXor8>(x, sg, s, dtype, y);
   uint32_t code = 0;
 #pragma unroll
   for (int j = 0; j < 8; ++j) code |= (y[j] >= 0.0f) ? (1u << j) : 0u;
@@ -108,55 +128,75 @@ __device__ __forceinline__ void enc_key_exact(const float (&x)[8], const float (
 // guarantee; a key that fails them is encoded by enc_key_exact instead.  The two square roots have no such
 // structure: the hardware square root (1 ulp) is used unless it lands within 4 ulp of a bf16 rounding boundary.
 
-constexpr int kMagTableBits = 10;                    // bf16 patterns 0x3C00 .. 0x3FFF: 2^-7 <= |u| < 2
-constexpr uint32_t kMagTableLo = 0x3C000000u, kMagTableHi = 0x3FFF0000u;
+// What the bf16 chain does with one component u of a block's direction depends on the bf16 pattern of |u| alone:
+// its magnitude code t (the number of thresholds below |u|) and its term of the weight's denominator,
+// bf16(centre[t] * |u|).  Both come from one 8-byte table entry indexed by the low 11 bits of the pattern, which
+// covers 2^-15 <= |u| < 2 (patterns 0x3800 .. 0x3FFF); |u| never reaches 2, and a wave that holds a smaller |u|
+// recomputes those terms by the formula (code 0, centre[0]).  The table is a constant of the library's device image;
+// a workgroup copies its 16 KB into LDS.
+constexpr int kMagTableBits = 11;
+constexpr int kMagEntries = 1 << kMagTableBits;
+constexpr uint32_t kMagTableLo = 0x38000000u;  // 2^-15
+constexpr float kMagTableLoF = 0x1p-15f;
+
+constexpr uint32_t enc_cx_bf16_round_bits(float f) {  // round to nearest even; positive normal numbers
+  uint32_t b = __builtin_bit_cast(uint32_t, f);
+  b += 0x7fffu + ((b >> 16) & 1u);
+  return b & 0xffff0000u;
+}
+struct EncTables {
+  uint32_t mag[2 * kMagEntries];  // {magnitude code, bf16(centre * |u|) as fp32 bits} for pattern kMagTableLo >> 16 + i
+  uint32_t spread[256];           // bit j of the index moved to bit 4j + 3
+  constexpr EncTables() : mag{}, spread{} {
+    for (int i = 0; i < kMagEntries; ++i) {
+      const float v = __builtin_bit_cast(float, kMagTableLo + ((uint32_t)i << 16));
+      int t = 0;
+      for (int k = 0; k < 7; ++k) t += (kEncThresholds[k] < v) ? 1 : 0;
+      mag[2 * i] = (uint32_t)t;
+      mag[2 * i + 1] = enc_cx_bf16_round_bits(kEncCenters[t] * v);
+    }
+    for (int c = 0; c < 256; ++c) {
+      uint32_t sp = 0;
+      for (int j = 0; j < 8; ++j) sp |= ((uint32_t)(c >> j) & 1u) << (4 * j + 3);
+      spread[c] = sp;
+    }
+  }
+};
+__device__ __align__(16) const EncTables g_enc_tables = EncTables();
 
 template <int CTRL>
 __device__ __forceinline__ float enc_dpp(float v) {  // bound_ctrl set, so that the move folds into the add that uses it
   return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), CTRL, 0xf, 0xf, true));
 }
-__device__ __forceinline__ float enc_flip(float v, uint32_t sign_mask) {
-  return __uint_as_float(__float_as_uint(v) ^ sign_mask);
-}
-
-// v + (value of lane ^ 4): banks 0 and 2 of a row of 16 lanes read four lanes up, banks 1 and 3 four lanes down.
-// The leading wait covers the two states the hardware needs between a vector write and a lane-crossing read of
-// the same register.
-__device__ __forceinline__ float enc_sum_xor4(float v) {
-  float d;
+// One Walsh-Hadamard stage across lanes in one instruction per value: held' = held(partner) * c + held with
+// c = +1 in the lanes whose block index has the stage's bit clear and -1 in the others.  Where c = +1 that is the
+// stage's own sum; where c = -1 it is own - partner, the NEGATIVE of the stage's partner - own (negation commutes
+// with rounding to nearest).  A lane therefore carries its value times (-1)^(number of set bits among the stages
+// done so far), the same factor in both lanes of every later pair, and the factor left after the four stages, the
+// parity of the block index, is taken out by the sign of the lane's final scale.  (A difference that is exactly zero
+// keeps +0 where the negated form would hold -0; zeros that reach the result send the key to enc_key_exact.)
+// The compiler does not fold the move into a fused multiply-add, hence the assembly: the four stages of eight values.
+// The leading wait covers the two states the hardware needs between a vector write and a lane-crossing read of the
+// same register; inside the block a value is read eight instructions after it was written.
+#define PKV_ENC_STAGE(CTL, C)                                   \
+  "v_fmac_f32_dpp %0, %0, " C " " CTL " row_mask:0xf bank_mask:0xf\n\t" \
+  "v_fmac_f32_dpp %1, %1, " C " " CTL " row_mask:0xf bank_mask:0xf\n\t" \
+  "v_fmac_f32_dpp %2, %2, " C " " CTL " row_mask:0xf bank_mask:0xf\n\t" \
+  "v_fmac_f32_dpp %3, %3, " C " " CTL " row_mask:0xf bank_mask:0xf\n\t" \
+  "v_fmac_f32_dpp %4, %4, " C " " CTL " row_mask:0xf bank_mask:0xf\n\t" \
+  "v_fmac_f32_dpp %5, %5, " C " " CTL " row_mask:0xf bank_mask:0xf\n\t" \
+  "v_fmac_f32_dpp %6, %6, " C " " CTL " row_mask:0xf bank_mask:0xf\n\t" \
+  "v_fmac_f32_dpp %7, %7, " C " " CTL " row_mask:0xf bank_mask:0xf\n\t"
+__device__ __forceinline__ void enc_lane_stages(float (&t)[8], float c1, float c2, float c4, float c8) {
   asm("s_nop 1\n\t"
-      "v_add_f32_dpp %0, %1, %1 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
-      "v_add_f32_dpp %0, %1, %1 row_shr:4 row_mask:0xf bank_mask:0xa"
-      : "=&v"(d)
-      : "v"(v));
-  return d;
+      PKV_ENC_STAGE("quad_perm:[1,0,3,2]", "%8")
+      PKV_ENC_STAGE("quad_perm:[2,3,0,1]", "%9")
+      PKV_ENC_STAGE("row_half_mirror", "%10")
+      PKV_ENC_STAGE("row_mirror", "%11")
+      : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(t[4]), "+v"(t[5]), "+v"(t[6]), "+v"(t[7])
+      : "v"(c1), "v"(c2), "v"(c4), "v"(c8));
 }
-
-// Walsh-Hadamard stage across lane ^ 4 for eight values: lanes with bit 2 clear get t + other, the rest other - t.
-__device__ __forceinline__ void enc_butterfly_xor4(float (&t)[8]) {
-  float d[8];
-  asm("s_nop 1\n\t"
-      "v_add_f32_dpp %0, %8, %8 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
-      "v_sub_f32_dpp %0, %8, %8 row_shr:4 row_mask:0xf bank_mask:0xa\n\t"
-      "v_add_f32_dpp %1, %9, %9 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
-      "v_sub_f32_dpp %1, %9, %9 row_shr:4 row_mask:0xf bank_mask:0xa\n\t"
-      "v_add_f32_dpp %2, %10, %10 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
-      "v_sub_f32_dpp %2, %10, %10 row_shr:4 row_mask:0xf bank_mask:0xa\n\t"
-      "v_add_f32_dpp %3, %11, %11 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
-      "v_sub_f32_dpp %3, %11, %11 row_shr:4 row_mask:0xf bank_mask:0xa\n\t"
-      "v_add_f32_dpp %4, %12, %12 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
-      "v_sub_f32_dpp %4, %12, %12 row_shr:4 row_mask:0xf bank_mask:0xa\n\t"
-      "v_add_f32_dpp %5, %13, %13 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
-      "v_sub_f32_dpp %5, %13, %13 row_shr:4 row_mask:0xf bank_mask:0xa\n\t"
-      "v_add_f32_dpp %6, %14, %14 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
-      "v_sub_f32_dpp %6, %14, %14 row_shr:4 row_mask:0xf bank_mask:0xa\n\t"
-      "v_add_f32_dpp %7, %15, %15 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
-      "v_sub_f32_dpp %7, %15, %15 row_shr:4 row_mask:0xf bank_mask:0xa"
-      : "=&v"(d[0]), "=&v"(d[1]), "=&v"(d[2]), "=&v"(d[3]), "=&v"(d[4]), "=&v"(d[5]), "=&v"(d[6]), "=&v"(d[7])
-      : "v"(t[0]), "v"(t[1]), "v"(t[2]), "v"(t[3]), "v"(t[4]), "v"(t[5]), "v"(t[6]), "v"(t[7]));
-#pragma unroll
-  for (int j = 0; j < 8; ++j) t[j] = d[j];
-}
+#undef PKV_ENC_STAGE
 
 // bf16(sqrt(a)) from the hardware square root (1 ulp); where the fp32 root lies within 4 ulp of a bf16 rounding
 // boundary the correctly rounded root decides.
@@ -179,11 +219,10 @@ __device__ __forceinline__ float enc_min_abs8(const float (&v)[8]) {
 // The bf16 chain of enc_key_exact without a division.  w[] = the lane's eight bf16 components as loaded (two per
 // word), sgw[] = the SRHT sign bits in the same packing.  Returns true when this lane's key needs enc_key_exact
 // (norm or radius outside [1e-8, 2^60], or a component below 2^-40 in magnitude, zero included); o is then
-// unspecified.  sm1/sm2/sm8 = the sign bit where the lane's block index has bit 0/1/3 set.  s_mag[p - 0x3C00] =
-// {magnitude code, magnitude centre} for the bf16 pattern p of |u|; s_spread[c] = bit j of the sign code c moved to
-// bit 4j + 3.
-__device__ __forceinline__ bool enc_key_fast(const uint32_t (&w)[4], const uint32_t (&sgw)[4], uint32_t sm1,
-                                             uint32_t sm2, uint32_t sm8, bool rerank, const uint2 *s_mag,
+// unspecified.  c1/c2/c4/c8 = -1 where the lane's block index has bit 0/1/2/3 set, else +1; scale = 1/sqrt(128)
+// with the sign (-1)^(set bits of the block index).  s_mag / s_spread = the workgroup's copy of g_enc_tables.
+__device__ __forceinline__ bool enc_key_fast(const uint32_t (&w)[4], const uint32_t (&sgw)[4], float c1, float c2,
+                                             float c4, float c8, float scale, bool rerank, const uint2 *s_mag,
                                              const uint32_t *s_spread, EncOut &o) {
   float x[8];  // components times their SRHT sign: the sign commutes with the division and its rounding
 #pragma unroll
@@ -198,10 +237,10 @@ __device__ __forceinline__ bool enc_key_fast(const uint32_t (&w)[4], const uint3
   float acc = x[0] * x[0];
 #pragma unroll
   for (int j = 1; j < 8; ++j) acc = __builtin_fmaf(x[j], x[j], acc);
-  acc = enc_dpp<0xB1>(acc) + acc;   // lane ^ 1
-  acc = enc_dpp<0x4E>(acc) + acc;   // lane ^ 2
-  acc = enc_sum_xor4(acc);
-  acc = enc_dpp<0x128>(acc) + acc;  // lane ^ 8
+  acc = enc_dpp<0xB1>(acc) + acc;   // block ^ 1: lane ^ 1
+  acc = enc_dpp<0x4E>(acc) + acc;   // block ^ 2: lane ^ 2
+  acc = enc_dpp<0x141>(acc) + acc;  // block ^ 4: lane ^ 7 (row_half_mirror)
+  acc = enc_dpp<0x140>(acc) + acc;  // block ^ 8: lane ^ 15 (row_mirror)
   const float n = enc_sqrt_bf16(acc);
   bool bad = !(n >= 1e-8f) || n > 0x1p60f;
   bad |= enc_min_abs8(x) < 0x1p-40f;
@@ -220,44 +259,48 @@ __device__ __forceinline__ bool enc_key_fast(const uint32_t (&w)[4], const uint3
       }
     }
   }
-#pragma unroll
-  for (int j = 0; j < 8; ++j) t[j] = enc_dpp<0xB1>(t[j]) + enc_flip(t[j], sm1);
-#pragma unroll
-  for (int j = 0; j < 8; ++j) t[j] = enc_dpp<0x4E>(t[j]) + enc_flip(t[j], sm2);
-  enc_butterfly_xor4(t);
-#pragma unroll
-  for (int j = 0; j < 8; ++j) t[j] = enc_dpp<0x128>(t[j]) + enc_flip(t[j], sm8);
+  enc_lane_stages(t, c1, c2, c4, c8);
   float y[8];
 #pragma unroll
-  for (int j = 0; j < 8; ++j) y[j] = pkv_bf16_round(t[j] * PKV_HADAMARD_SCALE);
-  bad |= enc_min_abs8(y) < 0x1p-40f;  // no zeros from here on: y >= 0 is the sign bit
+  for (int j = 0; j < 8; ++j) y[j] = pkv_bf16_round(t[j] * scale);
+  // y >= 0 is read off the sign bit, which is wrong for a zero: a key with |y| < 2^-40 somewhere, zero included, goes
+  // to enc_key_exact.  With the rerank outputs that test is made further down, and only in waves that need it.
   uint32_t sneg = 0;
 #pragma unroll
   for (int j = 7; j >= 0; --j) sneg = __builtin_amdgcn_alignbit(sneg, __float_as_uint(y[j]), 31);
   o.code = ~sneg & 0xffu;
-  if (!rerank) return bad;
+  if (!rerank) return bad | (enc_min_abs8(y) < 0x1p-40f);
 
-  float r2 = y[0] * y[0];  // y: bf16 values, magnitudes checked above: exact squares again
+  // y: bf16 values.  Their squares are exact again unless a |y| is below 2^-40, and such a y has |u| = |y| / r below
+  // 2^-15 (r <= 2^-24 is sent to enc_key_exact as well), which the test on |u| below catches.
+  float r2 = y[0] * y[0];
 #pragma unroll
   for (int j = 1; j < 8; ++j) r2 = __builtin_fmaf(y[j], y[j], r2);
   const float r = enc_sqrt_bf16(r2);
-  bad |= !(r >= 1e-8f) || r > 0x1p60f;
+  bad |= !(r >= 0x1p-24f) || r > 0x1p60f;
   const float r_inv = __builtin_amdgcn_rcpf(r);
-  float au[8];
+  float u[8];
   uint2 e[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    au[j] = fabsf(pkv_bf16_round(y[j] * r_inv));
-    const float cl = __builtin_amdgcn_fmed3f(au[j], __uint_as_float(kMagTableLo), __uint_as_float(kMagTableHi));
-    const uint32_t byte_off = __builtin_amdgcn_ubfe(__float_as_uint(cl), 13, kMagTableBits + 3);  // 8 * (pattern - 0x3C00)
+    u[j] = pkv_bf16_round(y[j] * r_inv);
+    const uint32_t byte_off = __builtin_amdgcn_ubfe(__float_as_uint(u[j]), 13, kMagTableBits + 3);  // 8 * (pattern & 0x7ff)
     e[j] = *(const uint2 *)((const char *)s_mag + byte_off);
+  }
+  if (__builtin_amdgcn_ballot_w64(enc_min_abs8(u) < kMagTableLoF) != 0) {  // about one wave in thirty
+    bad |= enc_min_abs8(y) < 0x1p-40f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float au = fabsf(u[j]);
+      if (au < kMagTableLoF) e[j] = make_uint2(0u, __float_as_uint(pkv_bf16_round(kEncCenters[0] * au)));
+    }
   }
   uint32_t mags = 0;
   float alpha = 0.f;
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     mags = __builtin_amdgcn_alignbit(e[j].x, mags, 4);  // the code enters at the top nibble; after 8 steps code j sits in nibble j
-    const float p = pkv_bf16_round(__uint_as_float(e[j].y) * au[j]);
+    const float p = __uint_as_float(e[j].y);
     alpha = (j == 0) ? p : alpha + p;
   }
   if (alpha < 1e-6f) alpha = 1e-6f;
@@ -270,40 +313,37 @@ __device__ __forceinline__ bool enc_key_fast(const uint32_t (&w)[4], const uint3
   return bad;
 }
 
-template <bool BF16>
-__global__ __launch_bounds__(kEncThreads) __attribute__((amdgpu_waves_per_eu(6, 6))) void pkv_encode_kernel(
+// ALL: codes, 4-bit records, weights and cluster sizes are all written (the caller's pointers are all set), so the
+// loop body has no branch around a store.  Loads and stores retire through one in-order counter; with a store that
+// may or may not have been issued after the load of the next key, the only safe wait for that key is "everything
+// outstanding", stores included.  Without the branches the wait names the exact count and the stores stay in flight.
+template <bool BF16, bool ALL>
+__global__ __launch_bounds__(kEncThreads) __attribute__((amdgpu_waves_per_eu(kEncWavesPerSimd, kEncWavesPerSimd))) void pkv_encode_kernel(
     const void *__restrict__ keys, int n_kv_heads, int64_t n_keys, int64_t k_stride_b, int64_t k_stride_h,
     int64_t k_stride_key, const float *__restrict__ signs, uint8_t *__restrict__ codes, int64_t cs_b, int64_t cs_h,
     int64_t cs_key, int64_t cs_sub, uint8_t *__restrict__ nib, int64_t ns_b, int64_t ns_h, int64_t ns_key,
     int64_t ns_sub, uint16_t *__restrict__ weight, int64_t ws_b, int64_t ws_h, int64_t ws_key, int64_t ws_sub,
     int32_t *__restrict__ cluster_counts, int64_t cc_b, int64_t cc_h, int keys_per_wg) {
+  const bool has_nib = ALL || nib, has_weight = ALL || weight, has_hist = ALL || cluster_counts;
   const int row = blockIdx.y;
   const int b = row / n_kv_heads, h = row % n_kv_heads;
   const int tid = threadIdx.x;
-  const int s = tid & 15;   // block (subspace) owned by this lane
+  const int s = enc_block_of_lane(tid & 15);  // block (subspace) owned by this lane
   const int kq = tid >> 4;  // key slot inside the iteration
 
   __shared__ uint32_t s_hist[16 * 256];
-  __shared__ uint2 s_mag[BF16 ? (1 << kMagTableBits) : 1];
+  __shared__ __align__(16) uint2 s_mag[BF16 ? kMagEntries : 2];
   __shared__ float s_centers[8];  // magnitude centres, looked up by code (an LDS read instead of a load from constant memory)
   __shared__ uint32_t s_spread[BF16 ? 256 : 1];
   if (tid < 8) s_centers[tid] = c_centers[tid];
   if (BF16) {
-    uint32_t sp = 0;
+    if (tid < 256) s_spread[tid] = g_enc_tables.spread[tid];
+    const pkv_u32x4 *src = (const pkv_u32x4 *)g_enc_tables.mag;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) sp |= ((uint32_t)(tid >> j) & 1u) << (4 * j + 3);
-    s_spread[tid] = sp;  // kEncThreads == 256: one entry per thread
+    for (int i = 0; i < kMagEntries / 2 / kEncThreads; ++i)
+      ((pkv_u32x4 *)s_mag)[tid + i * kEncThreads] = src[tid + i * kEncThreads];
   }
-  if (BF16) {
-    for (int i = tid; i < (1 << kMagTableBits); i += kEncThreads) {
-      const float v = __uint_as_float(kMagTableLo + ((uint32_t)i << 16));
-      int t = 0;
-#pragma unroll
-      for (int k = 0; k < 7; ++k) t += (c_thresholds[k] < v) ? 1 : 0;
-      s_mag[i] = make_uint2((uint32_t)t, __float_as_uint(c_centers[t]));
-    }
-  }
-  if (cluster_counts)
+  if (has_hist)
     for (int i = tid; i < 16 * 256; i += kEncThreads) s_hist[i] = 0;
   __syncthreads();
 
@@ -314,45 +354,64 @@ __global__ __launch_bounds__(kEncThreads) __attribute__((amdgpu_waves_per_eu(6, 
 #pragma unroll
   for (int p = 0; p < 4; ++p)
     sgw[p] = ((__float_as_uint(sg[2 * p]) >> 16) & 0x8000u) | (__float_as_uint(sg[2 * p + 1]) & 0x80000000u);
-  const uint32_t sm1 = (s & 1) ? 0x80000000u : 0u, sm2 = (s & 2) ? 0x80000000u : 0u, sm8 = (s & 8) ? 0x80000000u : 0u;
-  const bool rerank = nib || weight;
+  const float c1 = (s & 1) ? -1.f : 1.f, c2 = (s & 2) ? -1.f : 1.f, c4 = (s & 4) ? -1.f : 1.f, c8 = (s & 8) ? -1.f : 1.f;
+  const float scale = (__builtin_popcount((unsigned)s) & 1) ? -PKV_HADAMARD_SCALE : PKV_HADAMARD_SCALE;
+  const bool rerank = ALL || nib || weight;
 
-  // every pointer advances by one iteration's 16 keys; lanes past the end of a ragged last block reload its last
-  // key (all lanes take part in the shuffles) and store nothing
+  // Addresses are a wave-uniform base, which advances by one iteration's 16 keys through scalar adds, plus a
+  // 32-bit lane offset that never changes (the launcher checks that the offsets fit).  Lanes past the end of a
+  // ragged last block load its last key (all lanes take part in the lane-crossing steps) and store nothing.
   const int64_t key_begin = (int64_t)blockIdx.x * keys_per_wg;  // < n_keys by the grid's construction
   const int last = (int)((n_keys - key_begin < keys_per_wg) ? n_keys - key_begin : keys_per_wg) - 1;
   constexpr int esize = BF16 ? 2 : 4;
-  const char *krow = (const char *)keys + ((int64_t)b * k_stride_b + (int64_t)h * k_stride_h + key_begin * k_stride_key + 8 * s) * esize;
-  const char *kp = krow + (int64_t)kq * k_stride_key * esize;
-  const char *kp_last = krow + (int64_t)last * k_stride_key * esize;
-  uint8_t *cp = codes + (int64_t)b * cs_b + (int64_t)h * cs_h + (key_begin + kq) * cs_key + (int64_t)s * cs_sub;
-  uint8_t *np = nib ? nib + (int64_t)b * ns_b + (int64_t)h * ns_h + (key_begin + kq) * ns_key + (int64_t)s * ns_sub : nullptr;
-  uint16_t *wp = weight ? weight + (int64_t)b * ws_b + (int64_t)h * ws_h + (key_begin + kq) * ws_key + (int64_t)s * ws_sub : nullptr;
+  const char *k_base = (const char *)keys + ((int64_t)b * k_stride_b + (int64_t)h * k_stride_h + key_begin * k_stride_key) * esize;
+  uint8_t *c_base = codes + (int64_t)b * cs_b + (int64_t)h * cs_h + key_begin * cs_key;
+  uint8_t *n_base = has_nib ? nib + (int64_t)b * ns_b + (int64_t)h * ns_h + key_begin * ns_key : nullptr;
+  char *w_base = has_weight ? (char *)(weight + (int64_t)b * ws_b + (int64_t)h * ws_h + key_begin * ws_key) : nullptr;
+  const uint32_t key_bytes = (uint32_t)(k_stride_key * esize), blk_off = (uint32_t)(8 * s * esize);
+  const uint32_t k_lane = (uint32_t)kq * key_bytes + blk_off;
+  const uint32_t c_lane = (uint32_t)(kq * cs_key + s * cs_sub), n_lane = (uint32_t)(kq * ns_key + s * ns_sub),
+                 w_lane = (uint32_t)(2 * (kq * ws_key + s * ws_sub));
   const int64_t k_step = (int64_t)kEncKeysPerIter * k_stride_key * esize, c_step = (int64_t)kEncKeysPerIter * cs_key,
-                n_step = (int64_t)kEncKeysPerIter * ns_key, w_step = (int64_t)kEncKeysPerIter * ws_key;
-  pkv_u32x4 raw[BF16 ? 1 : 2];  // the next iteration's key, loaded one iteration ahead
-  {
-    const char *src = kq <= last ? kp : kp_last;
-    raw[0] = *(const pkv_u32x4 *)src;
-    if (!BF16) raw[BF16 ? 0 : 1] = *(const pkv_u32x4 *)(src + 16);
+                n_step = (int64_t)kEncKeysPerIter * ns_key, w_step = (int64_t)kEncKeysPerIter * ws_key * 2;
+  // A wave has the keys of its next kEncAhead iterations in flight (one iteration is about two microseconds of vector
+  // work for the four waves of a SIMD).
+  constexpr int kW = BF16 ? 1 : 2;  // 16-byte words per lane and key
+  pkv_u32x4 raw[kEncAhead][kW];
+#pragma unroll
+  for (int a = 0; a < kEncAhead; ++a) {
+    const int rel = a * kEncKeysPerIter + kq;
+    if (a * kEncKeysPerIter <= last) {  // uniform
+      const uint32_t off = rel <= last ? (uint32_t)a * kEncKeysPerIter * key_bytes + k_lane : (uint32_t)last * key_bytes + blk_off;
+      raw[a][0] = *(const pkv_u32x4 *)(k_base + off);
+      if (!BF16) raw[a][kW - 1] = *(const pkv_u32x4 *)(k_base + off + 16);
+    }
   }
-  for (int rel = kq; rel - kq <= last; rel += kEncKeysPerIter, cp += c_step, np += n_step, wp += w_step) {
-    const bool active = rel <= last;
-    pkv_u32x4 cur[BF16 ? 1 : 2];
-    cur[0] = raw[0];
-    if (!BF16) cur[BF16 ? 0 : 1] = raw[BF16 ? 0 : 1];
-    kp += k_step;
-    if (rel - kq + kEncKeysPerIter <= last) {  // uniform: another iteration follows
-      const char *src = rel + kEncKeysPerIter <= last ? kp : kp_last;
-      raw[0] = *(const pkv_u32x4 *)src;
-      if (!BF16) raw[BF16 ? 0 : 1] = *(const pkv_u32x4 *)(src + 16);
+  k_base += (kEncAhead - 1) * k_step;
+  for (int first = 0; first <= last; first += kEncKeysPerIter, c_base += c_step, n_base += n_step, w_base += w_step) {
+    const bool active = kq <= last - first;
+    pkv_u32x4 cur[kW];
+#pragma unroll
+    for (int q = 0; q < kW; ++q) cur[q] = raw[0][q];
+#pragma unroll
+    for (int a = 0; a + 1 < kEncAhead; ++a)
+#pragma unroll
+      for (int q = 0; q < kW; ++q) raw[a][q] = raw[a + 1][q];
+    k_base += k_step;
+    // the iteration loaded now holds the block's keys first + 16 * kEncAhead .. + lim
+    const int lim = last - first - kEncAhead * kEncKeysPerIter;
+    if (lim >= 0) {  // uniform: that iteration exists
+      uint32_t off = k_lane;
+      if (lim < kEncKeysPerIter - 1) off = kq <= lim ? k_lane : (uint32_t)lim * key_bytes + blk_off;  // uniform: it is ragged
+      raw[kEncAhead - 1][0] = *(const pkv_u32x4 *)(k_base + off);
+      if (!BF16) raw[kEncAhead - 1][kW - 1] = *(const pkv_u32x4 *)(k_base + off + 16);
     }
     EncOut o;
     bool exact = true;
     float x[8];
     if (BF16) {
       const uint32_t w[4] = {cur[0].x, cur[0].y, cur[0].z, cur[0].w};
-      exact = __builtin_amdgcn_ballot_w64(enc_key_fast(w, sgw, sm1, sm2, sm8, rerank, s_mag, s_spread, o)) != 0;
+      exact = __builtin_amdgcn_ballot_w64(enc_key_fast(w, sgw, c1, c2, c4, c8, scale, rerank, s_mag, s_spread, o)) != 0;
       if (exact) {
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
@@ -364,7 +423,7 @@ __global__ __launch_bounds__(kEncThreads) __attribute__((amdgpu_waves_per_eu(6, 
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         x[j] = __uint_as_float(cur[0][j]);
-        x[4 + j] = __uint_as_float(cur[BF16 ? 0 : 1][j]);
+        x[4 + j] = __uint_as_float(cur[kW - 1][j]);
       }
     }
     if (exact) {  // the whole wave: every lane takes part in the shuffles
@@ -375,14 +434,32 @@ __global__ __launch_bounds__(kEncThreads) __attribute__((amdgpu_waves_per_eu(6, 
       enc_key_exact<BF16>(x, sg, s, rerank, s_centers, o);
     }
 
-    if (active) {
-      *cp = (uint8_t)o.code;
-      if (cluster_counts) atomicAdd(&s_hist[s * 256 + o.code], 1u);
-      if (nib) *(uint32_t *)np = o.packed;
-      if (weight) *wp = (uint16_t)o.wbits;
+    // the empty statement keeps the lane offsets apart from the bases, so that the stores address
+    // scalar base + lane offset instead of three 64-bit lane pointers that would each need an add per iteration
+    uint32_t c_off = c_lane, n_off = n_lane, w_off = w_lane;
+    if (ALL) {
+      // No branch around the stores (see above): a lane past the end of a ragged block holds the block's last key
+      // and writes that key's results once more, to the same place.
+      if (last - first < kEncKeysPerIter - 1) {  // uniform
+        const uint32_t kk = (uint32_t)(kq < last - first ? kq : last - first);
+        c_off = kk * (uint32_t)cs_key + (uint32_t)(s * cs_sub);
+        n_off = kk * (uint32_t)ns_key + (uint32_t)(s * ns_sub);
+        w_off = 2 * (kk * (uint32_t)ws_key + (uint32_t)(s * ws_sub));
+      }
+      asm volatile("" : "+v"(c_off), "+v"(n_off), "+v"(w_off));
+      c_base[c_off] = (uint8_t)o.code;
+      *(uint32_t *)(n_base + n_off) = o.packed;
+      *(uint16_t *)(w_base + w_off) = (uint16_t)o.wbits;
+      if (active) atomicAdd(&s_hist[s * 256 + o.code], 1u);
+    } else if (active) {
+      asm volatile("" : "+v"(c_off), "+v"(n_off), "+v"(w_off));
+      c_base[c_off] = (uint8_t)o.code;
+      if (has_hist) atomicAdd(&s_hist[s * 256 + o.code], 1u);
+      if (has_nib) *(uint32_t *)(n_base + n_off) = o.packed;
+      if (has_weight) *(uint16_t *)(w_base + w_off) = (uint16_t)o.wbits;
     }
   }
-  if (cluster_counts) {
+  if (has_hist) {
     __syncthreads();
     pkv_flush_cluster_hist(s_hist, cluster_counts + (int64_t)b * cc_b + (int64_t)h * cc_h, tid, kEncThreads);
   }
@@ -430,16 +507,28 @@ extern "C" int pkv_encode_append(const void *keys, int dtype, int bs, int n_kv_h
               "keys must be 16-byte aligned with 16-byte-multiple strides");
   PKV_REQUIRE(!nib || (pkv_aligned(nib, 4) && ns_b % 4 == 0 && ns_h % 4 == 0 && ns_key % 4 == 0 && ns_sub % 4 == 0),
               "packed 4-bit blocks must be 4-byte aligned");
-  // 256 keys per workgroup: measured against 64 .. 1024 and against one resident set of larger workgroups, this
-  // balances the per-workgroup set-up (tables, histogram flush) against the partial last round of workgroups.
+  // a lane's byte offsets inside one iteration's keys and 16 blocks are kept in 32 bits
+  const int64_t lim = (int64_t)1 << 31;
+  PKV_REQUIRE(k_stride_key >= 0 && cs_key >= 0 && cs_sub >= 0 && ns_key >= 0 && ns_sub >= 0 && ws_key >= 0 && ws_sub >= 0,
+              "pkv_encode_append: negative key or block strides are not supported");
+  PKV_REQUIRE(kEncKeysPerIter * k_stride_key * 4 + 512 < lim && kEncKeysPerIter * cs_key + 16 * cs_sub < lim &&
+                  kEncKeysPerIter * ns_key + 16 * ns_sub < lim && 2 * (kEncKeysPerIter * ws_key + 16 * ws_sub) < lim,
+              "pkv_encode_append: key or block strides too large (a lane's offsets inside one iteration's keys must stay below 2 GiB)");
+  // 256 keys per workgroup: measured against 128 .. 4096, this balances the per-workgroup set-up (tables,
+  // histogram flush) against the partial last round of workgroups.
   const int64_t rows = (int64_t)bs * n_kv_heads;
   const int64_t per_wg = kEncKeysPerWg;
   dim3 grid((unsigned)((n_keys + per_wg - 1) / per_wg), (unsigned)rows);
-#define PKV_ENC(BF)                                                                                                  \
-  hipLaunchKernelGGL(pkv_encode_kernel<BF>, grid, dim3(kEncThreads), 0, (hipStream_t)stream, keys, n_kv_heads, n_keys, \
-                     k_stride_b, k_stride_h, k_stride_key, signs, codes, cs_b, cs_h, cs_key, cs_sub, nib, ns_b, ns_h,  \
-                     ns_key, ns_sub, weight, ws_b, ws_h, ws_key, ws_sub, cluster_counts, cc_b, cc_h, (int)per_wg)
-  if (dtype == PKV_DTYPE_BF16) PKV_ENC(true); else PKV_ENC(false);
+#define PKV_ENC(BF, ALL)                                                                                               \
+  hipLaunchKernelGGL((pkv_encode_kernel<BF, ALL>), grid, dim3(kEncThreads), 0, (hipStream_t)stream, keys, n_kv_heads,  \
+                     n_keys, k_stride_b, k_stride_h, k_stride_key, signs, codes, cs_b, cs_h, cs_key, cs_sub, nib, ns_b, \
+                     ns_h, ns_key, ns_sub, weight, ws_b, ws_h, ws_key, ws_sub, cluster_counts, cc_b, cc_h, (int)per_wg)
+  const bool all = nib && weight && cluster_counts;
+  if (dtype == PKV_DTYPE_BF16) {
+    if (all) PKV_ENC(true, true); else PKV_ENC(true, false);
+  } else {
+    if (all) PKV_ENC(false, true); else PKV_ENC(false, false);
+  }
 #undef PKV_ENC
   PKV_LAUNCH_CHECK("pkv_encode_kernel");
   return PKV_OK;
