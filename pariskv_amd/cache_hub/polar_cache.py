@@ -25,7 +25,7 @@ from typing import Optional
 
 import torch
 
-from .. import ops
+from .. import ops, ranges
 from .cache import KV_Cache
 from .zones import LayerZones
 
@@ -267,9 +267,11 @@ class polar_cache(KV_Cache):
         if n == 0:
             return
         sl = slice(abs0, abs0 + n)
+        ranges.push("batch_encode+cluster_count")  # the reference's prefill_step1_batch_encode / prefill_step3_cluster_count
         ops.encode_append(keys_bhsd, self._srht_signs, self.codebook_gpu[layer_idx][b0:b1, :, :, sl],
                           self.key_4bit_packed_gpu[layer_idx][b0:b1, :, :, sl], self.key_block_weight_gpu[layer_idx][b0:b1, :, :, sl],
                           self.cluster_key_counts_gpu[layer_idx][b0:b1])
+        ranges.pop()
 
     # ------------------------------------------------------------- prefill
     def prefill_update_kv_cache(self, query_states, key_states, value_states, layer_idx, batch_idx):
@@ -341,7 +343,8 @@ class polar_cache(KV_Cache):
         if layer_idx == 0:
             self.context += 1
         if refresh is not None:
-            self._update_polar_index(layer_idx, refresh)
+            with ranges.span("update_polar_index"):  # the reference's (commented-out) range, polar_cache_adaptivek_varlen.py:1214
+                self._update_polar_index(layer_idx, refresh)
         return None, None
 
     def _update_polar_index(self, layer_idx: int, r) -> None:
@@ -472,7 +475,12 @@ class polar_cache(KV_Cache):
             bound.segs[local_seg].n_rows = z.dense_tail_len
         self._wait_offload(layer_idx)
         self.last_topk_indices = out_ids  # the selected set; its order is fixed but not by score (the sort is left out)
-        return bound.launch(q)  # retrieval, gather and attention from one host call
+        # retrieval, gather and attention from one host call: the range covers what the reference's
+        # "collision_based_topk_batch", gather and attention ranges cover
+        if ranges.enabled:
+            with ranges.span("collision_topk+gather+attention"):
+                return bound.launch(q)
+        return bound.launch(q)
 
     def _bind_step(self, layer_idx, q, n_keys):
         """Build and validate the argument blocks of this layer's decode step; they stay valid until the next index

@@ -25,7 +25,7 @@ import os
 
 import torch
 
-from .. import ops
+from .. import ops, ranges
 from .polar_cache import polar_cache as _polar_cache_base
 
 
@@ -182,6 +182,11 @@ class polar_cache(_polar_cache_base):
         # (b, h) receives its own k rows at the head of its slice of the dense buffer) -> attention.  The reference
         # packs the indices and reads the largest k back to the host to size its launch (:1597-1644); the gather and
         # the attention take the per-row count from device memory instead, so the step never waits for the GPU.
+        # The range covers the reference's "collision_based_topk_batch", "adaptive_k0_pre", "adaptive_k1_qk_logits",
+        # "adaptive_k2_cuda_kernel", "pack_sink_local", "h2d_gather_kv_packed" and "compute_attention_varlen" (:1483-1771).
+        if ranges.enabled:
+            with ranges.span("collision_topk+adaptive_k+gather+attention_varlen"):
+                return bound.launch(q)
         return bound.launch(q)
 
     def _bind_adaptive_step(self, layer_idx, q, n_keys):

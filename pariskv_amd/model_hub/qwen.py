@@ -18,7 +18,7 @@ from dataclasses import dataclass
 import torch
 import torch.nn.functional as F
 
-from .. import ops
+from .. import ops, ranges
 from ..attn_hub import polar_decode_attn
 
 
@@ -154,8 +154,12 @@ class QwenModel:
             q = q.view(bsz, -1, self.num_heads, self.head_dim)
             k = k.view(bsz, -1, self.num_key_value_heads, self.head_dim)
         v = v.reshape(bsz, -1, self.num_key_value_heads, self.head_dim)
+        ranges.push("decode_update_kv_cache")
         k, v = self.kv_cache.decode_update_kv_cache(k, v, layer_idx)
+        ranges.pop()
+        ranges.push("decode_attention")
         attn_out = self.decode_attention(q, k, v, layer_idx)
+        ranges.pop()
         attn_out_dim = attn_out.shape[-2] * attn_out.shape[-1]
         hidden_states = residual + self.wo(attn_out, layer, bsz, seq_len, attn_out_dim)
         residual = hidden_states
@@ -176,8 +180,12 @@ class QwenModel:
                                 table_for=target)
         v = qkv[..., (self.num_heads + self.num_key_value_heads) * self.head_dim:].reshape(bsz, -1, self.num_key_value_heads,
                                                                                              self.head_dim)
+        ranges.push("decode_update_kv_cache")  # the reference's ranges of the same names, model_hub/LLM.py:173-183
         k, v = self.kv_cache.decode_update_kv_cache(k, v, layer_idx)
+        ranges.pop()
+        ranges.push("decode_attention")
         attn_out = self.decode_attention(q, k, v, layer_idx)
+        ranges.pop()
         return self.wo(attn_out, layer, bsz, seq_len, attn_out.shape[-2] * attn_out.shape[-1])
 
     def decode_forward(self, inputs_ids):

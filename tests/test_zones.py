@@ -101,3 +101,19 @@ def test_refresh_slots_match_reference_layer0():
         assert (r is not None) == (buf > 0 and buf % I == 0)
         if r is not None:
             pending = True
+
+
+def test_ranges_are_no_ops_when_switched_off():
+    """Range markers cost nothing and need no library unless PARISKV_RANGES=1 is set before the import."""
+    import importlib
+    import os
+
+    os.environ.pop("PARISKV_RANGES", None)
+    from pariskv_amd import ranges
+
+    ranges = importlib.reload(ranges)
+    assert ranges.enabled is False
+    ranges.push("a")
+    ranges.pop()
+    with ranges.span("b"):
+        pass
