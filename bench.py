@@ -791,10 +791,41 @@ def main():
         t_one, n_one, _ = time_torch(1, 12.0)
         torch.set_num_threads(default_threads)
         overlap = sum(len(np.intersect1d(tids.view(R, K)[r].numpy(), ref_ids[r])) for r in rows) / float(R * K)
+        # the gather alone by the reference's own host code (cache_hub/gather/gather_cpu.cpp, built into oracle/_ref)
+        from oracle import build_ref
+
+        ref_gather = None
+        ref_mod = build_ref.load()
+        if ref_mod is not None:
+            gids = torch.from_numpy(np.stack(ref_ids)).view(bs, H, K)
+            gk, gv = torch.empty(bs, H, K, D, dtype=kcpu.dtype), torch.empty(bs, H, K, D, dtype=kcpu.dtype)
+
+            def ref_gather_step():
+                ref_mod.gather_kv_out_cpu(kcpu, gids, gk)
+                ref_mod.gather_kv_out_cpu(vcpu, gids, gv)
+
+            ref_gather = {"kind": "reference", "bytes": 2 * R * K * D * 2}
+            for name, nt in (("default_threads", default_threads), ("one_thread", 1)):
+                torch.set_num_threads(nt)
+                ref_gather_step()
+                ts = []
+                for _ in range(20):
+                    t0 = time.perf_counter()
+                    ref_gather_step()
+                    ts.append(time.perf_counter() - t0)
+                ts.sort()
+                ref_gather[name] = {"value_us": round(ts[10] * 1e6, 1), "threads": nt}
+            torch.set_num_threads(default_threads)
+            step(0)  # the GPU's rows of the same layer and ids, gathered over PCIe
+            torch.cuda.synchronize()
+            ref_gather["rows_equal_the_uva_gather"] = bool(
+                parity and torch.equal(gk.view(torch.int16), dst_k.cpu().view(torch.int16)) and
+                torch.equal(gv.view(torch.int16), dst_v.cpu().view(torch.int16)))
         result["cpu_baseline"] = {"value": round(med * 1e6, 1), "unit": "us/layer/decode-step", "cores": 1, "kind": "port",
                                   "sample": f"all {R} rows of one layer at the full workload (C oracle, single thread, "
                                             f"host gather included), median of {len(times)} repetitions",
                                   "host_cpus": os.cpu_count(),
+                                  "host_gather_alone_by_the_reference_build": ref_gather,
                                   "torch_cpu_default_threads": {"value": round(t_def * 1e6, 1), "threads": default_threads,
                                                                 "repetitions": n_def},
                                   "torch_cpu_one_thread": {"value": round(t_one * 1e6, 1), "threads": 1,

@@ -98,3 +98,45 @@ def test_gather_cpu_host_function():
     idx[0, 0, 0] = 50
     with pytest.raises(RuntimeError, match="out of bounds"):
         ext.gather_kv_out_cpu(src, idx, out)
+
+
+def test_gather_cpu_equals_the_reference_build():
+    """pkv_gather_cpu and the oracle's gather_rows against the reference's own gather_cpu.cpp, compiled by
+    oracle/build_ref.py into oracle/_ref (skipped where that build is absent)."""
+    import numpy as np
+    import torch
+
+    from oracle import build_ref
+    from oracle import pkv_oracle as O
+    from pariskv_amd.cache_hub.gather import load_gather_ext
+
+    ref = build_ref.load()
+    if ref is None:
+        pytest.skip("oracle/_ref is not built (python oracle/build_ref.py needs the reference tree)")
+    ext = load_gather_ext()
+    g = torch.Generator().manual_seed(3)
+    for dtype, shape, K in ((torch.bfloat16, (2, 8, 3000, 128), 100), (torch.float32, (1, 3, 77, 128), 77),
+                            (torch.float16, (3, 2, 500, 64), 1)):
+        src = torch.randn(*shape, generator=g).to(dtype)
+        idx = torch.randint(0, shape[2], (shape[0], shape[1], K), generator=g)
+        want = torch.empty(shape[0], shape[1], K, shape[3], dtype=dtype)
+        got = torch.full_like(want, 7)
+        ref.gather_kv_out_cpu(src, idx, want)
+        ext.gather_kv_out_cpu(src, idx, got)
+        assert torch.equal(got.view(torch.uint8), want.view(torch.uint8))
+        for b in range(shape[0]):
+            for h in range(shape[1]):
+                rows = O.gather_rows(src[b, h].view(torch.uint8).numpy(), idx[b, h].numpy())
+                assert np.array_equal(rows, want[b, h].view(torch.uint8).numpy())
+    # rows that are not contiguous, and an output that is a slice of a larger buffer
+    src_t = torch.randn(2, 3, 128, 50, generator=g).transpose(2, 3)
+    idx = torch.randint(0, 50, (2, 3, 9), generator=g)
+    big_w, big_g = torch.zeros(2, 3, 20, 128), torch.zeros(2, 3, 20, 128)
+    ref.gather_kv_out_cpu(src_t, idx, big_w[:, :, 4:13])
+    ext.gather_kv_out_cpu(src_t, idx, big_g[:, :, 4:13])
+    assert torch.equal(big_g, big_w)
+    idx[1, 2, 8] = -1
+    with pytest.raises(RuntimeError, match="out of bounds"):
+        ref.gather_kv_out_cpu(src_t, idx, big_w[:, :, 4:13])
+    with pytest.raises(RuntimeError, match="out of bounds"):
+        ext.gather_kv_out_cpu(src_t, idx, big_g[:, :, 4:13])
