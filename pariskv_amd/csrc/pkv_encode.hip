@@ -22,9 +22,11 @@
 //   sum of squares: sequential inside a block, then a pairwise tree over blocks.
 //
 // The kernel sits between vector-instruction issue and the memory system (about
-// 3.4 TB/s of mixed traffic: 256 B read, 16 + 96 B written in pieces, 64 B of
+// 3.5 TB/s of mixed traffic: 256 B read, 16 + 96 B written in pieces, 64 B of
 // histogram atomics per key): forty more instructions per key cost 5 - 10 %, a
-// quarter fewer gained 5 %.  fp32 keys take enc_key_exact (correctly
+// quarter fewer gained 5 %; without the record stores it takes 90, without any
+// store and without the histogram 70 us per 2^20 keys, with everything 120 - 126.
+// fp32 keys take enc_key_exact (correctly
 // rounded divisions and roots, about 700 instructions per lane and key); bf16
 // keys take enc_key_fast (about 225), which reaches the same bits through
 // reciprocals, a table for the magnitude code and its term of the weight, and
@@ -41,7 +43,7 @@ constexpr int kEncThreads = 256;
 constexpr int kEncWavesPerSimd = 4;
 constexpr int kEncKeysPerIter = kEncThreads / 16;
 constexpr int kEncKeysPerWg = 16 * kEncKeysPerIter;
-constexpr int kEncAhead = 2;  // iterations whose keys a wave has in flight (1, 2 and 3 measure the same)
+constexpr int kEncAhead = 4;  // iterations whose keys a wave has in flight (1 / 2 / 4: 132 / 127 / 125 us per 1M key-heads)
 
 #define PKV_ENC_THRESHOLDS 0.08447265625f, 0.169921875f, 0.2578125f, 0.349609375f, 0.44921875f, 0.55859375f, 0.69140625f
 #define PKV_ENC_CENTERS 0.0419921875f, 0.126953125f, 0.212890625f, 0.302734375f, 0.396484375f, 0.5f, 0.6171875f, 0.76171875f
@@ -374,38 +376,30 @@ __global__ __launch_bounds__(kEncThreads) __attribute__((amdgpu_waves_per_eu(kEn
                  w_lane = (uint32_t)(2 * (kq * ws_key + s * ws_sub));
   const int64_t k_step = (int64_t)kEncKeysPerIter * k_stride_key * esize, c_step = (int64_t)kEncKeysPerIter * cs_key,
                 n_step = (int64_t)kEncKeysPerIter * ns_key, w_step = (int64_t)kEncKeysPerIter * ws_key * 2;
-  // A wave has the keys of its next kEncAhead iterations in flight (one iteration is about two microseconds of vector
-  // work for the four waves of a SIMD).
+  // A wave keeps the keys of its next kEncAhead iterations in flight, each in a register set of its own: set j holds
+  // iterations j, j + kEncAhead, ... and is refilled as soon as its key has been copied out.  (A ring whose sets are
+  // copied into each other waits for the newest load at every copy and hides one iteration of latency whatever its
+  // depth.)  Loads are never skipped - past the block's end they fetch its last iteration again - because a load that
+  // may or may not have been issued makes every later wait of the in-order counter a wait for everything.
   constexpr int kW = BF16 ? 1 : 2;  // 16-byte words per lane and key
+  const int n_iter = last / kEncKeysPerIter + 1;
   pkv_u32x4 raw[kEncAhead][kW];
-#pragma unroll
-  for (int a = 0; a < kEncAhead; ++a) {
-    const int rel = a * kEncKeysPerIter + kq;
-    if (a * kEncKeysPerIter <= last) {  // uniform
-      const uint32_t off = rel <= last ? (uint32_t)a * kEncKeysPerIter * key_bytes + k_lane : (uint32_t)last * key_bytes + blk_off;
-      raw[a][0] = *(const pkv_u32x4 *)(k_base + off);
-      if (!BF16) raw[a][kW - 1] = *(const pkv_u32x4 *)(k_base + off + 16);
-    }
-  }
-  k_base += (kEncAhead - 1) * k_step;
-  for (int first = 0; first <= last; first += kEncKeysPerIter, c_base += c_step, n_base += n_step, w_base += w_step) {
+  auto load_iter = [&](int it, pkv_u32x4 (&reg)[kW]) {
+    const int it_c = it < n_iter ? it : n_iter - 1;  // uniform
+    const char *base = k_base + (int64_t)it_c * k_step;
+    const int lim = last - it_c * kEncKeysPerIter;  // the iteration holds the block's keys 16 it_c .. 16 it_c + lim
+    uint32_t off = k_lane;
+    if (lim < kEncKeysPerIter - 1) off = kq <= lim ? k_lane : (uint32_t)lim * key_bytes + blk_off;  // uniform: it is ragged
+    reg[0] = *(const pkv_u32x4 *)(base + off);
+    if (!BF16) reg[kW - 1] = *(const pkv_u32x4 *)(base + off + 16);
+  };
+  auto iteration = [&](int it, pkv_u32x4 (&reg)[kW]) {
+    const int first = it * kEncKeysPerIter;
     const bool active = kq <= last - first;
     pkv_u32x4 cur[kW];
 #pragma unroll
-    for (int q = 0; q < kW; ++q) cur[q] = raw[0][q];
-#pragma unroll
-    for (int a = 0; a + 1 < kEncAhead; ++a)
-#pragma unroll
-      for (int q = 0; q < kW; ++q) raw[a][q] = raw[a + 1][q];
-    k_base += k_step;
-    // the iteration loaded now holds the block's keys first + 16 * kEncAhead .. + lim
-    const int lim = last - first - kEncAhead * kEncKeysPerIter;
-    if (lim >= 0) {  // uniform: that iteration exists
-      uint32_t off = k_lane;
-      if (lim < kEncKeysPerIter - 1) off = kq <= lim ? k_lane : (uint32_t)lim * key_bytes + blk_off;  // uniform: it is ragged
-      raw[kEncAhead - 1][0] = *(const pkv_u32x4 *)(k_base + off);
-      if (!BF16) raw[kEncAhead - 1][kW - 1] = *(const pkv_u32x4 *)(k_base + off + 16);
-    }
+    for (int q = 0; q < kW; ++q) cur[q] = reg[q];
+    load_iter(it + kEncAhead, reg);
     EncOut o;
     bool exact = true;
     float x[8];
@@ -436,6 +430,8 @@ __global__ __launch_bounds__(kEncThreads) __attribute__((amdgpu_waves_per_eu(kEn
 
     // the empty statement keeps the lane offsets apart from the bases, so that the stores address
     // scalar base + lane offset instead of three 64-bit lane pointers that would each need an add per iteration
+    uint8_t *cb = c_base + (int64_t)it * c_step, *nb = n_base + (int64_t)it * n_step;
+    char *wb = w_base + (int64_t)it * w_step;
     uint32_t c_off = c_lane, n_off = n_lane, w_off = w_lane;
     if (ALL) {
       // No branch around the stores (see above): a lane past the end of a ragged block holds the block's last key
@@ -447,18 +443,29 @@ __global__ __launch_bounds__(kEncThreads) __attribute__((amdgpu_waves_per_eu(kEn
         w_off = 2 * (kk * (uint32_t)ws_key + (uint32_t)(s * ws_sub));
       }
       asm volatile("" : "+v"(c_off), "+v"(n_off), "+v"(w_off));
-      c_base[c_off] = (uint8_t)o.code;
-      *(uint32_t *)(n_base + n_off) = o.packed;
-      *(uint16_t *)(w_base + w_off) = (uint16_t)o.wbits;
+      // written once and not read again by this launch: streaming stores (5 - 8 % on two of three shapes)
+      __builtin_nontemporal_store((uint8_t)o.code, cb + c_off);
+      __builtin_nontemporal_store(o.packed, (uint32_t *)(nb + n_off));
+      __builtin_nontemporal_store((uint16_t)o.wbits, (uint16_t *)(wb + w_off));
       if (active) atomicAdd(&s_hist[s * 256 + o.code], 1u);
     } else if (active) {
       asm volatile("" : "+v"(c_off), "+v"(n_off), "+v"(w_off));
-      c_base[c_off] = (uint8_t)o.code;
+      cb[c_off] = (uint8_t)o.code;
       if (has_hist) atomicAdd(&s_hist[s * 256 + o.code], 1u);
-      if (has_nib) *(uint32_t *)(n_base + n_off) = o.packed;
-      if (has_weight) *(uint16_t *)(w_base + w_off) = (uint16_t)o.wbits;
+      if (has_nib) *(uint32_t *)(nb + n_off) = o.packed;
+      if (has_weight) *(uint16_t *)(wb + w_off) = (uint16_t)o.wbits;
     }
+  };
+#pragma unroll
+  for (int j = 0; j < kEncAhead; ++j) load_iter(j, raw[j]);
+  int it = 0;
+  for (; it + kEncAhead <= n_iter; it += kEncAhead) {  // whole groups: no branch between the sets' loads and stores
+#pragma unroll
+    for (int j = 0; j < kEncAhead; ++j) iteration(it + j, raw[j]);
   }
+#pragma unroll
+  for (int j = 0; j < kEncAhead - 1; ++j)  // what a ragged block leaves: fewer than kEncAhead iterations
+    if (it + j < n_iter) iteration(it + j, raw[j]);
   if (has_hist) {
     __syncthreads();
     pkv_flush_cluster_hist(s_hist, cluster_counts + (int64_t)b * cc_b + (int64_t)h * cc_h, tid, kEncThreads);
