@@ -35,6 +35,27 @@ __device__ __forceinline__ void load_lut(uint32_t *s_lut, const uint8_t *__restr
   ((pkv_u32x4 *)s_lut)[threadIdx.x] = g[threadIdx.x];
 }
 
+// KPT * 256 whole keys from key k0 on, in the form the retrieval runs (one-byte counts out, histogram kept): every
+// load of the thread is issued before the first table lookup, and nothing in between is conditional, so the waits
+// of the in-order memory counter name exact counts and the lookups of one key run while the codes of the others are
+// still on their way.  Four keys per thread in flight, as in the general loop: with 8 or 16 the launch is slower at
+// a full grid (config 3: 36.8 us per step with 4, 38.0 with 8, 40.1 with 16; 37.2 with the general loop), faster
+// only where the grid leaves most of the chip idle.
+template <int KPT>
+__device__ __forceinline__ void scan_whole_keys(const pkv_u32x4 *__restrict__ base, int64_t k0, const uint8_t *l8,
+                                                uint8_t *__restrict__ out8, uint32_t *s_hist, int copy) {
+  const int64_t i0 = k0 + threadIdx.x;
+  pkv_u32x4 v[KPT];
+#pragma unroll
+  for (int u = 0; u < KPT; ++u) v[u] = __builtin_nontemporal_load(base + i0 + u * kScanThreads);
+#pragma unroll
+  for (int u = 0; u < KPT; ++u) {
+    const int c = lut_sum16(l8, v[u]);
+    out8[i0 + u * kScanThreads] = (uint8_t)c;
+    atomicAdd(&s_hist[c * kHistCopies + copy], 1u);
+  }
+}
+
 // Key-major codes ([key][16] bytes, 16-byte aligned).  grid (n_chunks, R).
 // sub_blocks = 1: workgroup c scans keys [c * chunk_keys, +chunk_keys) and leaves one suffix histogram.
 // sub_blocks = S > 1: the chunk is S pieces of chunk_keys / S keys spread over the row, workgroup c scans pieces
@@ -71,7 +92,11 @@ __global__ __launch_bounds__(kScanThreads) void pkv_scan_keymajor_kernel(
     const int64_t piece = (int64_t)chunk + (int64_t)j * n_chunks;
     const int64_t k0 = piece * piece_keys < n_keys ? piece * piece_keys : n_keys;
     const int64_t k1 = (k0 + piece_keys < n_keys) ? k0 + piece_keys : n_keys;
-    for (int64_t i0 = k0 + tid; i0 < k1; i0 += 4 * kScanThreads) {
+    int64_t kc = k0;
+    if (out8 && !out32 && chunk_suf) {  // uniform: the retrieval's form; whole runs of 1024 keys first
+      for (; kc + 4 * kScanThreads <= k1; kc += 4 * kScanThreads) scan_whole_keys<4>(base, kc, l8, out8, s_hist, copy);
+    }
+    for (int64_t i0 = kc + tid; i0 < k1; i0 += 4 * kScanThreads) {
       pkv_u32x4 v[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
