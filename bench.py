@@ -869,6 +869,18 @@ def main():
             r["headline"] = (f"decode_tokens_per_s with {pl['host_layers']} of 36 layers' K/V offloaded to pinned host "
                              f"memory and {pl['hbm_layers']} resident in HBM (the box pins at most ~65 GiB; the "
                              f"reference's enable_offload would put all 36 on the host)")
+            if pl["hbm_layers"] > 0:
+                # the same loop with every layer offloaded, at as many layers as the host budget holds: its time per
+                # layer is what a 36-layer all-offload run would show on a box that can pin the whole store
+                gc.collect()
+                torch.cuda.empty_cache()
+                n_l = pl["host_layers"] - pl["host_layers"] % 4
+                a = model_decode(torch, dev, n_l, 8, 65536, 136, 100, 8, True, None)
+                r["every_layer_offloaded"] = {"layers": n_l, "us_per_layer": a["us_per_layer"],
+                                              "ms_per_token": a["ms_per_token"],
+                                              "decode_tokens_per_s_at_that_many_layers": a["decode_tokens_per_s"],
+                                              "host_pinned_GiB": a["placement"]["host_pinned_GiB"],
+                                              "hbm_layers": a["placement"]["hbm_layers"]}
             return r
 
         leg("cfg5", cfg5)
