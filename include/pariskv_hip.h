@@ -524,9 +524,18 @@ int pkv_retrieve(const pkv_retrieve_args *args, void *ws, size_t ws_bytes, void 
  * 327-498 and cache_hub/polar_cache.py:1126-1162) with the cache update between them; nothing between them touches
  * the queries, the cluster sizes or the tier counts unless the update refreshes the index, after which the caller
  * must not set table_ready.  bf16 only; args->q is not read; n_q_heads = args->n_kv_heads * args->group. */
+/* `append` (NULL: none): the token's rows of the cache in the same launch - the finished key (as k_out) and the
+ * value head as it stands in qkv, behind the key heads, go to row `slot` of dst_k / dst_v [bs][kv_heads][rows][128]
+ * (strides in elements): the two slot writes of decode_update_kv_cache (cache_hub/polar_cache.py:848-856), i.e.
+ * what pkv_append_kv does with k_out and the value states in a launch of its own. */
+typedef struct pkv_kv_append {
+  void *dst_k, *dst_v;
+  int64_t stride_b, stride_h, rows, slot;
+} pkv_kv_append;
 int pkv_qk_norm_rope_table(const void *qkv, int64_t stride_b, int n_q_heads, const void *q_weight, const void *k_weight,
                            float eps, const void *cos_row, const void *sin_row, void *q_out, void *k_out,
-                           const pkv_retrieve_args *args, void *ws, size_t ws_bytes, void *stream);
+                           const pkv_retrieve_args *args, void *ws, size_t ws_bytes, const pkv_kv_append *append,
+                           void *stream);
 
 /* pkv_retrieve for callers that cannot allocate device memory (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc): the

@@ -35,6 +35,12 @@ class AttnArgs(C.Structure):
                 ("out", _vp), ("ws", _vp), ("ws_bytes", _sz)]
 
 
+class KvAppend(C.Structure):
+    """Mirror of ``pkv_kv_append``."""
+
+    _fields_ = [("dst_k", _vp), ("dst_v", _vp), ("stride_b", _i64), ("stride_h", _i64), ("rows", _i64), ("slot", _i64)]
+
+
 class RetrieveArgs(C.Structure):
     """Mirror of ``pkv_retrieve_args``."""
 
@@ -122,7 +128,8 @@ PROTOTYPES = {
     "pkv_silu_mul": (_i, [_vp, _i64, _i, _i, _vp, _vp]),
     "pkv_retrieve_ws_bytes": (_sz, [_i, _i64, _i64, _i64]),
     "pkv_retrieve": (_i, [C.POINTER(RetrieveArgs), _vp, _sz, _vp]),
-    "pkv_qk_norm_rope_table": (_i, [_vp, _i64, _i, _vp, _vp, C.c_float, _vp, _vp, _vp, _vp, C.POINTER(RetrieveArgs), _vp, _sz, _vp]),
+    "pkv_qk_norm_rope_table": (_i, [_vp, _i64, _i, _vp, _vp, C.c_float, _vp, _vp, _vp, _vp, C.POINTER(RetrieveArgs), _vp, _sz,
+                                    C.POINTER(KvAppend), _vp]),
     "pkv_retrieve_noalloc_max_bytes": (_sz, []),
     "pkv_retrieve_noalloc_prepare": (_i, []),
     "pkv_retrieve_noalloc": (_i, [C.POINTER(RetrieveArgs), _vp]),

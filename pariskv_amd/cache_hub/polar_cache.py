@@ -329,15 +329,25 @@ class polar_cache(KV_Cache):
         return key_states[:, vs:], value_states[:, vs:]
 
     # -------------------------------------------------------------- decode
-    def decode_update_kv_cache(self, key_states, value_states, layer_idx):
-        """Append one token ([bs,1,Hkv,D]); refresh the index when this layer's update buffer fills (:827-881)."""
+    def fused_append_target(self, layer_idx):
+        """(dst_k, dst_v, slot) of the next decoded token of this layer, for a caller whose own launch writes the rows
+        (``ops.qk_norm_rope(append=...)``) and then calls ``decode_update_kv_cache(..., appended=True)``; None where the
+        append does more than the two slot writes (subclasses that keep value norms) or the dtype is not bf16."""
+        if type(self)._append is not polar_cache._append or self.dtype != torch.bfloat16:
+            return None
+        return self.unified_keys_gpu[layer_idx], self.unified_values_gpu[layer_idx], self._zones[layer_idx].append_slot()
+
+    def decode_update_kv_cache(self, key_states, value_states, layer_idx, appended: bool = False):
+        """Append one token ([bs,1,Hkv,D]); refresh the index when this layer's update buffer fills (:827-881).
+        ``appended``: the rows are already at ``fused_append_target(layer_idx)`` (written on this stream)."""
         z = self._zones[layer_idx]
         if self.enable_offload and (self._prefill_stage[0] is not None or self._prefill_stage[1] is not None):
             self.release_prefill_staging()  # prefill is over: its staging pairs (two layers of K/V) go back to the allocator
         slot = z.append_slot()
-        if key_states.dtype != self.dtype or value_states.dtype != self.dtype:
-            key_states, value_states = key_states.to(self.dtype), value_states.to(self.dtype)
-        self._append(layer_idx, slot, key_states, value_states)
+        if not appended:
+            if key_states.dtype != self.dtype or value_states.dtype != self.dtype:
+                key_states, value_states = key_states.to(self.dtype), value_states.to(self.dtype)
+            self._append(layer_idx, slot, key_states, value_states)
         refresh = z.appended()
         self.current_seq_len[layer_idx] = z.seq_len
         if layer_idx == 0:

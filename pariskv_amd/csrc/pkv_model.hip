@@ -30,7 +30,10 @@ __device__ __forceinline__ void qk_norm_rope_task(int task, const uint16_t *__re
                                                   int n_kv_heads, const uint16_t *__restrict__ q_weight,
                                                   const uint16_t *__restrict__ k_weight, float eps,
                                                   const uint16_t *__restrict__ cos_row, const uint16_t *__restrict__ sin_row,
-                                                  uint16_t *__restrict__ q_out, uint16_t *__restrict__ k_out) {
+                                                  uint16_t *__restrict__ q_out, uint16_t *__restrict__ k_out,
+                                                  uint16_t *__restrict__ cache_k = nullptr,
+                                                  uint16_t *__restrict__ cache_v = nullptr, int64_t cache_stride_b = 0,
+                                                  int64_t cache_stride_h = 0, int64_t cache_slot = 0) {
   const int lane = pkv_lane();
   const int heads = n_q_heads + n_kv_heads;
   const int b = task / heads, head = task % heads;
@@ -43,6 +46,15 @@ __device__ __forceinline__ void qk_norm_rope_task(int task, const uint16_t *__re
                        : k_out + ((int64_t)b * n_kv_heads + (head - n_q_heads)) * 128;
   dst[lane] = pkv_f32_to_bf16_bits(y1);
   dst[lane + 64] = pkv_f32_to_bf16_bits(y2);
+  if (!is_q && cache_k) {  // the token's rows of the cache as well: the finished key, and the value head as it stands in qkv
+    const int kvh = head - n_q_heads;
+    const int64_t row = (int64_t)b * cache_stride_b + (int64_t)kvh * cache_stride_h + cache_slot * 128;
+    cache_k[row + lane] = pkv_f32_to_bf16_bits(y1);
+    cache_k[row + lane + 64] = pkv_f32_to_bf16_bits(y2);
+    const uint16_t *vsrc = qkv + (int64_t)b * stride_b + (int64_t)(heads + kvh) * 128;
+    cache_v[row + lane] = vsrc[lane];
+    cache_v[row + lane + 64] = vsrc[lane + 64];
+  }
 }
 
 __global__ __launch_bounds__(256) void pkv_qk_norm_rope_kernel(const uint16_t *__restrict__ qkv, int64_t stride_b, int n_q_heads,
@@ -69,12 +81,14 @@ __global__ __launch_bounds__(256) void pkv_qk_norm_rope_table_kernel(
     uint16_t *__restrict__ q_out, uint16_t *__restrict__ k_out, int n_tasks, int n_rope_blocks, int bs,
     const float *__restrict__ signs, const int32_t *__restrict__ cc, PkvTiers tiers, float *__restrict__ qhat,
     float *__restrict__ qnorm, uint8_t *__restrict__ lut, uint32_t *__restrict__ row_suf, uint32_t *__restrict__ zero_ptr,
-    int64_t zero_words) {
+    int64_t zero_words, uint16_t *__restrict__ cache_k, uint16_t *__restrict__ cache_v, int64_t cache_stride_b,
+    int64_t cache_stride_h, int64_t cache_slot) {
   const int tid = threadIdx.x;
   if ((int)blockIdx.x < n_rope_blocks) {
     const int task = blockIdx.x * 4 + tid / PKV_WAVE;
     if (task < n_tasks)
-      qk_norm_rope_task(task, qkv, stride_b, n_q_heads, n_kv_heads, q_weight, k_weight, eps, cos_row, sin_row, q_out, k_out);
+      qk_norm_rope_task(task, qkv, stride_b, n_q_heads, n_kv_heads, q_weight, k_weight, eps, cos_row, sin_row, q_out, k_out,
+                        cache_k, cache_v, cache_stride_b, cache_stride_h, cache_slot);
     return;
   }
   const int t = blockIdx.x - n_rope_blocks, n_table = 16 * bs * n_kv_heads;
@@ -231,8 +245,15 @@ int pkv_launch_qk_norm_rope_table(const void *qkv, int64_t stride_b, int bs, int
                                   const void *q_weight, const void *k_weight, float eps, const void *cos_row,
                                   const void *sin_row, void *q_out, void *k_out, const float *signs, const int32_t *cc,
                                   const PkvTiers &tiers, float *qhat, float *qnorm, uint8_t *lut, uint32_t *row_suf,
-                                  uint32_t *zero_ptr, int64_t zero_words, hipStream_t s) {
+                                  uint32_t *zero_ptr, int64_t zero_words, const pkv_kv_append *append, hipStream_t s) {
   PKV_REQUIRE(qkv && cos_row && sin_row && q_out && k_out, "pkv_qk_norm_rope_table: null pointer");
+  if (append) {
+    PKV_REQUIRE(append->dst_k && append->dst_v && append->rows > 0 && append->slot >= 0 && append->slot < append->rows &&
+                    append->stride_h >= append->rows * 128 && (bs == 1 || append->stride_b >= n_kv_heads * append->stride_h),
+                "pkv_qk_norm_rope_table: append needs dst_k / dst_v [bs][kv_heads][rows][128] and 0 <= slot < rows");
+    PKV_REQUIRE(stride_b >= (int64_t)(n_q_heads + 2 * n_kv_heads) * 128,
+                "pkv_qk_norm_rope_table: append reads the value heads behind the key heads of qkv");
+  }
   PKV_REQUIRE(bs > 0 && n_q_heads > 0 && n_kv_heads > 0 && n_q_heads % n_kv_heads == 0 &&
                   (int64_t)bs * (n_q_heads + n_kv_heads) < (1 << 24) && stride_b >= (int64_t)(n_q_heads + n_kv_heads) * 128,
               "pkv_qk_norm_rope_table: bad shape bs=%d heads=%d+%d stride=%lld", bs, n_q_heads, n_kv_heads, (long long)stride_b);
@@ -243,7 +264,9 @@ int pkv_launch_qk_norm_rope_table(const void *qkv, int64_t stride_b, int bs, int
                      (const uint16_t *)qkv, stride_b, n_q_heads, n_kv_heads, (const uint16_t *)q_weight,
                      (const uint16_t *)k_weight, eps, (const uint16_t *)cos_row, (const uint16_t *)sin_row, (uint16_t *)q_out,
                      (uint16_t *)k_out, n_tasks, n_rope_blocks, bs, signs, cc, tiers, qhat, qnorm, lut, row_suf, zero_ptr,
-                     zero_ptr ? zero_words : 0);
+                     zero_ptr ? zero_words : 0, append ? (uint16_t *)append->dst_k : nullptr,
+                     append ? (uint16_t *)append->dst_v : nullptr, append ? append->stride_b : 0,
+                     append ? append->stride_h : 0, append ? append->slot : 0);
   PKV_LAUNCH_CHECK("pkv_qk_norm_rope_table_kernel");
   return PKV_OK;
 }

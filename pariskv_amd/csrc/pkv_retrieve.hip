@@ -15,7 +15,7 @@ PKV_INTERNAL int pkv_launch_qk_norm_rope_table(const void *qkv, int64_t stride_b
                                   const void *q_weight, const void *k_weight, float eps, const void *cos_row,
                                   const void *sin_row, void *q_out, void *k_out, const float *signs, const int32_t *cc,
                                   const PkvTiers &tiers, float *qhat, float *qnorm, uint8_t *lut, uint32_t *row_suf,
-                                  uint32_t *zero_ptr, int64_t zero_words, hipStream_t s);
+                                  uint32_t *zero_ptr, int64_t zero_words, const pkv_kv_append *append, hipStream_t s);
 PKV_INTERNAL size_t pkv_fused_sync_bytes(int rows, int64_t n_chunks);
 PKV_INTERNAL bool pkv_fused_usable(int rows, int64_t n_keys, int chunk_keys, hipStream_t s);
 PKV_INTERNAL int pkv_launch_fused_retrieve(const void *q, int dtype, int bs, int n_kv_heads, int group, const float *signs,
@@ -234,7 +234,8 @@ static int retrieve_impl(const pkv_retrieve_args *a, void *ws, size_t ws_bytes, 
 
 extern "C" int pkv_qk_norm_rope_table(const void *qkv, int64_t stride_b, int n_q_heads, const void *q_weight,
                                       const void *k_weight, float eps, const void *cos_row, const void *sin_row, void *q_out,
-                                      void *k_out, const pkv_retrieve_args *a, void *ws, size_t ws_bytes, void *stream) {
+                                      void *k_out, const pkv_retrieve_args *a, void *ws, size_t ws_bytes,
+                                      const pkv_kv_append *append, void *stream) {
   PKV_REQUIRE(a != nullptr, "pkv_qk_norm_rope_table: null retrieval arguments");
   PKV_REQUIRE(a->dtype == PKV_DTYPE_BF16 && a->bs > 0 && a->n_kv_heads > 0 && a->group > 0 &&
                   n_q_heads == a->n_kv_heads * a->group,
@@ -258,7 +259,8 @@ extern "C" int pkv_qk_norm_rope_table(const void *qkv, int64_t stride_b, int n_q
   return pkv_launch_qk_norm_rope_table(qkv, stride_b, a->bs, n_q_heads, a->n_kv_heads, q_weight, k_weight, eps, cos_row,
                                        sin_row, q_out, k_out, a->signs, a->cluster_counts, t, (float *)(base + w.qhat),
                                        (float *)(base + w.qnorm), (uint8_t *)(base + w.lut), (uint32_t *)(base + w.rowsuf),
-                                       ctl_words ? (uint32_t *)(base + w.topk) : nullptr, ctl_words, (hipStream_t)stream);
+                                       ctl_words ? (uint32_t *)(base + w.topk) : nullptr, ctl_words, append,
+                                       (hipStream_t)stream);
 }
 
 extern "C" int pkv_retrieve(const pkv_retrieve_args *a, void *ws, size_t ws_bytes, void *stream) {

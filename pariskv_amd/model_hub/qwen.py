@@ -175,13 +175,19 @@ class QwenModel:
         pos = self._position
         # where this layer's step will retrieve, its vote table is built by the same launch that finishes the queries
         target = self.kv_cache.query_table_target(layer_idx) if hasattr(self.kv_cache, "query_table_target") else None
+        # ... and it writes the token's K/V rows into the cache as well, where the cache's append is nothing more
+        slot_rows = (self.kv_cache.fused_append_target(layer_idx)
+                     if target is not None and hasattr(self.kv_cache, "fused_append_target") else None)
         q, k = ops.qk_norm_rope(qkv, self.num_heads, self.num_key_value_heads, layer.q_norm_weight, layer.k_norm_weight,
                                 layer.q_norm_variance_epsilon or 0.0, self.cos_cache[pos], self.sin_cache[pos],
-                                table_for=target)
+                                table_for=target, append=slot_rows)
         v = qkv[..., (self.num_heads + self.num_key_value_heads) * self.head_dim:].reshape(bsz, -1, self.num_key_value_heads,
                                                                                              self.head_dim)
         ranges.push("decode_update_kv_cache")  # the reference's ranges of the same names, model_hub/LLM.py:173-183
-        k, v = self.kv_cache.decode_update_kv_cache(k, v, layer_idx)
+        if slot_rows is not None:
+            k, v = self.kv_cache.decode_update_kv_cache(k, v, layer_idx, appended=True)
+        else:
+            k, v = self.kv_cache.decode_update_kv_cache(k, v, layer_idx)
         ranges.pop()
         ranges.push("decode_attention")
         attn_out = self.decode_attention(q, k, v, layer_idx)

@@ -606,13 +606,16 @@ class DecodeAttention:
 
 
 def qk_norm_rope(qkv: torch.Tensor, n_q_heads: int, n_kv_heads: int, q_weight, k_weight, eps: float,
-                 cos_row: torch.Tensor, sin_row: torch.Tensor, table_for=None):
+                 cos_row: torch.Tensor, sin_row: torch.Tensor, table_for=None, append=None):
     """Per-head RMSNorm of q and k plus rotary embedding for one decode token per sequence, one launch
     (model_hub/qwen.py:327-340, 410-431, 434-498).  qkv bf16 [bs,1,(Hq+2Hkv)*128] (last dim contiguous); cos_row /
     sin_row bf16 [64] of the token's position.  Returns (q [bs,1,Hq,128], k [bs,1,Hkv,128]).
     ``table_for``: a :class:`BoundStep` / :class:`BoundAdaptiveStep` whose retrieval will run on the returned q next:
     the same launch then also leaves the retrieval's rotated query and vote table in that step's workspace
-    (pkv_qk_norm_rope_table) and the step's next launch skips its query-prep kernel."""
+    (pkv_qk_norm_rope_table) and the step's next launch skips its query-prep kernel.
+    ``append`` (with ``table_for`` only): (dst_k, dst_v, slot) - the launch also writes the token's key (as returned) and
+    value (as it stands in qkv) to row ``slot`` of the cache's dense bf16 K/V tensors [bs,Hkv,rows,128], which is
+    what :func:`append_kv` does with them in a launch of its own."""
     bs = qkv.shape[0]
     _need(qkv.is_cuda and qkv.dtype == torch.bfloat16 and qkv.stride(-1) == 1 and qkv.numel() == bs * qkv.shape[-1] and
           qkv.shape[-1] >= (n_q_heads + 2 * n_kv_heads) * HEAD_DIM, "qkv: bf16 [bs,1,(Hq+2Hkv)*128]")
@@ -623,10 +626,21 @@ def qk_norm_rope(qkv: torch.Tensor, n_q_heads: int, n_kv_heads: int, q_weight, k
               "norm weights: bf16 [128]")
     q = torch.empty(bs, 1, n_q_heads, HEAD_DIM, dtype=torch.bfloat16, device=qkv.device)
     k = torch.empty(bs, 1, n_kv_heads, HEAD_DIM, dtype=torch.bfloat16, device=qkv.device)
+    _need(append is None or table_for is not None, "append rides on the launch that builds the vote table")
     if table_for is not None:
+        app = None
+        if append is not None:
+            dk, dv, slot = append
+            _need(dk.is_cuda and dv.is_cuda and dk.dtype == torch.bfloat16 and dv.dtype == torch.bfloat16 and
+                  dk.shape == dv.shape and dk.stride() == dv.stride() and dk.dim() == 4 and
+                  tuple(dk.shape[:2]) == (bs, n_kv_heads) and dk.shape[3] == HEAD_DIM and dk.stride(3) == 1 and
+                  dk.stride(2) == HEAD_DIM and 0 <= slot < dk.shape[2],
+                  "append: dst_k, dst_v bf16 [bs,Hkv,rows,128] with contiguous rows, 0 <= slot < rows")
+            ka = _lib.KvAppend(dk.data_ptr(), dv.data_ptr(), dk.stride(0), dk.stride(1), dk.shape[2], int(slot))
+            app = C.byref(ka)
         _lib.check(_lib.lib().pkv_qk_norm_rope_table(_p(qkv), qkv.stride(0), n_q_heads, _p(q_weight), _p(k_weight), float(eps),
                                                      _p(cos_row), _p(sin_row), _p(q), _p(k), table_for._ra, table_for._ws,
-                                                     table_for._ws_bytes, _stream(qkv)))
+                                                     table_for._ws_bytes, app, _stream(qkv)))
         table_for.a.table_ready = 1   # consumed (and reset) by the step's next launch
         return q, k
     _lib.check(_lib.lib().pkv_qk_norm_rope(_p(qkv), qkv.stride(0), bs, n_q_heads, n_kv_heads, _p(q_weight), _p(k_weight),

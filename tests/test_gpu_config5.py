@@ -74,10 +74,10 @@ def test_config5_full_size_decode_with_split_placement():
     appended = {l: [] for l in probe_layers}    # the decode tokens' keys of the probe layers, as the model produced them
     inner_update = cache.decode_update_kv_cache
 
-    def spy_update(key_states, value_states, layer_idx):
+    def spy_update(key_states, value_states, layer_idx, **kw):   # kw: appended=True where the glue wrote the rows itself
         if layer_idx in appended:
             appended[layer_idx].append(key_states.clone())
-        return inner_update(key_states, value_states, layer_idx)
+        return inner_update(key_states, value_states, layer_idx, **kw)
 
     cache.decode_update_kv_cache = spy_update
     ids = torch.randint(0, cfg.vocab_size, (bs, 1), generator=g, device=DEV)

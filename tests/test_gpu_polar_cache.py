@@ -738,6 +738,62 @@ def test_qk_norm_rope_with_the_vote_table_in_the_same_launch():
         assert used >= 15, used
 
 
+def test_qk_norm_rope_writes_the_tokens_rows_into_the_cache():
+    """ops.qk_norm_rope(append=...) + decode_update_kv_cache(appended=True) against the ordinary append, two caches
+    side by side over 40 tokens and two index refreshes (offload and no-offload): the dense K/V tensors, the zone
+    counters, the attention outputs and the selected ids stay identical; an adaptive-k cache declines the fused form."""
+    from pariskv_amd import ops
+    from pariskv_amd.cache_hub.polar_cache import polar_cache
+    from pariskv_amd.cache_hub.polar_cache_adaptivek_varlen import polar_cache as adaptive_cache
+
+    bs, Hq, Hkv, D, S = 2, 8, 2, 128, 3000
+    g = torch.Generator(device=DEV).manual_seed(11)
+    for offload in (True, False):
+        a = _make_cache(offload, bs, Hkv, Hq, 1, S, 64, 4, 64, 16, 100)
+        b = _make_cache(offload, bs, Hkv, Hq, 1, S, 64, 4, 64, 16, 100)
+        k, v = _synth_kv(torch.Generator().manual_seed(1), bs, S, Hkv)
+        for c in (a, b):
+            c.prefill_update_kv_cache(None, k.to(DEV), v.to(DEV), 0, 0)
+        width = (Hq + 2 * Hkv) * D
+        qw = (1 + 0.1 * torch.randn(D, generator=g, device=DEV)).to(torch.bfloat16)
+        kw = (1 + 0.1 * torch.randn(D, generator=g, device=DEV)).to(torch.bfloat16)
+        ang = torch.rand(D // 2, generator=g, device=DEV) * 6.28
+        cos, sin = ang.cos().to(torch.bfloat16), ang.sin().to(torch.bfloat16)
+        fused = 0
+        for step in range(40):
+            qkv = torch.randn(bs, 1, width, generator=g, device=DEV).to(torch.bfloat16)
+            vv = qkv[..., (Hq + Hkv) * D:].reshape(bs, 1, Hkv, D)
+            # cache a: the glue's way; cache b: separate launches
+            target = a.query_table_target(0)
+            rows = a.fused_append_target(0) if target is not None else None
+            qa, ka = ops.qk_norm_rope(qkv, Hq, Hkv, qw, kw, 1e-6, cos, sin, table_for=target, append=rows)
+            if rows is not None:
+                fused += 1
+                assert rows[2] == b._zones[0].append_slot()
+                a.decode_update_kv_cache(ka, vv, 0, appended=True)
+            else:
+                a.decode_update_kv_cache(ka, vv, 0)
+            qb, kb = ops.qk_norm_rope(qkv, Hq, Hkv, qw, kw, 1e-6, cos, sin)
+            b.decode_update_kv_cache(kb, vv, 0)
+            out_a, out_b = a.compute(qa, 0), b.compute(qb, 0)
+            torch.cuda.synchronize()
+            assert torch.equal(a.unified_keys_gpu[0], b.unified_keys_gpu[0]), f"step {step}: key rows differ"
+            assert torch.equal(a.unified_values_gpu[0], b.unified_values_gpu[0]), f"step {step}: value rows differ"
+            assert torch.equal(out_a, out_b), f"step {step}: attention output differs"
+            assert a._zones[0].seq_len == b._zones[0].seq_len and a.current_seq_len == b.current_seq_len
+            if getattr(a, "last_topk_indices", None) is not None and b.last_topk_indices is not None:
+                assert torch.equal(a.last_topk_indices, b.last_topk_indices)
+        assert fused >= 30, fused
+    # bad slot / shapes are refused, and the adaptive-k cache (its append also writes value norms) opts out
+    with pytest.raises(Exception):
+        ops.qk_norm_rope(qkv, Hq, Hkv, qw, kw, 1e-6, cos, sin, table_for=a.query_table_target(0),
+                         append=(a.unified_keys_gpu[0], a.unified_values_gpu[0], a.unified_keys_gpu[0].shape[2]))
+    with pytest.raises(Exception):
+        ops.qk_norm_rope(qkv, Hq, Hkv, qw, kw, 1e-6, cos, sin, append=(a.unified_keys_gpu[0], a.unified_values_gpu[0], 0))
+    assert adaptive_cache.fused_append_target is polar_cache.fused_append_target
+    assert adaptive_cache._append is not polar_cache._append   # which is what makes fused_append_target return None there
+
+
 def test_add_rmsnorm_and_silu_mul_match_torch_ops():
     """The two fused element-wise kernels of the decode glue against the torch op sequences they replace (bf16 add then
     F.rms_norm; F.silu then multiply), element for element up to one bf16 rounding."""
