@@ -261,3 +261,46 @@ def test_query_prep_matches_library_restatement(oracle, signs, dtype_name):
         assert abs(np.linalg.norm(qhat.astype(np.float64)) - 1.0) < (2e-2 if bf else 1e-5)  # rotation keeps the unit norm
     if bf:  # bf16 rounding hides the summation order except at rounding boundaries
         assert bad <= 20 * 128 * 0.02
+
+
+def test_one_instruction_butterfly_stages_carry_only_a_sign(oracle):
+    """The encoder's lane-crossing Walsh-Hadamard stages as the HIP kernel runs them, simulated in float32: block s of
+    a key sits in lane s0*1 ^ s1*2 ^ s2*7 ^ s3*15 (every partner then is one lane-permute move away), a stage is
+    held' = held[partner] * c + held with c = -1 where the block's stage bit is set, and what is left is the sign
+    (-1)^(set bits of s), taken out by the sign of the final scale.  Bit for bit the natural butterfly
+    (t + o where the bit is clear, o - t where it is set) followed by the plain scale."""
+    lane_of = lambda s: ((s & 1) * 1) ^ (((s >> 1) & 1) * 2) ^ (((s >> 2) & 1) * 7) ^ (((s >> 3) & 1) * 15)
+    lanes = [lane_of(s) for s in range(16)]
+    assert sorted(lanes) == list(range(16))                                   # a placement: every lane holds one block
+    block_of = lambda l: l ^ (3 if l & 4 else 0) ^ (4 if l & 8 else 0)        # the kernel's inverse map
+    assert all(block_of(lane_of(s)) == s for s in range(16))
+    partner_xor = {1: 1, 2: 2, 4: 7, 8: 15}                                   # quad_perm, quad_perm, row_half_mirror, row_mirror
+    for bit, x in partner_xor.items():
+        assert all(lane_of(s ^ bit) == lane_of(s) ^ x for s in range(16))
+    rng = np.random.default_rng(7)
+    scale = np.float32(0.08838834764831845)
+    for trial in range(200):
+        v = (rng.standard_normal(16) * np.exp2(rng.integers(-20, 20))).astype(np.float32)
+        if trial % 5 == 0:
+            v[rng.integers(0, 16, size=4)] = v[0]                            # equal pairs: exact zeros on the way
+        # natural form, block s in slot s
+        t = v.copy()
+        for bit in (1, 2, 4, 8):
+            o = t[np.arange(16) ^ bit]
+            t = np.where(np.arange(16) & bit, o - t, t + o).astype(np.float32)
+        want = (t * scale).astype(np.float32)
+        # the kernel's form, in lanes
+        held = np.empty(16, np.float32)
+        for s in range(16):
+            held[lane_of(s)] = v[s]
+        blocks = np.array([block_of(l) for l in range(16)])
+        for bit, x in partner_xor.items():
+            c = np.where(blocks & bit, np.float32(-1), np.float32(1)).astype(np.float32)
+            prod = (held[np.arange(16) ^ x] * c).astype(np.float32)          # exact: c is +-1, so the fused form rounds once
+            held = (prod + held).astype(np.float32)
+        parity = np.array([bin(b).count("1") & 1 for b in blocks])
+        got_lanes = (held * np.where(parity, -scale, scale).astype(np.float32)).astype(np.float32)
+        got = np.array([got_lanes[lane_of(s)] for s in range(16)], np.float32)
+        nz = want != 0                                                        # zeros take the kernel's exact path
+        assert np.array_equal(got[nz].view(np.uint32), want[nz].view(np.uint32)), trial
+        assert np.all(got[~nz] == 0)
