@@ -362,7 +362,8 @@ __global__ __launch_bounds__(kEncThreads) __attribute__((amdgpu_waves_per_eu(kEn
 
   // Addresses are a wave-uniform base, which advances by one iteration's 16 keys through scalar adds, plus a
   // 32-bit lane offset that never changes (the launcher checks that the offsets fit).  Lanes past the end of a
-  // ragged last block load its last key (all lanes take part in the lane-crossing steps) and store nothing.
+  // ragged last block load its last key (all lanes take part in the lane-crossing steps); they store nothing, or,
+  // in the ALL form, that key's results once more.
   const int64_t key_begin = (int64_t)blockIdx.x * keys_per_wg;  // < n_keys by the grid's construction
   const int last = (int)((n_keys - key_begin < keys_per_wg) ? n_keys - key_begin : keys_per_wg) - 1;
   constexpr int esize = BF16 ? 2 : 4;
