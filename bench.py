@@ -340,17 +340,19 @@ def cfg4_leg(torch, ops, _lib, dev):
             "parity_checked": "adaptive k and the first k ids of the last step, layer " + str(l)}
 
 
-def encoder_leg(torch, ops, dev, shapes=((8, 8, 65536), (1, 8, 131072)), reps=10):
-    """The index build of a prefill or refresh (`pkv_encode_append`: bf16 keys -> codes, 4-bit records, weights,
-    cluster sizes) on synthetic keys, per shape (batch, kv heads, keys per head): microseconds per 2^20 key-heads and
-    the rate over the 368 bytes a key-head must move (256 read, 112 written)."""
+def encoder_leg(torch, ops, dev, shapes=((8, 8, 65536, "bf16"), (1, 8, 131072, "bf16"), (1, 8, 131072, "f32")), reps=10):
+    """The index build of a prefill or refresh (`pkv_encode_append`: keys -> codes, 4-bit records, weights, cluster
+    sizes) on synthetic keys, per shape (batch, kv heads, keys per head, key dtype): microseconds per 2^20 key-heads
+    and the rate over the bytes a key-head must move (bf16 keys: 256 read + 112 written = 368; fp32 keys: 512 + 112
+    = 624)."""
     signs = ops.srht_signs(dev)
     out = []
-    for bs, H, N in shapes:
+    for bs, H, N, dt in shapes:
         g = torch.Generator(device=dev).manual_seed(5)
         keys = torch.randn(bs, H, N, 128, generator=g, device=dev)
         keys[..., [7, 31, 64, 101]] *= 10.0
-        kb = keys.to(torch.bfloat16)
+        kb = keys.to(torch.bfloat16) if dt == "bf16" else keys
+        nbytes = 368 if dt == "bf16" else 624
         del keys
         _, _, _, cb, k4, kw = ops.alloc_keymajor(bs, H, N, dev)
         cc = torch.zeros(bs, H, 16, 256, dtype=torch.int32, device=dev)
@@ -358,12 +360,12 @@ def encoder_leg(torch, ops, dev, shapes=((8, 8, 65536), (1, 8, 131072)), reps=10
             ops.encode_append(kb, signs, cb, k4, kw, cc)
         us = timed_us(torch, lambda i: ops.encode_append(kb, signs, cb, k4, kw, cc), reps)
         kh = bs * H * N
-        out.append({"batch": bs, "kv_heads": H, "keys_per_head": N, "us_per_launch": round(us, 1),
+        out.append({"batch": bs, "kv_heads": H, "keys_per_head": N, "key_dtype": dt, "us_per_launch": round(us, 1),
                     "us_per_2^20_key_heads": round(us / kh * 2**20, 1),
-                    "GBps_over_368B_per_key_head": round(kh * 368 / us / 1e3, 1),
-                    "hbm_fraction": round(kh * 368 / us / 1e3 / HBM_PEAK_GBPS, 4)})
+                    f"GBps_over_{nbytes}B_per_key_head": round(kh * nbytes / us / 1e3, 1),
+                    "hbm_fraction": round(kh * nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)})
         del kb, cb, k4, kw, cc
-    return {"kernel": "pkv_encode_kernel<bf16>", "bound": "between vector issue (about 225 instructions per key and 16-lane group) and the memory system",
+    return {"kernel": "pkv_encode_kernel", "bound": "between vector issue (about 225 instructions per key and 16-lane group for bf16 keys, 295 for fp32 keys) and the memory system",
             "shapes": out}
 
 

@@ -26,13 +26,16 @@
 // histogram atomics per key): forty more instructions per key cost 5 - 10 %, a
 // quarter fewer gained 5 %; without the record stores it takes 90, without any
 // store and without the histogram 70 us per 2^20 keys, with everything 120 - 126.
-// fp32 keys take enc_key_exact (correctly
-// rounded divisions and roots, about 700 instructions per lane and key); bf16
-// keys take enc_key_fast (about 225), which reaches the same bits through
-// reciprocals, a table for the magnitude code and its term of the weight, and
-// lane-crossing butterflies of one instruction per value, and hands a wave
-// over to enc_key_exact when one of its keys is outside the range where that
-// is proven.
+// enc_key_exact is the chain as written (correctly rounded divisions and roots,
+// about 580 vector instructions per lane and key).  bf16 keys take enc_key_fast
+// (about 225), which reaches the same bits through reciprocals, a table for the
+// magnitude code and its term of the weight, and lane-crossing butterflies of
+// one instruction per value; fp32 keys take enc_key_fast_f32 (about 295): the
+// compiler's own division sequence with the reciprocal refinement shared by the
+// eight quotients of a denominator and without its range scaling, the same
+// butterflies, and a small banded table for the magnitude code.  Either hands a
+// wave over to enc_key_exact when one of its keys is outside the range where
+// that is proven.
 #include "pkv_common.h"
 
 namespace {
@@ -43,7 +46,9 @@ constexpr int kEncThreads = 256;
 constexpr int kEncWavesPerSimd = 4;
 constexpr int kEncKeysPerIter = kEncThreads / 16;
 constexpr int kEncKeysPerWg = 16 * kEncKeysPerIter;
-constexpr int kEncAhead = 4;  // iterations whose keys a wave has in flight (1 / 2 / 4: 132 / 127 / 125 us per 1M key-heads)
+// iterations whose keys a wave has in flight (bf16 keys, 1 / 2 / 4: 132 / 127 / 125 us per 1M key-heads); an fp32
+// key takes two 16-byte words per lane, so half as many iterations hold the same bytes in as many registers
+constexpr int kEncAheadBf16 = 4, kEncAheadF32 = 2;
 
 #define PKV_ENC_THRESHOLDS 0.08447265625f, 0.169921875f, 0.2578125f, 0.349609375f, 0.44921875f, 0.55859375f, 0.69140625f
 #define PKV_ENC_CENTERS 0.0419921875f, 0.126953125f, 0.212890625f, 0.302734375f, 0.396484375f, 0.5f, 0.6171875f, 0.76171875f
@@ -146,10 +151,34 @@ constexpr uint32_t enc_cx_bf16_round_bits(float f) {  // round to nearest even; 
   b += 0x7fffu + ((b >> 16) & 1u);
   return b & 0xffff0000u;
 }
+// fp32 keys: |u| is not a pattern one can index by, but thresholds lie further apart than 0.08, so a band of that
+// width holds at most one of them: entry k, for k = floor(12.5 |u|) (<= 12 as |u| <= 1 up to rounding; 16 entries, the
+// index is masked), names the number of thresholds below the band, the one threshold inside it (or infinity) and the
+// centres on either side of that threshold.  The code is the count plus one comparison.  The product 12.5 |u| is
+// rounded, so a |u| next to a band's edge may land in the neighbouring band: every entry is valid for the band widened
+// by kMagBandSlop on both sides (checked below: still at most one threshold).
+constexpr int kMagBands = 16;
+constexpr float kMagBandsPerUnit = 12.5f, kMagBandSlop = 1e-4f;
 struct EncTables {
   uint32_t mag[2 * kMagEntries];  // {magnitude code, bf16(centre * |u|) as fp32 bits} for pattern kMagTableLo >> 16 + i
   uint32_t spread[256];           // bit j of the index moved to bit 4j + 3
-  constexpr EncTables() : mag{}, spread{} {
+  uint32_t band[4 * kMagBands];   // {thresholds below the band, threshold inside it, centre below it, centre above it}
+  bool bands_ok;
+  constexpr EncTables() : mag{}, spread{}, band{}, bands_ok(true) {
+    for (int k = 0; k < kMagBands; ++k) {
+      const float lo = (float)k / kMagBandsPerUnit - kMagBandSlop, hi = (float)(k + 1) / kMagBandsPerUnit + kMagBandSlop;
+      int below = 0, inside = 0;
+      float th = __builtin_huge_valf();
+      for (int i = 0; i < 7; ++i) {
+        if (kEncThresholds[i] <= lo) ++below;
+        else if (kEncThresholds[i] < hi) ++inside, th = kEncThresholds[i];
+      }
+      if (inside > 1) bands_ok = false;
+      band[4 * k] = (uint32_t)below;
+      band[4 * k + 1] = __builtin_bit_cast(uint32_t, th);
+      band[4 * k + 2] = __builtin_bit_cast(uint32_t, kEncCenters[below]);
+      band[4 * k + 3] = __builtin_bit_cast(uint32_t, kEncCenters[below + (inside ? 1 : 0)]);
+    }
     for (int i = 0; i < kMagEntries; ++i) {
       const float v = __builtin_bit_cast(float, kMagTableLo + ((uint32_t)i << 16));
       int t = 0;
@@ -165,6 +194,7 @@ struct EncTables {
   }
 };
 __device__ __align__(16) const EncTables g_enc_tables = EncTables();
+static_assert(EncTables().bands_ok, "a band of |u| holds two magnitude thresholds");
 
 template <int CTRL>
 __device__ __forceinline__ float enc_dpp(float v) {  // bound_ctrl set, so that the move folds into the add that uses it
@@ -209,6 +239,37 @@ __device__ __forceinline__ float enc_sqrt_bf16(float a) {
     r = sqrtf(a);
   }
   return pkv_bf16_round(r);
+}
+
+// fp32 keys.  a / d as the compiler's own expansion of a correctly rounded division computes it (reciprocal, one
+// Newton step on it, quotient, two residual corrections), without the operand scaling and the special-case fix-up
+// around it: both are the identity while d and a are normal, 1 / d is normal and the quotient and its residuals
+// stay clear of the denormals, which the callers' range checks see to.  The refined reciprocal depends on d alone
+// and is shared by the eight quotients of one key and lane.
+struct EncRcp {
+  float neg_d, y;
+};
+__device__ __forceinline__ EncRcp enc_rcp_refined(float d) {
+  EncRcp r;
+  const float y0 = __builtin_amdgcn_rcpf(d);
+  r.neg_d = -d;
+  r.y = __builtin_fmaf(__builtin_fmaf(r.neg_d, y0, 1.0f), y0, y0);
+  return r;
+}
+__device__ __forceinline__ float enc_div_shared(float a, const EncRcp &r) {
+  float q = a * r.y;
+  q = __builtin_fmaf(__builtin_fmaf(r.neg_d, q, a), r.y, q);
+  return __builtin_fmaf(__builtin_fmaf(r.neg_d, q, a), r.y, q);
+}
+// sqrt(a), correctly rounded, for 2^-90 <= a <= 2^120: the hardware root (1 ulp) moved to a neighbour where the
+// residuals say so, again the compiler's expansion without its scaling of tiny arguments and its special cases.
+__device__ __forceinline__ float enc_sqrt_rn(float a) {
+  const float s = __builtin_amdgcn_sqrtf(a);
+  const float dn = __uint_as_float(__float_as_uint(s) - 1u), up = __uint_as_float(__float_as_uint(s) + 1u);
+  const float r_dn = __builtin_fmaf(-dn, s, a), r_up = __builtin_fmaf(-up, s, a);
+  float r = (0.0f >= r_dn) ? dn : s;
+  r = (0.0f < r_up) ? up : r;
+  return r;
 }
 
 __device__ __forceinline__ float enc_min_abs8(const float (&v)[8]) {
@@ -315,6 +376,86 @@ __device__ __forceinline__ bool enc_key_fast(const uint32_t (&w)[4], const uint3
   return bad;
 }
 
+// The fp32 chain of enc_key_exact in fewer instructions, same bits: the sixteen quotients of a key and lane share
+// two refined reciprocals (enc_div_shared), the roots skip the compiler's range scaling (enc_sqrt_rn), the
+// lane-crossing butterflies take one instruction per value (enc_lane_stages), signs are read off the sign bit and
+// the weight's division is done only near a bf16 rounding boundary.  Sums, products and comparisons are the exact
+// path's own.  xr[] = the lane's eight components as loaded, sg[] = the SRHT signs of its block.  Returns true when
+// this lane's key needs enc_key_exact (norm or radius outside [1e-8, 2^60], or a component of the key or of its
+// rotation below 2^-40 in magnitude, zero included); o is then unspecified.  A zero whose sign differs from the
+// exact path's (the butterflies' negated differences) can only end as a zero of the rotation, which that test sees.
+__device__ __forceinline__ bool enc_key_fast_f32(const float (&xr)[8], const float (&sg)[8], float c1, float c2,
+                                                 float c4, float c8, float scale, bool rerank,
+                                                 const pkv_u32x4 *s_band, const uint32_t *s_spread, EncOut &o) {
+  float x[8];  // components times their SRHT sign (+-1): the sign commutes with the division and its rounding
+#pragma unroll
+  for (int j = 0; j < 8; ++j) x[j] = xr[j] * sg[j];
+  float acc = x[0] * x[0];
+#pragma unroll
+  for (int j = 1; j < 8; ++j) acc = acc + x[j] * x[j];
+  acc = enc_dpp<0xB1>(acc) + acc;   // block ^ 1: lane ^ 1
+  acc = enc_dpp<0x4E>(acc) + acc;   // block ^ 2: lane ^ 2
+  acc = enc_dpp<0x141>(acc) + acc;  // block ^ 4: lane ^ 7 (row_half_mirror)
+  acc = enc_dpp<0x140>(acc) + acc;  // block ^ 8: lane ^ 15 (row_mirror)
+  const float n = enc_sqrt_rn(acc);  // acc outside the root's range gives an n outside the range tested next
+  bool bad = !(n >= 1e-8f) || n > 0x1p60f;
+  bad |= enc_min_abs8(x) < 0x1p-40f;
+  const EncRcp n_rcp = enc_rcp_refined(n);
+  float t[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) t[j] = enc_div_shared(x[j], n_rcp);
+#pragma unroll
+  for (int hh = 1; hh < 8; hh <<= 1) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if ((i & hh) == 0) {
+        const float a = t[i], c = t[i + hh];
+        t[i] = a + c;
+        t[i + hh] = a - c;
+      }
+    }
+  }
+  enc_lane_stages(t, c1, c2, c4, c8);
+  float y[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) y[j] = t[j] * scale;
+  uint32_t sneg = 0;
+#pragma unroll
+  for (int j = 7; j >= 0; --j) sneg = __builtin_amdgcn_alignbit(sneg, __float_as_uint(y[j]), 31);
+  o.code = ~sneg & 0xffu;
+  bad |= enc_min_abs8(y) < 0x1p-40f;
+  if (!rerank) return bad;
+
+  float r2 = y[0] * y[0];
+#pragma unroll
+  for (int j = 1; j < 8; ++j) r2 = r2 + y[j] * y[j];
+  const float r = enc_sqrt_rn(r2);
+  bad |= !(r >= 1e-8f) || r > 0x1p60f;
+  const EncRcp r_rcp = enc_rcp_refined(r);
+  uint32_t mags = 0;
+  float alpha = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float au = fabsf(enc_div_shared(y[j], r_rcp));
+    // 16 bytes per band: floor(200 |u|) without its low four bits = 16 floor(12.5 |u|); the mask also bounds the index
+    const uint32_t band_off = (uint32_t)(au * (16.0f * kMagBandsPerUnit)) & (16u * (kMagBands - 1));
+    const pkv_u32x4 e = *(const pkv_u32x4 *)((const char *)s_band + band_off);
+    const bool above = __uint_as_float(e.y) < au;
+    const uint32_t tc = e.x + (above ? 1u : 0u);
+    mags = __builtin_amdgcn_alignbit(tc, mags, 4);  // the code enters at the top nibble; after 8 steps code j sits in nibble j
+    const float p = __uint_as_float(above ? e.w : e.z) * au;
+    alpha = (j == 0) ? p : alpha + p;
+  }
+  if (alpha < 1e-6f) alpha = 1e-6f;
+  o.packed = (mags & 0x77777777u) | s_spread[o.code];  // bit 3 of nibble j = bit j of the sign code
+  // (r / alpha) * n: both forms are within 2^-22 of the exact value, at most 6 ulp apart; the reciprocal form
+  // decides the bf16 rounding unless it lies within 8 ulp of a rounding boundary
+  float wt = (r * __builtin_amdgcn_rcpf(alpha)) * n;
+  if ((__float_as_uint(wt) & 0xffffu) - 0x7ff8u < 17u) wt = (r / alpha) * n;
+  o.wbits = pkv_f32_to_bf16_bits(wt);
+  return bad;
+}
+
 // ALL: codes, 4-bit records, weights and cluster sizes are all written (the caller's pointers are all set), so the
 // loop body has no branch around a store.  Loads and stores retire through one in-order counter; with a store that
 // may or may not have been issued after the load of the next key, the only safe wait for that key is "everything
@@ -336,10 +477,12 @@ __global__ __launch_bounds__(kEncThreads) __attribute__((amdgpu_waves_per_eu(kEn
   __shared__ uint32_t s_hist[16 * 256];
   __shared__ __align__(16) uint2 s_mag[BF16 ? kMagEntries : 2];
   __shared__ float s_centers[8];  // magnitude centres, looked up by code (an LDS read instead of a load from constant memory)
-  __shared__ uint32_t s_spread[BF16 ? 256 : 1];
+  __shared__ uint32_t s_spread[256];
+  __shared__ __align__(16) pkv_u32x4 s_band[BF16 ? 1 : kMagBands];
   if (tid < 8) s_centers[tid] = c_centers[tid];
+  if (!BF16 && tid < kMagBands) s_band[tid] = ((const pkv_u32x4 *)g_enc_tables.band)[tid];
+  if (tid < 256) s_spread[tid] = g_enc_tables.spread[tid];
   if (BF16) {
-    if (tid < 256) s_spread[tid] = g_enc_tables.spread[tid];
     const pkv_u32x4 *src = (const pkv_u32x4 *)g_enc_tables.mag;
 #pragma unroll
     for (int i = 0; i < kMagEntries / 2 / kEncThreads; ++i)
@@ -383,6 +526,7 @@ __global__ __launch_bounds__(kEncThreads) __attribute__((amdgpu_waves_per_eu(kEn
   // depth.)  Loads are never skipped - past the block's end they fetch its last iteration again - because a load that
   // may or may not have been issued makes every later wait of the in-order counter a wait for everything.
   constexpr int kW = BF16 ? 1 : 2;  // 16-byte words per lane and key
+  constexpr int kEncAhead = BF16 ? kEncAheadBf16 : kEncAheadF32;
   const int n_iter = last / kEncKeysPerIter + 1;
   pkv_u32x4 raw[kEncAhead][kW];
   auto load_iter = [&](int it, pkv_u32x4 (&reg)[kW]) {
@@ -420,6 +564,7 @@ __global__ __launch_bounds__(kEncThreads) __attribute__((amdgpu_waves_per_eu(kEn
         x[j] = __uint_as_float(cur[0][j]);
         x[4 + j] = __uint_as_float(cur[kW - 1][j]);
       }
+      exact = __builtin_amdgcn_ballot_w64(enc_key_fast_f32(x, sg, c1, c2, c4, c8, scale, rerank, s_band, s_spread, o)) != 0;
     }
     if (exact) {  // the whole wave: every lane takes part in the shuffles
       if (BF16) {  // rare: the signs are fetched again instead of being held in registers across the loop

@@ -111,8 +111,8 @@ def test_encode_ragged_block_stays_inside_its_keys(ops, S):
     assert bool((rec[0, 0] == 0xAB).all()) and bool((rec[0, 1, S:] == 0xAB).all()) and bool((rec[0, 1, :, 96:] == 0xAB).all())
 
 
-def _adversarial_bf16_keys(n, seed):
-    """bf16 keys that stress every rounding decision of the encoder: magnitudes from 2^-30 to 2^30, outlier dims,
+def _adversarial_keys(n, seed, bf16=True):
+    """Keys that stress every rounding decision of the encoder: magnitudes from 2^-30 to 2^30, outlier dims,
     exact zeros and components far below the norm, powers of two, one-hot and constant vectors, tiny norms."""
     rng = np.random.default_rng(seed)
     k = rng.standard_normal((n, 128)).astype(np.float32)
@@ -129,7 +129,12 @@ def _adversarial_bf16_keys(n, seed):
     k[kind == 12] *= 1e-9                                                                                      # norm below the 1e-8 clamp
     k[kind == 13] = np.round(k[kind == 13] * 4.0) / 4.0                                                        # many exact ties and zeros
     k[kind == 14] *= 3e-8                                                                                      # norm just above the clamp
-    return O.bf16_round(k.astype(np.float32))
+    k = k.astype(np.float32)
+    return O.bf16_round(k) if bf16 else k
+
+
+def _adversarial_bf16_keys(n, seed):
+    return _adversarial_keys(n, seed, True)
 
 
 def test_encode_bf16_bit_exact_on_adversarial_keys(ops):
@@ -148,6 +153,36 @@ def test_encode_bf16_bit_exact_on_adversarial_keys(ops):
         codes, nib, w = O.encode(keys[0, h], signs, O.BF16)
         bad = np.where((cb[0, h].cpu().numpy().T != codes).any(axis=1))[0]
         assert bad.size == 0, f"codes differ at keys {bad[:8]} (kinds {bad[:8] % 16})"
+        bad = np.where((k4[0, h].cpu().numpy().transpose(1, 0, 2) != nib).any(axis=(1, 2)))[0]
+        assert bad.size == 0, f"4-bit codes differ at keys {bad[:8]} (kinds {bad[:8] % 16})"
+        got_w = kw[0, h].float().cpu().numpy().T
+        bad = np.where((got_w.view(np.uint32) != w.astype(np.float32).view(np.uint32)).any(axis=1))[0]
+        assert bad.size == 0, f"weights differ at keys {bad[:8]} (kinds {bad[:8] % 16})"
+        assert np.array_equal(cc[0, h].cpu().numpy(), O.count_cluster_keys(codes))
+
+
+def test_encode_f32_bit_exact_on_adversarial_keys(ops):
+    """The fp32 encoder shares one refined reciprocal among the quotients of a denominator and leaves out the range
+    scaling of divisions and roots inside a checked range, falling back to the plain correctly rounded operations per
+    wave elsewhere; both routes must equal the oracle bit for bit."""
+    H, S = 4, 16384 + 5
+    signs = O.srht_signs(42)
+    keys = np.stack([_adversarial_keys(S, 900 + h, bf16=False) for h in range(H)]).reshape(1, H, S, 128)
+    keys[0, 1] *= np.float32(2.0) ** np.random.default_rng(3).integers(-70, 50, size=(S, 1)).astype(np.float32)  # beyond the checked range too
+    _say(f"encode adversarial fp32 keys {keys.shape}")
+    tk = torch.from_numpy(keys).to(DEV)
+    _, _, _, cb, k4, kw = ops.alloc_keymajor(1, H, S, DEV)
+    cc = torch.zeros(1, H, 16, 256, dtype=torch.int32, device=DEV)
+    ops.encode_append(tk, torch.from_numpy(signs).to(DEV), cb, k4, kw, cc)
+    cb2 = torch.zeros(1, H, 16, S, dtype=torch.uint8, device=DEV)
+    ops.encode_append(tk, torch.from_numpy(signs).to(DEV), cb2, None, None, None)  # codes only: the other kernel form
+    torch.cuda.synchronize()
+    for h in range(H):
+        codes, nib, w = O.encode(keys[0, h], signs, O.F32)
+        bad = np.where((cb[0, h].cpu().numpy().T != codes).any(axis=1))[0]
+        assert bad.size == 0, f"codes differ at keys {bad[:8]} (kinds {bad[:8] % 16})"
+        bad = np.where((cb2[0, h].cpu().numpy().T != codes).any(axis=1))[0]
+        assert bad.size == 0, f"codes of the codes-only form differ at keys {bad[:8]} (kinds {bad[:8] % 16})"
         bad = np.where((k4[0, h].cpu().numpy().transpose(1, 0, 2) != nib).any(axis=(1, 2)))[0]
         assert bad.size == 0, f"4-bit codes differ at keys {bad[:8]} (kinds {bad[:8] % 16})"
         got_w = kw[0, h].float().cpu().numpy().T
