@@ -304,3 +304,91 @@ def test_one_instruction_butterfly_stages_carry_only_a_sign(oracle):
         nz = want != 0                                                        # zeros take the kernel's exact path
         assert np.array_equal(got[nz].view(np.uint32), want[nz].view(np.uint32)), trial
         assert np.all(got[~nz] == 0)
+
+
+def _rn32(fr):
+    """A rational rounded to the nearest float32 (ties to even), as a Fraction; normal range only."""
+    from fractions import Fraction
+    if fr == 0:
+        return Fraction(0)
+    sign, a = (-1 if fr < 0 else 1), abs(fr)
+    e = a.numerator.bit_length() - a.denominator.bit_length()
+    if Fraction(2) ** e > a:
+        e -= 1                                            # 2^e <= a < 2^(e+1)
+    q = a / Fraction(2) ** (e - 23)                       # in [2^23, 2^24)
+    n = q.numerator // q.denominator
+    rem = q - n
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and n & 1):
+        n += 1
+    return sign * n * Fraction(2) ** (e - 23)
+
+
+def test_shared_reciprocal_division_and_unscaled_root_are_correctly_rounded():
+    """What the GPU encoder's fp32 chain rests on, in exact rational arithmetic: from ANY reciprocal estimate within
+    one ulp, one Newton step and two residual corrections (each a fused multiply-add, rounded once) give the
+    correctly rounded quotient, and the hardware root (within one ulp) moved by the signs of two residuals gives the
+    correctly rounded root.  The refined reciprocal depends on the denominator alone, so eight quotients share it."""
+    from fractions import Fraction
+    rng = np.random.default_rng(11)
+    F = lambda v: Fraction(float(v))
+    fma = lambda a, b, c: _rn32(a * b + c)
+    ulp = lambda v: Fraction(2) ** ((v.numerator.bit_length() - v.denominator.bit_length() - (Fraction(2) ** (v.numerator.bit_length() - v.denominator.bit_length()) > v)) - 23)
+    dens = np.concatenate([rng.uniform(1.0, 2.0, 300), [1.0, 1.5, 2.0 - 2.0 ** -23, 1.0 + 2.0 ** -23]]).astype(np.float32)
+    for d32 in dens:
+        d = F(d32) * Fraction(2) ** int(rng.integers(-20, 40))
+        for off in (-1, 0, 1):                            # the reciprocal instruction: anything within one ulp
+            y0 = _rn32(1 / d)
+            y0 = y0 + off * ulp(y0)
+            y = fma(fma(-d, y0, Fraction(1)), y0, y0)
+            for a32 in rng.uniform(-2.0, 2.0, 6).astype(np.float32):
+                a = F(a32) * Fraction(2) ** int(rng.integers(-30, 30))
+                q = _rn32(a * y)
+                q = fma(fma(-d, q, a), y, q)
+                q = fma(fma(-d, q, a), y, q)
+                assert q == _rn32(a / d), (float(a), float(d), off)
+    for a32 in np.concatenate([rng.uniform(1.0, 4.0, 600), [1.0, 2.0, 4.0 - 2.0 ** -22, 1.0 + 2.0 ** -23]]).astype(np.float32):
+        a = F(a32) * Fraction(4) ** int(rng.integers(-20, 30))
+        root = F(np.sqrt(np.float64(float(a))))           # double: far closer than the decisions below need
+        want = _rn32(root)
+        assert (want - ulp(want) / 2) ** 2 < a < (want + ulp(want) / 2) ** 2 or want ** 2 == a
+        prv, nxt = (lambda v: v - ulp(v - ulp(v) / 2)), (lambda v: v + ulp(v))  # the neighbouring floats (bit pattern -1 / +1)
+        for s in (prv(want), want, nxt(want)):
+            off = float(s - want)
+            dn, up = prv(s), nxt(s)
+            r_dn, r_up = fma(-dn, s, a), fma(-up, s, a)
+            r = dn if r_dn <= 0 else s
+            r = up if r_up > 0 else r
+            assert r == want, (float(a), off)
+
+
+def test_banded_magnitude_table_counts_thresholds(oracle):
+    """The fp32 encoder's magnitude code: entry floor(12.5 |u|) of a 16-entry table names the thresholds below its
+    band of width 0.08, the one threshold inside and the centres either side; code = count + (threshold < |u|).
+    Simulated in float32 (the index is floor(200 |u|) with its low four bits cleared, the product rounded as the
+    GPU rounds it) against the plain count, on every float32 within 3000 ulp of a band edge or a threshold and on a
+    random sample."""
+    thr, cen = oracle.mag_constants()
+    thr, cen = thr.astype(np.float32), cen.astype(np.float32)
+    slop = 1e-4
+    below, inside_thr, c_lo, c_hi = [], [], [], []
+    for k in range(16):
+        lo, hi = np.float32(k) / np.float32(12.5) - np.float32(slop), np.float32(k + 1) / np.float32(12.5) + np.float32(slop)
+        b = int((thr <= lo).sum())
+        ins = thr[(thr > lo) & (thr < hi)]
+        assert ins.size <= 1, k
+        below.append(b)
+        inside_thr.append(ins[0] if ins.size else np.float32(np.inf))
+        c_lo.append(cen[b])
+        c_hi.append(cen[b + (1 if ins.size else 0)])
+    below, inside_thr, c_lo, c_hi = map(np.asarray, (below, inside_thr, c_lo, c_hi))
+    rng = np.random.default_rng(5)
+    anchors = np.concatenate([np.arange(1, 14, dtype=np.float32) / np.float32(12.5), thr, [np.float32(1.0)]]).astype(np.float32)
+    near = (anchors.view(np.uint32)[:, None] + np.arange(-3000, 3001)[None, :]).astype(np.uint32).view(np.float32).ravel()
+    au = np.concatenate([near, rng.uniform(0, 1.0000005, 200000).astype(np.float32), np.float32([0.0, 1e-30, 1.0000001])])
+    au = au[au <= np.float32(1.001)]
+    idx = ((au * np.float32(200.0)).astype(np.float32).astype(np.uint32) & 0xF0) >> 4
+    above = inside_thr[idx] < au
+    code = below[idx] + above
+    want = (thr[None, :] < au[:, None]).sum(axis=1)
+    assert np.array_equal(code, want)
+    assert np.array_equal(np.where(above, c_hi[idx], c_lo[idx]), cen[want])
