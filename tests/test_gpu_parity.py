@@ -85,23 +85,24 @@ def test_encode_append_bit_exact(ops, dtype, layout):
     assert torch.equal(cc2, cc)
 
 
+@pytest.mark.parametrize("dtype", [O.BF16, O.F32])
 @pytest.mark.parametrize("S", [1, 15, 16, 17, 255, 256, 257, 300])
-def test_encode_ragged_block_stays_inside_its_keys(ops, S):
+def test_encode_ragged_block_stays_inside_its_keys(ops, S, dtype):
     """The lanes past the end of a ragged block repeat its last key's stores: nothing beyond key S - 1 may change, and
     the cluster sizes count every key once."""
-    _say(f"encode ragged S={S}")
+    _say(f"encode ragged S={S} dtype={dtype}")
     cap = S + 40
     signs = O.srht_signs(42)
-    keys = O.synth_keys(S, 31 + S, bf16=True).reshape(1, 1, S, 128)
+    keys = O.synth_keys(S, 31 + S, bf16=dtype == O.BF16).reshape(1, 1, S, 128)
     codes_km, nib_km, w_km, cb, k4, kw = ops.alloc_keymajor(1, 2, cap, DEV)
     rec = nib_km.as_strided((1, 2, cap, 128), nib_km.stride(), nib_km.storage_offset())  # the whole 128-byte records
     codes_km.fill_(0xAB)
     rec.fill_(0xAB)
     cc = torch.zeros(1, 2, 16, 256, dtype=torch.int32, device=DEV)
-    tk = torch.from_numpy(keys).to(torch.bfloat16).to(DEV)
+    tk = torch.from_numpy(keys).to(torch.bfloat16 if dtype == O.BF16 else torch.float32).to(DEV)
     ops.encode_append(tk, torch.from_numpy(signs).to(DEV), cb[:, 1:, :, :S], k4[:, 1:, :, :S], kw[:, 1:, :, :S], cc[:, 1:])
     torch.cuda.synchronize()
-    codes, nib, w = O.encode(keys[0, 0], signs, O.BF16)
+    codes, nib, w = O.encode(keys[0, 0], signs, dtype)
     assert np.array_equal(cb[0, 1, :, :S].cpu().numpy().T, codes)
     assert np.array_equal(k4[0, 1, :, :S].cpu().numpy().transpose(1, 0, 2), nib)
     assert np.array_equal(kw[0, 1, :, :S].float().cpu().numpy().T, w)
