@@ -365,7 +365,7 @@ def encoder_leg(torch, ops, dev, shapes=((8, 8, 65536, "bf16"), (1, 8, 131072, "
                     f"GBps_over_{nbytes}B_per_key_head": round(kh * nbytes / us / 1e3, 1),
                     "hbm_fraction": round(kh * nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)})
         del kb, cb, k4, kw, cc
-    return {"kernel": "pkv_encode_kernel", "bound": "between vector issue (about 225 instructions per key and 16-lane group for bf16 keys, 295 for fp32 keys) and the memory system",
+    return {"kernel": "pkv_encode_kernel", "bound": "between vector issue (about 225 instructions per key and 16-lane group for bf16 keys, 345 for fp32 keys) and the memory system",
             "shapes": out}
 
 

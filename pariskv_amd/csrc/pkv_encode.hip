@@ -27,10 +27,10 @@
 // quarter fewer gained 5 %; without the record stores it takes 90, without any
 // store and without the histogram 70 us per 2^20 keys, with everything 120 - 126.
 // enc_key_exact is the chain as written (correctly rounded divisions and roots,
-// about 580 vector instructions per lane and key).  bf16 keys take enc_key_fast
+// about 660 vector instructions per lane and key).  bf16 keys take enc_key_fast
 // (about 225), which reaches the same bits through reciprocals, a table for the
 // magnitude code and its term of the weight, and lane-crossing butterflies of
-// one instruction per value; fp32 keys take enc_key_fast_f32 (about 295): the
+// one instruction per value; fp32 keys take enc_key_fast_f32 (about 345): the
 // compiler's own division sequence with the reciprocal refinement shared by the
 // eight quotients of a denominator and without its range scaling, the same
 // butterflies, and a small banded table for the magnitude code.  Either hands a
